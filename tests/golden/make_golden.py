@@ -1,0 +1,145 @@
+"""Writes tests/golden/golden.json (+ c1_recv.bin) by running the REAL reference functions.
+
+Runs only in the build container: it needs oracle/_ref/ref_driver (`make -C oracle ref`, which
+compiles the reference's sources from /root/reference with the image's MPICH) and mpiexec.
+Each case regenerates its inputs from a seed through rbruck_alltoallv_amd.workloads, hands the
+count matrix to `mpiexec -n P ref_driver ...` and records the per-rank FNV-1a digests of the
+receive blocks the reference produced (and, for the P=8 plumbing case, every byte of every
+rank's recvbuf).  The fixtures are data only; the tests rebuild the same inputs from the same
+seeds and never need the reference again.
+
+    python tests/golden/make_golden.py
+"""
+from __future__ import annotations
+
+import json
+import os
+import subprocess
+import sys
+import tempfile
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
+sys.path.insert(0, ROOT)
+from rbruck_alltoallv_amd import workloads as W  # noqa: E402
+
+DRIVER = os.path.join(ROOT, "oracle", "_ref", "ref_driver")
+MPIEXEC = "/opt/conda/bin/mpiexec"
+HERE = os.path.dirname(os.path.abspath(__file__))
+
+
+def counts_for(spec: dict) -> np.ndarray:
+    kind = spec["kind"]
+    if kind == "uniform_random":
+        c = W.counts_uniform_random(spec["P"], spec["hi"], spec["seed"])
+    elif kind == "zipf":
+        c = W.counts_zipf(spec["P"], spec["max"], 1.2, 5, spec["seed"])
+    elif kind == "normal":
+        c = W.counts_normal(spec["P"], spec["mean"], spec["sd"], 0, spec["hi"], spec["seed"])
+    elif kind == "fft":
+        c = W.counts_fft_rows(spec["P"], spec["row_len"], spec["count"])
+    elif kind == "zeros":
+        c = np.zeros((spec["P"], spec["P"]), dtype=np.int32)
+    else:
+        raise ValueError(kind)
+    if spec.get("sparsify"):
+        c = c.copy()
+        c[c % spec["sparsify"] == 0] = 0
+    return c
+
+
+def cases() -> list[dict]:
+    out = []
+
+    def add(cid, func, counts, esz, r=2, b=0, n=0, bblock=0, layout=0, payload=W.PAYLOAD_HASH, seed=1, count=0):
+        out.append(dict(id=cid, func=func, counts=counts, esz=esz, r=r, b=b, n=n, bblock=bblock, layout=layout,
+                        payload=payload, seed=seed, count=count))
+
+    c1 = dict(kind="uniform_random", P=8, hi=64, seed=0)
+    for f in ("twophase", "om", "tuna"):
+        add(f"C1-{f}", f, c1, 4, r=2, b=1, payload=W.PAYLOAD_SELFDESC32)
+    for f in ("ttpl", "ttpl_s1"):
+        add(f"C1-{f}", f, c1, 4, r=2, n=4, payload=W.PAYLOAD_SELFDESC32)
+    c2 = dict(kind="uniform_random", P=64, hi=256, seed=0)
+    for r in (2, 4, 8):
+        for f in ("twophase", "om", "tuna"):
+            add(f"C2s-{f}-r{r}", f, c2, 1, r=r, b=2)
+    c3 = dict(kind="zipf", P=64, max=2048, seed=0)
+    for f in ("twophase", "om", "tuna"):
+        add(f"C3s-{f}-r16", f, c3, 4, r=16, b=0)
+    c4 = dict(kind="normal", P=128, mean=64.0, sd=16.0, hi=256, seed=0)
+    add("C4s-ttpl", "ttpl", c4, 1, r=32, n=32, bblock=0)
+    add("C4s-ttpl-b3", "ttpl", c4, 1, r=32, n=32, bblock=3)
+    add("C4s-ttpl_s1", "ttpl_s1", c4, 1, r=32, n=32, bblock=0)
+    add("C4s-ttpl_s1-r4", "ttpl_s1", c4, 1, r=4, n=32, bblock=40)
+    add("C4s-ttpl-r2", "ttpl", c4, 1, r=2, n=32, bblock=0)
+    c5 = dict(kind="fft", P=64, row_len=8, count=96)
+    for r in (2, 8, 32, 64):
+        add(f"C5s-tuna-r{r}", "tuna", c5, 8, r=r, b=0)
+    add("C5s-tuna-r8-b1", "tuna", c5, 8, r=8, b=1)
+    # odd sizes, gaps, zeros
+    for P, r in ((12, 3), (17, 5), (27, 3), (7, 7), (49, 7), (5, 99)):
+        cg = dict(kind="uniform_random", P=P, hi=9, seed=P, sparsify=4)
+        for f in ("twophase", "om", "tuna"):
+            add(f"odd-P{P}-{f}-r{r}", f, cg, 2, r=r, b=3, layout=1)
+    for P, n, r in ((12, 4, 2), (12, 3, 3), (27, 9, 3), (16, 8, 3), (16, 16, 4)):
+        cg = dict(kind="uniform_random", P=P, hi=9, seed=P, sparsify=5)
+        add(f"odd-P{P}-n{n}-ttpl-r{r}", "ttpl", cg, 2, r=r, n=n, bblock=2, layout=1)
+        add(f"odd-P{P}-n{n}-ttpl_s1-r{r}", "ttpl_s1", cg, 2, r=r, n=n, bblock=5, layout=1)
+    zz = dict(kind="zeros", P=8)
+    for f in ("twophase", "om", "tuna"):
+        add(f"zeros-{f}", f, zz, 4, r=2, b=1)
+    add("zeros-ttpl", "ttpl", zz, 4, r=2, n=4)
+    add("zeros-ttpl_s1", "ttpl_s1", zz, 4, r=2, n=4)
+    # uniform two-layer functions
+    for P, n, r in ((16, 4, 2), (16, 4, 3), (16, 4, 4), (12, 3, 2), (64, 8, 4), (64, 16, 3)):
+        add(f"uni-spread-P{P}-n{n}-r{r}", "uniform_spreadout", None, 4, r=r, n=n, count=5)
+        add(f"uni-isplit-P{P}-n{n}-r{r}", "uniform_isplit", None, 4, r=r, n=n, count=5)
+    return out
+
+
+def run_case(case: dict, tmp: str) -> dict:
+    uniform = case["func"].startswith("uniform")
+    if uniform:
+        P = int(case["id"].split("-P")[1].split("-")[0])
+        counts_arg = str(case["count"])
+    else:
+        counts = counts_for(case["counts"])
+        P = counts.shape[0]
+        counts_arg = os.path.join(tmp, "counts.bin")
+        counts.astype("<i4").tofile(counts_arg)
+    outp = os.path.join(tmp, "out")
+    cmd = [MPIEXEC, "-n", str(P), DRIVER, case["func"], counts_arg, str(case["esz"]), str(case["r"]), str(case["b"]),
+           str(case["n"]), str(case["bblock"]), str(case["layout"]), str(case["payload"]), str(case["seed"]), "1", outp]
+    res = subprocess.run(cmd, capture_output=True, text=True, timeout=600)
+    line = res.stdout.strip().splitlines()[-1] if res.stdout.strip() else ""
+    if res.returncode != 0:
+        raise RuntimeError(f"{case['id']}: reference run failed ({res.returncode}): {line} {res.stderr[-400:]}")
+    digests = open(outp + ".digests").read().split()
+    rec = dict(case)
+    rec["P"] = P
+    rec["digests"] = digests
+    rec["reference_says"] = line
+    if case["id"] == "C1-twophase":
+        os.replace(outp + ".recv.bin", os.path.join(HERE, "c1_recv.bin"))
+    return rec
+
+
+def main() -> None:
+    if not os.path.exists(DRIVER):
+        raise SystemExit("build the reference driver first: make -C oracle ref")
+    recs = []
+    with tempfile.TemporaryDirectory() as tmp:
+        for case in cases():
+            rec = run_case(case, tmp)
+            print(rec["id"], rec["reference_says"], flush=True)
+            recs.append(rec)
+    with open(os.path.join(HERE, "golden.json"), "w") as f:
+        json.dump({"made_by": "tests/golden/make_golden.py", "mpi": "MPICH 3.3.2 (/opt/conda), mpiexec -n P, oversubscribed on 8 cores",
+                   "cases": recs}, f, indent=1)
+    print(f"{len(recs)} cases written")
+
+
+if __name__ == "__main__":
+    main()

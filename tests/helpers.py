@@ -1,0 +1,82 @@
+"""Shared by the CPU and GPU tests: rebuild a golden case's inputs and run one function on the oracle."""
+from __future__ import annotations
+
+import json
+import os
+
+import numpy as np
+
+from rbruck_alltoallv_amd import workloads as W
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+GOLDEN_DIR = os.path.join(ROOT, "tests", "golden")
+
+
+def load_golden() -> list[dict]:
+    with open(os.path.join(GOLDEN_DIR, "golden.json")) as f:
+        return json.load(f)["cases"]
+
+
+def counts_for(spec: dict) -> np.ndarray:
+    kind = spec["kind"]
+    if kind == "uniform_random":
+        c = W.counts_uniform_random(spec["P"], spec["hi"], spec["seed"])
+    elif kind == "zipf":
+        c = W.counts_zipf(spec["P"], spec["max"], 1.2, 5, spec["seed"])
+    elif kind == "normal":
+        c = W.counts_normal(spec["P"], spec["mean"], spec["sd"], 0, spec["hi"], spec["seed"])
+    elif kind == "fft":
+        c = W.counts_fft_rows(spec["P"], spec["row_len"], spec["count"])
+    elif kind == "zeros":
+        c = np.zeros((spec["P"], spec["P"]), dtype=np.int32)
+    else:
+        raise ValueError(kind)
+    if spec.get("sparsify"):
+        c = c.copy()
+        c[c % spec["sparsify"] == 0] = 0
+    return c
+
+
+def problem_for_case(case: dict) -> W.Problem:
+    """The inputs tests/golden/make_golden.py gave the reference for this case."""
+    if case["func"].startswith("uniform"):
+        return W.make_uniform_problem(case["P"], case["count"], case["esz"])
+    counts = counts_for(case["counts"])
+    recv_layout = 0 if case["func"] == "ttpl" else case["layout"]
+    return W.make_problem(counts, case["esz"], case["layout"], recv_layout)
+
+
+def run_on(backend, case: dict, prob: W.Problem, send, recv) -> int:
+    """Dispatch one golden case to a backend exposing the reference's function names
+    (oracle.oracle_py on numpy arenas, or the GPU package on device arenas)."""
+    f = case["func"]
+    if f == "twophase":
+        return backend.twophase_rbruck_alltoallv(case["r"], prob, send, recv)
+    if f == "om":
+        return backend.twophase_rbruck_alltoallv_om(case["r"], prob, send, recv)
+    if f == "tuna":
+        return backend.tuna_algorithm(case["r"], case["b"], prob, send, recv)
+    if f == "ttpl":
+        return backend.TTPL_BT_alltoallv(case["n"], case["r"], case["bblock"], prob, send, recv)
+    if f == "ttpl_s1":
+        return backend.TTPL_BT_alltoallv_s1(case["n"], case["r"], case["bblock"], prob, send, recv)
+    if f == "uniform_spreadout":
+        return backend.uniform_spreadout_twolayer(case["n"], case["r"], prob, case["count"], send, recv)
+    if f == "uniform_isplit":
+        return backend.uniform_inverse_isplit_r_bruck(case["n"], case["r"], case["b"], prob, case["count"], send, recv)
+    raise ValueError(f)
+
+
+def fnv1a64_blocks(prob: W.Problem, recv: np.ndarray) -> list[str]:
+    """Per-rank FNV-1a 64 over the receive blocks in source order (numpy restatement of the digest the
+    MPI driver around the reference wrote)."""
+    out = []
+    for t in range(prob.P):
+        h = 0xCBF29CE484222325
+        for s in range(prob.P):
+            nb = int(prob.recvcounts[t, s]) * prob.esz
+            at = int(prob.rbase[t]) + int(prob.rdispls[t, s]) * prob.esz
+            for byte in recv[at:at + nb].tolist():
+                h = ((h ^ byte) * 0x100000001B3) & 0xFFFFFFFFFFFFFFFF
+        out.append(f"{h:016x}")
+    return out
