@@ -1,0 +1,157 @@
+/*
+ * rbruck_vc.h — C ABI of the MI355X-native radix-r Bruck alltoallv library
+ * (librbruck_vc.so): the alltoallv data path of KokoFan16/rbruck_alltoallv for
+ * a VIRTUAL COMMUNICATOR of P ranks whose send, receive and staging buffers all
+ * live in the HBM of one GPU.
+ *
+ * The collective entry points keep the reference's names and argument order
+ * (src/rbruckv.h).  Three things change, uniformly:
+ *   - one call serves all P ranks.  `sendbuf` / `recvbuf` are DEVICE pointers
+ *     to arenas; rank p's buffer starts at sbase[p] / rbase[p] bytes into them
+ *     (vc_comm_set_bases).  `sendcounts`, `sdispls`, `recvcounts`, `rdispls`
+ *     are DEVICE pointers to [P][P] row-major int32 tables whose row p is the
+ *     array rank p would have passed; units are elements, as in the reference;
+ *   - MPI_Datatype becomes the element size in bytes (the reference only ever
+ *     calls MPI_Type_size on it, src/twophase_tunable_rbruckv.cpp:28; the
+ *     receive type is ignored there and here);
+ *   - MPI_Comm becomes a vc_comm_t handle.
+ * Calls are blocking like the reference's: the result is in `recvbuf` when the
+ * function returns (the comm's stream has been synchronised).
+ *
+ * Return codes: 0 success; -1 radix < 2 where the reference returns -1;
+ * further negative codes below for conditions under which the reference hangs,
+ * aborts or overflows.
+ */
+#ifndef RBRUCK_VC_H_
+#define RBRUCK_VC_H_
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct vc_comm *vc_comm_t;
+
+#define VC_OK 0
+#define VC_ERR_RADIX (-1)      /* r < 2 (src/twophase_tunable_rbruckv.cpp:16, twophase_twolayer_rbruck.cpp:242,472) */
+#define VC_ERR_GROUP (-2)      /* n does not divide P (the reference truncates P/n and hangs), or n >= P for the uniform functions (MPI_Abort, src/twolayer_rbruck.cpp:18-22) */
+#define VC_ERR_TOO_FEW_RANKS (-3) /* tuna_algorithm with P < 3 (src/tuna.cpp:20,28 never returns) */
+#define VC_ERR_HIP (-4)        /* a HIP runtime call failed; vc_last_error_string() says which */
+#define VC_ERR_ARG (-5)        /* null handle / pointer, element size < 1, bases not set */
+#define VC_ERR_NO_DEVICE (-6)  /* no HIP device */
+
+/* ---- communicator (replaces MPI_Comm; MPI_Comm_size/MPI_Comm_rank have no per-rank analogue) ---- */
+
+/* Creates a virtual communicator of `nranks` ranks on the current HIP device. */
+int vc_comm_create(int nranks, vc_comm_t *comm_out);
+int vc_comm_free(vc_comm_t comm);
+int vc_comm_size(vc_comm_t comm);
+
+/* Stream every kernel of this communicator is launched on (a hipStream_t; NULL = the default stream). */
+int vc_comm_set_stream(vc_comm_t comm, void *hip_stream);
+
+/* Where each rank's buffers start inside the arenas: two DEVICE arrays of P int64 byte offsets.  They are
+ * read on the device at every call (not copied), so they must stay valid.  Required before any collective. */
+int vc_comm_set_bases(vc_comm_t comm, const int64_t *sbase_bytes, const int64_t *rbase_bytes);
+
+/* Text of the most recent failure on this thread ("" if none). */
+const char *vc_last_error_string(void);
+
+/* ---- caller-side steps of the reference drivers, as kernels ---- */
+
+/* MPI_Alltoall of one int per pair (examples/rbruckv_example.cpp:76): recvcounts[t][s] = sendcounts[s][t].
+ * LDS-tiled P x P transpose. */
+int vc_alltoall_counts(const int *sendcounts, int *recvcounts, vc_comm_t comm);
+
+/* Exclusive prefix sum of every rank's counts (examples/rbruckv_example.cpp:69-72,77-82): displs[p][i] =
+ * sum_{k<i} counts[p][k].  extent_out (may be NULL) receives each rank's total, P int64 elements. */
+int vc_displs_from_counts(const int *counts, int *displs, int64_t *extent_out, vc_comm_t comm);
+
+/* Packed arena bases: base[p] = sum_{q<p} roundup(extent[q] * elem_size, align); total_out (device, 1 int64,
+ * may be NULL) receives the arena size in bytes. */
+int vc_bases_from_extents(const int64_t *extent, int elem_size, int64_t align, int64_t *base_out, int64_t *total_out,
+                          vc_comm_t comm);
+
+/* The reference's MPI_Allreduce(MAX) of the block length (src/twophase_tunable_rbruckv.cpp:40-44): max_out is
+ * one device int.  Kept for interface parity; the GPU path sizes its staging by prefix sums instead. */
+int vc_allreduce_max_count(const int *sendcounts, int *max_out, vc_comm_t comm);
+
+/* ---- the alltoallv family (reference: src/rbruckv.h:24-26, 84-96, 39-45, 28-33) ---- */
+
+/* src/twophase_tunable_rbruckv.cpp:13-152 — radix-r Bruck, most significant digit first. */
+int twophase_rbruck_alltoallv(int r, char *sendbuf, int *sendcounts, int *sdispls, int sendtype_size, char *recvbuf,
+                              int *recvcounts, int *rdispls, int recvtype_size, vc_comm_t comm);
+
+/* src/twophase_tunable_rbruckv-om.cpp:10-157 — least significant digit first; single-block rounds go straight
+ * from sendbuf to recvbuf. */
+int twophase_rbruck_alltoallv_om(int r, char *sendbuf, int *sendcounts, int *sdispls, int sendtype_size, char *recvbuf,
+                                 int *recvcounts, int *rdispls, int recvtype_size, vc_comm_t comm);
+
+/* src/tuna.cpp:10-177 — as _om with r clamped to [2, P-1] and b rounds of a digit in flight together
+ * (here: b rounds per kernel launch; b <= 0 or b > P means all of them). */
+int tuna_algorithm(int r, int b, char *sendbuf, int *sendcounts, int *sdispls, int sendtype_size, char *recvbuf,
+                   int *recvcounts, int *rdispls, int recvtype_size, vc_comm_t comm);
+
+/* src/twophase_twolayer_rbruck.cpp:237-463 — two-layer, coalesced inter-node messages, bblock groups in flight.
+ * Like the reference it ignores rdispls: rank t's blocks land back to back in source-rank order. */
+int TTPL_BT_alltoallv(int n, int r, int bblock, char *sendbuf, int *sendcounts, int *sdispls, int sendtype_size,
+                      char *recvbuf, int *recvcounts, int *rdispls, int recvtype_size, vc_comm_t comm);
+
+/* src/twophase_twolayer_rbruck.cpp:467-681 — two-layer, one inter-node message per block ("staggered"),
+ * bblock of them in flight; honours rdispls. */
+int TTPL_BT_alltoallv_s1(int n, int r, int bblock, char *sendbuf, int *sendcounts, int *sdispls, int sendtype_size,
+                         char *recvbuf, int *recvcounts, int *rdispls, int recvtype_size, vc_comm_t comm);
+
+/* src/twolayer_rbruck.cpp:10-134 — equal blocks of sendcount elements; rank p's buffers hold P blocks.
+ * The reference scrambles sendbuf (and needs recvbuf[0..P) free of '1' bytes); this one leaves sendbuf intact. */
+int uniform_spreadout_twolayer(int n, int r, char *sendbuf, int sendcount, int sendtype_size, char *recvbuf,
+                               int recvcount, int recvtype_size, vc_comm_t comm);
+
+/* src/twolayer_rbruck.cpp:137-277 — as above with a group-level Bruck whose radix the reference forces to the
+ * number of groups (:158), i.e. one digit of direct rounds.  The reference returns void; this returns a code. */
+int uniform_inverse_isplit_r_bruck(int n, int r1, int r2, char *sendbuf, int sendcount, int sendtype_size,
+                                   char *recvbuf, int recvcount, int recvtype_size, vc_comm_t comm);
+
+/* ---- measurement and inspection (the reference's global phase timers, src/rbruckv.h:13-18) ---- */
+
+#define VC_MAX_LAUNCHES 1024
+
+typedef struct {
+    int32_t n_launches;          /* data-moving kernel launches of the last call */
+    int32_t n_digits;            /* digit phases among them */
+    int64_t payload_bytes;       /* S: sum of all blocks */
+    int64_t moved_bytes;         /* sum over launches of the bytes copied (each counted once) */
+    int64_t staging_bytes;       /* staging arena the call needed */
+    float plan_ms;               /* metadata kernels (valid when timing is on) */
+    float total_ms;              /* whole call on the stream (valid when timing is on) */
+    int64_t launch_bytes[VC_MAX_LAUNCHES];
+    float launch_ms[VC_MAX_LAUNCHES];  /* per data-moving launch, HIP events on the comm's stream */
+} vc_stats_t;
+
+/* Per-launch HIP-event timing of the following calls (0 = off, default). */
+int vc_comm_set_timing(vc_comm_t comm, int enable);
+int vc_comm_last_stats(vc_comm_t comm, vc_stats_t *out);
+
+/* Route of the last call: for launch `launch`, the bytes sent from every rank to every rank, as a HOST
+ * [P][P] int64 matrix (row = sender).  For tests that pin the route against the oracle's message trace. */
+int vc_comm_last_traffic(vc_comm_t comm, int launch, int64_t *matrix_out);
+
+/* ---- harness utilities (payload of the reference drivers, examples/rbruckv_example.cpp:88-92, and a
+ * receiver-side check in the spirit of src/utils.cpp:31-46, but exact) ---- */
+
+/* Fills every send block: mode 0: byte k of block (s,d) = byte (k & 7) of H(seed, s, d, k >> 3), H = three chained
+ * splitmix64 rounds; mode 1: int32 word idx = s*2^20 + d*2^10 + idx. */
+int vc_fill_payload(int mode, uint64_t seed, char *sendbuf, const int *sendcounts, const int *sdispls, int elem_size,
+                    vc_comm_t comm);
+
+/* Counts the bytes of recvbuf that differ from the textbook definition recv_t[rdispls_t[s] + k] =
+ * send_s[sdispls_s[t] + k] into *mismatch_out (host).  packed_recv != 0 checks the packed layout of TTPL_BT_alltoallv. */
+int vc_verify_alltoallv(const char *sendbuf, const int *sendcounts, const int *sdispls, int elem_size,
+                        const char *recvbuf, const int *recvcounts, const int *rdispls, int packed_recv,
+                        int64_t *mismatch_out, vc_comm_t comm);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* RBRUCK_VC_H_ */

@@ -1,0 +1,150 @@
+"""Host-side mirror of the reference's function interface (src/rbruckv.h) over the C ABI.
+
+Same names, same argument meaning, same return codes as the reference functions; one call
+serves all P virtual ranks.  PyTorch is used only to own device memory and to hand out
+pointers and the current stream; all work happens in librbruck_vc.so.
+"""
+from __future__ import annotations
+
+import ctypes as C
+
+import numpy as np
+import torch
+
+from . import _lib
+from .workloads import Problem
+
+
+class VcError(RuntimeError):
+    pass
+
+
+class VirtualComm:
+    """vc_comm_t: the stand-in for MPI_Comm — P virtual ranks on one GPU."""
+
+    def __init__(self, nranks: int, device: str = "cuda:0"):
+        self.lib = _lib.load()
+        self.device = torch.device(device)
+        torch.cuda.set_device(self.device)
+        h = C.c_void_p()
+        rc = self.lib.vc_comm_create(nranks, C.byref(h))
+        if rc != 0:
+            raise VcError(f"vc_comm_create: {rc} {self.lib.vc_last_error_string().decode()}")
+        self.handle = h
+        self.P = nranks
+        self._keep = []
+        self.lib.vc_comm_set_stream(self.handle, C.c_void_p(torch.cuda.current_stream(self.device).cuda_stream))
+
+    def set_bases(self, sbase: torch.Tensor, rbase: torch.Tensor) -> None:
+        assert sbase.dtype == torch.int64 and rbase.dtype == torch.int64 and sbase.is_cuda and rbase.is_cuda
+        self._keep = [sbase, rbase]
+        self._check(self.lib.vc_comm_set_bases(self.handle, sbase.data_ptr(), rbase.data_ptr()))
+
+    def set_timing(self, on: bool) -> None:
+        self._check(self.lib.vc_comm_set_timing(self.handle, int(on)))
+
+    def last_stats(self) -> _lib.VcStats:
+        s = _lib.VcStats()
+        self._check(self.lib.vc_comm_last_stats(self.handle, C.byref(s)))
+        return s
+
+    def last_traffic(self, launch: int) -> np.ndarray:
+        m = np.zeros((self.P, self.P), dtype=np.int64)
+        self._check(self.lib.vc_comm_last_traffic(self.handle, launch, m.ctypes.data_as(C.c_void_p)))
+        return m
+
+    def error(self) -> str:
+        return self.lib.vc_last_error_string().decode()
+
+    def _check(self, rc: int) -> None:
+        if rc != 0:
+            raise VcError(f"librbruck_vc returned {rc}: {self.error()}")
+
+    def free(self) -> None:
+        if self.handle:
+            self.lib.vc_comm_free(self.handle)
+            self.handle = None
+
+    def __del__(self):
+        try:
+            self.free()
+        except Exception:
+            pass
+
+
+class DeviceProblem:
+    """Rank-major tables and arena bases of a Problem, resident in HBM, plus its communicator."""
+
+    def __init__(self, prob: Problem, device: str = "cuda:0", comm: VirtualComm | None = None):
+        self.host = prob
+        self.P, self.esz = prob.P, prob.esz
+        dev = torch.device(device)
+        self.sendcounts = torch.from_numpy(prob.sendcounts).to(dev)
+        self.sdispls = torch.from_numpy(prob.sdispls).to(dev)
+        self.recvcounts = torch.from_numpy(prob.recvcounts).to(dev)
+        self.rdispls = torch.from_numpy(prob.rdispls).to(dev)
+        self.sbase = torch.from_numpy(prob.sbase).to(dev)
+        self.rbase = torch.from_numpy(prob.rbase).to(dev)
+        self.comm = comm or VirtualComm(prob.P, device)
+        self.comm.set_bases(self.sbase, self.rbase)
+
+    def new_send_arena(self) -> torch.Tensor:
+        return torch.zeros(self.host.send_bytes, dtype=torch.uint8, device=self.sbase.device)
+
+    def new_recv_arena(self, fill: int = 0xEE) -> torch.Tensor:
+        return torch.full((self.host.recv_bytes,), fill, dtype=torch.uint8, device=self.sbase.device)
+
+    def fill_payload(self, mode: int, seed: int, send: torch.Tensor) -> None:
+        c = self.comm
+        c._check(c.lib.vc_fill_payload(mode, seed, send.data_ptr(), self.sendcounts.data_ptr(), self.sdispls.data_ptr(),
+                                       self.esz, c.handle))
+
+    def verify(self, send: torch.Tensor, recv: torch.Tensor, packed_recv: bool = False) -> int:
+        c = self.comm
+        bad = C.c_int64(-1)
+        c._check(c.lib.vc_verify_alltoallv(send.data_ptr(), self.sendcounts.data_ptr(), self.sdispls.data_ptr(), self.esz,
+                                           recv.data_ptr(), self.recvcounts.data_ptr(), self.rdispls.data_ptr(),
+                                           int(packed_recv), C.byref(bad), c.handle))
+        return bad.value
+
+
+def _tail(p: DeviceProblem, send: torch.Tensor, recv: torch.Tensor):
+    return (send.data_ptr(), p.sendcounts.data_ptr(), p.sdispls.data_ptr(), p.esz, recv.data_ptr(),
+            p.recvcounts.data_ptr(), p.rdispls.data_ptr(), p.esz, p.comm.handle)
+
+
+def twophase_rbruck_alltoallv(r: int, p: DeviceProblem, send: torch.Tensor, recv: torch.Tensor) -> int:
+    """src/twophase_tunable_rbruckv.cpp:13-152"""
+    return p.comm.lib.twophase_rbruck_alltoallv(r, *_tail(p, send, recv))
+
+
+def twophase_rbruck_alltoallv_om(r: int, p: DeviceProblem, send: torch.Tensor, recv: torch.Tensor) -> int:
+    """src/twophase_tunable_rbruckv-om.cpp:10-157"""
+    return p.comm.lib.twophase_rbruck_alltoallv_om(r, *_tail(p, send, recv))
+
+
+def tuna_algorithm(r: int, b: int, p: DeviceProblem, send: torch.Tensor, recv: torch.Tensor) -> int:
+    """src/tuna.cpp:10-177"""
+    return p.comm.lib.tuna_algorithm(r, b, *_tail(p, send, recv))
+
+
+def TTPL_BT_alltoallv(n: int, r: int, bblock: int, p: DeviceProblem, send: torch.Tensor, recv: torch.Tensor) -> int:
+    """src/twophase_twolayer_rbruck.cpp:237-463"""
+    return p.comm.lib.TTPL_BT_alltoallv(n, r, bblock, *_tail(p, send, recv))
+
+
+def TTPL_BT_alltoallv_s1(n: int, r: int, bblock: int, p: DeviceProblem, send: torch.Tensor, recv: torch.Tensor) -> int:
+    """src/twophase_twolayer_rbruck.cpp:467-681"""
+    return p.comm.lib.TTPL_BT_alltoallv_s1(n, r, bblock, *_tail(p, send, recv))
+
+
+def uniform_spreadout_twolayer(n: int, r: int, p: DeviceProblem, count: int, send: torch.Tensor, recv: torch.Tensor) -> int:
+    """src/twolayer_rbruck.cpp:10-134"""
+    return p.comm.lib.uniform_spreadout_twolayer(n, r, send.data_ptr(), count, p.esz, recv.data_ptr(), count, p.esz, p.comm.handle)
+
+
+def uniform_inverse_isplit_r_bruck(n: int, r1: int, r2: int, p: DeviceProblem, count: int, send: torch.Tensor,
+                                   recv: torch.Tensor) -> int:
+    """src/twolayer_rbruck.cpp:137-277"""
+    return p.comm.lib.uniform_inverse_isplit_r_bruck(n, r1, r2, send.data_ptr(), count, p.esz, recv.data_ptr(), count,
+                                                     p.esz, p.comm.handle)

@@ -1,0 +1,30 @@
+"""Builds librbruck_vc.so (HIP kernels + C ABI) in-tree with hipcc for gfx950."""
+from __future__ import annotations
+
+import os
+import subprocess
+
+PKG_DIR = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(PKG_DIR, "csrc")
+LIB_PATH = os.path.join(PKG_DIR, "librbruck_vc.so")
+SOURCES = ["vc_meta.hip", "vc_plan.hip", "vc_copy.hip", "vc_api.hip"]
+HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+# packed FP32 instructions stay off for every HIP translation unit of this library
+FLAGS = ["--offload-arch=gfx950", "-O3", "-fPIC", "-shared", "-std=c++17", "-Wall",
+         "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+
+
+def build_library(verbose: bool = False) -> str:
+    cmd = [HIPCC, *FLAGS, "-o", LIB_PATH, *[os.path.join(CSRC, s) for s in SOURCES]]
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    if verbose or res.returncode != 0:
+        print(" ".join(cmd))
+        print(res.stdout)
+        print("\n".join(l for l in res.stderr.splitlines() if "packed-fp32-ops" not in l))
+    if res.returncode != 0:
+        raise RuntimeError("hipcc failed building librbruck_vc.so")
+    return LIB_PATH
+
+
+if __name__ == "__main__":
+    print(build_library(verbose=True))

@@ -1,0 +1,376 @@
+// vc_api.hip — host side of librbruck_vc: the C ABI declared in include/rbruck_vc.h.
+//
+// Every collective entry point does what the reference function of the same name
+// does on each of the P ranks, for all ranks at once:
+//   1. clamp / validate the tunables exactly as the reference does,
+//   2. derive the schedule: which digit phases exist, which rounds share a launch,
+//   3. plan on the device (staging prefix sums, one copy descriptor per block hop),
+//   4. run one copy kernel per launch,
+//   5. synchronise the stream (the reference functions are blocking).
+#include <hip/hip_runtime.h>
+
+#include <algorithm>
+#include <cstdio>
+#include <cstring>
+#include <string>
+#include <vector>
+
+#include "../../include/rbruck_vc.h"
+#include "vc_common.h"
+#include "vc_sched.h"
+
+static thread_local std::string g_last_error;
+
+static int fail_hip(hipError_t e, const char *what, int line) {
+    char buf[256];
+    snprintf(buf, sizeof buf, "%s failed at vc_api.hip:%d: %s", what, line, hipGetErrorString(e));
+    g_last_error = buf;
+    return VC_ERR_HIP;
+}
+
+#define HIP_TRY(expr)                                                   \
+    do {                                                                \
+        hipError_t e_ = (expr);                                         \
+        if (e_ != hipSuccess) return fail_hip(e_, #expr, __LINE__);     \
+    } while (0)
+
+static int fail_arg(const char *msg, int code = VC_ERR_ARG) {
+    g_last_error = msg;
+    return code;
+}
+
+extern "C" const char *vc_last_error_string(void) { return g_last_error.c_str(); }
+
+// Grow-only device buffer.
+struct DevBuf {
+    void *p = nullptr;
+    size_t cap = 0;
+    hipError_t reserve(size_t bytes) {
+        if (bytes <= cap) return hipSuccess;
+        if (p) { hipError_t e = hipFree(p); p = nullptr; cap = 0; if (e != hipSuccess) return e; }
+        size_t want = std::max(bytes, (size_t)256);
+        hipError_t e = hipMalloc(&p, want);
+        if (e == hipSuccess) cap = want;
+        return e;
+    }
+    void release() { if (p) (void)hipFree(p); p = nullptr; cap = 0; }
+    template <class T> T *as() const { return static_cast<T *>(p); }
+};
+
+struct vc_comm {
+    int P = 0;
+    int device = 0;
+    hipStream_t stream = nullptr;
+    const int64_t *sbase = nullptr, *rbase = nullptr;
+    bool timing = false;
+    DevBuf slot_off, row_tot, row_base, desc, header, launches, stage, rd_packed, uni_counts, uni_displs, scratch;
+    int64_t *h_header = nullptr;          // pinned
+    VcLaunchInfo *h_launches = nullptr;   // pinned
+    std::vector<hipEvent_t> events;
+    vc_stats_t stats;
+    int last_nlaunch = 0;
+};
+
+// ------------------------------------------------------------------ communicator
+
+extern "C" int vc_comm_create(int nranks, vc_comm_t *comm_out) {
+    if (!comm_out || nranks < 1) return fail_arg("vc_comm_create: need nranks >= 1 and an output pointer");
+    int ndev = 0;
+    if (hipGetDeviceCount(&ndev) != hipSuccess || ndev < 1) return fail_arg("no HIP device", VC_ERR_NO_DEVICE);
+    vc_comm *c = new vc_comm();
+    c->P = nranks;
+    HIP_TRY(hipGetDevice(&c->device));
+    HIP_TRY(hipHostMalloc((void **)&c->h_header, sizeof(int64_t) * (2 + VC_MAX_LAUNCHES), hipHostMallocDefault));
+    HIP_TRY(hipHostMalloc((void **)&c->h_launches, sizeof(VcLaunchInfo) * VC_MAX_LAUNCHES, hipHostMallocDefault));
+    memset(&c->stats, 0, sizeof c->stats);
+    *comm_out = c;
+    return VC_OK;
+}
+
+extern "C" int vc_comm_free(vc_comm_t c) {
+    if (!c) return VC_OK;
+    (void)hipStreamSynchronize(c->stream);
+    for (DevBuf *b : {&c->slot_off, &c->row_tot, &c->row_base, &c->desc, &c->header, &c->launches, &c->stage, &c->rd_packed,
+                      &c->uni_counts, &c->uni_displs, &c->scratch})
+        b->release();
+    for (hipEvent_t e : c->events) (void)hipEventDestroy(e);
+    if (c->h_header) (void)hipHostFree(c->h_header);
+    if (c->h_launches) (void)hipHostFree(c->h_launches);
+    delete c;
+    return VC_OK;
+}
+
+extern "C" int vc_comm_size(vc_comm_t c) { return c ? c->P : VC_ERR_ARG; }
+
+extern "C" int vc_comm_set_stream(vc_comm_t c, void *hip_stream) {
+    if (!c) return fail_arg("null communicator");
+    c->stream = static_cast<hipStream_t>(hip_stream);
+    return VC_OK;
+}
+
+extern "C" int vc_comm_set_bases(vc_comm_t c, const int64_t *sbase, const int64_t *rbase) {
+    if (!c || !sbase || !rbase) return fail_arg("vc_comm_set_bases: null argument");
+    c->sbase = sbase;
+    c->rbase = rbase;
+    return VC_OK;
+}
+
+extern "C" int vc_comm_set_timing(vc_comm_t c, int enable) {
+    if (!c) return fail_arg("null communicator");
+    c->timing = enable != 0;
+    return VC_OK;
+}
+
+extern "C" int vc_comm_last_stats(vc_comm_t c, vc_stats_t *out) {
+    if (!c || !out) return fail_arg("vc_comm_last_stats: null argument");
+    *out = c->stats;
+    return VC_OK;
+}
+
+// ------------------------------------------------------------ caller-side steps
+
+extern "C" int vc_alltoall_counts(const int *sendcounts, int *recvcounts, vc_comm_t c) {
+    if (!c || !sendcounts || !recvcounts) return fail_arg("vc_alltoall_counts: null argument");
+    HIP_TRY(vc_launch_transpose(sendcounts, recvcounts, c->P, c->stream));
+    HIP_TRY(hipStreamSynchronize(c->stream));
+    return VC_OK;
+}
+
+extern "C" int vc_displs_from_counts(const int *counts, int *displs, int64_t *extent_out, vc_comm_t c) {
+    if (!c || !counts || !displs) return fail_arg("vc_displs_from_counts: null argument");
+    HIP_TRY(vc_launch_row_scan(counts, displs, extent_out, c->P, c->stream));
+    HIP_TRY(hipStreamSynchronize(c->stream));
+    return VC_OK;
+}
+
+extern "C" int vc_bases_from_extents(const int64_t *extent, int elem_size, int64_t align, int64_t *base_out, int64_t *total_out,
+                                     vc_comm_t c) {
+    if (!c || !extent || !base_out || elem_size < 1 || align < 1) return fail_arg("vc_bases_from_extents: bad argument");
+    HIP_TRY(vc_launch_bases(extent, elem_size, align, base_out, total_out, c->P, c->stream));
+    HIP_TRY(hipStreamSynchronize(c->stream));
+    return VC_OK;
+}
+
+extern "C" int vc_allreduce_max_count(const int *sendcounts, int *max_out, vc_comm_t c) {
+    if (!c || !sendcounts || !max_out) return fail_arg("vc_allreduce_max_count: null argument");
+    HIP_TRY(vc_launch_max(sendcounts, max_out, (int64_t)c->P * c->P, c->stream));
+    HIP_TRY(hipStreamSynchronize(c->stream));
+    return VC_OK;
+}
+
+// ------------------------------------------------------------- plan and run
+
+static int ensure_events(vc_comm *c, size_t n) {
+    while (c->events.size() < n) {
+        hipEvent_t e;
+        HIP_TRY(hipEventCreate(&e));
+        c->events.push_back(e);
+    }
+    return VC_OK;
+}
+
+// Steps 3-5 for any schedule.
+static int run_schedule(vc_comm *c, VcSched S, std::vector<VcLaunchInfo> &L, const char *sendbuf, char *recvbuf, VcTables T) {
+    const int P = S.P;
+    const int nl = (int)L.size();
+    if (nl > VC_MAX_LAUNCHES) return fail_arg("more than VC_MAX_LAUNCHES launches: raise b / bblock");
+    hipStream_t st = c->stream;
+    const size_t PP = (size_t)P * P;
+
+    HIP_TRY(c->slot_off.reserve(sizeof(int64_t) * PP * std::max(S.w, 1)));
+    HIP_TRY(c->row_tot.reserve(sizeof(int64_t) * (size_t)P * std::max(S.w, 1)));
+    HIP_TRY(c->row_base.reserve(sizeof(int64_t) * (size_t)P * std::max(S.w, 1)));
+    HIP_TRY(c->desc.reserve(sizeof(VcDesc) * PP * nl));
+    HIP_TRY(c->header.reserve(sizeof(int64_t) * (2 + VC_MAX_LAUNCHES)));
+    HIP_TRY(c->launches.reserve(sizeof(VcLaunchInfo) * VC_MAX_LAUNCHES));
+    if (c->timing) { int rc = ensure_events(c, (size_t)nl + 4); if (rc) return rc; }
+
+    if (c->timing) HIP_TRY(hipEventRecord(c->events[0], st));
+    memcpy(c->h_launches, L.data(), sizeof(VcLaunchInfo) * nl);
+    HIP_TRY(hipMemcpyAsync(c->launches.p, c->h_launches, sizeof(VcLaunchInfo) * nl, hipMemcpyHostToDevice, st));
+    if (S.packed_recv) {
+        HIP_TRY(c->rd_packed.reserve(sizeof(int) * PP));
+        HIP_TRY(vc_launch_row_scan(T.rc, c->rd_packed.as<int>(), nullptr, P, st));
+        T.rd_packed = c->rd_packed.as<int>();
+    }
+    HIP_TRY(vc_launch_plan(S, c->launches.as<VcLaunchInfo>(), nl, T, c->slot_off.as<int64_t>(), c->row_tot.as<int64_t>(),
+                           c->row_base.as<int64_t>(), c->desc.as<VcDesc>(), c->header.as<int64_t>(), st));
+    HIP_TRY(hipMemcpyAsync(c->h_header, c->header.p, sizeof(int64_t) * (2 + nl), hipMemcpyDeviceToHost, st));
+    if (c->timing) HIP_TRY(hipEventRecord(c->events[1], st));
+    HIP_TRY(hipStreamSynchronize(st));     // the staging arena is sized from the plan
+
+    const int64_t stage_bytes = c->h_header[0];
+    HIP_TRY(c->stage.reserve((size_t)stage_bytes + 64));
+
+    for (int k = 0; k < nl; k++) {
+        if (c->timing) HIP_TRY(hipEventRecord(c->events[2 + k], st));
+        HIP_TRY(vc_launch_copy_dense(c->desc.as<VcDesc>() + PP * k, (int64_t)PP, sendbuf, recvbuf, c->stage.as<char>(), st));
+    }
+    if (c->timing) HIP_TRY(hipEventRecord(c->events[2 + nl], st));
+    HIP_TRY(hipStreamSynchronize(st));
+
+    vc_stats_t &s = c->stats;
+    s.n_launches = nl;
+    s.n_digits = S.w;
+    s.staging_bytes = stage_bytes;
+    s.payload_bytes = c->h_header[1];
+    s.moved_bytes = 0;
+    s.plan_ms = s.total_ms = 0.f;
+    for (int k = 0; k < nl; k++) {
+        s.launch_bytes[k] = c->h_header[2 + k];
+        s.moved_bytes += s.launch_bytes[k];
+        s.launch_ms[k] = 0.f;
+        if (c->timing) HIP_TRY(hipEventElapsedTime(&s.launch_ms[k], c->events[2 + k], c->events[3 + k]));
+    }
+    if (c->timing) {
+        HIP_TRY(hipEventElapsedTime(&s.plan_ms, c->events[0], c->events[1]));
+        HIP_TRY(hipEventElapsedTime(&s.total_ms, c->events[0], c->events[2 + nl]));
+    }
+    c->last_nlaunch = nl;
+    return VC_OK;
+}
+
+static int check_common(vc_comm *c, const void *sendbuf, const void *recvbuf, int esz) {
+    if (!c) return fail_arg("null communicator");
+    if (!sendbuf || !recvbuf) return fail_arg("null buffer");
+    if (esz < 1) return fail_arg("element size must be >= 1");
+    if (!c->sbase || !c->rbase) return fail_arg("vc_comm_set_bases has not been called");
+    return VC_OK;
+}
+
+static VcTables make_tables(vc_comm *c, const int *sc, const int *sd, const int *rc, const int *rd) {
+    VcTables T;
+    T.sc = sc; T.sd = sd; T.rc = rc; T.rd = rd; T.sbase = c->sbase; T.rbase = c->rbase; T.rd_packed = nullptr;
+    return T;
+}
+
+static int schedule_error(int code) {
+    switch (code) {
+    case VC_ERR_RADIX: g_last_error = "radix must be >= 2"; break;
+    case VC_ERR_GROUP: g_last_error = "the ranks per node must divide the rank count (uniform functions: 2 <= n < P)"; break;
+    case VC_ERR_TOO_FEW_RANKS: g_last_error = "tuna_algorithm needs at least 3 ranks"; break;
+    default: break;
+    }
+    return code;
+}
+
+// The alltoallv-shaped functions.
+static int run_v(VcFunc f, int n, int r, int batch, vc_comm *c, char *sendbuf, int *sendcounts, int *sdispls, int esz,
+                 char *recvbuf, int *recvcounts, int *rdispls) {
+    int rc = check_common(c, sendbuf, recvbuf, esz);
+    if (rc) return rc;
+    if (!sendcounts || !sdispls || !recvcounts || (f != VC_F_TTPL && !rdispls)) return fail_arg("null table");
+    VcSched S;
+    std::vector<VcLaunchInfo> L;
+    rc = vc_make_schedule(f, c->P, n, r, batch, esz, 0, S, L);
+    if (rc) return schedule_error(rc);
+    S.recv_lo = (int)((uintptr_t)recvbuf & 15);
+    return run_schedule(c, S, L, sendbuf, recvbuf, make_tables(c, sendcounts, sdispls, recvcounts, rdispls));
+}
+
+extern "C" int twophase_rbruck_alltoallv(int r, char *sendbuf, int *sendcounts, int *sdispls, int sendtype_size, char *recvbuf,
+                                         int *recvcounts, int *rdispls, int recvtype_size, vc_comm_t c) {
+    (void)recvtype_size;
+    return run_v(VC_F_TWOPHASE, 0, r, 0, c, sendbuf, sendcounts, sdispls, sendtype_size, recvbuf, recvcounts, rdispls);
+}
+
+extern "C" int twophase_rbruck_alltoallv_om(int r, char *sendbuf, int *sendcounts, int *sdispls, int sendtype_size, char *recvbuf,
+                                            int *recvcounts, int *rdispls, int recvtype_size, vc_comm_t c) {
+    (void)recvtype_size;
+    return run_v(VC_F_OM, 0, r, 0, c, sendbuf, sendcounts, sdispls, sendtype_size, recvbuf, recvcounts, rdispls);
+}
+
+extern "C" int tuna_algorithm(int r, int b, char *sendbuf, int *sendcounts, int *sdispls, int sendtype_size, char *recvbuf,
+                              int *recvcounts, int *rdispls, int recvtype_size, vc_comm_t c) {
+    (void)recvtype_size;
+    return run_v(VC_F_TUNA, 0, r, b, c, sendbuf, sendcounts, sdispls, sendtype_size, recvbuf, recvcounts, rdispls);
+}
+
+extern "C" int TTPL_BT_alltoallv(int n, int r, int bblock, char *sendbuf, int *sendcounts, int *sdispls, int sendtype_size,
+                                 char *recvbuf, int *recvcounts, int *rdispls, int recvtype_size, vc_comm_t c) {
+    (void)recvtype_size;
+    return run_v(VC_F_TTPL, n, r, bblock, c, sendbuf, sendcounts, sdispls, sendtype_size, recvbuf, recvcounts, rdispls);
+}
+
+extern "C" int TTPL_BT_alltoallv_s1(int n, int r, int bblock, char *sendbuf, int *sendcounts, int *sdispls, int sendtype_size,
+                                    char *recvbuf, int *recvcounts, int *rdispls, int recvtype_size, vc_comm_t c) {
+    (void)recvtype_size;
+    return run_v(VC_F_TTPL_S1, n, r, bblock, c, sendbuf, sendcounts, sdispls, sendtype_size, recvbuf, recvcounts, rdispls);
+}
+
+// The alltoall-shaped (equal blocks) functions: the count tables are implied.
+static int run_uniform(VcFunc f, int n, int r, vc_comm *c, char *sendbuf, int sendcount, int esz, char *recvbuf) {
+    int rc = check_common(c, sendbuf, recvbuf, esz);
+    if (rc) return rc;
+    if (sendcount < 0) return fail_arg("negative block length");
+    VcSched S;
+    std::vector<VcLaunchInfo> L;
+    rc = vc_make_schedule(f, c->P, n, r, 0, esz, sendcount, S, L);
+    if (rc) return schedule_error(rc);
+    S.recv_lo = (int)((uintptr_t)recvbuf & 15);
+    const size_t PP = (size_t)c->P * c->P;
+    HIP_TRY(c->uni_counts.reserve(sizeof(int) * PP));
+    HIP_TRY(c->uni_displs.reserve(sizeof(int) * PP));
+    HIP_TRY(vc_launch_uniform_tables(c->uni_counts.as<int>(), c->uni_displs.as<int>(), sendcount, c->P, c->stream));
+    const int *cnt = c->uni_counts.as<int>(), *dsp = c->uni_displs.as<int>();
+    return run_schedule(c, S, L, sendbuf, recvbuf, make_tables(c, cnt, dsp, cnt, dsp));
+}
+
+extern "C" int uniform_spreadout_twolayer(int n, int r, char *sendbuf, int sendcount, int sendtype_size, char *recvbuf,
+                                          int recvcount, int recvtype_size, vc_comm_t c) {
+    (void)recvcount; (void)recvtype_size;
+    return run_uniform(VC_F_UNIFORM_SPREADOUT, n, r, c, sendbuf, sendcount, sendtype_size, recvbuf);
+}
+
+extern "C" int uniform_inverse_isplit_r_bruck(int n, int r1, int r2, char *sendbuf, int sendcount, int sendtype_size,
+                                              char *recvbuf, int recvcount, int recvtype_size, vc_comm_t c) {
+    (void)recvcount; (void)recvtype_size; (void)r2;          // r2 is overwritten with the group count (:158)
+    return run_uniform(VC_F_UNIFORM_ISPLIT, n, r1, c, sendbuf, sendcount, sendtype_size, recvbuf);
+}
+
+// ------------------------------------------------------------------ inspection
+
+extern "C" int vc_comm_last_traffic(vc_comm_t c, int launch, int64_t *matrix_out) {
+    if (!c || !matrix_out) return fail_arg("vc_comm_last_traffic: null argument");
+    if (launch < 0 || launch >= c->last_nlaunch) return fail_arg("vc_comm_last_traffic: no such launch");
+    const size_t PP = (size_t)c->P * c->P;
+    HIP_TRY(c->scratch.reserve(sizeof(int64_t) * PP));
+    HIP_TRY(hipMemsetAsync(c->scratch.p, 0, sizeof(int64_t) * PP, c->stream));
+    HIP_TRY(vc_launch_traffic(c->desc.as<VcDesc>() + PP * launch, (int64_t)PP, c->scratch.as<int64_t>(), c->P, c->stream));
+    HIP_TRY(hipMemcpyAsync(matrix_out, c->scratch.p, sizeof(int64_t) * PP, hipMemcpyDeviceToHost, c->stream));
+    HIP_TRY(hipStreamSynchronize(c->stream));
+    return VC_OK;
+}
+
+// ------------------------------------------------------------ harness utilities
+
+extern "C" int vc_fill_payload(int mode, uint64_t seed, char *sendbuf, const int *sendcounts, const int *sdispls, int elem_size,
+                               vc_comm_t c) {
+    if (!c || !sendbuf || !sendcounts || !sdispls || elem_size < 1 || !c->sbase) return fail_arg("vc_fill_payload: bad argument");
+    HIP_TRY(vc_launch_fill_payload(mode, seed, sendbuf, sendcounts, sdispls, c->sbase, elem_size, c->P, c->stream));
+    HIP_TRY(hipStreamSynchronize(c->stream));
+    return VC_OK;
+}
+
+extern "C" int vc_verify_alltoallv(const char *sendbuf, const int *sendcounts, const int *sdispls, int elem_size,
+                                   const char *recvbuf, const int *recvcounts, const int *rdispls, int packed_recv,
+                                   int64_t *mismatch_out, vc_comm_t c) {
+    if (!c || !sendbuf || !recvbuf || !sendcounts || !sdispls || !recvcounts || !mismatch_out || elem_size < 1 || !c->sbase)
+        return fail_arg("vc_verify_alltoallv: bad argument");
+    if (!packed_recv && !rdispls) return fail_arg("vc_verify_alltoallv: rdispls needed");
+    const size_t PP = (size_t)c->P * c->P;
+    VcTables T = make_tables(c, sendcounts, sdispls, recvcounts, rdispls);
+    if (packed_recv) {
+        HIP_TRY(c->rd_packed.reserve(sizeof(int) * PP));
+        HIP_TRY(vc_launch_row_scan(recvcounts, c->rd_packed.as<int>(), nullptr, c->P, c->stream));
+        T.rd_packed = c->rd_packed.as<int>();
+    }
+    HIP_TRY(c->scratch.reserve(sizeof(int64_t) * PP));
+    HIP_TRY(hipMemsetAsync(c->scratch.p, 0, sizeof(unsigned long long), c->stream));
+    HIP_TRY(vc_launch_verify(sendbuf, recvbuf, T, elem_size, c->P, packed_recv, c->scratch.as<unsigned long long>(), c->stream));
+    unsigned long long bad = 0;
+    HIP_TRY(hipMemcpyAsync(&bad, c->scratch.p, sizeof bad, hipMemcpyDeviceToHost, c->stream));
+    HIP_TRY(hipStreamSynchronize(c->stream));
+    *mismatch_out = (int64_t)bad;
+    return VC_OK;
+}

@@ -1,0 +1,83 @@
+// vc_common.h — types shared by the host side and the kernels of librbruck_vc.
+//
+// Vocabulary (follows the reference): a *block* is the data one rank sends to one
+// other rank; its *offset* is j = (source - destination) mod span and never
+// changes; the *slot* a block occupies on whichever rank currently holds it is
+// id = g*n + (j + local_rank) % n (src/twophase_twolayer_rbruck.cpp:322; with one
+// group this is (j + rank) % P, src/twophase_tunable_rbruckv.cpp:81).  A *digit
+// phase* x moves every block whose base-r digit x of j is non-zero by z*r^x ranks.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#define VC_THREADS 256
+
+// Location of a byte range: which arena (top bits) and the byte offset inside it.
+#define VC_SPACE_SHIFT 60
+#define VC_SPACE_SEND (0ll << VC_SPACE_SHIFT)
+#define VC_SPACE_RECV (1ll << VC_SPACE_SHIFT)
+#define VC_SPACE_STAGE (2ll << VC_SPACE_SHIFT)
+#define VC_OFFSET_MASK ((1ll << VC_SPACE_SHIFT) - 1)
+
+// One block copy: `len` bytes from `src` to `dst` (space-tagged offsets), sent by
+// virtual rank `from` to virtual rank `to`.
+struct VcDesc {
+    int64_t src;
+    int64_t dst;
+    int64_t len;
+    int32_t from;
+    int32_t to;
+};
+
+// What kind of algorithm the call runs; fixed for the whole call.
+struct VcSched {
+    int P;            // ranks
+    int n;            // ranks per node (P for the one-layer variants)
+    int G;            // nodes = P / n
+    int r;            // radix of the intra-node digits (already clamped)
+    int w;            // digits of n-1 in base r (0 when n == 1)
+    int msd;          // 1: most significant digit first (twophase_rbruck_alltoallv, uniform intra phase)
+    int esz;          // element size in bytes
+    int packed_recv;  // 1: receive side is the packed source-ordered layout (TTPL_BT_alltoallv ignores rdispls)
+    int uniform;      // >0: equal blocks of this many elements, tables are implied (uniform_* functions)
+    int recv_lo;      // low 4 bits of the recvbuf pointer (staging slots copy the final destination's 16-byte phase)
+};
+
+// One data-moving kernel launch.
+struct VcLaunchInfo {
+    int kind;      // 0: rounds of intra-node digit x with digit value in [zlo, zhi]; 1: inter-node messages
+    int x;         // digit
+    int dist;      // r^x
+    int zlo, zhi;
+    int qlo, qhi;  // inter-node: (group distance)*n + source local index in [qlo, qhi)
+    int self;      // also performs every rank's copy to itself
+};
+
+struct VcTables {
+    const int *sc, *sd, *rc, *rd;    // [P][P] row-major, elements
+    const int64_t *sbase, *rbase;    // [P] bytes
+    const int *rd_packed;            // [P][P] exclusive scan of rc rows (only when packed_recv)
+};
+
+// ---- launchers implemented in the .hip files (all asynchronous on `st`) ----
+
+// vc_meta.hip
+hipError_t vc_launch_transpose(const int *in, int *out, int P, hipStream_t st);
+hipError_t vc_launch_row_scan(const int *counts, int *displs, int64_t *extent, int P, hipStream_t st);
+hipError_t vc_launch_bases(const int64_t *extent, int esz, int64_t align, int64_t *base, int64_t *total, int P, hipStream_t st);
+hipError_t vc_launch_max(const int *counts, int *out, int64_t nelem, hipStream_t st);
+hipError_t vc_launch_fill_payload(int mode, uint64_t seed, char *sendbuf, const int *sc, const int *sd, const int64_t *sbase,
+                                  int esz, int P, hipStream_t st);
+hipError_t vc_launch_verify(const char *sendbuf, const char *recvbuf, VcTables t, int esz, int P, int packed,
+                            unsigned long long *mismatch, hipStream_t st);
+hipError_t vc_launch_uniform_tables(int *counts, int *displs, int count, int P, hipStream_t st);
+
+// vc_plan.hip
+// header layout (int64): [0] staging bytes, [1] payload bytes, [2 + L] bytes moved by launch L
+hipError_t vc_launch_plan(const VcSched &S, const VcLaunchInfo *launches_dev, int nlaunch, VcTables T, int64_t *slot_off,
+                          int64_t *row_tot, int64_t *row_base, VcDesc *desc, int64_t *header, hipStream_t st);
+hipError_t vc_launch_traffic(const VcDesc *desc, int64_t ndesc, int64_t *matrix, int P, hipStream_t st);
+
+// vc_copy.hip
+hipError_t vc_launch_copy_dense(const VcDesc *desc, int64_t ndesc, const char *sendbuf, char *recvbuf, char *stage, hipStream_t st);

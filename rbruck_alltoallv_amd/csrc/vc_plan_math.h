@@ -1,0 +1,153 @@
+// vc_plan_math.h — index arithmetic of the Bruck family, shared by the planning
+// kernels and by host code (the CPU build used to check the plan without a GPU).
+//
+// Which block sits in slot `id` of rank p before digit x follows from the
+// residency invariant of the digit order:
+//   least significant digit first: its source is (j mod r^x) ranks above the holder,
+//   most significant digit first:  its source is (j div r^(x+1)) * r^(x+1) ranks above.
+#pragma once
+
+#include "vc_common.h"
+
+#if defined(__HIPCC__)
+#define VC_HD __host__ __device__ __forceinline__
+#else
+#define VC_HD inline
+#endif
+
+struct VcBlock {
+    int s, t;        // source and destination rank of the block
+    int from;        // rank that holds it before this hop
+    int z;           // digit value (0: does not move in this digit)
+    int xprev;       // digit in which it last moved (-1: still in sendbuf)
+    int id_from;     // its slot on `from`
+    bool to_stage;   // lands in the receiver's staging area (else in recvbuf)
+};
+
+VC_HD int vc_top_digit(int v, int r) {     // position of the highest non-zero digit, v > 0
+    int x = -1;
+    while (v) { v /= r; x++; }
+    return x;
+}
+
+VC_HD int vc_low_digit(int v, int r) {     // position of the lowest non-zero digit, v > 0
+    int x = 0;
+    while (v % r == 0) { v /= r; x++; }
+    return x;
+}
+
+// Block that arrives in slot `id` of rank `to` during digit x (dist = r^x), if any.
+VC_HD bool vc_intra_block(const VcSched &S, int x, int dist, int to, int id, VcBlock &b) {
+    const int n = S.n, r = S.r;
+    const int gs = to / n, lr = to % n;
+    const int g = id / n;
+    const int j = (id % n - lr + n) % n;
+    b.z = 0;
+    if (j == 0) return false;
+    const int z = (j / dist) % r;
+    if (z == 0) return false;
+    const int lfrom = (lr + z * dist) % n;
+    const int64_t nd = (int64_t)dist * r;
+    int above;        // how far the source is above the sender
+    bool last;
+    if (!S.msd) {
+        above = j % dist;
+        last = j < nd;
+        b.xprev = above ? vc_top_digit(above, r) : -1;
+    } else {
+        above = (int)((j / nd) * nd);
+        last = (j % dist) == 0;
+        b.xprev = above ? vc_low_digit(above, r) : -1;
+    }
+    const int ls = (lfrom + above) % n;
+    b.s = gs * n + ls;
+    b.t = g * n + (ls - j + n) % n;
+    b.from = gs * n + lfrom;
+    b.z = z;
+    b.id_from = g * n + (j + lfrom) % n;
+    b.to_stage = !(last && g == gs);
+    return true;
+}
+
+VC_HD int64_t vc_recv_offset(const VcSched &S, const VcTables &T, int s, int t) {
+    const int *rd = S.packed_recv ? T.rd_packed : T.rd;
+    return T.rbase[t] + (int64_t)rd[(int64_t)t * S.P + s] * S.esz;
+}
+
+// Staging slots start 16-byte aligned; the data inside starts at the 16-byte phase
+// of the block's final address in recvbuf, so that every later hop copies between
+// equally aligned addresses.
+VC_HD int vc_phase16(const VcSched &S, const VcTables &T, int s, int t) {
+    return (int)((vc_recv_offset(S, T, s, t) + S.recv_lo) & 15);
+}
+
+
+// Bytes the staging slot `id` of rank `to` needs for the block that arrives in digit x
+// (0 if nothing arrives there, or if it goes to recvbuf).  Always a multiple of 16.
+VC_HD int64_t vc_stage_slot_size(const VcSched &S, const VcTables &T, int x, int dist, int to, int id) {
+    VcBlock b;
+    if (!vc_intra_block(S, x, dist, to, id, b) || !b.to_stage) return 0;
+    const int64_t len = (int64_t)T.sc[(int64_t)b.s * S.P + b.t] * S.esz;
+    return len ? ((len + vc_phase16(S, T, b.s, b.t) + 15) & ~15ll) : 0;
+}
+
+// Address (inside the staging arena) of the data of block (s, t) while it sits in slot `id`
+// of `holder`, having arrived there in digit x.
+VC_HD int64_t vc_stage_addr(const VcSched &S, const VcTables &T, const int64_t *slot_off, const int64_t *row_base,
+                            int x, int holder, int id, int s, int t) {
+    const int64_t row = (int64_t)x * S.P + holder;
+    return row_base[row] + slot_off[row * S.P + id] + vc_phase16(S, T, s, t);
+}
+
+VC_HD int64_t vc_send_offset(const VcSched &S, const VcTables &T, int s, int t) {
+    return T.sbase[s] + (int64_t)T.sd[(int64_t)s * S.P + t] * S.esz;
+}
+
+// The copy that entry (`to`, `id`) of a launch stands for; len = 0 if none.
+// Intra-node launches index by the receiver's slot, inter-node launches by the source rank.
+VC_HD VcDesc vc_emit_entry(const VcSched &S, const VcLaunchInfo &info, const VcTables &T, const int64_t *slot_off,
+                           const int64_t *row_base, int to, int id) {
+    const int P = S.P, n = S.n;
+    VcDesc d;
+    d.src = 0; d.dst = 0; d.len = 0; d.from = -1; d.to = to;
+    if (info.self && id == to) {
+        // a rank's block to itself (src/twophase_tunable_rbruckv.cpp:63)
+        d.len = (int64_t)T.sc[(int64_t)to * P + to] * S.esz;
+        d.src = VC_SPACE_SEND | vc_send_offset(S, T, to, to);
+        d.dst = VC_SPACE_RECV | vc_recv_offset(S, T, to, to);
+        d.from = to;
+    } else if (info.kind == 0) {
+        VcBlock b;
+        if (vc_intra_block(S, info.x, info.dist, to, id, b) && b.z >= info.zlo && b.z <= info.zhi) {
+            d.len = (int64_t)T.sc[(int64_t)b.s * P + b.t] * S.esz;
+            d.from = b.from;
+            d.src = b.xprev < 0 ? (VC_SPACE_SEND | vc_send_offset(S, T, b.s, b.t))
+                                : (VC_SPACE_STAGE | vc_stage_addr(S, T, slot_off, row_base, b.xprev, b.from, b.id_from, b.s, b.t));
+            d.dst = b.to_stage ? (VC_SPACE_STAGE | vc_stage_addr(S, T, slot_off, row_base, info.x, to, id, b.s, b.t))
+                               : (VC_SPACE_RECV | vc_recv_offset(S, T, b.s, b.t));
+        }
+    } else {
+        // inter-node: `id` is the source rank s; the block waits on the rank of s's node that has
+        // the receiver's local index (src/twophase_twolayer_rbruck.cpp:430-453, 634-671)
+        const int s = id, t = to;
+        const int gs = s / n, gt = t / n, ls = s % n, lt = t % n;
+        if (gs != gt) {
+            const int q = ((gs - gt + S.G) % S.G) * n + ls;
+            if (q >= info.qlo && q < info.qhi) {
+                const int holder = gs * n + lt;
+                const int j = (ls - lt + n) % n;
+                d.len = (int64_t)T.sc[(int64_t)s * P + t] * S.esz;
+                d.from = holder;
+                if (j == 0) {
+                    d.src = VC_SPACE_SEND | vc_send_offset(S, T, s, t);
+                } else {
+                    const int xlast = S.msd ? vc_low_digit(j, S.r) : vc_top_digit(j, S.r);
+                    d.src = VC_SPACE_STAGE | vc_stage_addr(S, T, slot_off, row_base, xlast, holder, gt * n + ls, s, t);
+                }
+                d.dst = VC_SPACE_RECV | vc_recv_offset(S, T, s, t);
+            }
+        }
+    }
+    if (d.len == 0) d.from = -1;
+    return d;
+}

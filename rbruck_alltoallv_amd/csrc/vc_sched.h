@@ -1,0 +1,128 @@
+// vc_sched.h — host-side derivation of the schedule of one collective call: the
+// reference's clamping and validation of its tunables, the digit phases, and which
+// rounds share a kernel launch.  Plain C++ (no HIP calls) so that it can also be
+// compiled into a CPU-only check of the plan.
+#pragma once
+
+#include <algorithm>
+#include <cstring>
+#include <vector>
+
+#include "../../include/rbruck_vc.h"
+#include "vc_common.h"
+
+enum VcFunc {
+    VC_F_TWOPHASE,           // twophase_rbruck_alltoallv
+    VC_F_OM,                 // twophase_rbruck_alltoallv_om
+    VC_F_TUNA,               // tuna_algorithm
+    VC_F_TTPL,               // TTPL_BT_alltoallv
+    VC_F_TTPL_S1,            // TTPL_BT_alltoallv_s1
+    VC_F_UNIFORM_SPREADOUT,  // uniform_spreadout_twolayer
+    VC_F_UNIFORM_ISPLIT      // uniform_inverse_isplit_r_bruck
+};
+
+// Digits of span-1 in base r and the number of unused values of the top digit, in
+// integer arithmetic (src/tuna.cpp:28-31).  The float-log form of
+// src/twophase_tunable_rbruckv.cpp:30-32 gives the same rounds: where it differs it
+// adds a top digit with no rounds.
+inline void vc_radix_params(int span, int r, int &w, int &d) {
+    w = 0;
+    for (int top = span - 1; top; top /= r) w++;
+    int nlpow = 1;
+    for (int i = 0; i < w - 1; i++) nlpow *= r;
+    d = w ? (nlpow * r - span) / nlpow : 0;
+}
+
+// One launch per digit, or per `batch` rounds of a digit (TuNA's b, src/tuna.cpp:69).
+inline void vc_add_intra_launches(std::vector<VcLaunchInfo> &out, const VcSched &S, int d, int batch) {
+    for (int k = 0; k < S.w; k++) {
+        const int x = S.msd ? S.w - 1 - k : k;
+        int dist = 1;
+        for (int i = 0; i < x; i++) dist *= S.r;
+        const int ze = (x == S.w - 1) ? S.r - d : S.r;      // digit values 1 .. ze-1 occur
+        if (ze - 1 < 1) continue;
+        const int step = (batch <= 0 || batch > ze - 1) ? ze - 1 : batch;
+        for (int zlo = 1; zlo < ze; zlo += step) {
+            VcLaunchInfo li;
+            memset(&li, 0, sizeof li);
+            li.kind = 0; li.x = x; li.dist = dist; li.zlo = zlo; li.zhi = std::min(zlo + step - 1, ze - 1);
+            out.push_back(li);
+        }
+    }
+}
+
+// Inter-node messages, `qstep` (group distance, source local index) pairs per launch.
+inline void vc_add_inter_launches(std::vector<VcLaunchInfo> &out, const VcSched &S, int qstep) {
+    if (S.G <= 1) return;
+    if (qstep <= 0 || qstep > S.P) qstep = S.P;
+    for (int q = 0; q < S.P; q += qstep) {
+        VcLaunchInfo li;
+        memset(&li, 0, sizeof li);
+        li.kind = 1; li.x = -1; li.qlo = q; li.qhi = std::min(q + qstep, S.P);
+        out.push_back(li);
+    }
+}
+
+// Fills S and L for function f.  `r`, `batch` (b of tuna_algorithm, bblock of the TTPL functions) and `n`
+// are the caller's raw values.  Returns VC_OK or the code the entry point must return.
+inline int vc_make_schedule(VcFunc f, int P, int n, int r, int batch, int esz, int uniform_count, VcSched &S,
+                            std::vector<VcLaunchInfo> &L) {
+    memset(&S, 0, sizeof S);
+    L.clear();
+    S.P = P; S.esz = esz; S.uniform = uniform_count;
+    int d = 0;
+    switch (f) {
+    case VC_F_TWOPHASE:
+    case VC_F_OM:
+        if (r < 2) return VC_ERR_RADIX;                     // src/twophase_tunable_rbruckv.cpp:16, -om.cpp:13
+        if (r > P) r = P;                                   // :22, :19
+        S.n = P; S.G = 1; S.r = r; S.msd = (f == VC_F_TWOPHASE);
+        vc_radix_params(P, S.r, S.w, d);
+        vc_add_intra_launches(L, S, d, 0);
+        break;
+    case VC_F_TUNA:
+        if (P < 3) return VC_ERR_TOO_FEW_RANKS;             // src/tuna.cpp:20,28 never returns
+        if (r < 2) r = 2;                                   // :13
+        if (r > P - 1) r = P - 1;                           // :20
+        if (batch <= 0 || batch > P) batch = P;             // :21
+        S.n = P; S.G = 1; S.r = r; S.msd = 0;
+        vc_radix_params(P, S.r, S.w, d);
+        vc_add_intra_launches(L, S, d, batch);
+        break;
+    case VC_F_TTPL:
+    case VC_F_TTPL_S1:
+        if (r < 2) return VC_ERR_RADIX;                     // src/twophase_twolayer_rbruck.cpp:242, :472
+        if (n < 1 || P % n != 0) return VC_ERR_GROUP;       // the reference truncates P/n (:260) and hangs
+        if (r > n) r = n;                                   // :248
+        S.n = n; S.G = P / n; S.r = std::max(r, 2); S.msd = 0;
+        S.packed_recv = (f == VC_F_TTPL);                   // the coalesced variant never reads rdispls
+        vc_radix_params(n, S.r, S.w, d);
+        vc_add_intra_launches(L, S, d, 0);
+        if (f == VC_F_TTPL_S1) {
+            vc_add_inter_launches(L, S, (batch <= 0 || batch > P) ? P : batch);                 // :621
+        } else {
+            const int groups = (batch <= 0 || batch > S.G) ? S.G : batch;                      // :421
+            vc_add_inter_launches(L, S, groups * n);
+        }
+        break;
+    case VC_F_UNIFORM_SPREADOUT:
+    case VC_F_UNIFORM_ISPLIT:
+        if (f == VC_F_UNIFORM_SPREADOUT && r < 2) return VC_ERR_RADIX;   // src/twolayer_rbruck.cpp:12
+        if (r < 2) r = 2;                                                // :143
+        if (n < 2 || n >= P || P % n != 0) return VC_ERR_GROUP;          // :18-22, :145-149 MPI_Abort
+        if (r > n) r = n;
+        S.n = n; S.G = P / n; S.r = r; S.msd = 1;           // intra-node phase is most significant digit first (:69)
+        vc_radix_params(n, S.r, S.w, d);
+        vc_add_intra_launches(L, S, d, 0);
+        vc_add_inter_launches(L, S, P);                     // every group at once (:107-128; :243-274 with r2 = ngroup)
+        break;
+    }
+    if (L.empty()) {                                        // a single rank: only the copy to itself
+        VcLaunchInfo li;
+        memset(&li, 0, sizeof li);
+        li.kind = 0; li.dist = 1; li.zlo = 1; li.zhi = 0;
+        L.push_back(li);
+    }
+    L[0].self = 1;
+    return VC_OK;
+}

@@ -1,0 +1,93 @@
+"""Loads tests/plan_emulator.cpp (CPU build of the library's schedule + plan arithmetic) and exposes the
+reference's function names on numpy arenas, like oracle.oracle_py does for the oracle."""
+from __future__ import annotations
+
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+SRC = os.path.join(HERE, "plan_emulator.cpp")
+LIB = os.path.join(HERE, "_build", "libplan_emulator.so")
+CSRC = os.path.join(os.path.dirname(HERE), "rbruck_alltoallv_amd", "csrc")
+
+F_TWOPHASE, F_OM, F_TUNA, F_TTPL, F_TTPL_S1, F_UNIFORM_SPREADOUT, F_UNIFORM_ISPLIT = range(7)
+MAX_LAUNCHES = 64
+
+
+def build() -> str:
+    deps = [SRC] + [os.path.join(CSRC, f) for f in ("vc_plan_math.h", "vc_sched.h", "vc_common.h")]
+    if not os.path.exists(LIB) or os.path.getmtime(LIB) < max(os.path.getmtime(d) for d in deps):
+        os.makedirs(os.path.dirname(LIB), exist_ok=True)
+        subprocess.run(["/opt/rocm/bin/hipcc", "-O1", "-g", "-std=c++17", "-fPIC", "-shared", "-o", LIB, SRC],
+                       check=True, capture_output=True)
+    return LIB
+
+
+_lib = None
+
+
+def _p(a):
+    return a.ctypes.data_as(C.c_void_p) if a is not None else None
+
+
+class Result:
+    def __init__(self, rc, stats, traffic):
+        self.rc, self.nlaunch, self.stage_bytes, self.moved, self.errors = rc, int(stats[0]), int(stats[1]), int(stats[2]), int(stats[3])
+        self.traffic = traffic[: self.nlaunch] if rc == 0 else None
+
+
+def emulate(func, prob, send, recv, n=0, r=2, batch=0, uniform_count=0, recv_lo=0) -> Result:
+    global _lib
+    if _lib is None:
+        _lib = C.CDLL(build())
+    P = prob.P
+    stats = np.zeros(4, dtype=np.int64)
+    traffic = np.zeros((MAX_LAUNCHES, P, P), dtype=np.int64)
+    rc = _lib.plan_emulate(C.c_int(func), C.c_int(P), C.c_int(n), C.c_int(r), C.c_int(batch), C.c_int(prob.esz),
+                           C.c_int(uniform_count), _p(send), C.c_int64(send.size), _p(recv), C.c_int64(recv.size),
+                           _p(prob.sbase), _p(prob.rbase), _p(prob.sendcounts), _p(prob.sdispls), _p(prob.recvcounts),
+                           _p(prob.rdispls), C.c_int(recv_lo), _p(stats), _p(traffic), C.c_int(MAX_LAUNCHES))
+    return Result(rc, stats, traffic)
+
+
+# the reference's names, returning the return code and remembering the last Result
+last = None
+
+
+def _run(*a, **k):
+    global last
+    last = emulate(*a, **k)
+    if last.rc == 0 and last.errors:
+        return 1000 + last.errors
+    return last.rc
+
+
+def twophase_rbruck_alltoallv(r, prob, send, recv):
+    return _run(F_TWOPHASE, prob, send, recv, r=r)
+
+
+def twophase_rbruck_alltoallv_om(r, prob, send, recv):
+    return _run(F_OM, prob, send, recv, r=r)
+
+
+def tuna_algorithm(r, b, prob, send, recv):
+    return _run(F_TUNA, prob, send, recv, r=r, batch=b)
+
+
+def TTPL_BT_alltoallv(n, r, bblock, prob, send, recv):
+    return _run(F_TTPL, prob, send, recv, n=n, r=r, batch=bblock)
+
+
+def TTPL_BT_alltoallv_s1(n, r, bblock, prob, send, recv):
+    return _run(F_TTPL_S1, prob, send, recv, n=n, r=r, batch=bblock)
+
+
+def uniform_spreadout_twolayer(n, r, prob, count, send, recv):
+    return _run(F_UNIFORM_SPREADOUT, prob, send, recv, n=n, r=r, uniform_count=count)
+
+
+def uniform_inverse_isplit_r_bruck(n, r1, r2, prob, count, send, recv):
+    return _run(F_UNIFORM_ISPLIT, prob, send, recv, n=n, r=r1, uniform_count=count)

@@ -1,0 +1,115 @@
+// plan_emulator.cpp — CPU build of the library's schedule and plan arithmetic.
+//
+// Test infrastructure: compiles the SAME headers the GPU library uses
+// (csrc/vc_sched.h for the schedule, csrc/vc_plan_math.h for the per-entry index
+// arithmetic) as host code, replaces the three planning kernels by plain loops
+// and the copy kernel by memcpy, and checks every copy before doing it:
+//   - source and destination ranges lie inside their arenas,
+//   - staged bytes are read only after they were written,
+//   - within one launch no destination overlaps another destination or a source.
+// This is how indexing mistakes are found without a GPU.
+#include <algorithm>
+#include <cstdint>
+#include <cstdio>
+#include <cstring>
+#include <vector>
+
+#include "../rbruck_alltoallv_amd/csrc/vc_plan_math.h"
+#include "../rbruck_alltoallv_amd/csrc/vc_sched.h"
+
+struct Range { int64_t lo, hi; int space; };
+
+static int count_overlaps(std::vector<Range> &dst, std::vector<Range> &src) {
+    int bad = 0;
+    auto key = [](const Range &a, const Range &b) { return a.space != b.space ? a.space < b.space : a.lo < b.lo; };
+    std::sort(dst.begin(), dst.end(), key);
+    for (size_t i = 1; i < dst.size(); i++)
+        if (dst[i].space == dst[i - 1].space && dst[i].lo < dst[i - 1].hi) bad++;
+    for (const Range &s : src)
+        for (const Range &d : dst)
+            if (d.space == s.space && d.lo < s.hi && s.lo < d.hi) { bad++; break; }
+    return bad;
+}
+
+extern "C" int plan_emulate(int func, int P, int n, int r, int batch, int esz, int uniform_count, const char *send,
+                            int64_t send_bytes, char *recv, int64_t recv_bytes, const int64_t *sbase, const int64_t *rbase,
+                            const int *sc, const int *sd, const int *rc, const int *rd, int recv_lo, int64_t *stats_out,
+                            int64_t *traffic_out, int max_launches) {
+    VcSched S;
+    std::vector<VcLaunchInfo> L;
+    int code = vc_make_schedule((VcFunc)func, P, n, r, batch, esz, uniform_count, S, L);
+    if (code) return code;
+    S.recv_lo = recv_lo;
+    const int64_t PP = (int64_t)P * P;
+
+    std::vector<int> ucnt, udsp, rdp;
+    VcTables T;
+    T.sbase = sbase; T.rbase = rbase; T.rd_packed = nullptr;
+    if (uniform_count > 0 || func == VC_F_UNIFORM_SPREADOUT || func == VC_F_UNIFORM_ISPLIT) {
+        ucnt.assign(PP, uniform_count); udsp.resize(PP);
+        for (int64_t i = 0; i < PP; i++) udsp[i] = (int)(i % P) * uniform_count;
+        T.sc = T.rc = ucnt.data(); T.sd = T.rd = udsp.data();
+    } else {
+        T.sc = sc; T.sd = sd; T.rc = rc; T.rd = rd;
+    }
+    if (S.packed_recv) {
+        rdp.resize(PP);
+        for (int t = 0; t < P; t++) { int acc = 0; for (int s = 0; s < P; s++) { rdp[(int64_t)t * P + s] = acc; acc += T.rc[(int64_t)t * P + s]; } }
+        T.rd_packed = rdp.data();
+    }
+
+    // passes 1 and 2 of the planner
+    const int w = std::max(S.w, 1);
+    std::vector<int64_t> slot_off(PP * w, 0), row_base((int64_t)P * w, 0);
+    int64_t stage_bytes = 0;
+    for (int x = 0; x < S.w; x++) {
+        int dist = 1;
+        for (int k = 0; k < x; k++) dist *= S.r;
+        for (int to = 0; to < P; to++) {
+            row_base[(int64_t)x * P + to] = stage_bytes;
+            int64_t acc = 0;
+            for (int id = 0; id < P; id++) {
+                slot_off[((int64_t)x * P + to) * P + id] = acc;
+                acc += vc_stage_slot_size(S, T, x, dist, to, id);
+            }
+            stage_bytes += acc;
+        }
+    }
+    std::vector<char> stage((size_t)stage_bytes + 64, (char)0xCD);
+    std::vector<char> written((size_t)stage_bytes + 64, 0);
+
+    int64_t errors = 0, moved = 0;
+    const int nl = (int)L.size();
+    for (int k = 0; k < nl; k++) {
+        std::vector<VcDesc> descs;
+        std::vector<Range> dst_ranges, src_ranges;
+        for (int to = 0; to < P; to++)
+            for (int id = 0; id < P; id++) {
+                VcDesc d = vc_emit_entry(S, L[k], T, slot_off.data(), row_base.data(), to, id);
+                if (d.len <= 0) continue;
+                const int sspace = (int)(d.src >> VC_SPACE_SHIFT), dspace = (int)(d.dst >> VC_SPACE_SHIFT);
+                const int64_t so = d.src & VC_OFFSET_MASK, dof = d.dst & VC_OFFSET_MASK;
+                const int64_t slim = sspace == 0 ? send_bytes : (sspace == 2 ? stage_bytes : -1);
+                const int64_t dlim = dspace == 1 ? recv_bytes : (dspace == 2 ? stage_bytes : -1);
+                if (so < 0 || so + d.len > slim || dof < 0 || dof + d.len > dlim) { errors++; continue; }
+                if (d.from < 0 || d.from >= P || d.to != to) errors++;
+                if (sspace == 2)
+                    for (int64_t b = 0; b < d.len; b++) errors += !written[so + b];
+                descs.push_back(d);
+                dst_ranges.push_back({dof, dof + d.len, dspace});
+                src_ranges.push_back({so, so + d.len, sspace});
+                if (traffic_out && k < max_launches) traffic_out[((int64_t)k * P + d.from) * P + d.to] += d.len;
+            }
+        errors += count_overlaps(dst_ranges, src_ranges);
+        for (const VcDesc &d : descs) {
+            const int sspace = (int)(d.src >> VC_SPACE_SHIFT), dspace = (int)(d.dst >> VC_SPACE_SHIFT);
+            const char *from = (sspace == 0 ? send : stage.data()) + (d.src & VC_OFFSET_MASK);
+            char *to = (dspace == 1 ? recv : stage.data()) + (d.dst & VC_OFFSET_MASK);
+            memcpy(to, from, (size_t)d.len);
+            if (dspace == 2) memset(written.data() + (d.dst & VC_OFFSET_MASK), 1, (size_t)d.len);
+            moved += d.len;
+        }
+    }
+    stats_out[0] = nl; stats_out[1] = stage_bytes; stats_out[2] = moved; stats_out[3] = errors;
+    return 0;
+}

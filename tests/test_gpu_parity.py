@@ -1,0 +1,169 @@
+"""Parity of the HIP path with the oracle, through the C ABI, on a real MI355X (pytest -m gpu).
+
+Bit-exact bar: every byte of every virtual rank's receive arena — blocks and the untouched gaps between
+them — equals what the CPU oracle produced from the same seeded inputs; the per-rank digests equal the ones
+the real reference produced under mpiexec (tests/golden/golden.json)."""
+import numpy as np
+import pytest
+
+from oracle import oracle_py as O
+from rbruck_alltoallv_amd import workloads as W
+from tests.helpers import load_golden, problem_for_case, run_on
+
+pytestmark = pytest.mark.gpu
+
+CASES = load_golden()
+
+
+@pytest.fixture(scope="module")
+def api():
+    import torch
+    assert torch.cuda.is_available(), "these tests need the GPU"
+    from rbruck_alltoallv_amd import api as A
+    return A
+
+
+def _to_dev(api, arr):
+    import torch
+    return torch.from_numpy(arr).to("cuda:0")
+
+
+@pytest.mark.parametrize("case", CASES, ids=[c["id"] for c in CASES])
+def test_golden_case(api, case):
+    print("case", case["id"], flush=True)
+    prob = problem_for_case(case)
+    send = W.fill_send_arena(prob, case["payload"], case["seed"])
+    want = np.full(prob.recv_bytes, 0xEE, dtype=np.uint8)
+    assert run_on(O, case, prob, send.copy(), want) == 0
+    dp = api.DeviceProblem(prob)
+    dsend = dp.new_send_arena()
+    dp.fill_payload(case["payload"], case["seed"], dsend)            # the GPU fill must equal the host fill
+    assert np.array_equal(dsend.cpu().numpy(), send)
+    drecv = dp.new_recv_arena(0xEE)
+    rc = run_on(api, case, dp, dsend, drecv)
+    assert rc == 0, dp.comm.error()
+    got = drecv.cpu().numpy()
+    assert np.array_equal(got, want)
+    assert [f"{int(h):016x}" for h in O.digest_recv(prob, got)] == case["digests"]
+    assert np.array_equal(dsend.cpu().numpy(), send), "sendbuf must stay intact"
+    assert dp.verify(dsend, drecv, packed_recv=(case["func"] == "ttpl")) == 0
+    dp.comm.free()
+
+
+@pytest.mark.parametrize("P", [1, 2, 3, 5, 8, 12, 17, 27, 50])
+def test_flat_variants_odd_sizes(api, P):
+    print("flat P", P, flush=True)
+    for layout in (0, 1):
+        for esz in (1, 4):
+            counts = W.counts_uniform_random(P, 40, seed=P)
+            counts[counts % 4 == 0] = 0
+            prob = W.make_problem(counts, esz, layout, layout)
+            send = W.fill_send_arena(prob, 0, 5)
+            want = W.expected_recv_arena(prob, send)
+            dp = api.DeviceProblem(prob)
+            dsend = _to_dev(api, send)
+            for r in sorted({2, 3, 5, P, P + 3} - {1}):
+                for name, fn in (("twophase", lambda d: api.twophase_rbruck_alltoallv(r, dp, dsend, d)),
+                                 ("om", lambda d: api.twophase_rbruck_alltoallv_om(r, dp, dsend, d)),
+                                 ("tuna2", lambda d: api.tuna_algorithm(r, 2, dp, dsend, d)),
+                                 ("tunaP", lambda d: api.tuna_algorithm(r, 0, dp, dsend, d))):
+                    drecv = dp.new_recv_arena(0xEE)
+                    rc = fn(drecv)
+                    if name.startswith("tuna") and P < 3:
+                        assert rc == -3
+                        continue
+                    assert rc == 0, (name, P, r, dp.comm.error())
+                    assert np.array_equal(drecv.cpu().numpy(), want), (name, P, layout, esz, r)
+            dp.comm.free()
+
+
+def test_error_codes(api):
+    counts = W.counts_uniform_random(8, 9, seed=3)
+    prob = W.make_problem(counts, 4, 0, 0)
+    dp = api.DeviceProblem(prob)
+    s, d = dp.new_send_arena(), dp.new_recv_arena()
+    for r in (0, 1, -5):
+        assert api.twophase_rbruck_alltoallv(r, dp, s, d) == -1
+        assert api.twophase_rbruck_alltoallv_om(r, dp, s, d) == -1
+        assert api.TTPL_BT_alltoallv(4, r, 0, dp, s, d) == -1
+        assert api.TTPL_BT_alltoallv_s1(4, r, 0, dp, s, d) == -1
+        assert api.tuna_algorithm(r, 1, dp, s, d) == 0
+    assert api.TTPL_BT_alltoallv(3, 2, 0, dp, s, d) == -2
+    assert api.TTPL_BT_alltoallv_s1(5, 2, 0, dp, s, d) == -2
+    assert api.uniform_spreadout_twolayer(8, 2, dp, 1, s, d) == -2
+    assert api.uniform_spreadout_twolayer(4, 1, dp, 1, s, d) == -1
+    # without bases: a clear error instead of a wild access
+    c2 = api.VirtualComm(8)
+    rc = c2.lib.twophase_rbruck_alltoallv(2, s.data_ptr(), dp.sendcounts.data_ptr(), dp.sdispls.data_ptr(), 4, d.data_ptr(),
+                                          dp.recvcounts.data_ptr(), dp.rdispls.data_ptr(), 4, c2.handle)
+    assert rc == -5 and "bases" in c2.error()
+    c2.free()
+    dp.comm.free()
+
+
+def _oracle_traffic(rec, P, select):
+    m = np.zeros((P, P), dtype=np.int64)
+    for t in rec[select]:
+        m[int(t["src"]), int(t["dst"])] += int(t["bytes"])
+    return m
+
+
+@pytest.mark.parametrize("func,P,r", [("twophase", 27, 3), ("om", 64, 4), ("tuna", 30, 29), ("tuna", 17, 5)])
+def test_route_on_gpu_equals_oracle_trace(api, func, P, r):
+    """The launches of the GPU call carry, rank to rank, the bytes of the reference's rounds digit by digit."""
+    counts = W.counts_uniform_random(P, 20, seed=P * 7 + r)
+    counts[counts % 3 == 0] = 0
+    prob = W.make_problem(counts, 2, 0, 0)
+    send = W.fill_send_arena(prob, 0, 2)
+    recv = np.zeros(prob.recv_bytes, dtype=np.uint8)
+    ofn = {"twophase": lambda: O.twophase_rbruck_alltoallv(r, prob, send, recv),
+           "om": lambda: O.twophase_rbruck_alltoallv_om(r, prob, send, recv),
+           "tuna": lambda: O.tuna_algorithm(r, 0, prob, send, recv)}[func]
+    with O.trace() as t:
+        assert ofn() == 0
+    rec = t.records
+    dp = api.DeviceProblem(prob)
+    ds, dr = _to_dev(api, send), dp.new_recv_arena()
+    gfn = {"twophase": lambda: api.twophase_rbruck_alltoallv(r, dp, ds, dr),
+           "om": lambda: api.twophase_rbruck_alltoallv_om(r, dp, ds, dr),
+           "tuna": lambda: api.tuna_algorithm(r, 0, dp, ds, dr)}[func]
+    assert gfn() == 0
+    st = dp.comm.last_stats()
+    digits = list(dict.fromkeys(rec[rec["kind"] != 4]["digit"].tolist()))
+    assert st.n_launches == len(digits)
+    for k, x in enumerate(digits):
+        want = _oracle_traffic(rec, P, (rec["digit"] == x) & (rec["kind"] != 4))
+        if k == 0:
+            want += _oracle_traffic(rec, P, rec["kind"] == 4)
+        assert np.array_equal(dp.comm.last_traffic(k), want)
+        assert st.launch_bytes[k] == int(want.sum())
+    assert st.payload_bytes == prob.payload_bytes
+    assert st.moved_bytes * 2 == W.algorithmic_bytes(prob.sendcounts, prob.esz, W.hops_flat(P, min(r, P - 1) if func == "tuna" else r))
+    dp.comm.free()
+
+
+def test_caller_side_metadata_kernels(api):
+    """Count-matrix exchange (transpose), displacement prefix sums, bases and global maximum against numpy."""
+    import ctypes as C
+    import torch
+    for P in (1, 5, 32, 33, 100, 257, 1024):
+        counts = W.counts_uniform_random(P, 5000, seed=P)
+        comm = api.VirtualComm(P)
+        dc = _to_dev(api, counts)
+        out = torch.zeros_like(dc)
+        assert comm.lib.vc_alltoall_counts(dc.data_ptr(), out.data_ptr(), comm.handle) == 0
+        assert np.array_equal(out.cpu().numpy(), counts.T)
+        displs = torch.zeros_like(dc)
+        ext = torch.zeros(P, dtype=torch.int64, device="cuda:0")
+        assert comm.lib.vc_displs_from_counts(dc.data_ptr(), displs.data_ptr(), ext.data_ptr(), comm.handle) == 0
+        want_d, want_e = W.layout_displs(counts, 0)
+        assert np.array_equal(displs.cpu().numpy(), want_d) and np.array_equal(ext.cpu().numpy(), want_e)
+        base = torch.zeros(P, dtype=torch.int64, device="cuda:0")
+        tot = torch.zeros(1, dtype=torch.int64, device="cuda:0")
+        assert comm.lib.vc_bases_from_extents(ext.data_ptr(), 4, 256, base.data_ptr(), tot.data_ptr(), comm.handle) == 0
+        wb, wt = W.aligned_bases(want_e * 4, 256)
+        assert np.array_equal(base.cpu().numpy(), wb) and int(tot.item()) == wt
+        mx = torch.zeros(1, dtype=torch.int32, device="cuda:0")
+        assert comm.lib.vc_allreduce_max_count(dc.data_ptr(), mx.data_ptr(), comm.handle) == 0
+        assert int(mx.item()) == int(counts.max())
+        comm.free()

@@ -1,0 +1,156 @@
+"""Host logic of the product without a GPU: the schedule builder (csrc/vc_sched.h) and the per-entry plan
+arithmetic (csrc/vc_plan_math.h) compiled for the CPU (tests/plan_emulator.cpp), checked against the reference's
+golden digests, the textbook alltoallv and the oracle's message trace (the route)."""
+import numpy as np
+import pytest
+
+from oracle import oracle_py as O
+from rbruck_alltoallv_amd import workloads as W
+from tests import emulator as E
+from tests.helpers import load_golden, problem_for_case, run_on
+
+CASES = load_golden()
+
+
+@pytest.mark.parametrize("case", CASES, ids=[c["id"] for c in CASES])
+def test_plan_reproduces_reference_digests(case):
+    prob = problem_for_case(case)
+    send = W.fill_send_arena(prob, case["payload"], case["seed"])
+    recv = np.full(prob.recv_bytes, 0xEE, dtype=np.uint8)
+    keep = send.copy()
+    assert run_on(E, case, prob, send, recv) == 0
+    assert E.last.errors == 0
+    assert [f"{int(h):016x}" for h in O.digest_recv(prob, recv)] == case["digests"]
+    assert np.array_equal(recv, W.expected_recv_arena(prob, send))       # gaps between blocks stay untouched
+    assert np.array_equal(send, keep)
+
+
+def _prob(P, layout, esz, seed, recv_layout=None):
+    counts = W.counts_uniform_random(P, 9, seed=seed)
+    counts[counts % 4 == 0] = 0
+    return W.make_problem(counts, esz, layout, layout if recv_layout is None else recv_layout)
+
+
+@pytest.mark.parametrize("P", [1, 2, 3, 4, 5, 6, 7, 8, 9, 12, 16, 17, 27, 32, 50])
+def test_flat_plans_all_radices(P):
+    for layout in (0, 1):
+        for esz in (1, 4):
+            prob = _prob(P, layout, esz, seed=P)
+            send = W.fill_send_arena(prob, 0, 5)
+            want = W.expected_recv_arena(prob, send)
+            for r in sorted({2, 3, 4, 5, 8, P, P + 3, max(2, P - 1)} - {1}):
+                for name, fn in (("twophase", lambda d: E.twophase_rbruck_alltoallv(r, prob, send, d)),
+                                 ("om", lambda d: E.twophase_rbruck_alltoallv_om(r, prob, send, d)),
+                                 ("tuna1", lambda d: E.tuna_algorithm(r, 1, prob, send, d)),
+                                 ("tuna3", lambda d: E.tuna_algorithm(r, 3, prob, send, d)),
+                                 ("tunaP", lambda d: E.tuna_algorithm(r, 0, prob, send, d))):
+                    recv = np.full(prob.recv_bytes, 0xEE, dtype=np.uint8)
+                    rc = fn(recv)
+                    if name.startswith("tuna") and P < 3:
+                        assert rc == -3
+                        continue
+                    assert rc == 0 and E.last.errors == 0, (name, P, layout, esz, r, rc)
+                    assert np.array_equal(recv, want), (name, P, layout, esz, r)
+
+
+@pytest.mark.parametrize("P,n", [(4, 2), (6, 2), (6, 3), (8, 2), (8, 4), (9, 3), (12, 4), (16, 8), (32, 8), (8, 8), (8, 1), (27, 9)])
+def test_twolayer_plans(P, n):
+    for layout in (0, 1):
+        for esz in (1, 8):
+            for r in sorted({2, 3, 4, n, n + 1} - {1}):
+                for bblock in (0, 1, 3):
+                    for name, fn in (("ttpl", E.TTPL_BT_alltoallv), ("s1", E.TTPL_BT_alltoallv_s1)):
+                        prob = _prob(P, layout, esz, seed=P + 100, recv_layout=0 if name == "ttpl" else layout)
+                        send = W.fill_send_arena(prob, 0, 5)
+                        recv = np.full(prob.recv_bytes, 0xEE, dtype=np.uint8)
+                        assert fn(n, r, bblock, prob, send, recv) == 0, (name, layout, esz, r, bblock)
+                        assert np.array_equal(recv, W.expected_recv_arena(prob, send)), (name, layout, esz, r, bblock)
+
+
+def test_error_codes_match_the_oracle():
+    prob = _prob(8, 0, 4, seed=3)
+    send = W.fill_send_arena(prob, 0, 1)
+    recv = np.zeros(prob.recv_bytes, dtype=np.uint8)
+    for backend in (E, O):
+        for r in (0, 1, -5):
+            assert backend.twophase_rbruck_alltoallv(r, prob, send, recv) == -1
+            assert backend.twophase_rbruck_alltoallv_om(r, prob, send, recv) == -1
+            assert backend.TTPL_BT_alltoallv(4, r, 0, prob, send, recv) == -1
+            assert backend.TTPL_BT_alltoallv_s1(4, r, 0, prob, send, recv) == -1
+            assert backend.tuna_algorithm(r, 1, prob, send, recv) == 0
+        assert backend.TTPL_BT_alltoallv(3, 2, 0, prob, send, recv) == -2
+        assert backend.TTPL_BT_alltoallv_s1(5, 2, 0, prob, send, recv) == -2
+        up = W.make_uniform_problem(8, 2, 4)
+        us = W.fill_send_arena(up, 0, 1)
+        ur = np.zeros(up.recv_bytes, dtype=np.uint8)
+        assert backend.uniform_spreadout_twolayer(4, 1, up, 2, us.copy(), ur) == -1
+        assert backend.uniform_spreadout_twolayer(8, 2, up, 2, us.copy(), ur) == -2
+        assert backend.uniform_spreadout_twolayer(3, 2, up, 2, us.copy(), ur) == -2
+        assert backend.uniform_inverse_isplit_r_bruck(8, 2, 2, up, 2, us.copy(), ur) == -2
+    p2 = _prob(2, 0, 1, seed=1)
+    s2 = W.fill_send_arena(p2, 0, 1)
+    r2 = np.zeros(p2.recv_bytes, dtype=np.uint8)
+    assert E.tuna_algorithm(2, 1, p2, s2, r2) == O.tuna_algorithm(2, 1, p2, s2, r2) == -3
+
+
+def _oracle_traffic(rec, P, select):
+    m = np.zeros((P, P), dtype=np.int64)
+    for t in rec[select]:
+        m[int(t["src"]), int(t["dst"])] += int(t["bytes"])
+    return m
+
+
+@pytest.mark.parametrize("P,r", [(8, 2), (12, 3), (17, 5), (27, 3), (64, 4), (49, 7), (30, 29)])
+@pytest.mark.parametrize("func", ["twophase", "om", "tuna"])
+def test_route_equals_the_oracles_message_trace(P, r, func):
+    """Per digit phase, the bytes every rank sends to every other rank are those of the reference's rounds of
+    that digit — the plan really walks the Bruck route instead of gathering in one pass."""
+    counts = W.counts_uniform_random(P, 20, seed=P * 7 + r)
+    counts[counts % 3 == 0] = 0
+    prob = W.make_problem(counts, 2, 0, 0)
+    send = W.fill_send_arena(prob, 0, 2)
+    recv = np.zeros(prob.recv_bytes, dtype=np.uint8)
+    ofn = {"twophase": lambda: O.twophase_rbruck_alltoallv(r, prob, send, recv),
+           "om": lambda: O.twophase_rbruck_alltoallv_om(r, prob, send, recv),
+           "tuna": lambda: O.tuna_algorithm(r, 0, prob, send, recv)}[func]
+    with O.trace() as t:
+        assert ofn() == 0
+    rec = t.records
+    efn = {"twophase": lambda: E.twophase_rbruck_alltoallv(r, prob, send, recv),
+           "om": lambda: E.twophase_rbruck_alltoallv_om(r, prob, send, recv),
+           "tuna": lambda: E.tuna_algorithm(r, 0, prob, send, recv)}[func]
+    assert efn() == 0
+    res = E.last
+    digits = list(dict.fromkeys(rec[rec["kind"] != 4]["digit"].tolist()))      # order the oracle visited them
+    assert res.nlaunch == len(digits)
+    for k, x in enumerate(digits):
+        want = _oracle_traffic(rec, P, (rec["digit"] == x) & (rec["kind"] != 4))
+        if k == 0:
+            want += _oracle_traffic(rec, P, rec["kind"] == 4)                  # self copies ride in the first launch
+        assert np.array_equal(res.traffic[k], want), (func, x)
+    assert res.moved * 2 == W.algorithmic_bytes(prob.sendcounts, prob.esz, W.hops_flat(P, min(r, P - 1) if func == "tuna" else min(r, P)))
+
+
+@pytest.mark.parametrize("P,n,r", [(8, 4, 2), (12, 4, 2), (27, 9, 3), (64, 16, 4), (64, 32, 32), (16, 8, 3)])
+def test_twolayer_route_equals_the_oracles_trace(P, n, r):
+    counts = W.counts_uniform_random(P, 20, seed=P + n + r)
+    counts[counts % 3 == 0] = 0
+    prob = W.make_problem(counts, 1, 0, 0)
+    send = W.fill_send_arena(prob, 0, 2)
+    recv = np.zeros(prob.recv_bytes, dtype=np.uint8)
+    with O.trace() as t:
+        assert O.TTPL_BT_alltoallv_s1(n, r, 0, prob, send, recv) == 0
+    rec = t.records
+    assert E.TTPL_BT_alltoallv_s1(n, r, 0, prob, send, recv) == 0
+    res = E.last
+    digits = list(dict.fromkeys(rec[rec["kind"] == 0]["digit"].tolist()))
+    assert res.nlaunch == len(digits) + (1 if P > n else 0)
+    for k, x in enumerate(digits):
+        got = res.traffic[k].copy()
+        if k == 0:
+            got[np.arange(P), np.arange(P)] = 0                                  # self copies
+        # the staggered reference sends own-node finals inside the intra rounds too: identical matrices
+        assert np.array_equal(got, _oracle_traffic(rec, P, (rec["digit"] == x) & (rec["kind"] == 0))), x
+    if P > n:
+        assert np.array_equal(res.traffic[len(digits)], _oracle_traffic(rec, P, rec["kind"] == 3))
+    assert res.moved * 2 == W.algorithmic_bytes(prob.sendcounts, prob.esz, W.hops_twolayer(P, n, r))
