@@ -197,7 +197,7 @@ def main() -> None:
         "one_pass_floor_fraction": round(2 * S / (elapsed / args.steps) / 1e9 / HBM_PEAK_GBPS, 4),
         "plan_ms_per_step": round(plan_ms / args.steps, 4),
         "mismatched_bytes": int(bad),
-        "roofline": {"bound": "hbm", "kernel": "vc_copy_dense_kernel", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
+        "roofline": {"bound": "hbm", "kernel": "vc_copy_items_kernel", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
                      "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None,
                      "avg_launch_ms": round(kern_ms / max(nkern, 1), 4),
                      "algorithmic_bytes_per_launch": int(kern_bytes / max(nkern, 1))},

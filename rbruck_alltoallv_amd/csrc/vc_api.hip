@@ -63,12 +63,14 @@ struct vc_comm {
     hipStream_t stream = nullptr;
     const int64_t *sbase = nullptr, *rbase = nullptr;
     bool timing = false;
-    DevBuf slot_off, row_tot, row_base, desc, header, launches, stage, rd_packed, uni_counts, uni_displs, scratch;
+    DevBuf slot_off, row_tot, row_base, item_row_tot, item_row_base, row_bytes, desc, header, launches, stage, rd_packed,
+        uni_counts, uni_displs, scratch;
     int64_t *h_header = nullptr;          // pinned
     VcLaunchInfo *h_launches = nullptr;   // pinned
     std::vector<hipEvent_t> events;
     vc_stats_t stats;
     int last_nlaunch = 0;
+    int64_t launch_first[VC_MAX_LAUNCHES], launch_items[VC_MAX_LAUNCHES];   // work items of the last call
 };
 
 // ------------------------------------------------------------------ communicator
@@ -80,7 +82,7 @@ extern "C" int vc_comm_create(int nranks, vc_comm_t *comm_out) {
     vc_comm *c = new vc_comm();
     c->P = nranks;
     HIP_TRY(hipGetDevice(&c->device));
-    HIP_TRY(hipHostMalloc((void **)&c->h_header, sizeof(int64_t) * (2 + VC_MAX_LAUNCHES), hipHostMallocDefault));
+    HIP_TRY(hipHostMalloc((void **)&c->h_header, sizeof(int64_t) * VC_HEADER_WORDS(VC_MAX_LAUNCHES), hipHostMallocDefault));
     HIP_TRY(hipHostMalloc((void **)&c->h_launches, sizeof(VcLaunchInfo) * VC_MAX_LAUNCHES, hipHostMallocDefault));
     memset(&c->stats, 0, sizeof c->stats);
     *comm_out = c;
@@ -90,7 +92,7 @@ extern "C" int vc_comm_create(int nranks, vc_comm_t *comm_out) {
 extern "C" int vc_comm_free(vc_comm_t c) {
     if (!c) return VC_OK;
     (void)hipStreamSynchronize(c->stream);
-    for (DevBuf *b : {&c->slot_off, &c->row_tot, &c->row_base, &c->desc, &c->header, &c->launches, &c->stage, &c->rd_packed,
+    for (DevBuf *b : {&c->slot_off, &c->row_tot, &c->row_base, &c->item_row_tot, &c->item_row_base, &c->row_bytes, &c->desc, &c->header, &c->launches, &c->stage, &c->rd_packed,
                       &c->uni_counts, &c->uni_displs, &c->scratch})
         b->release();
     for (hipEvent_t e : c->events) (void)hipEventDestroy(e);
@@ -176,12 +178,15 @@ static int run_schedule(vc_comm *c, VcSched S, std::vector<VcLaunchInfo> &L, con
     if (nl > VC_MAX_LAUNCHES) return fail_arg("more than VC_MAX_LAUNCHES launches: raise b / bblock");
     hipStream_t st = c->stream;
     const size_t PP = (size_t)P * P;
+    const size_t wmax = (size_t)std::max(S.w, 1);
 
-    HIP_TRY(c->slot_off.reserve(sizeof(int64_t) * PP * std::max(S.w, 1)));
-    HIP_TRY(c->row_tot.reserve(sizeof(int64_t) * (size_t)P * std::max(S.w, 1)));
-    HIP_TRY(c->row_base.reserve(sizeof(int64_t) * (size_t)P * std::max(S.w, 1)));
-    HIP_TRY(c->desc.reserve(sizeof(VcDesc) * PP * nl));
-    HIP_TRY(c->header.reserve(sizeof(int64_t) * (2 + VC_MAX_LAUNCHES)));
+    HIP_TRY(c->slot_off.reserve(sizeof(int64_t) * PP * wmax));
+    HIP_TRY(c->row_tot.reserve(sizeof(int64_t) * (size_t)P * wmax));
+    HIP_TRY(c->row_base.reserve(sizeof(int64_t) * (size_t)P * wmax));
+    HIP_TRY(c->item_row_tot.reserve(sizeof(int64_t) * (size_t)P * nl));
+    HIP_TRY(c->item_row_base.reserve(sizeof(int64_t) * (size_t)P * nl));
+    HIP_TRY(c->row_bytes.reserve(sizeof(int64_t) * (size_t)P * (nl + 1)));
+    HIP_TRY(c->header.reserve(sizeof(int64_t) * VC_HEADER_WORDS(VC_MAX_LAUNCHES)));
     HIP_TRY(c->launches.reserve(sizeof(VcLaunchInfo) * VC_MAX_LAUNCHES));
     if (c->timing) { int rc = ensure_events(c, (size_t)nl + 4); if (rc) return rc; }
 
@@ -193,18 +198,23 @@ static int run_schedule(vc_comm *c, VcSched S, std::vector<VcLaunchInfo> &L, con
         HIP_TRY(vc_launch_row_scan(T.rc, c->rd_packed.as<int>(), nullptr, P, st));
         T.rd_packed = c->rd_packed.as<int>();
     }
-    HIP_TRY(vc_launch_plan(S, c->launches.as<VcLaunchInfo>(), nl, T, c->slot_off.as<int64_t>(), c->row_tot.as<int64_t>(),
-                           c->row_base.as<int64_t>(), c->desc.as<VcDesc>(), c->header.as<int64_t>(), st));
-    HIP_TRY(hipMemcpyAsync(c->h_header, c->header.p, sizeof(int64_t) * (2 + nl), hipMemcpyDeviceToHost, st));
-    if (c->timing) HIP_TRY(hipEventRecord(c->events[1], st));
-    HIP_TRY(hipStreamSynchronize(st));     // the staging arena is sized from the plan
+    HIP_TRY(vc_launch_plan_sizes(S, c->launches.as<VcLaunchInfo>(), nl, T, c->slot_off.as<int64_t>(), c->row_tot.as<int64_t>(),
+                                 c->row_base.as<int64_t>(), c->item_row_tot.as<int64_t>(), c->item_row_base.as<int64_t>(),
+                                 c->row_bytes.as<int64_t>(), c->header.as<int64_t>(), st));
+    HIP_TRY(hipMemcpyAsync(c->h_header, c->header.p, sizeof(int64_t) * VC_HEADER_WORDS(nl), hipMemcpyDeviceToHost, st));
+    HIP_TRY(hipStreamSynchronize(st));     // the staging arena and the item list are sized from the plan
 
-    const int64_t stage_bytes = c->h_header[0];
+    const int64_t *h = c->h_header;
+    const int64_t stage_bytes = h[0], nitems = h[2];
     HIP_TRY(c->stage.reserve((size_t)stage_bytes + 64));
+    HIP_TRY(c->desc.reserve(sizeof(VcDesc) * (size_t)std::max<int64_t>(nitems, 1)));
+    HIP_TRY(vc_launch_plan_emit(S, c->launches.as<VcLaunchInfo>(), nl, T, c->slot_off.as<int64_t>(), c->row_base.as<int64_t>(),
+                                c->item_row_base.as<int64_t>(), c->desc.as<VcDesc>(), st));
+    if (c->timing) HIP_TRY(hipEventRecord(c->events[1], st));
 
     for (int k = 0; k < nl; k++) {
         if (c->timing) HIP_TRY(hipEventRecord(c->events[2 + k], st));
-        HIP_TRY(vc_launch_copy_dense(c->desc.as<VcDesc>() + PP * k, (int64_t)PP, sendbuf, recvbuf, c->stage.as<char>(), st));
+        HIP_TRY(vc_launch_copy_items(c->desc.as<VcDesc>() + h[3 + nl + k], h[3 + 2 * nl + k], sendbuf, recvbuf, c->stage.as<char>(), st));
     }
     if (c->timing) HIP_TRY(hipEventRecord(c->events[2 + nl], st));
     HIP_TRY(hipStreamSynchronize(st));
@@ -213,13 +223,15 @@ static int run_schedule(vc_comm *c, VcSched S, std::vector<VcLaunchInfo> &L, con
     s.n_launches = nl;
     s.n_digits = S.w;
     s.staging_bytes = stage_bytes;
-    s.payload_bytes = c->h_header[1];
+    s.payload_bytes = h[1];
     s.moved_bytes = 0;
     s.plan_ms = s.total_ms = 0.f;
     for (int k = 0; k < nl; k++) {
-        s.launch_bytes[k] = c->h_header[2 + k];
+        s.launch_bytes[k] = h[3 + k];
         s.moved_bytes += s.launch_bytes[k];
         s.launch_ms[k] = 0.f;
+        c->launch_first[k] = h[3 + nl + k];
+        c->launch_items[k] = h[3 + 2 * nl + k];
         if (c->timing) HIP_TRY(hipEventElapsedTime(&s.launch_ms[k], c->events[2 + k], c->events[3 + k]));
     }
     if (c->timing) {
@@ -336,7 +348,8 @@ extern "C" int vc_comm_last_traffic(vc_comm_t c, int launch, int64_t *matrix_out
     const size_t PP = (size_t)c->P * c->P;
     HIP_TRY(c->scratch.reserve(sizeof(int64_t) * PP));
     HIP_TRY(hipMemsetAsync(c->scratch.p, 0, sizeof(int64_t) * PP, c->stream));
-    HIP_TRY(vc_launch_traffic(c->desc.as<VcDesc>() + PP * launch, (int64_t)PP, c->scratch.as<int64_t>(), c->P, c->stream));
+    HIP_TRY(vc_launch_traffic(c->desc.as<VcDesc>() + c->launch_first[launch], c->launch_items[launch], c->scratch.as<int64_t>(), c->P,
+                              c->stream));
     HIP_TRY(hipMemcpyAsync(matrix_out, c->scratch.p, sizeof(int64_t) * PP, hipMemcpyDeviceToHost, c->stream));
     HIP_TRY(hipStreamSynchronize(c->stream));
     return VC_OK;

@@ -12,6 +12,8 @@
 #include <stdint.h>
 
 #define VC_THREADS 256
+// bytes one workgroup of the copy kernel moves: 256 lanes x 2 vectors x 16 bytes
+#define VC_CHUNK 8192
 
 // Location of a byte range: which arena (top bits) and the byte offset inside it.
 #define VC_SPACE_SHIFT 60
@@ -74,10 +76,18 @@ hipError_t vc_launch_verify(const char *sendbuf, const char *recvbuf, VcTables t
 hipError_t vc_launch_uniform_tables(int *counts, int *displs, int count, int P, hipStream_t st);
 
 // vc_plan.hip
-// header layout (int64): [0] staging bytes, [1] payload bytes, [2 + L] bytes moved by launch L
-hipError_t vc_launch_plan(const VcSched &S, const VcLaunchInfo *launches_dev, int nlaunch, VcTables T, int64_t *slot_off,
-                          int64_t *row_tot, int64_t *row_base, VcDesc *desc, int64_t *header, hipStream_t st);
+// header layout (int64), nl = number of launches:
+//   [0] staging bytes   [1] payload bytes   [2] work items of all launches
+//   [3 + L] bytes moved by launch L   [3 + nl + L] first work item of launch L   [3 + 2 nl + L] its item count
+#define VC_HEADER_WORDS(nl) (3 + 3 * (nl))
+// Passes 1 and 2: staging prefix sums and the number of work items of every launch (sizes only).
+hipError_t vc_launch_plan_sizes(const VcSched &S, const VcLaunchInfo *launches_dev, int nlaunch, VcTables T, int64_t *slot_off,
+                                int64_t *row_tot, int64_t *row_base, int64_t *item_row_tot, int64_t *item_row_base,
+                                int64_t *row_bytes, int64_t *header, hipStream_t st);
+// Pass 3: writes the work items (needs the item buffer, sized from the header).
+hipError_t vc_launch_plan_emit(const VcSched &S, const VcLaunchInfo *launches_dev, int nlaunch, VcTables T, const int64_t *slot_off,
+                               const int64_t *row_base, const int64_t *item_row_base, VcDesc *items, hipStream_t st);
 hipError_t vc_launch_traffic(const VcDesc *desc, int64_t ndesc, int64_t *matrix, int P, hipStream_t st);
 
 // vc_copy.hip
-hipError_t vc_launch_copy_dense(const VcDesc *desc, int64_t ndesc, const char *sendbuf, char *recvbuf, char *stage, hipStream_t st);
+hipError_t vc_launch_copy_items(const VcDesc *items, int64_t nitems, const char *sendbuf, char *recvbuf, char *stage, hipStream_t st);

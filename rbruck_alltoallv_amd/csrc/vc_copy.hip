@@ -1,15 +1,28 @@
-// vc_copy.hip — the data movers.  A Bruck round on P virtual ranks is a set of
+// vc_copy.hip — the data mover.  A Bruck round on P virtual ranks is a set of
 // independent block copies inside HBM: the reference's pack (memcpy into
 // temp_send_buffer), MPI_Sendrecv and unpack (memcpy out of temp_recv_buffer)
 // (src/twophase_tunable_rbruckv.cpp:90-100,119,126-139) collapse into one read of
 // the block where the sender holds it and one write where the receiver wants it.
+//
+// Shape of the kernel, chosen by measurement on MI355X: one 256-lane workgroup per
+// work item (a piece of at most VC_CHUNK = 8 KiB of one block), every lane moving
+// up to two 16-byte vectors whose loads are both issued before the stores,
+// non-temporal on both sides (the data is touched once per hop).  Many small
+// workgroups beat persistent or wider ones for a plain copy on this chip, and the
+// same holds for the scattered variable-size blocks of an alltoallv.
 #include "vc_common.h"
 
-struct __attribute__((packed, aligned(1))) VcU128 { uint32_t a, b, c, d; };
+typedef unsigned int vc_u32x4 __attribute__((ext_vector_type(4)));
+struct __attribute__((packed, aligned(1))) VcU128 { vc_u32x4 v; };
 
-__device__ __forceinline__ uint4 vc_load16_unaligned(const char *p) {
-    VcU128 v = *reinterpret_cast<const VcU128 *>(p);
-    return make_uint4(v.a, v.b, v.c, v.d);
+// 16-byte load from any byte address (one global_load_dwordx4; the hardware handles the misalignment)
+__device__ __forceinline__ vc_u32x4 vc_load16(const char *p) {
+    return __builtin_nontemporal_load(&reinterpret_cast<const VcU128 *>(p)->v);
+}
+
+// 16-byte store to a 16-byte aligned address
+__device__ __forceinline__ void vc_store16(char *p, vc_u32x4 v) {
+    __builtin_nontemporal_store(v, reinterpret_cast<vc_u32x4 *>(p));
 }
 
 __device__ __forceinline__ char *vc_resolve(int64_t loc, const char *sendbuf, char *recvbuf, char *stage) {
@@ -19,33 +32,34 @@ __device__ __forceinline__ char *vc_resolve(int64_t loc, const char *sendbuf, ch
     return base + off;
 }
 
-// Copies len bytes with a whole workgroup: byte stores up to the first 16-byte
-// boundary of dst, then aligned 16-byte stores fed by (possibly unaligned)
-// 16-byte loads, then the tail.
-__device__ __forceinline__ void vc_copy_block(char *__restrict__ dst, const char *__restrict__ src, int64_t len) {
+// One workgroup per work item: byte stores up to the first 16-byte boundary of dst,
+// aligned 16-byte stores fed by (possibly unaligned) 16-byte loads, then the tail.
+__global__ __launch_bounds__(VC_THREADS) void vc_copy_items_kernel(const VcDesc *__restrict__ items, const char *__restrict__ sendbuf,
+                                                                   char *__restrict__ recvbuf, char *__restrict__ stage) {
+    const VcDesc d = items[blockIdx.x];
+    const int64_t len = d.len;
+    if (len <= 0) return;
+    const char *src = vc_resolve(d.src, sendbuf, recvbuf, stage);
+    char *dst = vc_resolve(d.dst, sendbuf, recvbuf, stage);
+    const int t = threadIdx.x;
     int64_t head = (16 - ((uintptr_t)dst & 15)) & 15;
     if (head > len) head = len;
-    if ((int64_t)threadIdx.x < head) dst[threadIdx.x] = src[threadIdx.x];
-    const int64_t nvec = (len - head) >> 4;
+    const int64_t nvec = (len - head) >> 4;                 // at most VC_CHUNK / 16 = 2 * VC_THREADS
     const char *s2 = src + head;
     char *d2 = dst + head;
-    for (int64_t i = threadIdx.x; i < nvec; i += VC_THREADS)
-        *reinterpret_cast<uint4 *>(d2 + (i << 4)) = vc_load16_unaligned(s2 + (i << 4));
+    vc_u32x4 v0, v1;
+    const bool has0 = t < nvec, has1 = t + VC_THREADS < nvec;
+    if (has0) v0 = vc_load16(s2 + ((int64_t)t << 4));
+    if (has1) v1 = vc_load16(s2 + ((int64_t)(t + VC_THREADS) << 4));
+    if (t < head) dst[t] = src[t];
     const int64_t done = head + (nvec << 4);
-    const int64_t tail = len - done;
-    if ((int64_t)threadIdx.x < tail) dst[done + threadIdx.x] = src[done + threadIdx.x];
+    if (t < len - done) dst[done + t] = src[done + t];
+    if (has0) vc_store16(d2 + ((int64_t)t << 4), v0);
+    if (has1) vc_store16(d2 + ((int64_t)(t + VC_THREADS) << 4), v1);
 }
 
-// One workgroup per descriptor; empty descriptors return at once.
-__global__ __launch_bounds__(VC_THREADS) void vc_copy_dense_kernel(const VcDesc *__restrict__ desc, const char *__restrict__ sendbuf,
-                                                                   char *__restrict__ recvbuf, char *__restrict__ stage) {
-    const VcDesc d = desc[blockIdx.x];
-    if (d.len <= 0) return;
-    vc_copy_block(vc_resolve(d.dst, sendbuf, recvbuf, stage), vc_resolve(d.src, sendbuf, recvbuf, stage), d.len);
-}
-
-hipError_t vc_launch_copy_dense(const VcDesc *desc, int64_t ndesc, const char *sendbuf, char *recvbuf, char *stage, hipStream_t st) {
-    if (ndesc <= 0) return hipSuccess;
-    hipLaunchKernelGGL(vc_copy_dense_kernel, dim3((unsigned)ndesc), dim3(VC_THREADS), 0, st, desc, sendbuf, recvbuf, stage);
+hipError_t vc_launch_copy_items(const VcDesc *items, int64_t nitems, const char *sendbuf, char *recvbuf, char *stage, hipStream_t st) {
+    if (nitems <= 0) return hipSuccess;
+    hipLaunchKernelGGL(vc_copy_items_kernel, dim3((unsigned)nitems), dim3(VC_THREADS), 0, st, items, sendbuf, recvbuf, stage);
     return hipGetLastError();
 }

@@ -1,85 +1,152 @@
-// vc_plan.hip — turns the count tables into the list of block copies of every
-// launch.
+// vc_plan.hip — turns the count tables into the work items of every launch.
 //
 // The reference learns the size of each incoming block from a metadata
 // MPI_Sendrecv before every data round ("two-phase", src/twophase_tunable_rbruckv.cpp:110).
 // With all P ranks' tables in one address space the size of a block is simply
-// sendcounts[s][t] of the (s, t) it belongs to, and which (s, t) sits in slot
-// `id` of rank p before digit x follows from the residency invariant:
-//   least significant digit first: s is (j mod r^x) ranks above the holder,
-//   most significant digit first:  s is (j div r^(x+1)) * r^(x+1) ranks above it.
-// Staging offsets (the reference's fixed-stride extra_buffer, :59) become
-// exclusive prefix sums over the blocks that arrive in a rank's staging area in a
-// digit phase, so the staging arena is compact.
+// sendcounts[s][t] of the (s, t) it belongs to, and which (s, t) sits in a slot
+// follows from the residency invariant (vc_plan_math.h).  Staging offsets (the
+// reference's fixed-stride extra_buffer, :59) become exclusive prefix sums over
+// the blocks that arrive in a rank's staging area in a digit phase, so the
+// staging arena is compact; a second family of prefix sums numbers the work
+// items (block pieces of at most VC_CHUNK bytes) so that every launch gets a
+// dense list with no empty entries.
 #include "vc_common.h"
 #include "vc_scan.h"
 
 #include "vc_plan_math.h"
 
-// ---- pass 1: per (digit, receiving rank) exclusive scan of the staging sizes ----
-// grid (P, w).  slot_off[(x*P + to)*P + id] = offset of the slot inside the row.
-__global__ __launch_bounds__(VC_THREADS) void vc_plan_stage_rows(VcSched S, VcTables T, int64_t *__restrict__ slot_off,
-                                                                 int64_t *__restrict__ row_tot) {
+// ---- pass 1: row-wise prefix sums ----
+// grid (P, w + nl).  Rows y < w: staging sizes of digit y, slot_off[(y*P + to)*P + id] = offset of the
+// slot inside the row.  Rows y >= w: work-item count, moved bytes (and, for the first launch, payload)
+// of launch y - w.
+__global__ __launch_bounds__(VC_THREADS) void vc_plan_rows(VcSched S, const VcLaunchInfo *__restrict__ launches, int nl, VcTables T,
+                                                           int64_t *__restrict__ slot_off, int64_t *__restrict__ row_tot,
+                                                           int64_t *__restrict__ item_row_tot, int64_t *__restrict__ row_bytes) {
     __shared__ int64_t lds[VC_WAVES_PER_BLOCK];
-    const int to = blockIdx.x, x = blockIdx.y, P = S.P;
-    int dist = 1;
-    for (int k = 0; k < x; k++) dist *= S.r;
-    int64_t carry = 0;
-    for (int base = 0; base < P; base += VC_THREADS) {
-        const int id = base + threadIdx.x;
-        int64_t total;
-        const int64_t v = (id < P) ? vc_stage_slot_size(S, T, x, dist, to, id) : 0;
-        int64_t ex = vc_block_exclusive_scan(v, lds, total);
-        if (id < P) slot_off[((int64_t)x * P + to) * P + id] = carry + ex;
-        carry += total;
+    const int to = blockIdx.x, P = S.P;
+    if ((int)blockIdx.y < S.w) {
+        const int x = blockIdx.y;
+        int dist = 1;
+        for (int k = 0; k < x; k++) dist *= S.r;
+        int64_t carry = 0;
+        for (int base = 0; base < P; base += VC_THREADS) {
+            const int id = base + threadIdx.x;
+            int64_t total;
+            const int64_t v = (id < P) ? vc_stage_slot_size(S, T, x, dist, to, id) : 0;
+            const int64_t ex = vc_block_exclusive_scan(v, lds, total);
+            if (id < P) slot_off[((int64_t)x * P + to) * P + id] = carry + ex;
+            carry += total;
+        }
+        if (threadIdx.x == 0) row_tot[(int64_t)x * P + to] = carry;
+        return;
     }
-    if (threadIdx.x == 0) row_tot[(int64_t)x * P + to] = carry;
+    const int L = blockIdx.y - S.w;
+    const VcLaunchInfo info = launches[L];
+    int64_t items = 0, bytes = 0, payload = 0;
+    for (int id = threadIdx.x; id < P; id += VC_THREADS) {
+        VcEntry e;
+        if (vc_entry_block(S, info, to, id, e)) {
+            const int64_t len = vc_entry_len(S, T, e);
+            items += vc_chunk_count(len);
+            bytes += len;
+        }
+        if (L == 0) payload += (int64_t)T.rc[(int64_t)to * P + id] * S.esz;
+    }
+    items = vc_block_sum(items, lds);
+    bytes = vc_block_sum(bytes, lds);
+    if (L == 0) payload = vc_block_sum(payload, lds);
+    if (threadIdx.x == 0) {
+        item_row_tot[(int64_t)L * P + to] = items;
+        row_bytes[(int64_t)L * P + to] = bytes;
+        if (L == 0) row_bytes[(int64_t)nl * P + to] = payload;
+    }
 }
 
-// ---- pass 2: exclusive scan of the row totals; one workgroup ----
-__global__ __launch_bounds__(VC_THREADS) void vc_plan_stage_bases(const int64_t *__restrict__ row_tot, int64_t *__restrict__ row_base,
-                                                                  int64_t nrows, int64_t *__restrict__ header, int nheader) {
+// ---- pass 2: prefix sums over the rows; one workgroup ----
+__global__ __launch_bounds__(VC_THREADS) void vc_plan_bases(int P, int w, int nl, const int64_t *__restrict__ row_tot,
+                                                            int64_t *__restrict__ row_base, const int64_t *__restrict__ item_row_tot,
+                                                            int64_t *__restrict__ item_row_base, const int64_t *__restrict__ row_bytes,
+                                                            int64_t *__restrict__ header) {
     __shared__ int64_t lds[VC_WAVES_PER_BLOCK];
     int64_t carry = 0;
+    const int64_t nrows = (int64_t)w * P;
     for (int64_t b0 = 0; b0 < nrows; b0 += VC_THREADS) {
-        int64_t i = b0 + threadIdx.x, total;
-        int64_t v = (i < nrows) ? row_tot[i] : 0;
-        int64_t ex = vc_block_exclusive_scan(v, lds, total);
+        const int64_t i = b0 + threadIdx.x;
+        int64_t total;
+        const int64_t v = (i < nrows) ? row_tot[i] : 0;
+        const int64_t ex = vc_block_exclusive_scan(v, lds, total);
         if (i < nrows) row_base[i] = carry + ex;
         carry += total;
     }
-    for (int i = threadIdx.x; i < nheader; i += VC_THREADS) header[i] = (i == 0) ? carry : 0;
+    if (threadIdx.x == 0) header[0] = carry;
+    int64_t icarry = 0;
+    for (int L = 0; L <= nl; L++) {          // L == nl: the payload row of launch 0
+        int64_t bytes = 0;
+        const int64_t first = icarry;
+        for (int b0 = 0; b0 < P; b0 += VC_THREADS) {
+            const int i = b0 + threadIdx.x;
+            int64_t total = 0;
+            bytes += (i < P) ? row_bytes[(int64_t)L * P + i] : 0;
+            if (L < nl) {
+                const int64_t v = (i < P) ? item_row_tot[(int64_t)L * P + i] : 0;
+                const int64_t ex = vc_block_exclusive_scan(v, lds, total);
+                if (i < P) item_row_base[(int64_t)L * P + i] = icarry + ex;
+                icarry += total;
+            }
+        }
+        bytes = vc_block_sum(bytes, lds);
+        if (threadIdx.x == 0) {
+            if (L < nl) {
+                header[3 + L] = bytes;
+                header[3 + nl + L] = first;
+                header[3 + 2 * nl + L] = icarry - first;
+            } else {
+                header[1] = bytes;
+                header[2] = icarry;
+            }
+        }
+    }
 }
 
-// ---- pass 3: one descriptor per (launch, receiving rank, slot) ----
-// grid (P, nlaunch).  Inactive entries get len = 0.
+// ---- pass 3: the work items ----
+// grid (P, nl).  Repeats the row scan of pass 1 to place every block's pieces.
 __global__ __launch_bounds__(VC_THREADS) void vc_plan_emit(VcSched S, const VcLaunchInfo *__restrict__ launches, VcTables T,
                                                            const int64_t *__restrict__ slot_off, const int64_t *__restrict__ row_base,
-                                                           VcDesc *__restrict__ desc, int64_t *__restrict__ header) {
+                                                           const int64_t *__restrict__ item_row_base, VcDesc *__restrict__ items) {
     __shared__ int64_t lds[VC_WAVES_PER_BLOCK];
     const int to = blockIdx.x, L = blockIdx.y, P = S.P;
     const VcLaunchInfo info = launches[L];
-    int64_t moved = 0, payload = 0;
-    for (int id = threadIdx.x; id < P; id += VC_THREADS) {
-        if (L == 0) payload += (int64_t)T.rc[(int64_t)to * P + id] * S.esz;
-        const VcDesc d = vc_emit_entry(S, info, T, slot_off, row_base, to, id);
-        moved += d.len;
-        desc[((int64_t)L * P + to) * P + id] = d;
-    }
-    moved = vc_block_sum(moved, lds);
-    if (threadIdx.x == 0 && moved) atomicAdd((unsigned long long *)&header[2 + L], (unsigned long long)moved);
-    if (L == 0) {
-        payload = vc_block_sum(payload, lds);
-        if (threadIdx.x == 0 && payload) atomicAdd((unsigned long long *)&header[1], (unsigned long long)payload);
+    int64_t carry = item_row_base[(int64_t)L * P + to];
+    for (int base = 0; base < P; base += VC_THREADS) {
+        const int id = base + threadIdx.x;
+        VcEntry e;
+        const bool active = id < P && vc_entry_block(S, info, to, id, e);
+        const int64_t len = active ? vc_entry_len(S, T, e) : 0;
+        const int64_t cnt = vc_chunk_count(len);
+        int64_t total;
+        const int64_t at = carry + vc_block_exclusive_scan(cnt, lds, total);
+        if (cnt) {
+            const VcDesc whole = vc_entry_desc(S, T, slot_off, row_base, e, to);
+            for (int64_t c = 0; c < cnt; c++) items[at + c] = vc_chunk_of(whole, c);
+        }
+        carry += total;
     }
 }
 
-hipError_t vc_launch_plan(const VcSched &S, const VcLaunchInfo *launches_dev, int nlaunch, VcTables T, int64_t *slot_off,
-                          int64_t *row_tot, int64_t *row_base, VcDesc *desc, int64_t *header, hipStream_t st) {
-    if (S.w > 0)
-        hipLaunchKernelGGL(vc_plan_stage_rows, dim3(S.P, S.w), dim3(VC_THREADS), 0, st, S, T, slot_off, row_tot);
-    hipLaunchKernelGGL(vc_plan_stage_bases, dim3(1), dim3(VC_THREADS), 0, st, row_tot, row_base, (int64_t)S.w * S.P, header, 2 + nlaunch);
-    hipLaunchKernelGGL(vc_plan_emit, dim3(S.P, nlaunch), dim3(VC_THREADS), 0, st, S, launches_dev, T, slot_off, row_base, desc, header);
+hipError_t vc_launch_plan_sizes(const VcSched &S, const VcLaunchInfo *launches_dev, int nlaunch, VcTables T, int64_t *slot_off,
+                                int64_t *row_tot, int64_t *row_base, int64_t *item_row_tot, int64_t *item_row_base,
+                                int64_t *row_bytes, int64_t *header, hipStream_t st) {
+    hipLaunchKernelGGL(vc_plan_rows, dim3(S.P, S.w + nlaunch), dim3(VC_THREADS), 0, st, S, launches_dev, nlaunch, T, slot_off, row_tot,
+                       item_row_tot, row_bytes);
+    hipLaunchKernelGGL(vc_plan_bases, dim3(1), dim3(VC_THREADS), 0, st, S.P, S.w, nlaunch, row_tot, row_base, item_row_tot,
+                       item_row_base, row_bytes, header);
+    return hipGetLastError();
+}
+
+hipError_t vc_launch_plan_emit(const VcSched &S, const VcLaunchInfo *launches_dev, int nlaunch, VcTables T, const int64_t *slot_off,
+                               const int64_t *row_base, const int64_t *item_row_base, VcDesc *items, hipStream_t st) {
+    hipLaunchKernelGGL(vc_plan_emit, dim3(S.P, nlaunch), dim3(VC_THREADS), 0, st, S, launches_dev, T, slot_off, row_base, item_row_base,
+                       items);
     return hipGetLastError();
 }
 

@@ -103,51 +103,70 @@ VC_HD int64_t vc_send_offset(const VcSched &S, const VcTables &T, int s, int t) 
     return T.sbase[s] + (int64_t)T.sd[(int64_t)s * S.P + t] * S.esz;
 }
 
-// The copy that entry (`to`, `id`) of a launch stands for; len = 0 if none.
-// Intra-node launches index by the receiver's slot, inter-node launches by the source rank.
-VC_HD VcDesc vc_emit_entry(const VcSched &S, const VcLaunchInfo &info, const VcTables &T, const int64_t *slot_off,
-                           const int64_t *row_base, int to, int id) {
-    const int P = S.P, n = S.n;
-    VcDesc d;
-    d.src = 0; d.dst = 0; d.len = 0; d.from = -1; d.to = to;
+// One entry of a launch before addresses are known: which block it moves and between which arenas.
+struct VcEntry {
+    int s, t;          // the block
+    int from;          // rank that holds it before the hop
+    int xprev;         // digit in which it arrived in `from`'s staging area (-1: still in sendbuf)
+    int id_from;       // its slot there
+    int xdst;          // digit phase whose staging region receives it (-1: it goes to recvbuf)
+    int id_to;         // its slot on the receiver
+};
+
+// Entry (`to`, `id`) of a launch: intra-node launches index by the receiver's slot, inter-node
+// launches by the source rank.  Returns false if the entry moves nothing in this launch.
+VC_HD bool vc_entry_block(const VcSched &S, const VcLaunchInfo &info, int to, int id, VcEntry &e) {
+    const int n = S.n;
     if (info.self && id == to) {
         // a rank's block to itself (src/twophase_tunable_rbruckv.cpp:63)
-        d.len = (int64_t)T.sc[(int64_t)to * P + to] * S.esz;
-        d.src = VC_SPACE_SEND | vc_send_offset(S, T, to, to);
-        d.dst = VC_SPACE_RECV | vc_recv_offset(S, T, to, to);
-        d.from = to;
-    } else if (info.kind == 0) {
-        VcBlock b;
-        if (vc_intra_block(S, info.x, info.dist, to, id, b) && b.z >= info.zlo && b.z <= info.zhi) {
-            d.len = (int64_t)T.sc[(int64_t)b.s * P + b.t] * S.esz;
-            d.from = b.from;
-            d.src = b.xprev < 0 ? (VC_SPACE_SEND | vc_send_offset(S, T, b.s, b.t))
-                                : (VC_SPACE_STAGE | vc_stage_addr(S, T, slot_off, row_base, b.xprev, b.from, b.id_from, b.s, b.t));
-            d.dst = b.to_stage ? (VC_SPACE_STAGE | vc_stage_addr(S, T, slot_off, row_base, info.x, to, id, b.s, b.t))
-                               : (VC_SPACE_RECV | vc_recv_offset(S, T, b.s, b.t));
-        }
-    } else {
-        // inter-node: `id` is the source rank s; the block waits on the rank of s's node that has
-        // the receiver's local index (src/twophase_twolayer_rbruck.cpp:430-453, 634-671)
-        const int s = id, t = to;
-        const int gs = s / n, gt = t / n, ls = s % n, lt = t % n;
-        if (gs != gt) {
-            const int q = ((gs - gt + S.G) % S.G) * n + ls;
-            if (q >= info.qlo && q < info.qhi) {
-                const int holder = gs * n + lt;
-                const int j = (ls - lt + n) % n;
-                d.len = (int64_t)T.sc[(int64_t)s * P + t] * S.esz;
-                d.from = holder;
-                if (j == 0) {
-                    d.src = VC_SPACE_SEND | vc_send_offset(S, T, s, t);
-                } else {
-                    const int xlast = S.msd ? vc_low_digit(j, S.r) : vc_top_digit(j, S.r);
-                    d.src = VC_SPACE_STAGE | vc_stage_addr(S, T, slot_off, row_base, xlast, holder, gt * n + ls, s, t);
-                }
-                d.dst = VC_SPACE_RECV | vc_recv_offset(S, T, s, t);
-            }
-        }
+        e.s = e.t = e.from = to; e.xprev = -1; e.id_from = id; e.xdst = -1; e.id_to = id;
+        return true;
     }
-    if (d.len == 0) d.from = -1;
+    if (info.kind == 0) {
+        VcBlock b;
+        if (!vc_intra_block(S, info.x, info.dist, to, id, b) || b.z < info.zlo || b.z > info.zhi) return false;
+        e.s = b.s; e.t = b.t; e.from = b.from; e.xprev = b.xprev; e.id_from = b.id_from;
+        e.xdst = b.to_stage ? info.x : -1; e.id_to = id;
+        return true;
+    }
+    // inter-node: `id` is the source rank s; the block waits on the rank of s's node that has
+    // the receiver's local index (src/twophase_twolayer_rbruck.cpp:430-453, 634-671)
+    const int s = id, t = to;
+    const int gs = s / n, gt = t / n, ls = s % n, lt = t % n;
+    if (gs == gt) return false;
+    const int q = ((gs - gt + S.G) % S.G) * n + ls;
+    if (q < info.qlo || q >= info.qhi) return false;
+    const int j = (ls - lt + n) % n;
+    e.s = s; e.t = t; e.from = gs * n + lt;
+    e.xprev = j == 0 ? -1 : (S.msd ? vc_low_digit(j, S.r) : vc_top_digit(j, S.r));
+    e.id_from = gt * n + ls; e.xdst = -1; e.id_to = id;
+    return true;
+}
+
+VC_HD int64_t vc_entry_len(const VcSched &S, const VcTables &T, const VcEntry &e) {
+    return (int64_t)T.sc[(int64_t)e.s * S.P + e.t] * S.esz;
+}
+
+// The whole-block copy an entry stands for.
+VC_HD VcDesc vc_entry_desc(const VcSched &S, const VcTables &T, const int64_t *slot_off, const int64_t *row_base,
+                           const VcEntry &e, int to) {
+    VcDesc d;
+    d.len = vc_entry_len(S, T, e);
+    d.from = e.from; d.to = to;
+    d.src = e.xprev < 0 ? (VC_SPACE_SEND | vc_send_offset(S, T, e.s, e.t))
+                        : (VC_SPACE_STAGE | vc_stage_addr(S, T, slot_off, row_base, e.xprev, e.from, e.id_from, e.s, e.t));
+    d.dst = e.xdst < 0 ? (VC_SPACE_RECV | vc_recv_offset(S, T, e.s, e.t))
+                       : (VC_SPACE_STAGE | vc_stage_addr(S, T, slot_off, row_base, e.xdst, to, e.id_to, e.s, e.t));
+    return d;
+}
+
+// Blocks are copied in pieces of at most VC_CHUNK bytes, one workgroup each.
+VC_HD int64_t vc_chunk_count(int64_t len) { return (len + VC_CHUNK - 1) / VC_CHUNK; }
+
+VC_HD VcDesc vc_chunk_of(const VcDesc &whole, int64_t c) {
+    VcDesc d = whole;
+    d.src += c * VC_CHUNK; d.dst += c * VC_CHUNK;
+    const int64_t left = whole.len - c * VC_CHUNK;
+    d.len = left < VC_CHUNK ? left : VC_CHUNK;
     return d;
 }

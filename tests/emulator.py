@@ -36,6 +36,7 @@ def _p(a):
 class Result:
     def __init__(self, rc, stats, traffic):
         self.rc, self.nlaunch, self.stage_bytes, self.moved, self.errors = rc, int(stats[0]), int(stats[1]), int(stats[2]), int(stats[3])
+        self.items = int(stats[4])
         self.traffic = traffic[: self.nlaunch] if rc == 0 else None
 
 
@@ -44,7 +45,7 @@ def emulate(func, prob, send, recv, n=0, r=2, batch=0, uniform_count=0, recv_lo=
     if _lib is None:
         _lib = C.CDLL(build())
     P = prob.P
-    stats = np.zeros(4, dtype=np.int64)
+    stats = np.zeros(5, dtype=np.int64)
     traffic = np.zeros((MAX_LAUNCHES, P, P), dtype=np.int64)
     rc = _lib.plan_emulate(C.c_int(func), C.c_int(P), C.c_int(n), C.c_int(r), C.c_int(batch), C.c_int(prob.esz),
                            C.c_int(uniform_count), _p(send), C.c_int64(send.size), _p(recv), C.c_int64(recv.size),

@@ -7,6 +7,7 @@
 //   - source and destination ranges lie inside their arenas,
 //   - staged bytes are read only after they were written,
 //   - within one launch no destination overlaps another destination or a source.
+// Blocks are split into the same VC_CHUNK pieces the copy kernel gets.
 // This is how indexing mistakes are found without a GPU.
 #include <algorithm>
 #include <cstdint>
@@ -78,15 +79,21 @@ extern "C" int plan_emulate(int func, int P, int n, int r, int batch, int esz, i
     std::vector<char> stage((size_t)stage_bytes + 64, (char)0xCD);
     std::vector<char> written((size_t)stage_bytes + 64, 0);
 
-    int64_t errors = 0, moved = 0;
+    int64_t errors = 0, moved = 0, items = 0;
     const int nl = (int)L.size();
     for (int k = 0; k < nl; k++) {
         std::vector<VcDesc> descs;
         std::vector<Range> dst_ranges, src_ranges;
         for (int to = 0; to < P; to++)
             for (int id = 0; id < P; id++) {
-                VcDesc d = vc_emit_entry(S, L[k], T, slot_off.data(), row_base.data(), to, id);
-                if (d.len <= 0) continue;
+                VcEntry e;
+                if (!vc_entry_block(S, L[k], to, id, e)) continue;
+                const VcDesc whole = vc_entry_desc(S, T, slot_off.data(), row_base.data(), e, to);
+                const int64_t nchunks = vc_chunk_count(whole.len);
+                items += nchunks;
+                for (int64_t c = 0; c < nchunks; c++) {
+                const VcDesc d = vc_chunk_of(whole, c);
+                if (d.len <= 0 || d.len > VC_CHUNK) { errors++; continue; }
                 const int sspace = (int)(d.src >> VC_SPACE_SHIFT), dspace = (int)(d.dst >> VC_SPACE_SHIFT);
                 const int64_t so = d.src & VC_OFFSET_MASK, dof = d.dst & VC_OFFSET_MASK;
                 const int64_t slim = sspace == 0 ? send_bytes : (sspace == 2 ? stage_bytes : -1);
@@ -99,6 +106,7 @@ extern "C" int plan_emulate(int func, int P, int n, int r, int batch, int esz, i
                 dst_ranges.push_back({dof, dof + d.len, dspace});
                 src_ranges.push_back({so, so + d.len, sspace});
                 if (traffic_out && k < max_launches) traffic_out[((int64_t)k * P + d.from) * P + d.to] += d.len;
+                }
             }
         errors += count_overlaps(dst_ranges, src_ranges);
         for (const VcDesc &d : descs) {
@@ -110,6 +118,6 @@ extern "C" int plan_emulate(int func, int P, int n, int r, int batch, int esz, i
             moved += d.len;
         }
     }
-    stats_out[0] = nl; stats_out[1] = stage_bytes; stats_out[2] = moved; stats_out[3] = errors;
+    stats_out[0] = nl; stats_out[1] = stage_bytes; stats_out[2] = moved; stats_out[3] = errors; stats_out[4] = items;
     return 0;
 }

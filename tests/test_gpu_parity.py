@@ -167,3 +167,30 @@ def test_caller_side_metadata_kernels(api):
         assert comm.lib.vc_allreduce_max_count(dc.data_ptr(), mx.data_ptr(), comm.handle) == 0
         assert int(mx.item()) == int(counts.max())
         comm.free()
+
+
+@pytest.mark.parametrize("layout", [0, 1])
+def test_large_blocks_split_into_pieces(api, layout):
+    """Blocks far above the 8 KiB work-item size, odd lengths and alignments, zeros in between."""
+    P = 12
+    counts = (W.counts_uniform_random(P, 70000, seed=11) * (W.counts_uniform_random(P, 3, seed=12) > 0)).astype(np.int32)
+    prob = W.make_problem(counts, 1, layout, layout)
+    send = W.fill_send_arena(prob, 0, 9)
+    want = W.expected_recv_arena(prob, send)
+    dp = api.DeviceProblem(prob)
+    ds = _to_dev(api, send)
+    for name, fn in (("twophase r=3", lambda d: api.twophase_rbruck_alltoallv(3, dp, ds, d)),
+                     ("om r=2", lambda d: api.twophase_rbruck_alltoallv_om(2, dp, ds, d)),
+                     ("tuna r=4 b=2", lambda d: api.tuna_algorithm(4, 2, dp, ds, d)),
+                     ("s1 n=4 r=2", lambda d: api.TTPL_BT_alltoallv_s1(4, 2, 3, dp, ds, d))):
+        dr = dp.new_recv_arena(0xEE)
+        assert fn(dr) == 0, (name, dp.comm.error())
+        assert np.array_equal(dr.cpu().numpy(), want), name
+    prob2 = W.make_problem(counts, 1, layout, 0)
+    dp2 = api.DeviceProblem(prob2)
+    send2 = W.fill_send_arena(prob2, 0, 9)
+    dr = dp2.new_recv_arena(0xEE)
+    assert api.TTPL_BT_alltoallv(6, 3, 1, dp2, _to_dev(api, send2), dr) == 0
+    assert np.array_equal(dr.cpu().numpy(), W.expected_recv_arena(prob2, send2))
+    dp.comm.free()
+    dp2.comm.free()

@@ -154,3 +154,18 @@ def test_twolayer_route_equals_the_oracles_trace(P, n, r):
     if P > n:
         assert np.array_equal(res.traffic[len(digits)], _oracle_traffic(rec, P, rec["kind"] == 3))
     assert res.moved * 2 == W.algorithmic_bytes(prob.sendcounts, prob.esz, W.hops_twolayer(P, n, r))
+
+
+def test_large_blocks_split_into_pieces():
+    P = 12
+    counts = (W.counts_uniform_random(P, 70000, seed=11) * (W.counts_uniform_random(P, 3, seed=12) > 0)).astype(np.int32)
+    for layout in (0, 1):
+        prob = W.make_problem(counts, 1, layout, layout)
+        send = W.fill_send_arena(prob, 0, 9)
+        want = W.expected_recv_arena(prob, send)
+        for fn in (lambda d: E.twophase_rbruck_alltoallv(3, prob, send, d), lambda d: E.tuna_algorithm(4, 2, prob, send, d),
+                   lambda d: E.TTPL_BT_alltoallv_s1(4, 2, 3, prob, send, d)):
+            recv = np.full(prob.recv_bytes, 0xEE, dtype=np.uint8)
+            assert fn(recv) == 0 and E.last.errors == 0
+            assert np.array_equal(recv, want)
+            assert E.last.items > P * P          # pieces, not blocks
