@@ -140,6 +140,8 @@ def main() -> None:
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-budget", type=float, default=150.0)
+    ap.add_argument("--calibration-copy", type=int, default=0, metavar="MiB",
+                    help="also run one plain copy of this many MiB before the timed region (for scaling rocprofv3 --pmc byte counters)")
     args = ap.parse_args()
     if args.gpus != 1:
         raise SystemExit("bench.py: this build runs the virtual communicator on ONE GPU; --gpus N with N > 1 is not supported")
@@ -160,12 +162,20 @@ def main() -> None:
     dp.fill_payload(0, args.seed, send)
     dp.comm.set_timing(True)
 
+    if args.calibration_copy:
+        nb = args.calibration_copy << 20
+        a = torch.zeros(nb, dtype=torch.uint8, device="cuda:0")
+        b = torch.zeros(nb, dtype=torch.uint8, device="cuda:0")
+        dp.comm._check(dp.comm.lib.vc_calibration_copy(b.data_ptr(), a.data_ptr(), nb, dp.comm.handle))
+        del a, b
+
     for _ in range(args.warmup):
         rc = call(api, func, tun, dp, send, recv)
         assert rc == 0, dp.comm.error()
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     kern_ms, kern_bytes, nkern, plan_ms = 0.0, 0, 0, 0.0
+    per_launch_ms = None
     for _ in range(args.steps):
         rc = call(api, func, tun, dp, send, recv)
         assert rc == 0, dp.comm.error()
@@ -175,6 +185,9 @@ def main() -> None:
             kern_bytes += 2 * st.launch_bytes[k]
             nkern += 1
         plan_ms += st.plan_ms
+        if st.n_launches <= 16:
+            now = [st.launch_ms[k] for k in range(st.n_launches)]
+            per_launch_ms = now if per_launch_ms is None else [a + b for a, b in zip(per_launch_ms, now)]
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
     st = dp.comm.last_stats()
@@ -200,7 +213,10 @@ def main() -> None:
         "roofline": {"bound": "hbm", "kernel": "vc_copy_items_kernel", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
                      "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None,
                      "avg_launch_ms": round(kern_ms / max(nkern, 1), 4),
-                     "algorithmic_bytes_per_launch": int(kern_bytes / max(nkern, 1))},
+                     "algorithmic_bytes_per_launch": int(kern_bytes / max(nkern, 1)),
+                     "per_launch": None if per_launch_ms is None else [
+                         {"ms": round(m / args.steps, 4), "GBps": round(2 * st.launch_bytes[k] / (m / args.steps) / 1e6, 1) if m > 0 else 0.0}
+                         for k, m in enumerate(per_launch_ms)]},
     }
     if not args.no_cpu_baseline:
         del send, recv

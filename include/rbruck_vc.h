@@ -151,6 +151,10 @@ int vc_verify_alltoallv(const char *sendbuf, const int *sendcounts, const int *s
                         const char *recvbuf, const int *recvcounts, const int *rdispls, int packed_recv,
                         int64_t *mismatch_out, vc_comm_t comm);
 
+/* Plain contiguous copy of nbytes (multiple of 16, 16-byte aligned pointers) with the same 16-byte non-temporal
+ * accesses the block mover uses: the transfer of known size against which hardware byte counters are scaled. */
+int vc_calibration_copy(char *dst, const char *src, int64_t nbytes, vc_comm_t comm);
+
 #ifdef __cplusplus
 }
 #endif

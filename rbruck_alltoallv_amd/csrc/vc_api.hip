@@ -387,3 +387,11 @@ extern "C" int vc_verify_alltoallv(const char *sendbuf, const int *sendcounts, c
     *mismatch_out = (int64_t)bad;
     return VC_OK;
 }
+
+extern "C" int vc_calibration_copy(char *dst, const char *src, int64_t nbytes, vc_comm_t c) {
+    if (!c || !dst || !src || nbytes < 0 || (nbytes & 15) || ((uintptr_t)dst & 15) || ((uintptr_t)src & 15))
+        return fail_arg("vc_calibration_copy: 16-byte aligned pointers and size needed");
+    HIP_TRY(vc_launch_calibration_copy(src, dst, nbytes, c->stream));
+    HIP_TRY(hipStreamSynchronize(c->stream));
+    return VC_OK;
+}

@@ -91,3 +91,4 @@ hipError_t vc_launch_traffic(const VcDesc *desc, int64_t ndesc, int64_t *matrix,
 
 // vc_copy.hip
 hipError_t vc_launch_copy_items(const VcDesc *items, int64_t nitems, const char *sendbuf, char *recvbuf, char *stage, hipStream_t st);
+hipError_t vc_launch_calibration_copy(const char *src, char *dst, int64_t nbytes, hipStream_t st);

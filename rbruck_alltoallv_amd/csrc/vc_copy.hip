@@ -63,3 +63,18 @@ hipError_t vc_launch_copy_items(const VcDesc *items, int64_t nitems, const char 
     hipLaunchKernelGGL(vc_copy_items_kernel, dim3((unsigned)nitems), dim3(VC_THREADS), 0, st, items, sendbuf, recvbuf, stage);
     return hipGetLastError();
 }
+
+// Plain contiguous copy of a known size: one 16-byte vector per lane, 4 KiB per workgroup.  It exists so that
+// hardware counters (bytes fetched / written per dispatch) can be scaled against a transfer whose size is known.
+__global__ __launch_bounds__(VC_THREADS) void vc_calibration_copy_kernel(const vc_u32x4 *__restrict__ src, vc_u32x4 *__restrict__ dst, int64_t nvec) {
+    const int64_t i = (int64_t)blockIdx.x * VC_THREADS + threadIdx.x;
+    if (i < nvec) __builtin_nontemporal_store(__builtin_nontemporal_load(&src[i]), &dst[i]);
+}
+
+hipError_t vc_launch_calibration_copy(const char *src, char *dst, int64_t nbytes, hipStream_t st) {
+    const int64_t nvec = nbytes / 16;
+    if (nvec <= 0) return hipSuccess;
+    hipLaunchKernelGGL(vc_calibration_copy_kernel, dim3((unsigned)((nvec + VC_THREADS - 1) / VC_THREADS)), dim3(VC_THREADS), 0, st,
+                       reinterpret_cast<const vc_u32x4 *>(src), reinterpret_cast<vc_u32x4 *>(dst), nvec);
+    return hipGetLastError();
+}
