@@ -29,6 +29,10 @@ sys.path.insert(0, ROOT)
 from rbruck_alltoallv_amd import workloads as W  # noqa: E402
 
 HBM_PEAK_GBPS = 8000.0
+# HBM bytes per launch of the copy kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, each scaled by what the same
+# counter reads for a plain copy of known size (profiles/vc_copy_items_kernel_C4_pmc_fetch_write.txt); counters cannot
+# be read from inside this process, so workloads that were not profiled report null.
+MEASURED_TRAFFIC_PER_LAUNCH = {("C4", "TTPL_BT_alltoallv"): 8757560657}
 METRIC = "effective alltoallv GB/s + % HBM peak, P=64..1024 virtual ranks, 1 GPU"
 
 
@@ -211,7 +215,8 @@ def main() -> None:
         "plan_ms_per_step": round(plan_ms / args.steps, 4),
         "mismatched_bytes": int(bad),
         "roofline": {"bound": "hbm", "kernel": "vc_copy_items_kernel", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
-                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None,
+                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
+                     "traffic": MEASURED_TRAFFIC_PER_LAUNCH.get((args.workload, func)),
                      "avg_launch_ms": round(kern_ms / max(nkern, 1), 4),
                      "algorithmic_bytes_per_launch": int(kern_bytes / max(nkern, 1)),
                      "per_launch": None if per_launch_ms is None else [
