@@ -113,6 +113,30 @@ int uniform_spreadout_twolayer(int n, int r, char *sendbuf, int sendcount, int s
 int uniform_inverse_isplit_r_bruck(int n, int r1, int r2, char *sendbuf, int sendcount, int sendtype_size,
                                    char *recvbuf, int recvcount, int recvtype_size, vc_comm_t comm);
 
+/* ---- the linear comparators the reference drivers time beside the Bruck variants
+ * (examples/twophaseLayer_example.cpp:99-113).  On one GPU each is a single pass: every block goes straight from
+ * its source's sendbuf to its destination's recvbuf.  Same argument order as the reference. ---- */
+
+/* src/MPICH_scattered.cpp:11-76 — bblock messages per rank in flight (here: bblock rank distances per launch). */
+int MPICH_intra_scattered(int bblock, char *sendbuf, int *sendcounts, int *sdispls, int sendtype_size, char *recvbuf,
+                          int *recvcounts, int *rdispls, int recvtype_size, vc_comm_t comm);
+
+/* src/OpenMPI_basic_linear.cpp:10-77 */
+int ompi_alltoallv_intra_basic_linear(char *sendbuf, int *sendcounts, int *sdispls, int sendtype_size, char *recvbuf,
+                                      int *recvcounts, int *rdispls, int recvtype_size, vc_comm_t comm);
+
+/* src/OpenMPI_pairwise.cpp:14-64 — the P pairwise steps are independent here and share one launch. */
+int ompi_alltoallv_intra_pairwise(char *sendbuf, int *sendcounts, int *sdispls, int sendtype_size, char *recvbuf,
+                                  int *recvcounts, int *rdispls, int recvtype_size, vc_comm_t comm);
+
+/* src/exclusive_or_alltoallv.cpp:12-51 (name as spelled there) — returns -1 unless P is a power of two (:31). */
+int exclisive_or_alltoallv(char *sendbuf, int *sendcounts, int *sdispls, int sendtype_size, char *recvbuf,
+                           int *recvcounts, int *rdispls, int recvtype_size, vc_comm_t comm);
+
+/* benchmarks/common.cpp:10-37 (declared in src/rbruckv.h:88-89; returns void there). */
+int spreadout_alltoallv(char *sendbuf, int *sendcounts, int *sdispls, int sendtype_size, char *recvbuf,
+                        int *recvcounts, int *rdispls, int recvtype_size, vc_comm_t comm);
+
 /* ---- measurement and inspection (the reference's global phase timers, src/rbruckv.h:13-18) ---- */
 
 #define VC_MAX_LAUNCHES 1024

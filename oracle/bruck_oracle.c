@@ -700,6 +700,79 @@ int ora_uniform_inverse_isplit_r_bruck(int n, int r1, int r2, char *sendarena, c
     return 0;
 }
 
+/* ------------------------------------------------ linear comparators -------
+ * One message per (source, destination) pair, straight between the user buffers.
+ * They differ only in the order and batching of the messages and in which empty
+ * messages are skipped. */
+
+static void direct_message(const ora_ctx *c, int from, int to, int step) {
+    int64_t nbytes = (int64_t)SC(c, from, to) * c->esz;
+    memcpy(rbuf(c, to) + (int64_t)RD(c, to, from) * c->esz, sbuf(c, from) + (int64_t)SD(c, from, to) * c->esz, (size_t)nbytes);
+    trace_msg(5, -1, step, from, to, 1, nbytes);
+}
+
+/* benchmarks/common.cpp:10-37: rank p receives from p+i and sends to p-i for i = 0..P-1, one Waitall. */
+int ora_spreadout_alltoallv(char *sendarena, const int64_t *sbase, const int *sendcounts, const int *sdispls, int esz,
+                            char *recvarena, const int64_t *rbase, const int *recvcounts, const int *rdispls, int P) {
+    ora_ctx c = make_ctx(sendarena, sbase, sendcounts, sdispls, esz, recvarena, rbase, recvcounts, rdispls, P);
+    for (int p = 0; p < P; p++)
+        for (int i = 0; i < P; i++) direct_message(&c, p, (p - i + P) % P, i);
+    return 0;
+}
+
+/* src/MPICH_scattered.cpp:31-70: the same pairs, bblock at a time, empty messages not posted. */
+int ora_MPICH_intra_scattered(int bblock, char *sendarena, const int64_t *sbase, const int *sendcounts, const int *sdispls,
+                              int esz, char *recvarena, const int64_t *rbase, const int *recvcounts, const int *rdispls, int P) {
+    ora_ctx c = make_ctx(sendarena, sbase, sendcounts, sdispls, esz, recvarena, rbase, recvcounts, rdispls, P);
+    if (bblock <= 0 || bblock > P) bblock = P;                        /* :31 */
+    for (int ii = 0; ii < P; ii += bblock) {
+        int ss = P - ii < bblock ? P - ii : bblock;
+        for (int p = 0; p < P; p++)
+            for (int i = 0; i < ss; i++) {
+                int dst = (p - i - ii + 2 * P) % P;                   /* :56 */
+                if (SC(&c, p, dst)) direct_message(&c, p, dst, i + ii);
+            }
+    }
+    return 0;
+}
+
+/* src/OpenMPI_basic_linear.cpp:10-77: memcpy to self, then all receives and all sends of non-empty messages. */
+int ora_ompi_alltoallv_intra_basic_linear(char *sendarena, const int64_t *sbase, const int *sendcounts, const int *sdispls,
+                                          int esz, char *recvarena, const int64_t *rbase, const int *recvcounts,
+                                          const int *rdispls, int P) {
+    ora_ctx c = make_ctx(sendarena, sbase, sendcounts, sdispls, esz, recvarena, rbase, recvcounts, rdispls, P);
+    self_copies(&c);                                                   /* :28-30 */
+    for (int p = 0; p < P; p++) if (SC(&c, p, p) < 0) return -1;       /* :32 */
+    for (int p = 0; p < P; p++)
+        for (int i = 0; i < P; i++)
+            if (i != p && SC(&c, p, i) > 0) direct_message(&c, p, i, (p - i + P) % P);
+    return 0;
+}
+
+/* src/OpenMPI_pairwise.cpp:32-58: step = 0..P-1, send to rank+step, receive from rank-step. */
+int ora_ompi_alltoallv_intra_pairwise(char *sendarena, const int64_t *sbase, const int *sendcounts, const int *sdispls,
+                                      int esz, char *recvarena, const int64_t *rbase, const int *recvcounts,
+                                      const int *rdispls, int P) {
+    ora_ctx c = make_ctx(sendarena, sbase, sendcounts, sdispls, esz, recvarena, rbase, recvcounts, rdispls, P);
+    for (int step = 0; step < P; step++)
+        for (int p = 0; p < P; p++) {
+            int to = (p + step) % P;
+            if (SC(&c, p, to) > 0) direct_message(&c, p, to, step);
+        }
+    return 0;
+}
+
+/* src/exclusive_or_alltoallv.cpp:12-51: partner = rank XOR step; only for P a power of two (:31). */
+int ora_exclisive_or_alltoallv(char *sendarena, const int64_t *sbase, const int *sendcounts, const int *sdispls, int esz,
+                               char *recvarena, const int64_t *rbase, const int *recvcounts, const int *rdispls, int P) {
+    ora_ctx c = make_ctx(sendarena, sbase, sendcounts, sdispls, esz, recvarena, rbase, recvcounts, rdispls, P);
+    int w = (int)ceil(log((double)P) / (float)log(2.0));              /* :25 */
+    if (P != ora_pow(2, (unsigned)w)) return -1;                       /* :31 */
+    for (int step = 0; step < P; step++)
+        for (int p = 0; p < P; p++) direct_message(&c, p, p ^ step, step);
+    return 0;
+}
+
 /* ------------------------------------------------------- payload + digests */
 
 void ora_fill_payload(int mode, uint64_t seed, char *sendarena, const int64_t *sbase, const int *sendcounts,

@@ -33,7 +33,7 @@ extern "C" {
  * Isend/Irecv pair, or an inter-node message). */
 typedef struct {
     int32_t kind;    /* 0 staged Bruck round, 1 direct single-block round, 2 inter-node coalesced,
-                        3 inter-node staggered, 4 self copy */
+                        3 inter-node staggered, 4 self copy, 5 direct message of a linear comparator */
     int32_t digit;   /* x for kind 0/1, -1 otherwise */
     int32_t z;       /* digit value of the round (kind 0/1), group distance otherwise */
     int32_t from, to;
@@ -90,6 +90,20 @@ int ora_uniform_spreadout_twolayer(int n, int r, char *sendarena, const int64_t 
 /* src/twolayer_rbruck.cpp:137-277 */
 int ora_uniform_inverse_isplit_r_bruck(int n, int r1, int r2, char *sendarena, const int64_t *sbase,
                                        int sendcount, int esz, char *recvarena, const int64_t *rbase, int P);
+
+/* The linear comparators (kind 5 in the trace: one direct message per pair; z = the step or distance). */
+int ora_spreadout_alltoallv(char *sendarena, const int64_t *sbase, const int *sendcounts, const int *sdispls, int esz,
+                            char *recvarena, const int64_t *rbase, const int *recvcounts, const int *rdispls, int P);   /* benchmarks/common.cpp:10-37 */
+int ora_MPICH_intra_scattered(int bblock, char *sendarena, const int64_t *sbase, const int *sendcounts, const int *sdispls,
+                              int esz, char *recvarena, const int64_t *rbase, const int *recvcounts, const int *rdispls, int P); /* src/MPICH_scattered.cpp:11-76 */
+int ora_ompi_alltoallv_intra_basic_linear(char *sendarena, const int64_t *sbase, const int *sendcounts, const int *sdispls,
+                                          int esz, char *recvarena, const int64_t *rbase, const int *recvcounts,
+                                          const int *rdispls, int P);                                              /* src/OpenMPI_basic_linear.cpp:10-77 */
+int ora_ompi_alltoallv_intra_pairwise(char *sendarena, const int64_t *sbase, const int *sendcounts, const int *sdispls,
+                                      int esz, char *recvarena, const int64_t *rbase, const int *recvcounts,
+                                      const int *rdispls, int P);                                                  /* src/OpenMPI_pairwise.cpp:14-64 */
+int ora_exclisive_or_alltoallv(char *sendarena, const int64_t *sbase, const int *sendcounts, const int *sdispls, int esz,
+                               char *recvarena, const int64_t *rbase, const int *recvcounts, const int *rdispls, int P);  /* src/exclusive_or_alltoallv.cpp:12-51 */
 
 /* Synthetic payload (oracle/vc_synth.h) written into every rank's send blocks. */
 void ora_fill_payload(int mode, uint64_t seed, char *sendarena, const int64_t *sbase, const int *sendcounts,

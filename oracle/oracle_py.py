@@ -84,6 +84,26 @@ def uniform_inverse_isplit_r_bruck(n, r1, r2, prob, count, send, recv):
                                                     C.c_int(prob.P))
 
 
+def MPICH_intra_scattered(bblock, prob, send, recv):
+    return lib().ora_MPICH_intra_scattered(C.c_int(bblock), *_v_args(prob, send, recv))
+
+
+def ompi_alltoallv_intra_basic_linear(prob, send, recv):
+    return lib().ora_ompi_alltoallv_intra_basic_linear(*_v_args(prob, send, recv))
+
+
+def ompi_alltoallv_intra_pairwise(prob, send, recv):
+    return lib().ora_ompi_alltoallv_intra_pairwise(*_v_args(prob, send, recv))
+
+
+def exclisive_or_alltoallv(prob, send, recv):
+    return lib().ora_exclisive_or_alltoallv(*_v_args(prob, send, recv))
+
+
+def spreadout_alltoallv(prob, send, recv):
+    return lib().ora_spreadout_alltoallv(*_v_args(prob, send, recv))
+
+
 def fill_payload(mode, seed, prob, send):
     lib().ora_fill_payload(C.c_int(mode), C.c_uint64(seed), _p(send), _p(prob.sbase), _p(prob.sendcounts),
                            _p(prob.sdispls), C.c_int(prob.esz), C.c_int(prob.P))

@@ -12,7 +12,8 @@
  * compared with MPI_Alltoallv.
  *
  * usage: mpiexec -n P ref_driver FUNC COUNTS ESZ R B N BBLOCK LAYOUT PAYLOAD SEED ITERS OUT
- *   FUNC    twophase | om | tuna | ttpl | ttpl_s1 | uniform_spreadout | uniform_isplit
+ *   FUNC    twophase | om | tuna | ttpl | ttpl_s1 | uniform_spreadout | uniform_isplit |
+ *           scattered | ompi_linear | ompi_pairwise | xor | spreadout | mpi_alltoallv
  *   COUNTS  file of P*P int32 (row = sender); for the uniform functions the decimal block count
  *   LAYOUT  0 packed ascending displacements, 1 reversed order with gaps
  *   OUT     prefix: OUT.digests (one hex FNV-1a per rank), OUT.recv.bin (all recv extents, rank
@@ -115,6 +116,11 @@ int main(int argc, char **argv) {
         else if (func == "ttpl_s1") ret = TTPL_BT_alltoallv_s1(n, r, bblock, sb, sc, sd, dtype, rb, rc, rd, dtype, MPI_COMM_WORLD);
         else if (func == "uniform_spreadout") ret = uniform_spreadout_twolayer(n, r, sb, sendcounts[0], dtype, rb, recvcounts[0], dtype, MPI_COMM_WORLD);
         else if (func == "uniform_isplit") uniform_inverse_isplit_r_bruck(n, r, b, sb, sendcounts[0], dtype, rb, recvcounts[0], dtype, MPI_COMM_WORLD);
+        else if (func == "scattered") ret = MPICH_intra_scattered(bblock, sb, sc, sd, dtype, rb, rc, rd, dtype, MPI_COMM_WORLD);
+        else if (func == "ompi_linear") ret = ompi_alltoallv_intra_basic_linear(sb, sc, sd, dtype, rb, rc, rd, dtype, MPI_COMM_WORLD);
+        else if (func == "ompi_pairwise") ret = ompi_alltoallv_intra_pairwise(sb, sc, sd, dtype, rb, rc, rd, dtype, MPI_COMM_WORLD);
+        else if (func == "xor") ret = exclisive_or_alltoallv(sb, sc, sd, dtype, rb, rc, rd, dtype, MPI_COMM_WORLD);
+        else if (func == "spreadout") spreadout_alltoallv(sb, sc, sd, dtype, rb, rc, rd, dtype, MPI_COMM_WORLD);
         else if (func == "mpi_alltoallv") ret = MPI_Alltoallv(sb, sc, sd, dtype, rb, rc, rd, dtype, MPI_COMM_WORLD);
         else { if (rank_ == 0) fprintf(stderr, "unknown FUNC %s\n", func.c_str()); MPI_Abort(MPI_COMM_WORLD, 2); }
         double el = MPI_Wtime() - st, mx = 0;

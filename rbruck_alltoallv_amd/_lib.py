@@ -40,6 +40,11 @@ SYMBOLS = {
     "TTPL_BT_alltoallv_s1": (_I, [_I, _I, _I] + _V_TAIL),
     "uniform_spreadout_twolayer": (_I, [_I, _I, _P, _I, _I, _P, _I, _I, _P]),
     "uniform_inverse_isplit_r_bruck": (_I, [_I, _I, _I, _P, _I, _I, _P, _I, _I, _P]),
+    "MPICH_intra_scattered": (_I, [_I] + _V_TAIL),
+    "ompi_alltoallv_intra_basic_linear": (_I, _V_TAIL),
+    "ompi_alltoallv_intra_pairwise": (_I, _V_TAIL),
+    "exclisive_or_alltoallv": (_I, _V_TAIL),
+    "spreadout_alltoallv": (_I, _V_TAIL),
     "vc_comm_set_timing": (_I, [_P, _I]),
     "vc_comm_last_stats": (_I, [_P, C.POINTER(VcStats)]),
     "vc_comm_last_traffic": (_I, [_P, _I, _P]),

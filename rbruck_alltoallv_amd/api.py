@@ -148,3 +148,28 @@ def uniform_inverse_isplit_r_bruck(n: int, r1: int, r2: int, p: DeviceProblem, c
     """src/twolayer_rbruck.cpp:137-277"""
     return p.comm.lib.uniform_inverse_isplit_r_bruck(n, r1, r2, send.data_ptr(), count, p.esz, recv.data_ptr(), count,
                                                      p.esz, p.comm.handle)
+
+
+def MPICH_intra_scattered(bblock: int, p: DeviceProblem, send: torch.Tensor, recv: torch.Tensor) -> int:
+    """src/MPICH_scattered.cpp:11-76"""
+    return p.comm.lib.MPICH_intra_scattered(bblock, *_tail(p, send, recv))
+
+
+def ompi_alltoallv_intra_basic_linear(p: DeviceProblem, send: torch.Tensor, recv: torch.Tensor) -> int:
+    """src/OpenMPI_basic_linear.cpp:10-77"""
+    return p.comm.lib.ompi_alltoallv_intra_basic_linear(*_tail(p, send, recv))
+
+
+def ompi_alltoallv_intra_pairwise(p: DeviceProblem, send: torch.Tensor, recv: torch.Tensor) -> int:
+    """src/OpenMPI_pairwise.cpp:14-64"""
+    return p.comm.lib.ompi_alltoallv_intra_pairwise(*_tail(p, send, recv))
+
+
+def exclisive_or_alltoallv(p: DeviceProblem, send: torch.Tensor, recv: torch.Tensor) -> int:
+    """src/exclusive_or_alltoallv.cpp:12-51"""
+    return p.comm.lib.exclisive_or_alltoallv(*_tail(p, send, recv))
+
+
+def spreadout_alltoallv(p: DeviceProblem, send: torch.Tensor, recv: torch.Tensor) -> int:
+    """benchmarks/common.cpp:10-37"""
+    return p.comm.lib.spreadout_alltoallv(*_tail(p, send, recv))

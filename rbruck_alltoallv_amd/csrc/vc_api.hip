@@ -204,12 +204,14 @@ static int run_schedule(vc_comm *c, VcSched S, std::vector<VcLaunchInfo> &L, con
     HIP_TRY(hipMemcpyAsync(c->h_header, c->header.p, sizeof(int64_t) * VC_HEADER_WORDS(nl), hipMemcpyDeviceToHost, st));
     HIP_TRY(hipStreamSynchronize(st));     // the staging arena and the item list are sized from the plan
 
-    const int64_t *h = c->h_header;
-    const int64_t stage_bytes = h[0], nitems = h[2];
+    int64_t *h = c->h_header;
+    int64_t nitems = 0;
+    for (int k = 0; k < nl; k++) { h[3 + nl + k] = nitems; nitems += h[3 + 2 * nl + k]; }     // first item of every launch
+    const int64_t stage_bytes = h[0];
     HIP_TRY(c->stage.reserve((size_t)stage_bytes + 64));
     HIP_TRY(c->desc.reserve(sizeof(VcDesc) * (size_t)std::max<int64_t>(nitems, 1)));
     HIP_TRY(vc_launch_plan_emit(S, c->launches.as<VcLaunchInfo>(), nl, T, c->slot_off.as<int64_t>(), c->row_base.as<int64_t>(),
-                                c->item_row_base.as<int64_t>(), c->desc.as<VcDesc>(), st));
+                                c->item_row_base.as<int64_t>(), c->header.as<int64_t>(), c->desc.as<VcDesc>(), st));
     if (c->timing) HIP_TRY(hipEventRecord(c->events[1], st));
 
     for (int k = 0; k < nl; k++) {
@@ -258,7 +260,7 @@ static VcTables make_tables(vc_comm *c, const int *sc, const int *sd, const int 
 
 static int schedule_error(int code) {
     switch (code) {
-    case VC_ERR_RADIX: g_last_error = "radix must be >= 2"; break;
+    case VC_ERR_RADIX: g_last_error = "radix must be >= 2 (exclisive_or_alltoallv: the rank count must be a power of 2)"; break;
     case VC_ERR_GROUP: g_last_error = "the ranks per node must divide the rank count (uniform functions: 2 <= n < P)"; break;
     case VC_ERR_TOO_FEW_RANKS: g_last_error = "tuna_algorithm needs at least 3 ranks"; break;
     default: break;
@@ -308,6 +310,38 @@ extern "C" int TTPL_BT_alltoallv_s1(int n, int r, int bblock, char *sendbuf, int
                                     char *recvbuf, int *recvcounts, int *rdispls, int recvtype_size, vc_comm_t c) {
     (void)recvtype_size;
     return run_v(VC_F_TTPL_S1, n, r, bblock, c, sendbuf, sendcounts, sdispls, sendtype_size, recvbuf, recvcounts, rdispls);
+}
+
+// The linear comparators (src/MPICH_scattered.cpp, src/OpenMPI_basic_linear.cpp, src/OpenMPI_pairwise.cpp,
+// src/exclusive_or_alltoallv.cpp, benchmarks/common.cpp): one hop per block.
+extern "C" int MPICH_intra_scattered(int bblock, char *sendbuf, int *sendcounts, int *sdispls, int sendtype_size, char *recvbuf,
+                                     int *recvcounts, int *rdispls, int recvtype_size, vc_comm_t c) {
+    (void)recvtype_size;
+    return run_v(VC_F_MPICH_SCATTERED, 0, 2, bblock, c, sendbuf, sendcounts, sdispls, sendtype_size, recvbuf, recvcounts, rdispls);
+}
+
+extern "C" int ompi_alltoallv_intra_basic_linear(char *sendbuf, int *sendcounts, int *sdispls, int sendtype_size, char *recvbuf,
+                                                 int *recvcounts, int *rdispls, int recvtype_size, vc_comm_t c) {
+    (void)recvtype_size;
+    return run_v(VC_F_OMPI_LINEAR, 0, 2, 0, c, sendbuf, sendcounts, sdispls, sendtype_size, recvbuf, recvcounts, rdispls);
+}
+
+extern "C" int ompi_alltoallv_intra_pairwise(char *sendbuf, int *sendcounts, int *sdispls, int sendtype_size, char *recvbuf,
+                                             int *recvcounts, int *rdispls, int recvtype_size, vc_comm_t c) {
+    (void)recvtype_size;
+    return run_v(VC_F_OMPI_PAIRWISE, 0, 2, 0, c, sendbuf, sendcounts, sdispls, sendtype_size, recvbuf, recvcounts, rdispls);
+}
+
+extern "C" int exclisive_or_alltoallv(char *sendbuf, int *sendcounts, int *sdispls, int sendtype_size, char *recvbuf,
+                                      int *recvcounts, int *rdispls, int recvtype_size, vc_comm_t c) {
+    (void)recvtype_size;
+    return run_v(VC_F_XOR, 0, 2, 0, c, sendbuf, sendcounts, sdispls, sendtype_size, recvbuf, recvcounts, rdispls);
+}
+
+extern "C" int spreadout_alltoallv(char *sendbuf, int *sendcounts, int *sdispls, int sendtype_size, char *recvbuf,
+                                   int *recvcounts, int *rdispls, int recvtype_size, vc_comm_t c) {
+    (void)recvtype_size;
+    return run_v(VC_F_SPREADOUT, 0, 2, 0, c, sendbuf, sendcounts, sdispls, sendtype_size, recvbuf, recvcounts, rdispls);
 }
 
 // The alltoall-shaped (equal blocks) functions: the count tables are implied.

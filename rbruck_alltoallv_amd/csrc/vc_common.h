@@ -48,11 +48,11 @@ struct VcSched {
 
 // One data-moving kernel launch.
 struct VcLaunchInfo {
-    int kind;      // 0: rounds of intra-node digit x with digit value in [zlo, zhi]; 1: inter-node messages
+    int kind;      // 0: rounds of intra-node digit x with digit value in [zlo, zhi]; 1: inter-node messages; 2: direct messages
     int x;         // digit
     int dist;      // r^x
     int zlo, zhi;
-    int qlo, qhi;  // inter-node: (group distance)*n + source local index in [qlo, qhi)
+    int qlo, qhi;  // inter-node: (group distance)*n + source local index in [qlo, qhi); direct: rank distance in [qlo, qhi)
     int self;      // also performs every rank's copy to itself
 };
 
@@ -77,8 +77,8 @@ hipError_t vc_launch_uniform_tables(int *counts, int *displs, int count, int P, 
 
 // vc_plan.hip
 // header layout (int64), nl = number of launches:
-//   [0] staging bytes   [1] payload bytes   [2] work items of all launches
-//   [3 + L] bytes moved by launch L   [3 + nl + L] first work item of launch L   [3 + 2 nl + L] its item count
+//   [0] staging bytes   [1] payload bytes   [2] unused
+//   [3 + L] bytes moved by launch L   [3 + nl + L] unused on the device   [3 + 2 nl + L] work items of launch L
 #define VC_HEADER_WORDS(nl) (3 + 3 * (nl))
 // Passes 1 and 2: staging prefix sums and the number of work items of every launch (sizes only).
 hipError_t vc_launch_plan_sizes(const VcSched &S, const VcLaunchInfo *launches_dev, int nlaunch, VcTables T, int64_t *slot_off,
@@ -86,7 +86,8 @@ hipError_t vc_launch_plan_sizes(const VcSched &S, const VcLaunchInfo *launches_d
                                 int64_t *row_bytes, int64_t *header, hipStream_t st);
 // Pass 3: writes the work items (needs the item buffer, sized from the header).
 hipError_t vc_launch_plan_emit(const VcSched &S, const VcLaunchInfo *launches_dev, int nlaunch, VcTables T, const int64_t *slot_off,
-                               const int64_t *row_base, const int64_t *item_row_base, VcDesc *items, hipStream_t st);
+                               const int64_t *row_base, const int64_t *item_row_base, const int64_t *header, VcDesc *items,
+                               hipStream_t st);
 hipError_t vc_launch_traffic(const VcDesc *desc, int64_t ndesc, int64_t *matrix, int P, hipStream_t st);
 
 // vc_copy.hip

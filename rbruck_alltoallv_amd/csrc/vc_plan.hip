@@ -62,61 +62,57 @@ __global__ __launch_bounds__(VC_THREADS) void vc_plan_rows(VcSched S, const VcLa
     }
 }
 
-// ---- pass 2: prefix sums over the rows; one workgroup ----
+// ---- pass 2: prefix sums over the rows ----
+// grid (nl + 1).  Workgroup L < nl: item bases of launch L's rows (relative to the launch's first item), its item
+// count and moved bytes.  Workgroup nl: staging row bases, staging bytes, payload bytes.
 __global__ __launch_bounds__(VC_THREADS) void vc_plan_bases(int P, int w, int nl, const int64_t *__restrict__ row_tot,
                                                             int64_t *__restrict__ row_base, const int64_t *__restrict__ item_row_tot,
                                                             int64_t *__restrict__ item_row_base, const int64_t *__restrict__ row_bytes,
                                                             int64_t *__restrict__ header) {
     __shared__ int64_t lds[VC_WAVES_PER_BLOCK];
-    int64_t carry = 0;
-    const int64_t nrows = (int64_t)w * P;
-    for (int64_t b0 = 0; b0 < nrows; b0 += VC_THREADS) {
-        const int64_t i = b0 + threadIdx.x;
-        int64_t total;
-        const int64_t v = (i < nrows) ? row_tot[i] : 0;
-        const int64_t ex = vc_block_exclusive_scan(v, lds, total);
-        if (i < nrows) row_base[i] = carry + ex;
-        carry += total;
-    }
-    if (threadIdx.x == 0) header[0] = carry;
-    int64_t icarry = 0;
-    for (int L = 0; L <= nl; L++) {          // L == nl: the payload row of launch 0
-        int64_t bytes = 0;
-        const int64_t first = icarry;
-        for (int b0 = 0; b0 < P; b0 += VC_THREADS) {
-            const int i = b0 + threadIdx.x;
-            int64_t total = 0;
-            bytes += (i < P) ? row_bytes[(int64_t)L * P + i] : 0;
-            if (L < nl) {
-                const int64_t v = (i < P) ? item_row_tot[(int64_t)L * P + i] : 0;
-                const int64_t ex = vc_block_exclusive_scan(v, lds, total);
-                if (i < P) item_row_base[(int64_t)L * P + i] = icarry + ex;
-                icarry += total;
-            }
+    const int L = blockIdx.x;
+    int64_t carry = 0, bytes = 0;
+    if (L == nl) {
+        const int64_t nrows = (int64_t)w * P;
+        for (int64_t b0 = 0; b0 < nrows; b0 += VC_THREADS) {
+            const int64_t i = b0 + threadIdx.x;
+            int64_t total;
+            const int64_t v = (i < nrows) ? row_tot[i] : 0;
+            const int64_t ex = vc_block_exclusive_scan(v, lds, total);
+            if (i < nrows) row_base[i] = carry + ex;
+            carry += total;
         }
+        for (int i = threadIdx.x; i < P; i += VC_THREADS) bytes += row_bytes[(int64_t)nl * P + i];
         bytes = vc_block_sum(bytes, lds);
-        if (threadIdx.x == 0) {
-            if (L < nl) {
-                header[3 + L] = bytes;
-                header[3 + nl + L] = first;
-                header[3 + 2 * nl + L] = icarry - first;
-            } else {
-                header[1] = bytes;
-                header[2] = icarry;
-            }
-        }
+        if (threadIdx.x == 0) { header[0] = carry; header[1] = bytes; }
+        return;
     }
+    for (int b0 = 0; b0 < P; b0 += VC_THREADS) {
+        const int i = b0 + threadIdx.x;
+        int64_t total;
+        const int64_t v = (i < P) ? item_row_tot[(int64_t)L * P + i] : 0;
+        const int64_t ex = vc_block_exclusive_scan(v, lds, total);
+        if (i < P) item_row_base[(int64_t)L * P + i] = carry + ex;
+        carry += total;
+        bytes += (i < P) ? row_bytes[(int64_t)L * P + i] : 0;
+    }
+    bytes = vc_block_sum(bytes, lds);
+    if (threadIdx.x == 0) { header[3 + L] = bytes; header[3 + 2 * nl + L] = carry; }
 }
 
 // ---- pass 3: the work items ----
 // grid (P, nl).  Repeats the row scan of pass 1 to place every block's pieces.
 __global__ __launch_bounds__(VC_THREADS) void vc_plan_emit(VcSched S, const VcLaunchInfo *__restrict__ launches, VcTables T,
                                                            const int64_t *__restrict__ slot_off, const int64_t *__restrict__ row_base,
-                                                           const int64_t *__restrict__ item_row_base, VcDesc *__restrict__ items) {
+                                                           const int64_t *__restrict__ item_row_base, const int64_t *__restrict__ header,
+                                                           int nl, VcDesc *__restrict__ items) {
     __shared__ int64_t lds[VC_WAVES_PER_BLOCK];
     const int to = blockIdx.x, L = blockIdx.y, P = S.P;
     const VcLaunchInfo info = launches[L];
-    int64_t carry = item_row_base[(int64_t)L * P + to];
+    int64_t first = 0;                                    // items of the launches before this one
+    for (int k = threadIdx.x; k < L; k += VC_THREADS) first += header[3 + 2 * nl + k];
+    first = vc_block_sum(first, lds);
+    int64_t carry = first + item_row_base[(int64_t)L * P + to];
     for (int base = 0; base < P; base += VC_THREADS) {
         const int id = base + threadIdx.x;
         VcEntry e;
@@ -138,15 +134,16 @@ hipError_t vc_launch_plan_sizes(const VcSched &S, const VcLaunchInfo *launches_d
                                 int64_t *row_bytes, int64_t *header, hipStream_t st) {
     hipLaunchKernelGGL(vc_plan_rows, dim3(S.P, S.w + nlaunch), dim3(VC_THREADS), 0, st, S, launches_dev, nlaunch, T, slot_off, row_tot,
                        item_row_tot, row_bytes);
-    hipLaunchKernelGGL(vc_plan_bases, dim3(1), dim3(VC_THREADS), 0, st, S.P, S.w, nlaunch, row_tot, row_base, item_row_tot,
+    hipLaunchKernelGGL(vc_plan_bases, dim3(nlaunch + 1), dim3(VC_THREADS), 0, st, S.P, S.w, nlaunch, row_tot, row_base, item_row_tot,
                        item_row_base, row_bytes, header);
     return hipGetLastError();
 }
 
 hipError_t vc_launch_plan_emit(const VcSched &S, const VcLaunchInfo *launches_dev, int nlaunch, VcTables T, const int64_t *slot_off,
-                               const int64_t *row_base, const int64_t *item_row_base, VcDesc *items, hipStream_t st) {
+                               const int64_t *row_base, const int64_t *item_row_base, const int64_t *header, VcDesc *items,
+                               hipStream_t st) {
     hipLaunchKernelGGL(vc_plan_emit, dim3(S.P, nlaunch), dim3(VC_THREADS), 0, st, S, launches_dev, T, slot_off, row_base, item_row_base,
-                       items);
+                       header, nlaunch, items);
     return hipGetLastError();
 }
 

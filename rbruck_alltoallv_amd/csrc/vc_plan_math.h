@@ -117,6 +117,14 @@ struct VcEntry {
 // launches by the source rank.  Returns false if the entry moves nothing in this launch.
 VC_HD bool vc_entry_block(const VcSched &S, const VcLaunchInfo &info, int to, int id, VcEntry &e) {
     const int n = S.n;
+    if (info.kind == 2) {
+        // direct: `id` is the source rank; launches are batches of the distance (source - destination) mod P
+        // (src/MPICH_scattered.cpp:44-45: receive from rank + i + ii)
+        const int q = (id - to + S.P) % S.P;
+        if (q < info.qlo || q >= info.qhi) return false;
+        e.s = id; e.t = to; e.from = id; e.xprev = -1; e.id_from = to; e.xdst = -1; e.id_to = id;
+        return true;
+    }
     if (info.self && id == to) {
         // a rank's block to itself (src/twophase_tunable_rbruckv.cpp:63)
         e.s = e.t = e.from = to; e.xprev = -1; e.id_from = id; e.xdst = -1; e.id_to = id;

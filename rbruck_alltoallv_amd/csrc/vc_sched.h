@@ -18,7 +18,14 @@ enum VcFunc {
     VC_F_TTPL,               // TTPL_BT_alltoallv
     VC_F_TTPL_S1,            // TTPL_BT_alltoallv_s1
     VC_F_UNIFORM_SPREADOUT,  // uniform_spreadout_twolayer
-    VC_F_UNIFORM_ISPLIT      // uniform_inverse_isplit_r_bruck
+    VC_F_UNIFORM_ISPLIT,     // uniform_inverse_isplit_r_bruck
+    // the linear comparators the reference times next to the Bruck variants: every block goes straight from
+    // its source's sendbuf to its destination's recvbuf
+    VC_F_SPREADOUT,          // spreadout_alltoallv
+    VC_F_MPICH_SCATTERED,    // MPICH_intra_scattered
+    VC_F_OMPI_LINEAR,        // ompi_alltoallv_intra_basic_linear
+    VC_F_OMPI_PAIRWISE,      // ompi_alltoallv_intra_pairwise
+    VC_F_XOR                 // exclisive_or_alltoallv
 };
 
 // Digits of span-1 in base r and the number of unused values of the top digit, in
@@ -59,6 +66,17 @@ inline void vc_add_inter_launches(std::vector<VcLaunchInfo> &out, const VcSched 
         VcLaunchInfo li;
         memset(&li, 0, sizeof li);
         li.kind = 1; li.x = -1; li.qlo = q; li.qhi = std::min(q + qstep, S.P);
+        out.push_back(li);
+    }
+}
+
+// Direct (one-hop) messages, `qstep` rank distances (source - destination) mod P per launch.
+inline void vc_add_direct_launches(std::vector<VcLaunchInfo> &out, int P, int qstep) {
+    if (qstep <= 0 || qstep > P) qstep = P;
+    for (int q = 0; q < P; q += qstep) {
+        VcLaunchInfo li;
+        memset(&li, 0, sizeof li);
+        li.kind = 2; li.x = -1; li.qlo = q; li.qhi = std::min(q + qstep, P);
         out.push_back(li);
     }
 }
@@ -116,6 +134,19 @@ inline int vc_make_schedule(VcFunc f, int P, int n, int r, int batch, int esz, i
         vc_add_intra_launches(L, S, d, 0);
         vc_add_inter_launches(L, S, P);                     // every group at once (:107-128; :243-274 with r2 = ngroup)
         break;
+    case VC_F_XOR:
+        if ((P & (P - 1)) != 0) return VC_ERR_RADIX;        // src/exclusive_or_alltoallv.cpp:31 returns -1 unless P is a power of 2
+        /* fall through */
+    case VC_F_SPREADOUT:                                    // benchmarks/common.cpp:10-37: all 2P requests, one Waitall
+    case VC_F_OMPI_LINEAR:                                  // src/OpenMPI_basic_linear.cpp:10-77: self copy, then everything at once
+    case VC_F_OMPI_PAIRWISE:                                // src/OpenMPI_pairwise.cpp:32-58: P steps; independent, so one launch
+        S.n = P; S.G = 1; S.r = 2; S.msd = 0; S.w = 0;
+        vc_add_direct_launches(L, P, P);
+        break;
+    case VC_F_MPICH_SCATTERED:                              // src/MPICH_scattered.cpp:31-70: bblock requests in flight
+        S.n = P; S.G = 1; S.r = 2; S.msd = 0; S.w = 0;
+        vc_add_direct_launches(L, P, (batch <= 0 || batch > P) ? P : batch);
+        break;
     }
     if (L.empty()) {                                        // a single rank: only the copy to itself
         VcLaunchInfo li;
@@ -123,6 +154,6 @@ inline int vc_make_schedule(VcFunc f, int P, int n, int r, int batch, int esz, i
         li.kind = 0; li.dist = 1; li.zlo = 1; li.zhi = 0;
         L.push_back(li);
     }
-    L[0].self = 1;
+    if (L[0].kind != 2) L[0].self = 1;                      // direct launches carry the self block as distance 0
     return VC_OK;
 }

@@ -13,7 +13,8 @@ SRC = os.path.join(HERE, "plan_emulator.cpp")
 LIB = os.path.join(HERE, "_build", "libplan_emulator.so")
 CSRC = os.path.join(os.path.dirname(HERE), "rbruck_alltoallv_amd", "csrc")
 
-F_TWOPHASE, F_OM, F_TUNA, F_TTPL, F_TTPL_S1, F_UNIFORM_SPREADOUT, F_UNIFORM_ISPLIT = range(7)
+F_TWOPHASE, F_OM, F_TUNA, F_TTPL, F_TTPL_S1, F_UNIFORM_SPREADOUT, F_UNIFORM_ISPLIT, F_SPREADOUT, F_MPICH_SCATTERED, \
+    F_OMPI_LINEAR, F_OMPI_PAIRWISE, F_XOR = range(12)
 MAX_LAUNCHES = 64
 
 
@@ -92,3 +93,23 @@ def uniform_spreadout_twolayer(n, r, prob, count, send, recv):
 
 def uniform_inverse_isplit_r_bruck(n, r1, r2, prob, count, send, recv):
     return _run(F_UNIFORM_ISPLIT, prob, send, recv, n=n, r=r1, uniform_count=count)
+
+
+def MPICH_intra_scattered(bblock, prob, send, recv):
+    return _run(F_MPICH_SCATTERED, prob, send, recv, batch=bblock)
+
+
+def ompi_alltoallv_intra_basic_linear(prob, send, recv):
+    return _run(F_OMPI_LINEAR, prob, send, recv)
+
+
+def ompi_alltoallv_intra_pairwise(prob, send, recv):
+    return _run(F_OMPI_PAIRWISE, prob, send, recv)
+
+
+def exclisive_or_alltoallv(prob, send, recv):
+    return _run(F_XOR, prob, send, recv)
+
+
+def spreadout_alltoallv(prob, send, recv):
+    return _run(F_SPREADOUT, prob, send, recv)

@@ -92,6 +92,11 @@ def cases() -> list[dict]:
         add(f"zeros-{f}", f, zz, 4, r=2, b=1)
     add("zeros-ttpl", "ttpl", zz, 4, r=2, n=4)
     add("zeros-ttpl_s1", "ttpl_s1", zz, 4, r=2, n=4)
+    # linear comparators
+    for P in (8, 12, 32):
+        cg = dict(kind="uniform_random", P=P, hi=30, seed=P + 5, sparsify=4)
+        for f in ("scattered", "ompi_linear", "ompi_pairwise", "spreadout") + (("xor",) if P & (P - 1) == 0 else ()):
+            add(f"cmp-P{P}-{f}", f, cg, 4, bblock=3, layout=1)
     # uniform two-layer functions
     for P, n, r in ((16, 4, 2), (16, 4, 3), (16, 4, 4), (12, 3, 2), (64, 8, 4), (64, 16, 3)):
         add(f"uni-spread-P{P}-n{n}-r{r}", "uniform_spreadout", None, 4, r=r, n=n, count=5)

@@ -64,6 +64,16 @@ def run_on(backend, case: dict, prob: W.Problem, send, recv) -> int:
         return backend.uniform_spreadout_twolayer(case["n"], case["r"], prob, case["count"], send, recv)
     if f == "uniform_isplit":
         return backend.uniform_inverse_isplit_r_bruck(case["n"], case["r"], case["b"], prob, case["count"], send, recv)
+    if f == "scattered":
+        return backend.MPICH_intra_scattered(case["bblock"], prob, send, recv)
+    if f == "ompi_linear":
+        return backend.ompi_alltoallv_intra_basic_linear(prob, send, recv)
+    if f == "ompi_pairwise":
+        return backend.ompi_alltoallv_intra_pairwise(prob, send, recv)
+    if f == "xor":
+        return backend.exclisive_or_alltoallv(prob, send, recv)
+    if f == "spreadout":
+        return backend.spreadout_alltoallv(prob, send, recv)
     raise ValueError(f)
 
 

@@ -194,3 +194,31 @@ def test_large_blocks_split_into_pieces(api, layout):
     assert np.array_equal(dr.cpu().numpy(), W.expected_recv_arena(prob2, send2))
     dp.comm.free()
     dp2.comm.free()
+
+
+@pytest.mark.parametrize("P", [1, 5, 8, 32])
+def test_linear_comparators(api, P):
+    for layout in (0, 1):
+        counts = W.counts_uniform_random(P, 3000, seed=P + 40)
+        counts[counts % 4 == 0] = 0
+        prob = W.make_problem(counts, 2, layout, layout)
+        send = W.fill_send_arena(prob, 0, 3)
+        want = W.expected_recv_arena(prob, send)
+        dp = api.DeviceProblem(prob)
+        ds = _to_dev(api, send)
+        for name, fn in (("spreadout", lambda d: api.spreadout_alltoallv(dp, ds, d)),
+                         ("linear", lambda d: api.ompi_alltoallv_intra_basic_linear(dp, ds, d)),
+                         ("pairwise", lambda d: api.ompi_alltoallv_intra_pairwise(dp, ds, d)),
+                         ("xor", lambda d: api.exclisive_or_alltoallv(dp, ds, d)),
+                         ("scattered3", lambda d: api.MPICH_intra_scattered(3, dp, ds, d)),
+                         ("scattered0", lambda d: api.MPICH_intra_scattered(0, dp, ds, d))):
+            dr = dp.new_recv_arena(0xEE)
+            rc = fn(dr)
+            if name == "xor" and P & (P - 1):
+                assert rc == -1
+                continue
+            assert rc == 0, (name, dp.comm.error())
+            assert np.array_equal(dr.cpu().numpy(), want), (name, P, layout)
+            st = dp.comm.last_stats()
+            assert st.moved_bytes == prob.payload_bytes
+        dp.comm.free()

@@ -203,3 +203,34 @@ def test_route_of_twolayer_variants(P, n, r, func):
     cross = int(prob.sendcounts[(s // n) != (t // n)].astype(np.int64).sum()) * prob.esz
     own = int(prob.sendcounts[(s // n) == (t // n)].astype(np.int64).sum()) * prob.esz
     assert int(inter["bytes"].sum()) == cross + (own if func == "ttpl" else 0)
+
+
+@pytest.mark.parametrize("P", [1, 2, 3, 4, 5, 8, 12, 16, 27, 32])
+def test_linear_comparators_equal_textbook_alltoallv(P):
+    """src/MPICH_scattered.cpp, OpenMPI_basic_linear.cpp, OpenMPI_pairwise.cpp, exclusive_or_alltoallv.cpp,
+    benchmarks/common.cpp: one direct message per pair."""
+    for layout in (0, 1):
+        prob = _prob(P, layout, 2, seed=P + 40)
+        send = W.fill_send_arena(prob, W.PAYLOAD_HASH, 3)
+        want = W.expected_recv_arena(prob, send)
+        fns = {"spreadout": lambda d: O.spreadout_alltoallv(prob, send, d),
+               "linear": lambda d: O.ompi_alltoallv_intra_basic_linear(prob, send, d),
+               "pairwise": lambda d: O.ompi_alltoallv_intra_pairwise(prob, send, d),
+               "xor": lambda d: O.exclisive_or_alltoallv(prob, send, d)}
+        for bb in (0, 1, 3, P + 5):
+            fns[f"scattered{bb}"] = lambda d, bb=bb: O.MPICH_intra_scattered(bb, prob, send, d)
+        for name, fn in fns.items():
+            recv = np.full(prob.recv_bytes, 0xEE, dtype=np.uint8)
+            with O.trace() as t:
+                rc = fn(recv)
+            if name == "xor" and P & (P - 1):
+                assert rc == -1                     # exclusive_or_alltoallv.cpp:31
+                continue
+            assert rc == 0
+            assert np.array_equal(recv, want), (name, P, layout)
+            rec = t.records
+            direct = rec[rec["kind"] == 5]
+            # every non-empty pair exactly once, one hop: total traffic = payload
+            assert int(rec["bytes"].sum()) == prob.payload_bytes
+            pairs = set(zip(direct["src"].tolist(), direct["dst"].tolist()))
+            assert len(pairs) == len(direct)

@@ -169,3 +169,33 @@ def test_large_blocks_split_into_pieces():
             assert fn(recv) == 0 and E.last.errors == 0
             assert np.array_equal(recv, want)
             assert E.last.items > P * P          # pieces, not blocks
+
+
+@pytest.mark.parametrize("P", [1, 2, 5, 8, 12, 32])
+def test_linear_comparator_plans(P):
+    for layout in (0, 1):
+        counts = W.counts_uniform_random(P, 30, seed=P + 40)
+        counts[counts % 4 == 0] = 0
+        prob = W.make_problem(counts, 2, layout, layout)
+        send = W.fill_send_arena(prob, 0, 3)
+        want = W.expected_recv_arena(prob, send)
+        for name, fn, launches in (("spreadout", lambda d: E.spreadout_alltoallv(prob, send, d), 1),
+                                   ("linear", lambda d: E.ompi_alltoallv_intra_basic_linear(prob, send, d), 1),
+                                   ("pairwise", lambda d: E.ompi_alltoallv_intra_pairwise(prob, send, d), 1),
+                                   ("xor", lambda d: E.exclisive_or_alltoallv(prob, send, d), 1),
+                                   ("scattered3", lambda d: E.MPICH_intra_scattered(3, prob, send, d), -(-P // 3)),
+                                   ("scattered0", lambda d: E.MPICH_intra_scattered(0, prob, send, d), 1)):
+            recv = np.full(prob.recv_bytes, 0xEE, dtype=np.uint8)
+            rc = fn(recv)
+            if name == "xor" and P & (P - 1):
+                assert rc == -1
+                continue
+            assert rc == 0 and E.last.errors == 0, (name, P)
+            assert np.array_equal(recv, want), (name, P, layout)
+            assert E.last.nlaunch == launches
+            assert E.last.moved == prob.payload_bytes            # one hop per block
+            if name == "scattered3":
+                # launch k carries the rank distances 3k .. 3k+2, like the reference's batches (MPICH_scattered.cpp:38-45)
+                for k in range(E.last.nlaunch):
+                    src, dst = np.nonzero(E.last.traffic[k])
+                    assert np.all(((src - dst) % P >= 3 * k) & ((src - dst) % P < 3 * k + 3))
