@@ -37,7 +37,14 @@ METRIC = "effective alltoallv GB/s + % HBM peak, P=64..1024 virtual ranks, 1 GPU
 
 
 def workload(name: str, seed: int):
-    """(counts, esz, function name, tunables, hop matrix) of a BASELINE configuration."""
+    """(counts, esz, function name, tunables, hop matrix) of a BASELINE configuration, or of one of the reference's
+    own communication-pattern matrices (ML<P>: inputs/<P>proc, 1-byte elements, twophase_rbruck_alltoallv as in
+    examples/MLinputs_example.cpp:96)."""
+    if name.startswith("ML"):
+        P = int(name[2:])
+        counts = W.counts_from_npz(os.path.join(ROOT, "tests", "golden", "inputs", f"global_comm_pattern_{P}proc.npz"))
+        r = min(32, P)
+        return counts, 1, "twophase_rbruck_alltoallv", dict(r=r), W.hops_flat(P, r)
     counts, esz, tun = W.config_counts(name, seed)
     P = counts.shape[0]
     if name == "C4":
@@ -141,6 +148,7 @@ def main() -> None:
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="C4")
     ap.add_argument("--func", default=None, help="override the function (e.g. TTPL_BT_alltoallv_s1)")
+    ap.add_argument("--radix", type=int, default=0, help="override the radix r of the workload")
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-budget", type=float, default=150.0)
@@ -156,6 +164,10 @@ def main() -> None:
     counts, esz, func, tun, hops = workload(args.workload, args.seed)
     if args.func:
         func = args.func
+    if args.radix:
+        tun["r"] = args.radix
+        P_ = counts.shape[0]
+        hops = W.hops_twolayer(P_, tun["n"], args.radix) if "n" in tun else W.hops_flat(P_, min(args.radix, P_ - 1 if func == "tuna_algorithm" else P_))
     prob = W.make_problem(counts, esz, 0, 0)
     S = prob.payload_bytes
     A = W.algorithmic_bytes(counts, esz, hops)
@@ -219,7 +231,8 @@ def main() -> None:
         "metric": METRIC, "value": round(value, 2), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "u8", "data": "synthetic",
-        "config": {"workload": f"BASELINE config {args.workload[1:]}: {func}, P={prob.P} virtual ranks, "
+        "config": {"workload": (f"BASELINE config {args.workload[1:]}" if args.workload[0] == "C" else
+                                f"reference input matrix inputs/{prob.P}proc") + f": {func}, P={prob.P} virtual ranks, "
                                + ", ".join(f"{k}={v}" for k, v in tun.items()) + f", {esz}-byte elements",
                    "payload_bytes": S, "algorithmic_bytes": A, "launches_per_step": int(st.n_launches),
                    "staging_bytes": int(st.staging_bytes)},

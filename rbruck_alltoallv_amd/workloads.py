@@ -102,6 +102,15 @@ def counts_from_text(path: str) -> np.ndarray:
     return m
 
 
+def counts_from_npz(path: str, divide: int = 1) -> np.ndarray:
+    """A P x P byte-count matrix stored as the array `counts` of an .npz file (the binary form of the reference's
+    inputs/<P>proc matrices); `divide` > 1 scales the counts down for parity-test sizes."""
+    with np.load(path, allow_pickle=False) as z:
+        m = z["counts"].astype(np.int64)
+    assert m.ndim == 2 and m.shape[0] == m.shape[1]
+    return (m // divide).astype(np.int32)
+
+
 # ------------------------------------------------------------------ displacements
 
 def layout_displs(counts_rows: np.ndarray, layout: int) -> tuple[np.ndarray, np.ndarray]:

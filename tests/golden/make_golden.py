@@ -27,6 +27,7 @@ from rbruck_alltoallv_amd import workloads as W  # noqa: E402
 DRIVER = os.path.join(ROOT, "oracle", "_ref", "ref_driver")
 MPIEXEC = "/opt/conda/bin/mpiexec"
 HERE = os.path.dirname(os.path.abspath(__file__))
+INPUTS_DIR = os.path.join(HERE, "inputs")
 
 
 def counts_for(spec: dict) -> np.ndarray:
@@ -41,6 +42,9 @@ def counts_for(spec: dict) -> np.ndarray:
         c = W.counts_fft_rows(spec["P"], spec["row_len"], spec["count"])
     elif kind == "zeros":
         c = np.zeros((spec["P"], spec["P"]), dtype=np.int32)
+    elif kind == "ml":
+        # the reference's own communication-pattern matrices (inputs/<P>proc), scaled down
+        c = W.counts_from_npz(os.path.join(INPUTS_DIR, f"global_comm_pattern_{spec['P']}proc.npz"), spec["divide"])
     else:
         raise ValueError(kind)
     if spec.get("sparsify"):
@@ -92,6 +96,13 @@ def cases() -> list[dict]:
         add(f"zeros-{f}", f, zz, 4, r=2, b=1)
     add("zeros-ttpl", "ttpl", zz, 4, r=2, n=4)
     add("zeros-ttpl_s1", "ttpl_s1", zz, 4, r=2, n=4)
+    # the reference's own input matrices (examples/MLinputs_example.cpp: MPI_CHAR, packed displacements), scaled down
+    for P, div, r in ((4, 65536, 2), (8, 65536, 2), (16, 32768, 4), (32, 16384, 2), (64, 16384, 8), (128, 16384, 12)):
+        ml = dict(kind="ml", P=P, divide=div)
+        add(f"ml-P{P}-twophase-r{r}", "twophase", ml, 1, r=r)
+        add(f"ml-P{P}-tuna-r{r}", "tuna", ml, 1, r=r, b=0)
+    add("ml-P64-ttpl-n8", "ttpl", dict(kind="ml", P=64, divide=16384), 1, r=4, n=8)
+    add("ml-P128-ttpl_s1-n32", "ttpl_s1", dict(kind="ml", P=128, divide=16384), 1, r=32, n=32)
     # linear comparators
     for P in (8, 12, 32):
         cg = dict(kind="uniform_random", P=P, hi=30, seed=P + 5, sparsify=4)

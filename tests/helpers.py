@@ -10,6 +10,7 @@ from rbruck_alltoallv_amd import workloads as W
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 GOLDEN_DIR = os.path.join(ROOT, "tests", "golden")
+INPUTS_DIR = os.path.join(GOLDEN_DIR, "inputs")
 
 
 def load_golden() -> list[dict]:
@@ -29,6 +30,9 @@ def counts_for(spec: dict) -> np.ndarray:
         c = W.counts_fft_rows(spec["P"], spec["row_len"], spec["count"])
     elif kind == "zeros":
         c = np.zeros((spec["P"], spec["P"]), dtype=np.int32)
+    elif kind == "ml":
+        # the reference's own communication-pattern matrices (inputs/<P>proc), scaled down
+        c = W.counts_from_npz(os.path.join(INPUTS_DIR, f"global_comm_pattern_{spec['P']}proc.npz"), spec["divide"])
     else:
         raise ValueError(kind)
     if spec.get("sparsify"):
