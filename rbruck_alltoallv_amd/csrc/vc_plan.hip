@@ -113,6 +113,10 @@ __global__ __launch_bounds__(VC_THREADS) void vc_plan_emit(VcSched S, const VcLa
     for (int k = threadIdx.x; k < L; k += VC_THREADS) first += header[3 + 2 * nl + k];
     first = vc_block_sum(first, lds);
     int64_t carry = first + item_row_base[(int64_t)L * P + to];
+    // blocks of many pieces are written by the whole workgroup, not by the lane that owns the entry
+    __shared__ VcDesc big_whole[VC_THREADS];
+    __shared__ int64_t big_at[VC_THREADS], big_cnt[VC_THREADS];
+    __shared__ int nbig;
     for (int base = 0; base < P; base += VC_THREADS) {
         const int id = base + threadIdx.x;
         VcEntry e;
@@ -120,12 +124,26 @@ __global__ __launch_bounds__(VC_THREADS) void vc_plan_emit(VcSched S, const VcLa
         const int64_t len = active ? vc_entry_len(S, T, e) : 0;
         const int64_t cnt = vc_chunk_count(len);
         int64_t total;
-        const int64_t at = carry + vc_block_exclusive_scan(cnt, lds, total);
+        if (threadIdx.x == 0) nbig = 0;
+        const int64_t at = carry + vc_block_exclusive_scan(cnt, lds, total);    // (barriers inside order the reset of nbig)
         if (cnt) {
             const VcDesc whole = vc_entry_desc(S, T, slot_off, row_base, e, to);
-            for (int64_t c = 0; c < cnt; c++) items[at + c] = vc_chunk_of(whole, c);
+            if (cnt <= 4) {
+                for (int64_t c = 0; c < cnt; c++) items[at + c] = vc_chunk_of(whole, c);
+            } else {
+                const int k = atomicAdd(&nbig, 1);
+                big_whole[k] = whole; big_at[k] = at; big_cnt[k] = cnt;
+            }
+        }
+        __syncthreads();
+        const int nb = nbig;
+        for (int k = 0; k < nb; k++) {
+            const VcDesc whole = big_whole[k];
+            const int64_t at_k = big_at[k], cnt_k = big_cnt[k];
+            for (int64_t c = threadIdx.x; c < cnt_k; c += VC_THREADS) items[at_k + c] = vc_chunk_of(whole, c);
         }
         carry += total;
+        __syncthreads();                                  // everybody has read nbig and the list before they are reused
     }
 }
 
