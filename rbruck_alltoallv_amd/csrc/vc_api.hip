@@ -63,7 +63,7 @@ struct vc_comm {
     hipStream_t stream = nullptr;
     const int64_t *sbase = nullptr, *rbase = nullptr;
     bool timing = false;
-    DevBuf slot_off, row_tot, row_base, item_row_tot, item_row_base, row_bytes, desc, header, launches, stage, rd_packed,
+    DevBuf slot_off, row_tot, row_base, org_run_base, item_row_tot, item_row_base, row_bytes, desc, header, launches, stage, rd_packed,
         uni_counts, uni_displs, scratch;
     int64_t *h_header = nullptr;          // pinned
     VcLaunchInfo *h_launches = nullptr;   // pinned
@@ -92,7 +92,7 @@ extern "C" int vc_comm_create(int nranks, vc_comm_t *comm_out) {
 extern "C" int vc_comm_free(vc_comm_t c) {
     if (!c) return VC_OK;
     (void)hipStreamSynchronize(c->stream);
-    for (DevBuf *b : {&c->slot_off, &c->row_tot, &c->row_base, &c->item_row_tot, &c->item_row_base, &c->row_bytes, &c->desc, &c->header, &c->launches, &c->stage, &c->rd_packed,
+    for (DevBuf *b : {&c->slot_off, &c->row_tot, &c->row_base, &c->org_run_base, &c->item_row_tot, &c->item_row_base, &c->row_bytes, &c->desc, &c->header, &c->launches, &c->stage, &c->rd_packed,
                       &c->uni_counts, &c->uni_displs, &c->scratch})
         b->release();
     for (hipEvent_t e : c->events) (void)hipEventDestroy(e);
@@ -178,11 +178,12 @@ static int run_schedule(vc_comm *c, VcSched S, std::vector<VcLaunchInfo> &L, con
     if (nl > VC_MAX_LAUNCHES) return fail_arg("more than VC_MAX_LAUNCHES launches: raise b / bblock");
     hipStream_t st = c->stream;
     const size_t PP = (size_t)P * P;
-    const size_t wmax = (size_t)std::max(S.w, 1);
+    const size_t wmax = (size_t)std::max(S.w, 1) + 1;      // digit regions + the organized region
 
     HIP_TRY(c->slot_off.reserve(sizeof(int64_t) * PP * wmax));
     HIP_TRY(c->row_tot.reserve(sizeof(int64_t) * (size_t)P * wmax));
     HIP_TRY(c->row_base.reserve(sizeof(int64_t) * (size_t)P * wmax));
+    HIP_TRY(c->org_run_base.reserve(sizeof(int64_t) * (size_t)P * std::max(S.G, 1)));
     HIP_TRY(c->item_row_tot.reserve(sizeof(int64_t) * (size_t)P * nl));
     HIP_TRY(c->item_row_base.reserve(sizeof(int64_t) * (size_t)P * nl));
     HIP_TRY(c->row_bytes.reserve(sizeof(int64_t) * (size_t)P * (nl + 1)));
@@ -199,7 +200,8 @@ static int run_schedule(vc_comm *c, VcSched S, std::vector<VcLaunchInfo> &L, con
         T.rd_packed = c->rd_packed.as<int>();
     }
     HIP_TRY(vc_launch_plan_sizes(S, c->launches.as<VcLaunchInfo>(), nl, T, c->slot_off.as<int64_t>(), c->row_tot.as<int64_t>(),
-                                 c->row_base.as<int64_t>(), c->item_row_tot.as<int64_t>(), c->item_row_base.as<int64_t>(),
+                                 c->row_base.as<int64_t>(), c->org_run_base.as<int64_t>(), c->item_row_tot.as<int64_t>(),
+                                 c->item_row_base.as<int64_t>(),
                                  c->row_bytes.as<int64_t>(), c->header.as<int64_t>(), st));
     HIP_TRY(hipMemcpyAsync(c->h_header, c->header.p, sizeof(int64_t) * VC_HEADER_WORDS(nl), hipMemcpyDeviceToHost, st));
     HIP_TRY(hipStreamSynchronize(st));     // the staging arena and the item list are sized from the plan

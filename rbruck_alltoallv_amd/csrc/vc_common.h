@@ -44,11 +44,16 @@ struct VcSched {
     int packed_recv;  // 1: receive side is the packed source-ordered layout (TTPL_BT_alltoallv ignores rdispls)
     int uniform;      // >0: equal blocks of this many elements, tables are implied (uniform_* functions)
     int recv_lo;      // low 4 bits of the recvbuf pointer (staging slots copy the final destination's 16-byte phase)
+    int coalesce;     // 1: blocks that are about to leave their node wait in "organized" runs — the n blocks one rank
+                      //    holds for one destination rank back to back in source order — so that an inter-node message
+                      //    is a contiguous copy (TTPL_BT_alltoallv, src/twophase_twolayer_rbruck.cpp:388-398, 430-453).
+                      //    The organized region is staging region number w.
 };
 
 // One data-moving kernel launch.
 struct VcLaunchInfo {
-    int kind;      // 0: rounds of intra-node digit x with digit value in [zlo, zhi]; 1: inter-node messages; 2: direct messages
+    int kind;      // 0: rounds of intra-node digit x with digit value in [zlo, zhi]; 1: inter-node messages, one per block;
+                   // 2: direct messages; 3: inter-node messages, coalesced (entries are (source group, part) pairs)
     int x;         // digit
     int dist;      // r^x
     int zlo, zhi;
@@ -82,8 +87,8 @@ hipError_t vc_launch_uniform_tables(int *counts, int *displs, int count, int P, 
 #define VC_HEADER_WORDS(nl) (3 + 3 * (nl))
 // Passes 1 and 2: staging prefix sums and the number of work items of every launch (sizes only).
 hipError_t vc_launch_plan_sizes(const VcSched &S, const VcLaunchInfo *launches_dev, int nlaunch, VcTables T, int64_t *slot_off,
-                                int64_t *row_tot, int64_t *row_base, int64_t *item_row_tot, int64_t *item_row_base,
-                                int64_t *row_bytes, int64_t *header, hipStream_t st);
+                                int64_t *row_tot, int64_t *row_base, int64_t *org_run_base, int64_t *item_row_tot,
+                                int64_t *item_row_base, int64_t *row_bytes, int64_t *header, hipStream_t st);
 // Pass 3: writes the work items (needs the item buffer, sized from the header).
 hipError_t vc_launch_plan_emit(const VcSched &S, const VcLaunchInfo *launches_dev, int nlaunch, VcTables T, const int64_t *slot_off,
                                const int64_t *row_base, const int64_t *item_row_base, const int64_t *header, VcDesc *items,

@@ -43,15 +43,17 @@ __global__ __launch_bounds__(VC_THREADS) void vc_plan_rows(VcSched S, const VcLa
     const int L = blockIdx.y - S.w;
     const VcLaunchInfo info = launches[L];
     int64_t items = 0, bytes = 0, payload = 0;
-    for (int id = threadIdx.x; id < P; id += VC_THREADS) {
+    const int nent = vc_entries_per_rank(S, info);
+    for (int id = threadIdx.x; id < nent; id += VC_THREADS) {
         VcEntry e;
         if (vc_entry_block(S, info, to, id, e)) {
             const int64_t len = vc_entry_len(S, T, e);
             items += vc_chunk_count(len);
             bytes += len;
         }
-        if (L == 0) payload += (int64_t)T.rc[(int64_t)to * P + id] * S.esz;
     }
+    if (L == 0)
+        for (int id = threadIdx.x; id < P; id += VC_THREADS) payload += (int64_t)T.rc[(int64_t)to * P + id] * S.esz;
     items = vc_block_sum(items, lds);
     bytes = vc_block_sum(bytes, lds);
     if (L == 0) payload = vc_block_sum(payload, lds);
@@ -60,6 +62,27 @@ __global__ __launch_bounds__(VC_THREADS) void vc_plan_rows(VcSched S, const VcLa
         row_bytes[(int64_t)L * P + to] = bytes;
         if (L == 0) row_bytes[(int64_t)nl * P + to] = payload;
     }
+}
+
+// ---- pass 1b (S.coalesce): layout of the organized region, one workgroup per rank ----
+// Scan of the run sizes over the groups, then slot_off[(w*P + to)*P + id] for every slot; row_tot[w*P + to].
+__global__ __launch_bounds__(VC_THREADS) void vc_plan_org_rows(VcSched S, VcTables T, int64_t *__restrict__ slot_off,
+                                                               int64_t *__restrict__ row_tot, int64_t *__restrict__ org_run_base) {
+    __shared__ int64_t lds[VC_WAVES_PER_BLOCK];
+    const int to = blockIdx.x, P = S.P, G = S.G;
+    int64_t carry = 0;
+    for (int base = 0; base < G; base += VC_THREADS) {
+        const int g = base + threadIdx.x;
+        int64_t total;
+        const int64_t v = (g < G) ? vc_org_run_size(S, T, to, g) : 0;
+        const int64_t ex = vc_block_exclusive_scan(v, lds, total);
+        if (g < G) org_run_base[(int64_t)to * G + g] = carry + ex;
+        carry += total;
+    }
+    if (threadIdx.x == 0) row_tot[(int64_t)S.w * P + to] = carry;
+    __syncthreads();                                      // org_run_base of this rank is complete (same workgroup wrote it)
+    for (int id = threadIdx.x; id < P; id += VC_THREADS)
+        slot_off[((int64_t)S.w * P + to) * P + id] = org_run_base[(int64_t)to * G + id / S.n] + vc_org_slot_rel(S, T, to, id);
 }
 
 // ---- pass 2: prefix sums over the rows ----
@@ -73,7 +96,7 @@ __global__ __launch_bounds__(VC_THREADS) void vc_plan_bases(int P, int w, int nl
     const int L = blockIdx.x;
     int64_t carry = 0, bytes = 0;
     if (L == nl) {
-        const int64_t nrows = (int64_t)w * P;
+        const int64_t nrows = (int64_t)w * P;                 // w counts the organized region when there is one
         for (int64_t b0 = 0; b0 < nrows; b0 += VC_THREADS) {
             const int64_t i = b0 + threadIdx.x;
             int64_t total;
@@ -117,10 +140,11 @@ __global__ __launch_bounds__(VC_THREADS) void vc_plan_emit(VcSched S, const VcLa
     __shared__ VcDesc big_whole[VC_THREADS];
     __shared__ int64_t big_at[VC_THREADS], big_cnt[VC_THREADS];
     __shared__ int nbig;
-    for (int base = 0; base < P; base += VC_THREADS) {
+    const int nent = vc_entries_per_rank(S, info);
+    for (int base = 0; base < nent; base += VC_THREADS) {
         const int id = base + threadIdx.x;
         VcEntry e;
-        const bool active = id < P && vc_entry_block(S, info, to, id, e);
+        const bool active = id < nent && vc_entry_block(S, info, to, id, e);
         const int64_t len = active ? vc_entry_len(S, T, e) : 0;
         const int64_t cnt = vc_chunk_count(len);
         int64_t total;
@@ -148,11 +172,13 @@ __global__ __launch_bounds__(VC_THREADS) void vc_plan_emit(VcSched S, const VcLa
 }
 
 hipError_t vc_launch_plan_sizes(const VcSched &S, const VcLaunchInfo *launches_dev, int nlaunch, VcTables T, int64_t *slot_off,
-                                int64_t *row_tot, int64_t *row_base, int64_t *item_row_tot, int64_t *item_row_base,
-                                int64_t *row_bytes, int64_t *header, hipStream_t st) {
+                                int64_t *row_tot, int64_t *row_base, int64_t *org_run_base, int64_t *item_row_tot,
+                                int64_t *item_row_base, int64_t *row_bytes, int64_t *header, hipStream_t st) {
     hipLaunchKernelGGL(vc_plan_rows, dim3(S.P, S.w + nlaunch), dim3(VC_THREADS), 0, st, S, launches_dev, nlaunch, T, slot_off, row_tot,
                        item_row_tot, row_bytes);
-    hipLaunchKernelGGL(vc_plan_bases, dim3(nlaunch + 1), dim3(VC_THREADS), 0, st, S.P, S.w, nlaunch, row_tot, row_base, item_row_tot,
+    if (S.coalesce)
+        hipLaunchKernelGGL(vc_plan_org_rows, dim3(S.P), dim3(VC_THREADS), 0, st, S, T, slot_off, row_tot, org_run_base);
+    hipLaunchKernelGGL(vc_plan_bases, dim3(nlaunch + 1), dim3(VC_THREADS), 0, st, S.P, S.w + S.coalesce, nlaunch, row_tot, row_base, item_row_tot,
                        item_row_base, row_bytes, header);
     return hipGetLastError();
 }

@@ -22,6 +22,7 @@ struct VcBlock {
     int xprev;       // digit in which it last moved (-1: still in sendbuf)
     int id_from;     // its slot on `from`
     bool to_stage;   // lands in the receiver's staging area (else in recvbuf)
+    bool to_org;     // ... in its organized region (last intra-node hop of a block that still has to change node)
 };
 
 VC_HD int vc_top_digit(int v, int r) {     // position of the highest non-zero digit, v > 0
@@ -66,6 +67,7 @@ VC_HD bool vc_intra_block(const VcSched &S, int x, int dist, int to, int id, VcB
     b.z = z;
     b.id_from = g * n + (j + lfrom) % n;
     b.to_stage = !(last && g == gs);
+    b.to_org = S.coalesce && last && g != gs;
     return true;
 }
 
@@ -86,7 +88,7 @@ VC_HD int vc_phase16(const VcSched &S, const VcTables &T, int s, int t) {
 // (0 if nothing arrives there, or if it goes to recvbuf).  Always a multiple of 16.
 VC_HD int64_t vc_stage_slot_size(const VcSched &S, const VcTables &T, int x, int dist, int to, int id) {
     VcBlock b;
-    if (!vc_intra_block(S, x, dist, to, id, b) || !b.to_stage) return 0;
+    if (!vc_intra_block(S, x, dist, to, id, b) || !b.to_stage || b.to_org) return 0;
     const int64_t len = (int64_t)T.sc[(int64_t)b.s * S.P + b.t] * S.esz;
     return len ? ((len + vc_phase16(S, T, b.s, b.t) + 15) & ~15ll) : 0;
 }
@@ -103,6 +105,40 @@ VC_HD int64_t vc_send_offset(const VcSched &S, const VcTables &T, int s, int t) 
     return T.sbase[s] + (int64_t)T.sd[(int64_t)s * S.P + t] * S.esz;
 }
 
+// ---- organized region (S.coalesce) ----
+// Rank `to` = (gs, l) keeps, for every other group g, a run that mirrors byte for byte the part of rank (g, l)'s
+// packed recvbuf that comes from group gs: n blocks in source order.  The block of local rank l itself never
+// moves inside the node and leaves a hole of its length.  A run starts 16-byte aligned plus the 16-byte phase of
+// its image in recvbuf, so that the inter-node copy of a run is a copy between equally aligned addresses.
+
+// byte offset, inside rank t's recvbuf, of the first block coming from group gs (packed receive layout)
+VC_HD int64_t vc_org_run_dst(const VcSched &S, const VcTables &T, int gs, int t) {
+    return T.rbase[t] + (int64_t)T.rd_packed[(int64_t)t * S.P + gs * S.n] * S.esz;
+}
+
+// bytes of blocks [0, m) of the run, m in [0, n]
+VC_HD int64_t vc_org_run_prefix(const VcSched &S, const VcTables &T, int gs, int t, int m) {
+    const int64_t row = (int64_t)t * S.P, s0 = gs * S.n;
+    const int64_t end = m < S.n ? T.rd_packed[row + s0 + m] : (int64_t)T.rd_packed[row + s0 + S.n - 1] + T.rc[row + s0 + S.n - 1];
+    return (end - T.rd_packed[row + s0]) * S.esz;
+}
+
+// size of the run rank `to` keeps for group g (multiple of 16; 0 for its own group)
+VC_HD int64_t vc_org_run_size(const VcSched &S, const VcTables &T, int to, int g) {
+    const int gs = to / S.n, t = g * S.n + to % S.n;
+    if (g == gs) return 0;
+    const int64_t phase = (vc_org_run_dst(S, T, gs, t) + S.recv_lo) & 15;
+    return (phase + vc_org_run_prefix(S, T, gs, t, S.n) + 15) & ~15ll;
+}
+
+// 16-byte aligned part of the offset of slot id = g*n + m inside the run (vc_stage_addr adds the block's own phase)
+VC_HD int64_t vc_org_slot_rel(const VcSched &S, const VcTables &T, int to, int id) {
+    const int gs = to / S.n, g = id / S.n, m = id % S.n, t = g * S.n + to % S.n;
+    if (g == gs) return 0;
+    const int64_t phase = (vc_org_run_dst(S, T, gs, t) + S.recv_lo) & 15;
+    return (phase + vc_org_run_prefix(S, T, gs, t, m)) & ~15ll;
+}
+
 // One entry of a launch before addresses are known: which block it moves and between which arenas.
 struct VcEntry {
     int s, t;          // the block
@@ -111,12 +147,31 @@ struct VcEntry {
     int id_from;       // its slot there
     int xdst;          // digit phase whose staging region receives it (-1: it goes to recvbuf)
     int id_to;         // its slot on the receiver
+    int nblk;          // 1, or the number of consecutive source blocks of a coalesced inter-node message part
 };
+
+// Number of entries per receiving rank in a launch of this kind.
+VC_HD int vc_entries_per_rank(const VcSched &S, const VcLaunchInfo &info) { return info.kind == 3 ? 3 * S.G : S.P; }
 
 // Entry (`to`, `id`) of a launch: intra-node launches index by the receiver's slot, inter-node
 // launches by the source rank.  Returns false if the entry moves nothing in this launch.
 VC_HD bool vc_entry_block(const VcSched &S, const VcLaunchInfo &info, int to, int id, VcEntry &e) {
     const int n = S.n;
+    e.nblk = 1;
+    if (info.kind == 3) {
+        // coalesced inter-node message from rank (gs, lt) to rank `to` = (gt, lt), in three contiguous parts: the
+        // blocks of local ranks below lt (organized region), the block of lt itself (still in sendbuf), those above
+        const int gs = id / 3, part = id % 3, gt = to / n, lt = to % n;
+        if (gs == gt) return false;
+        const int q = ((gs - gt + S.G) % S.G) * n;
+        if (q < info.qlo || q >= info.qhi) return false;
+        const int m0 = part == 0 ? 0 : (part == 1 ? lt : lt + 1);
+        const int m1 = part == 0 ? lt : (part == 1 ? lt + 1 : n);
+        if (m1 <= m0) return false;
+        e.s = gs * n + m0; e.t = to; e.from = gs * n + lt; e.nblk = m1 - m0;
+        e.xprev = part == 1 ? -1 : S.w; e.id_from = gt * n + m0; e.xdst = -1; e.id_to = id;
+        return true;
+    }
     if (info.kind == 2) {
         // direct: `id` is the source rank; launches are batches of the distance (source - destination) mod P
         // (src/MPICH_scattered.cpp:44-45: receive from rank + i + ii)
@@ -134,7 +189,7 @@ VC_HD bool vc_entry_block(const VcSched &S, const VcLaunchInfo &info, int to, in
         VcBlock b;
         if (!vc_intra_block(S, info.x, info.dist, to, id, b) || b.z < info.zlo || b.z > info.zhi) return false;
         e.s = b.s; e.t = b.t; e.from = b.from; e.xprev = b.xprev; e.id_from = b.id_from;
-        e.xdst = b.to_stage ? info.x : -1; e.id_to = id;
+        e.xdst = b.to_org ? S.w : (b.to_stage ? info.x : -1); e.id_to = id;
         return true;
     }
     // inter-node: `id` is the source rank s; the block waits on the rank of s's node that has
@@ -152,7 +207,9 @@ VC_HD bool vc_entry_block(const VcSched &S, const VcLaunchInfo &info, int to, in
 }
 
 VC_HD int64_t vc_entry_len(const VcSched &S, const VcTables &T, const VcEntry &e) {
-    return (int64_t)T.sc[(int64_t)e.s * S.P + e.t] * S.esz;
+    if (e.nblk == 1) return (int64_t)T.sc[(int64_t)e.s * S.P + e.t] * S.esz;
+    const int gs = e.s / S.n, m0 = e.s % S.n;
+    return vc_org_run_prefix(S, T, gs, e.t, m0 + e.nblk) - vc_org_run_prefix(S, T, gs, e.t, m0);
 }
 
 // The whole-block copy an entry stands for.

@@ -120,7 +120,13 @@ inline int vc_make_schedule(VcFunc f, int P, int n, int r, int batch, int esz, i
             vc_add_inter_launches(L, S, (batch <= 0 || batch > P) ? P : batch);                 // :621
         } else {
             const int groups = (batch <= 0 || batch > S.G) ? S.G : batch;                      // :421
+            const size_t first_inter = L.size();
             vc_add_inter_launches(L, S, groups * n);
+            // coalesced messages need the organized region, which the intra-node launches fill
+            if (S.w > 0 && S.G > 1) {
+                S.coalesce = 1;
+                for (size_t k = first_inter; k < L.size(); k++) L[k].kind = 3;
+            }
         }
         break;
     case VC_F_UNIFORM_SPREADOUT:

@@ -60,7 +60,7 @@ extern "C" int plan_emulate(int func, int P, int n, int r, int batch, int esz, i
     }
 
     // passes 1 and 2 of the planner
-    const int w = std::max(S.w, 1);
+    const int w = std::max(S.w, 1) + 1;                   // digit regions + the organized region
     std::vector<int64_t> slot_off(PP * w, 0), row_base((int64_t)P * w, 0);
     int64_t stage_bytes = 0;
     for (int x = 0; x < S.w; x++) {
@@ -76,6 +76,16 @@ extern "C" int plan_emulate(int func, int P, int n, int r, int batch, int esz, i
             stage_bytes += acc;
         }
     }
+    if (S.coalesce)                                       // pass 1b: organized region
+        for (int to = 0; to < P; to++) {
+            row_base[(int64_t)S.w * P + to] = stage_bytes;
+            std::vector<int64_t> run_base(S.G);
+            int64_t acc = 0;
+            for (int g = 0; g < S.G; g++) { run_base[g] = acc; acc += vc_org_run_size(S, T, to, g); }
+            for (int id = 0; id < P; id++)
+                slot_off[((int64_t)S.w * P + to) * P + id] = run_base[id / S.n] + vc_org_slot_rel(S, T, to, id);
+            stage_bytes += acc;
+        }
     std::vector<char> stage((size_t)stage_bytes + 64, (char)0xCD);
     std::vector<char> written((size_t)stage_bytes + 64, 0);
 
@@ -84,8 +94,9 @@ extern "C" int plan_emulate(int func, int P, int n, int r, int batch, int esz, i
     for (int k = 0; k < nl; k++) {
         std::vector<VcDesc> descs;
         std::vector<Range> dst_ranges, src_ranges;
+        const int nent = vc_entries_per_rank(S, L[k]);
         for (int to = 0; to < P; to++)
-            for (int id = 0; id < P; id++) {
+            for (int id = 0; id < nent; id++) {
                 VcEntry e;
                 if (!vc_entry_block(S, L[k], to, id, e)) continue;
                 const VcDesc whole = vc_entry_desc(S, T, slot_off.data(), row_base.data(), e, to);

@@ -199,3 +199,38 @@ def test_linear_comparator_plans(P):
                 for k in range(E.last.nlaunch):
                     src, dst = np.nonzero(E.last.traffic[k])
                     assert np.all(((src - dst) % P >= 3 * k) & ((src - dst) % P < 3 * k + 3))
+
+
+@pytest.mark.parametrize("P,n,r,bblock", [(8, 4, 4, 0), (12, 4, 2, 2), (27, 9, 3, 0), (64, 16, 16, 3), (64, 32, 32, 0), (16, 2, 2, 0)])
+def test_coalesced_twolayer_route(P, n, r, bblock):
+    """TTPL_BT_alltoallv: intra-node launches as in the staggered variant; every inter-node message is the coalesced
+    one of the reference (src/twophase_twolayer_rbruck.cpp:430-453) — same rank pairs, same bytes — and is copied in
+    at most three contiguous parts instead of n blocks."""
+    counts = W.counts_uniform_random(P, 300, seed=P + n + r)
+    counts[counts % 3 == 0] = 0
+    prob = W.make_problem(counts, 1, 1, 0)
+    send = W.fill_send_arena(prob, 0, 2)
+    recv = np.full(prob.recv_bytes, 0xEE, dtype=np.uint8)
+    with O.trace() as t:
+        assert O.TTPL_BT_alltoallv(n, r, bblock, prob, send, recv) == 0
+    rec = t.records
+    want = recv.copy()
+    recv[:] = 0xEE
+    assert E.TTPL_BT_alltoallv(n, r, bblock, prob, send, recv) == 0 and E.last.errors == 0
+    assert np.array_equal(recv, want)
+    res = E.last
+    G = P // n
+    digits = list(dict.fromkeys(rec[rec["kind"] == 0]["digit"].tolist()))
+    groups = G if bblock <= 0 or bblock > G else bblock
+    n_inter = -(-G // groups)
+    assert res.nlaunch == len(digits) + n_inter
+    inter = rec[rec["kind"] == 2]
+    cross = inter[inter["src"] // n != inter["dst"] // n]          # the reference also sends a message to itself
+    got = sum(res.traffic[len(digits) + k] for k in range(n_inter))
+    assert np.array_equal(got, _oracle_traffic(cross, P, np.ones(len(cross), dtype=bool)))
+    # batches follow the group distance (src/twophase_twolayer_rbruck.cpp:425-447)
+    for k in range(n_inter):
+        src, dst = np.nonzero(res.traffic[len(digits) + k])
+        dist = (src // n - dst // n) % G
+        assert np.all((dist >= k * groups) & (dist < (k + 1) * groups))
+    assert res.moved * 2 == W.algorithmic_bytes(prob.sendcounts, prob.esz, W.hops_twolayer(P, n, r))
