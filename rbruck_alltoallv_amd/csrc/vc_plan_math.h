@@ -225,13 +225,21 @@ VC_HD VcDesc vc_entry_desc(const VcSched &S, const VcTables &T, const int64_t *s
     return d;
 }
 
-// Blocks are copied in pieces of at most VC_CHUNK bytes, one workgroup each.
-VC_HD int64_t vc_chunk_count(int64_t len) { return (len + VC_CHUNK - 1) / VC_CHUNK; }
+// Blocks are copied in pieces of at most VC_CHUNK bytes, one workgroup each.  Pieces are cut where the DESTINATION
+// address is a multiple of 16, so that only the first piece of a block has a byte-wise head and only the last one a
+// tail; every piece in between is whole aligned vectors.
 
-VC_HD VcDesc vc_chunk_of(const VcDesc &whole, int64_t c) {
+// 16-byte phase of the destination address of an entry's copy.  Staging slots and organized runs are laid out at
+// the phase of the block's final address, so this holds whichever arena the copy writes to.
+VC_HD int vc_entry_phase(const VcSched &S, const VcTables &T, const VcEntry &e) { return vc_phase16(S, T, e.s, e.t); }
+
+VC_HD int64_t vc_chunk_count(int64_t len, int phase) { return len > 0 ? (len + phase + VC_CHUNK - 1) / VC_CHUNK : 0; }
+
+VC_HD VcDesc vc_chunk_of(const VcDesc &whole, int64_t c, int phase) {
     VcDesc d = whole;
-    d.src += c * VC_CHUNK; d.dst += c * VC_CHUNK;
-    const int64_t left = whole.len - c * VC_CHUNK;
-    d.len = left < VC_CHUNK ? left : VC_CHUNK;
+    const int64_t lo = c == 0 ? 0 : c * VC_CHUNK - phase;
+    int64_t hi = (c + 1) * VC_CHUNK - phase;
+    if (hi > whole.len) hi = whole.len;
+    d.src += lo; d.dst += lo; d.len = hi - lo;
     return d;
 }

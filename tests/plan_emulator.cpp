@@ -100,11 +100,18 @@ extern "C" int plan_emulate(int func, int P, int n, int r, int batch, int esz, i
                 VcEntry e;
                 if (!vc_entry_block(S, L[k], to, id, e)) continue;
                 const VcDesc whole = vc_entry_desc(S, T, slot_off.data(), row_base.data(), e, to);
-                const int64_t nchunks = vc_chunk_count(whole.len);
+                const int phase = vc_entry_phase(S, T, e);
+                const int dst_lo = (int)(whole.dst >> VC_SPACE_SHIFT) == 1 ? recv_lo : 0;
+                if (whole.len > 0 && (int)(((whole.dst & VC_OFFSET_MASK) + dst_lo) & 15) != phase) errors++;
+                const int64_t nchunks = vc_chunk_count(whole.len, phase);
+                int64_t covered = 0;
                 items += nchunks;
                 for (int64_t c = 0; c < nchunks; c++) {
-                const VcDesc d = vc_chunk_of(whole, c);
-                if (d.len <= 0 || d.len > VC_CHUNK) { errors++; continue; }
+                const VcDesc d = vc_chunk_of(whole, c, phase);
+                if (d.len <= 0 || d.len > VC_CHUNK || d.src - whole.src != covered || d.dst - whole.dst != covered) { errors++; continue; }
+                // only the first piece may start off a 16-byte boundary of the destination
+                if (c > 0 && (((d.dst & VC_OFFSET_MASK) + dst_lo) & 15) != 0) errors++;
+                covered += d.len;
                 const int sspace = (int)(d.src >> VC_SPACE_SHIFT), dspace = (int)(d.dst >> VC_SPACE_SHIFT);
                 const int64_t so = d.src & VC_OFFSET_MASK, dof = d.dst & VC_OFFSET_MASK;
                 const int64_t slim = sspace == 0 ? send_bytes : (sspace == 2 ? stage_bytes : -1);
@@ -118,6 +125,7 @@ extern "C" int plan_emulate(int func, int P, int n, int r, int batch, int esz, i
                 src_ranges.push_back({so, so + d.len, sspace});
                 if (traffic_out && k < max_launches) traffic_out[((int64_t)k * P + d.from) * P + d.to] += d.len;
                 }
+                if (covered != whole.len) errors++;
             }
         errors += count_overlaps(dst_ranges, src_ranges);
         for (const VcDesc &d : descs) {

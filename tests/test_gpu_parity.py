@@ -222,3 +222,29 @@ def test_linear_comparators(api, P):
             st = dp.comm.last_stats()
             assert st.moved_bytes == prob.payload_bytes
         dp.comm.free()
+
+
+@pytest.mark.parametrize("shift", [(0, 0), (5, 0), (0, 7), (3, 13)])
+def test_arena_pointers_of_any_alignment(api, shift):
+    """sendbuf / recvbuf need not be 16-byte aligned."""
+    import torch
+    s_shift, r_shift = shift
+    counts = (W.counts_uniform_random(12, 30000, seed=5) * (W.counts_uniform_random(12, 3, seed=6) > 0)).astype(np.int32)
+    prob = W.make_problem(counts, 1, 1, 0)
+    send = W.fill_send_arena(prob, 0, 9)
+    want = W.expected_recv_arena(prob, send)
+    dp = api.DeviceProblem(prob)
+    sbig = torch.zeros(prob.send_bytes + 64, dtype=torch.uint8, device="cuda:0")
+    ds = sbig[s_shift:s_shift + prob.send_bytes]
+    ds.copy_(torch.from_numpy(send))
+    for name, fn in (("twophase r=3", lambda d: api.twophase_rbruck_alltoallv(3, dp, ds, d)),
+                     ("tuna r=2 b=1", lambda d: api.tuna_algorithm(2, 1, dp, ds, d)),
+                     ("ttpl n=4 r=4", lambda d: api.TTPL_BT_alltoallv(4, 4, 0, dp, ds, d)),
+                     ("s1 n=6 r=2", lambda d: api.TTPL_BT_alltoallv_s1(6, 2, 5, dp, ds, d)),
+                     ("spreadout", lambda d: api.spreadout_alltoallv(dp, ds, d))):
+        rbig = torch.full((prob.recv_bytes + 64,), 0xEE, dtype=torch.uint8, device="cuda:0")
+        dr = rbig[r_shift:r_shift + prob.recv_bytes]
+        assert fn(dr) == 0, (name, dp.comm.error())
+        assert np.array_equal(dr.cpu().numpy(), want), (name, shift)
+        assert bool((rbig[:r_shift] == 0xEE).all()) and bool((rbig[r_shift + prob.recv_bytes:] == 0xEE).all())
+    dp.comm.free()
