@@ -12,8 +12,10 @@
 #include <stdint.h>
 
 #define VC_THREADS 256
-// bytes one workgroup of the copy kernel moves: 256 lanes x 2 vectors x 16 bytes
+// most bytes one workgroup of the copy kernel moves: 256 lanes x 2 vectors x 16 bytes
 #define VC_CHUNK 8192
+// piece size for copies longer than that: 256 lanes x 1 vector x 16 bytes
+#define VC_PIECE 4096
 
 // Location of a byte range: which arena (top bits) and the byte offset inside it.
 #define VC_SPACE_SHIFT 60
