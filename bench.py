@@ -212,6 +212,24 @@ def main() -> None:
 
     bad = dp.verify(send, recv, packed_recv=(func == "TTPL_BT_alltoallv"))
 
+    # The same collective as a persistent plan (planned once, executed many times): what the path costs when the
+    # count tables do not change between calls.  Extra information; `value` stays the full call.
+    plan_kw = {"n": tun.get("n", 0), "r": tun.get("r", 2), "batch": tun.get("b", tun.get("bblock", 0))}
+    plan = api.Plan(func, dp, recv, **plan_kw)
+    plan_info = None
+    if plan.rc == 0:
+        assert plan.execute(send, recv) == 0, dp.comm.error()
+        torch.cuda.synchronize()
+        p0 = time.perf_counter()
+        for _ in range(args.steps):
+            assert plan.execute(send, recv) == 0
+        torch.cuda.synchronize()
+        plan_s = (time.perf_counter() - p0) / args.steps
+        plan_bad = dp.verify(send, recv, packed_recv=(func == "TTPL_BT_alltoallv"))
+        plan_info = {"ms_per_call": round(plan_s * 1e3, 4), "GBps_effective": round(S / plan_s / 1e9, 1),
+                     "hbm_frac": round(A / plan_s / 1e9 / HBM_PEAK_GBPS, 4), "mismatched_bytes": int(plan_bad)}
+        plan.free()
+
     # The linear comparator the reference drivers time beside the Bruck variants (examples/twophaseLayer_example.cpp:99-113
     # times MPI_Alltoallv): on one GPU it is a single pass over the payload.  Context only, not the metric.
     dp.comm.set_timing(False)
@@ -240,6 +258,7 @@ def main() -> None:
         "one_pass_floor_fraction": round(2 * S / (elapsed / args.steps) / 1e9 / HBM_PEAK_GBPS, 4),
         "plan_ms_per_step": round(plan_ms / args.steps, 4),
         "mismatched_bytes": int(bad),
+        "persistent_plan": plan_info,
         "one_pass_comparator": {"func": "spreadout_alltoallv", "ms_per_call": round(comp_s * 1e3, 4),
                                 "GBps_effective": round(S / comp_s / 1e9, 1),
                                 "hbm_frac": round(2 * S / comp_s / 1e9 / HBM_PEAK_GBPS, 4), "mismatched_bytes": int(comp_bad)},

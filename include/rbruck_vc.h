@@ -137,6 +137,24 @@ int exclisive_or_alltoallv(char *sendbuf, int *sendcounts, int *sdispls, int sen
 int spreadout_alltoallv(char *sendbuf, int *sendcounts, int *sdispls, int sendtype_size, char *recvbuf,
                         int *recvcounts, int *rdispls, int recvtype_size, vc_comm_t comm);
 
+/* ---- persistent plans: the analogue of MPI-4 persistent collectives (MPI_Alltoallv_init / MPI_Start).
+ * The reference re-exchanges its metadata in every call (src/twophase_tunable_rbruckv.cpp:110); when the same tables are
+ * used again, a plan keeps the schedule, the staging layout and the work items, and executing it launches only the
+ * copy kernels (no planning kernels, no host synchronisation before the final one).  No counterpart in the reference. ---- */
+
+typedef struct vc_plan *vc_plan_t;
+
+/* `function` is the name of one of the alltoallv-shaped entry points above ("twophase_rbruck_alltoallv", "tuna_algorithm",
+ * "TTPL_BT_alltoallv", "spreadout_alltoallv", ...); n, r and batch (b / bblock) are that function's tunables, ignored where
+ * it has none.  The tables are read now and not needed afterwards; the communicator's bases are read now too.
+ * recvbuf_low_bits = (address of the recvbuf that will be passed) & 15.  Same return codes as the function itself. */
+int vc_plan_create(const char *function, int n, int r, int batch, int *sendcounts, int *sdispls, int elem_size,
+                   int *recvcounts, int *rdispls, int recvbuf_low_bits, vc_comm_t comm, vc_plan_t *plan_out);
+
+/* Runs the planned collective; blocking.  One plan (or call) per communicator at a time. */
+int vc_plan_execute(vc_plan_t plan, char *sendbuf, char *recvbuf);
+int vc_plan_free(vc_plan_t plan);
+
 /* ---- measurement and inspection (the reference's global phase timers, src/rbruckv.h:13-18) ---- */
 
 #define VC_MAX_LAUNCHES 1024

@@ -45,6 +45,9 @@ SYMBOLS = {
     "ompi_alltoallv_intra_pairwise": (_I, _V_TAIL),
     "exclisive_or_alltoallv": (_I, _V_TAIL),
     "spreadout_alltoallv": (_I, _V_TAIL),
+    "vc_plan_create": (_I, [C.c_char_p, _I, _I, _I, _P, _P, _I, _P, _P, _I, _P, C.POINTER(_P)]),
+    "vc_plan_execute": (_I, [_P, _P, _P]),
+    "vc_plan_free": (_I, [_P]),
     "vc_comm_set_timing": (_I, [_P, _I]),
     "vc_comm_last_stats": (_I, [_P, C.POINTER(VcStats)]),
     "vc_comm_last_traffic": (_I, [_P, _I, _P]),

@@ -173,3 +173,24 @@ def exclisive_or_alltoallv(p: DeviceProblem, send: torch.Tensor, recv: torch.Ten
 def spreadout_alltoallv(p: DeviceProblem, send: torch.Tensor, recv: torch.Tensor) -> int:
     """benchmarks/common.cpp:10-37"""
     return p.comm.lib.spreadout_alltoallv(*_tail(p, send, recv))
+
+
+class Plan:
+    """vc_plan_t: a planned (persistent) collective for one set of tables."""
+
+    def __init__(self, function: str, p: DeviceProblem, recv: torch.Tensor, n: int = 0, r: int = 2, batch: int = 0):
+        self.problem = p
+        h = C.c_void_p()
+        rc = p.comm.lib.vc_plan_create(function.encode(), n, r, batch, p.sendcounts.data_ptr(), p.sdispls.data_ptr(), p.esz,
+                                       p.recvcounts.data_ptr(), p.rdispls.data_ptr(), recv.data_ptr() & 15, p.comm.handle,
+                                       C.byref(h))
+        self.rc = rc
+        self.handle = h if rc == 0 else None
+
+    def execute(self, send: torch.Tensor, recv: torch.Tensor) -> int:
+        return self.problem.comm.lib.vc_plan_execute(self.handle, send.data_ptr(), recv.data_ptr())
+
+    def free(self) -> None:
+        if self.handle:
+            self.problem.comm.lib.vc_plan_free(self.handle)
+            self.handle = None

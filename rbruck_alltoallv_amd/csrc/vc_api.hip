@@ -71,6 +71,7 @@ struct vc_comm {
     vc_stats_t stats;
     int last_nlaunch = 0;
     int64_t launch_first[VC_MAX_LAUNCHES], launch_items[VC_MAX_LAUNCHES];   // work items of the last call
+    const VcDesc *last_items = nullptr;
 };
 
 // ------------------------------------------------------------------ communicator
@@ -79,12 +80,17 @@ extern "C" int vc_comm_create(int nranks, vc_comm_t *comm_out) {
     if (!comm_out || nranks < 1) return fail_arg("vc_comm_create: need nranks >= 1 and an output pointer");
     int ndev = 0;
     if (hipGetDeviceCount(&ndev) != hipSuccess || ndev < 1) return fail_arg("no HIP device", VC_ERR_NO_DEVICE);
+    if (nranks > 32768) return fail_arg("vc_comm_create: at most 32768 ranks (P x P int32 tables)");
     vc_comm *c = new vc_comm();
     c->P = nranks;
-    HIP_TRY(hipGetDevice(&c->device));
-    HIP_TRY(hipHostMalloc((void **)&c->h_header, sizeof(int64_t) * VC_HEADER_WORDS(VC_MAX_LAUNCHES), hipHostMallocDefault));
-    HIP_TRY(hipHostMalloc((void **)&c->h_launches, sizeof(VcLaunchInfo) * VC_MAX_LAUNCHES, hipHostMallocDefault));
     memset(&c->stats, 0, sizeof c->stats);
+    hipError_t e = hipGetDevice(&c->device);
+    if (e == hipSuccess) e = hipHostMalloc((void **)&c->h_header, sizeof(int64_t) * VC_HEADER_WORDS(VC_MAX_LAUNCHES), hipHostMallocDefault);
+    if (e == hipSuccess) e = hipHostMalloc((void **)&c->h_launches, sizeof(VcLaunchInfo) * VC_MAX_LAUNCHES, hipHostMallocDefault);
+    if (e != hipSuccess) {
+        (void)vc_comm_free(c);
+        return fail_hip(e, "vc_comm_create", __LINE__);
+    }
     *comm_out = c;
     return VC_OK;
 }
@@ -171,8 +177,16 @@ static int ensure_events(vc_comm *c, size_t n) {
     return VC_OK;
 }
 
-// Steps 3-5 for any schedule.
-static int run_schedule(vc_comm *c, VcSched S, std::vector<VcLaunchInfo> &L, const char *sendbuf, char *recvbuf, VcTables T) {
+// What the planner leaves behind for the copy launches.
+struct PlanInfo {
+    int nl = 0, n_digits = 0;
+    int recv_lo = 0;
+    int64_t stage_bytes = 0, payload_bytes = 0;
+    std::vector<int64_t> first, count, bytes;       // per launch: first work item, item count, bytes moved
+};
+
+// Step 3: staging prefix sums, item counts (read back to size the buffers), then the work items into `items`.
+static int build_plan(vc_comm *c, VcSched S, std::vector<VcLaunchInfo> &L, VcTables T, DevBuf &items, PlanInfo &out) {
     const int P = S.P;
     const int nl = (int)L.size();
     if (nl > VC_MAX_LAUNCHES) return fail_arg("more than VC_MAX_LAUNCHES launches: raise b / bblock");
@@ -201,49 +215,71 @@ static int run_schedule(vc_comm *c, VcSched S, std::vector<VcLaunchInfo> &L, con
     }
     HIP_TRY(vc_launch_plan_sizes(S, c->launches.as<VcLaunchInfo>(), nl, T, c->slot_off.as<int64_t>(), c->row_tot.as<int64_t>(),
                                  c->row_base.as<int64_t>(), c->org_run_base.as<int64_t>(), c->item_row_tot.as<int64_t>(),
-                                 c->item_row_base.as<int64_t>(),
-                                 c->row_bytes.as<int64_t>(), c->header.as<int64_t>(), st));
+                                 c->item_row_base.as<int64_t>(), c->row_bytes.as<int64_t>(), c->header.as<int64_t>(), st));
     HIP_TRY(hipMemcpyAsync(c->h_header, c->header.p, sizeof(int64_t) * VC_HEADER_WORDS(nl), hipMemcpyDeviceToHost, st));
     HIP_TRY(hipStreamSynchronize(st));     // the staging arena and the item list are sized from the plan
 
-    int64_t *h = c->h_header;
+    const int64_t *h = c->h_header;
+    out.nl = nl; out.n_digits = S.w; out.recv_lo = S.recv_lo;
+    out.stage_bytes = h[0]; out.payload_bytes = h[1];
+    out.first.assign(nl, 0); out.count.assign(nl, 0); out.bytes.assign(nl, 0);
     int64_t nitems = 0;
-    for (int k = 0; k < nl; k++) { h[3 + nl + k] = nitems; nitems += h[3 + 2 * nl + k]; }     // first item of every launch
-    const int64_t stage_bytes = h[0];
-    HIP_TRY(c->stage.reserve((size_t)stage_bytes + 64));
-    HIP_TRY(c->desc.reserve(sizeof(VcDesc) * (size_t)std::max<int64_t>(nitems, 1)));
+    for (int k = 0; k < nl; k++) {
+        out.bytes[k] = h[3 + k];
+        out.first[k] = nitems;
+        out.count[k] = h[3 + 2 * nl + k];
+        nitems += out.count[k];
+    }
+    HIP_TRY(items.reserve(sizeof(VcDesc) * (size_t)std::max<int64_t>(nitems, 1)));
     HIP_TRY(vc_launch_plan_emit(S, c->launches.as<VcLaunchInfo>(), nl, T, c->slot_off.as<int64_t>(), c->row_base.as<int64_t>(),
-                                c->item_row_base.as<int64_t>(), c->header.as<int64_t>(), c->desc.as<VcDesc>(), st));
+                                c->item_row_base.as<int64_t>(), c->header.as<int64_t>(), items.as<VcDesc>(), st));
     if (c->timing) HIP_TRY(hipEventRecord(c->events[1], st));
+    return VC_OK;
+}
 
+// Steps 4-5: one copy kernel per launch, then the blocking synchronisation.  `planned_now` says whether events 0 and 1
+// (the planner's) belong to this call.
+static int run_items(vc_comm *c, const PlanInfo &pi, const VcDesc *items, const char *sendbuf, char *recvbuf, bool planned_now) {
+    hipStream_t st = c->stream;
+    const int nl = pi.nl;
+    HIP_TRY(c->stage.reserve((size_t)pi.stage_bytes + 64));
+    if (c->timing) { int rc = ensure_events(c, (size_t)nl + 4); if (rc) return rc; }
     for (int k = 0; k < nl; k++) {
         if (c->timing) HIP_TRY(hipEventRecord(c->events[2 + k], st));
-        HIP_TRY(vc_launch_copy_items(c->desc.as<VcDesc>() + h[3 + nl + k], h[3 + 2 * nl + k], sendbuf, recvbuf, c->stage.as<char>(), st));
+        HIP_TRY(vc_launch_copy_items(items + pi.first[k], pi.count[k], sendbuf, recvbuf, c->stage.as<char>(), st));
     }
     if (c->timing) HIP_TRY(hipEventRecord(c->events[2 + nl], st));
     HIP_TRY(hipStreamSynchronize(st));
 
     vc_stats_t &s = c->stats;
     s.n_launches = nl;
-    s.n_digits = S.w;
-    s.staging_bytes = stage_bytes;
-    s.payload_bytes = h[1];
+    s.n_digits = pi.n_digits;
+    s.staging_bytes = pi.stage_bytes;
+    s.payload_bytes = pi.payload_bytes;
     s.moved_bytes = 0;
     s.plan_ms = s.total_ms = 0.f;
     for (int k = 0; k < nl; k++) {
-        s.launch_bytes[k] = h[3 + k];
-        s.moved_bytes += s.launch_bytes[k];
+        s.launch_bytes[k] = pi.bytes[k];
+        s.moved_bytes += pi.bytes[k];
         s.launch_ms[k] = 0.f;
-        c->launch_first[k] = h[3 + nl + k];
-        c->launch_items[k] = h[3 + 2 * nl + k];
+        c->launch_first[k] = pi.first[k];
+        c->launch_items[k] = pi.count[k];
         if (c->timing) HIP_TRY(hipEventElapsedTime(&s.launch_ms[k], c->events[2 + k], c->events[3 + k]));
     }
     if (c->timing) {
-        HIP_TRY(hipEventElapsedTime(&s.plan_ms, c->events[0], c->events[1]));
-        HIP_TRY(hipEventElapsedTime(&s.total_ms, c->events[0], c->events[2 + nl]));
+        if (planned_now) HIP_TRY(hipEventElapsedTime(&s.plan_ms, c->events[0], c->events[1]));
+        HIP_TRY(hipEventElapsedTime(&s.total_ms, c->events[planned_now ? 0 : 2], c->events[2 + nl]));
     }
     c->last_nlaunch = nl;
+    c->last_items = items;
     return VC_OK;
+}
+
+static int run_schedule(vc_comm *c, VcSched S, std::vector<VcLaunchInfo> &L, const char *sendbuf, char *recvbuf, VcTables T) {
+    PlanInfo pi;
+    int rc = build_plan(c, S, L, T, c->desc, pi);
+    if (rc) return rc;
+    return run_items(c, pi, c->desc.as<VcDesc>(), sendbuf, recvbuf, true);
 }
 
 static int check_common(vc_comm *c, const void *sendbuf, const void *recvbuf, int esz) {
@@ -351,6 +387,7 @@ static int run_uniform(VcFunc f, int n, int r, vc_comm *c, char *sendbuf, int se
     int rc = check_common(c, sendbuf, recvbuf, esz);
     if (rc) return rc;
     if (sendcount < 0) return fail_arg("negative block length");
+    if ((int64_t)sendcount * c->P > 0x7FFFFFFF) return fail_arg("sendcount * P must fit the reference's int displacements");
     VcSched S;
     std::vector<VcLaunchInfo> L;
     rc = vc_make_schedule(f, c->P, n, r, 0, esz, sendcount, S, L);
@@ -376,6 +413,63 @@ extern "C" int uniform_inverse_isplit_r_bruck(int n, int r1, int r2, char *sendb
     return run_uniform(VC_F_UNIFORM_ISPLIT, n, r1, c, sendbuf, sendcount, sendtype_size, recvbuf);
 }
 
+// ------------------------------------------------------------- persistent plans
+
+struct vc_plan {
+    vc_comm *comm = nullptr;
+    PlanInfo info;
+    DevBuf items;
+};
+
+static bool func_by_name(const char *name, VcFunc &f) {
+    static const struct { const char *name; VcFunc f; } table[] = {
+        {"twophase_rbruck_alltoallv", VC_F_TWOPHASE}, {"twophase_rbruck_alltoallv_om", VC_F_OM}, {"tuna_algorithm", VC_F_TUNA},
+        {"TTPL_BT_alltoallv", VC_F_TTPL}, {"TTPL_BT_alltoallv_s1", VC_F_TTPL_S1}, {"spreadout_alltoallv", VC_F_SPREADOUT},
+        {"MPICH_intra_scattered", VC_F_MPICH_SCATTERED}, {"ompi_alltoallv_intra_basic_linear", VC_F_OMPI_LINEAR},
+        {"ompi_alltoallv_intra_pairwise", VC_F_OMPI_PAIRWISE}, {"exclisive_or_alltoallv", VC_F_XOR}};
+    for (const auto &e : table)
+        if (strcmp(name, e.name) == 0) { f = e.f; return true; }
+    return false;
+}
+
+extern "C" int vc_plan_create(const char *function, int n, int r, int batch, int *sendcounts, int *sdispls, int elem_size,
+                              int *recvcounts, int *rdispls, int recvbuf_low_bits, vc_comm_t c, vc_plan_t *plan_out) {
+    if (!c || !function || !plan_out) return fail_arg("vc_plan_create: null argument");
+    if (elem_size < 1) return fail_arg("element size must be >= 1");
+    if (!c->sbase || !c->rbase) return fail_arg("vc_comm_set_bases has not been called");
+    VcFunc f;
+    if (!func_by_name(function, f)) return fail_arg("vc_plan_create: unknown function name");
+    if (!sendcounts || !sdispls || !recvcounts || (f != VC_F_TTPL && !rdispls)) return fail_arg("null table");
+    VcSched S;
+    std::vector<VcLaunchInfo> L;
+    int rc = vc_make_schedule(f, c->P, n, r, batch, elem_size, 0, S, L);
+    if (rc) return schedule_error(rc);
+    S.recv_lo = recvbuf_low_bits & 15;
+    vc_plan *p = new vc_plan();
+    p->comm = c;
+    rc = build_plan(c, S, L, make_tables(c, sendcounts, sdispls, recvcounts, rdispls), p->items, p->info);
+    if (rc == VC_OK && hipStreamSynchronize(c->stream) != hipSuccess) rc = fail_arg("vc_plan_create: stream error", VC_ERR_HIP);
+    if (rc) { p->items.release(); delete p; return rc; }
+    *plan_out = p;
+    return VC_OK;
+}
+
+extern "C" int vc_plan_execute(vc_plan_t p, char *sendbuf, char *recvbuf) {
+    if (!p || !sendbuf || !recvbuf) return fail_arg("vc_plan_execute: null argument");
+    if ((int)((uintptr_t)recvbuf & 15) != p->info.recv_lo)
+        return fail_arg("vc_plan_execute: recvbuf must have the low address bits the plan was made for");
+    return run_items(p->comm, p->info, p->items.as<VcDesc>(), sendbuf, recvbuf, false);
+}
+
+extern "C" int vc_plan_free(vc_plan_t p) {
+    if (!p) return VC_OK;
+    (void)hipStreamSynchronize(p->comm->stream);
+    if (p->comm->last_items == p->items.as<VcDesc>()) { p->comm->last_items = nullptr; p->comm->last_nlaunch = 0; }
+    p->items.release();
+    delete p;
+    return VC_OK;
+}
+
 // ------------------------------------------------------------------ inspection
 
 extern "C" int vc_comm_last_traffic(vc_comm_t c, int launch, int64_t *matrix_out) {
@@ -384,7 +478,7 @@ extern "C" int vc_comm_last_traffic(vc_comm_t c, int launch, int64_t *matrix_out
     const size_t PP = (size_t)c->P * c->P;
     HIP_TRY(c->scratch.reserve(sizeof(int64_t) * PP));
     HIP_TRY(hipMemsetAsync(c->scratch.p, 0, sizeof(int64_t) * PP, c->stream));
-    HIP_TRY(vc_launch_traffic(c->desc.as<VcDesc>() + c->launch_first[launch], c->launch_items[launch], c->scratch.as<int64_t>(), c->P,
+    HIP_TRY(vc_launch_traffic(c->last_items + c->launch_first[launch], c->launch_items[launch], c->scratch.as<int64_t>(), c->P,
                               c->stream));
     HIP_TRY(hipMemcpyAsync(matrix_out, c->scratch.p, sizeof(int64_t) * PP, hipMemcpyDeviceToHost, c->stream));
     HIP_TRY(hipStreamSynchronize(c->stream));

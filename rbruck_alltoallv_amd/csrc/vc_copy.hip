@@ -59,8 +59,11 @@ __global__ __launch_bounds__(VC_THREADS) void vc_copy_items_kernel(const VcDesc 
 }
 
 hipError_t vc_launch_copy_items(const VcDesc *items, int64_t nitems, const char *sendbuf, char *recvbuf, char *stage, hipStream_t st) {
-    if (nitems <= 0) return hipSuccess;
-    hipLaunchKernelGGL(vc_copy_items_kernel, dim3((unsigned)nitems), dim3(VC_THREADS), 0, st, items, sendbuf, recvbuf, stage);
+    const int64_t max_grid = 0x7FFFFFFF;                  // gridDim.x limit; more items than that go in several launches
+    for (int64_t done = 0; done < nitems; done += max_grid) {
+        const int64_t now = nitems - done < max_grid ? nitems - done : max_grid;
+        hipLaunchKernelGGL(vc_copy_items_kernel, dim3((unsigned)now), dim3(VC_THREADS), 0, st, items + done, sendbuf, recvbuf, stage);
+    }
     return hipGetLastError();
 }
 

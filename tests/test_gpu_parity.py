@@ -248,3 +248,44 @@ def test_arena_pointers_of_any_alignment(api, shift):
         assert np.array_equal(dr.cpu().numpy(), want), (name, shift)
         assert bool((rbig[:r_shift] == 0xEE).all()) and bool((rbig[r_shift + prob.recv_bytes:] == 0xEE).all())
     dp.comm.free()
+
+
+def test_persistent_plans(api):
+    """A plan executes the same copies as the call it was made from, any number of times, on any arenas."""
+    import torch
+    counts = W.counts_uniform_random(24, 5000, seed=21)
+    counts[counts % 5 == 0] = 0
+    prob = W.make_problem(counts, 2, 1, 0)
+    send = W.fill_send_arena(prob, 0, 4)
+    want = W.expected_recv_arena(prob, send)
+    dp = api.DeviceProblem(prob)
+    ds = _to_dev(api, send)
+    for function, kw, direct in (
+        ("twophase_rbruck_alltoallv", dict(r=3), lambda d: api.twophase_rbruck_alltoallv(3, dp, ds, d)),
+        ("tuna_algorithm", dict(r=4, batch=2), lambda d: api.tuna_algorithm(4, 2, dp, ds, d)),
+        ("TTPL_BT_alltoallv", dict(n=6, r=6, batch=0), lambda d: api.TTPL_BT_alltoallv(6, 6, 0, dp, ds, d)),
+        ("TTPL_BT_alltoallv_s1", dict(n=4, r=2, batch=7), lambda d: api.TTPL_BT_alltoallv_s1(4, 2, 7, dp, ds, d)),
+        ("MPICH_intra_scattered", dict(batch=5), lambda d: api.MPICH_intra_scattered(5, dp, ds, d)),
+    ):
+        dr = dp.new_recv_arena(0xEE)
+        plan = api.Plan(function, dp, dr, **kw)
+        assert plan.rc == 0, dp.comm.error()
+        assert direct(dr) == 0
+        traffic_direct = [dp.comm.last_traffic(k) for k in range(dp.comm.last_stats().n_launches)]
+        for rep in range(3):
+            dr2 = dp.new_recv_arena(0xEE)
+            ds2 = ds.clone()
+            assert plan.execute(ds2, dr2) == 0, dp.comm.error()
+            assert np.array_equal(dr2.cpu().numpy(), want), (function, rep)
+        st = dp.comm.last_stats()
+        assert st.n_launches == len(traffic_direct) and st.payload_bytes == prob.payload_bytes
+        for k, m in enumerate(traffic_direct):
+            assert np.array_equal(dp.comm.last_traffic(k), m)
+        # a receive arena with other low address bits is refused, not mis-copied
+        rbig = torch.full((prob.recv_bytes + 16,), 0xEE, dtype=torch.uint8, device="cuda:0")
+        assert plan.execute(ds, rbig[3:]) == -5
+        plan.free()
+    bad = api.Plan("no_such_function", dp, dp.new_recv_arena())
+    assert bad.rc == -5
+    assert api.Plan("twophase_rbruck_alltoallv", dp, dp.new_recv_arena(), r=1).rc == -1
+    dp.comm.free()
