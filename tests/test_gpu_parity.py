@@ -289,3 +289,53 @@ def test_persistent_plans(api):
     assert bad.rc == -5
     assert api.Plan("twophase_rbruck_alltoallv", dp, dp.new_recv_arena(), r=1).rc == -1
     dp.comm.free()
+
+
+def _device_check(api, prob, seed, calls):
+    """Runs calls on device-filled payload and checks each with the exact on-device definition check."""
+    dp = api.DeviceProblem(prob)
+    ds = dp.new_send_arena()
+    dp.fill_payload(0, seed, ds)
+    for name, fn, packed in calls(dp, ds):
+        print("  ", name, flush=True)
+        dr = dp.new_recv_arena(0xEE)
+        assert fn(dr) == 0, (name, dp.comm.error())
+        assert dp.verify(ds, dr, packed_recv=packed) == 0, name
+        st = dp.comm.last_stats()
+        assert st.payload_bytes == prob.payload_bytes
+    dp.comm.free()
+
+
+def test_benchmark_shapes_at_reduced_size(api):
+    """The five benchmark shapes at their full rank counts with smaller blocks: many digits, many launches."""
+    c3 = W.counts_zipf(256, 4096, 1.2, 5, 0)
+    _device_check(api, W.make_problem(c3, 4, 0, 0), 1, lambda dp, ds: [
+        ("C3 twophase r=16", lambda d: api.twophase_rbruck_alltoallv(16, dp, ds, d), False),
+        ("C3 om r=2", lambda d: api.twophase_rbruck_alltoallv_om(2, dp, ds, d), False),
+        ("C3 tuna r=255 b=1 (255 launches)", lambda d: api.tuna_algorithm(255, 1, dp, ds, d), False)])
+    c4 = W.counts_normal(1024, 256.0, 64.0, 0, 1024, 0)
+    _device_check(api, W.make_problem(c4, 1, 0, 0), 2, lambda dp, ds: [
+        ("C4 ttpl n=32 r=32", lambda d: api.TTPL_BT_alltoallv(32, 32, 0, dp, ds, d), True),
+        ("C4 ttpl n=32 r=2 bblock=5", lambda d: api.TTPL_BT_alltoallv(32, 2, 5, dp, ds, d), True),
+        ("C4 s1 n=32 r=32 bblock=100", lambda d: api.TTPL_BT_alltoallv_s1(32, 32, 100, dp, ds, d), False),
+        ("C4 s1 n=64 r=8", lambda d: api.TTPL_BT_alltoallv_s1(64, 8, 0, dp, ds, d), False),
+        ("C4 twophase r=2 (10 digits)", lambda d: api.twophase_rbruck_alltoallv(2, dp, ds, d), False)])
+    c5 = W.counts_fft_rows(512, 32, 4096)
+    _device_check(api, W.make_problem(c5, 8, 0, 0), 3, lambda dp, ds: [
+        (f"C5 tuna r={r} b={b}", (lambda d, r=r, b=b: api.tuna_algorithm(r, b, dp, ds, d)), False)
+        for r, b in ((2, 0), (8, 0), (32, 0), (512, 0), (32, 7))])
+    up = W.make_uniform_problem(256, 300, 4)
+    _device_check(api, up, 4, lambda dp, ds: [
+        ("uniform spreadout n=16 r=4", lambda d: api.uniform_spreadout_twolayer(16, 4, dp, 300, ds, d), False),
+        ("uniform isplit n=32 r=3", lambda d: api.uniform_inverse_isplit_r_bruck(32, 3, 2, dp, 300, ds, d), False)])
+
+
+def test_reference_input_matrices(api):
+    """The reference's own communication patterns (inputs/<P>proc), scaled down, through the function its driver uses."""
+    import os
+    from tests.helpers import INPUTS_DIR
+    for P, div in ((256, 4096), (512, 2048), (1024, 1024)):
+        counts = W.counts_from_npz(os.path.join(INPUTS_DIR, f"global_comm_pattern_{P}proc.npz"), div)
+        _device_check(api, W.make_problem(counts, 1, 0, 0), 5, lambda dp, ds: [
+            (f"ML{P} twophase r=32", lambda d: api.twophase_rbruck_alltoallv(32, dp, ds, d), False),
+            (f"ML{P} tuna r=8", lambda d: api.tuna_algorithm(8, 0, dp, ds, d), False)])
