@@ -3,7 +3,7 @@
 
 A "step" is one complete collective call (planning kernels + every data-moving launch +
 stream synchronisation) over one synthetic batch that is already resident in HBM.  Default
-workload: BASELINE config 4 — TTPL_BT_alltoallv, P = 1024 virtual ranks, 32 per node, r = 32,
+workload: benchmark configuration 4 — TTPL_BT_alltoallv, P = 1024 virtual ranks, 32 per node, r = 32,
 1-byte elements, counts ~ Normal(4096, 1024) clipped to [0, 16384].
 
 Prints ONE JSON line: effective GB/s (payload bytes / time), the HBM roofline of the copy
@@ -37,7 +37,7 @@ METRIC = "effective alltoallv GB/s + % HBM peak, P=64..1024 virtual ranks, 1 GPU
 
 
 def workload(name: str, seed: int):
-    """(counts, esz, function name, tunables, hop matrix) of a BASELINE configuration, or of one of the reference's
+    """(counts, esz, function name, tunables, hop matrix) of one of the five benchmark configurations, or of one of the reference's
     own communication-pattern matrices (ML<P>: inputs/<P>proc, 1-byte elements, twophase_rbruck_alltoallv as in
     examples/MLinputs_example.cpp:96)."""
     if name.startswith("ML"):
@@ -249,7 +249,7 @@ def main() -> None:
         "metric": METRIC, "value": round(value, 2), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "u8", "data": "synthetic",
-        "config": {"workload": (f"BASELINE config {args.workload[1:]}" if args.workload[0] == "C" else
+        "config": {"workload": (f"benchmark configuration {args.workload[1:]}" if args.workload[0] == "C" else
                                 f"reference input matrix inputs/{prob.P}proc") + f": {func}, P={prob.P} virtual ranks, "
                                + ", ".join(f"{k}={v}" for k, v in tun.items()) + f", {esz}-byte elements",
                    "payload_bytes": S, "algorithmic_bytes": A, "launches_per_step": int(st.n_launches),

@@ -205,7 +205,7 @@ def expected_recv_arena(prob: Problem, send_arena: np.ndarray, fill: int = 0xEE,
     return out
 
 
-# ----------------------------------------------------------------- BASELINE configs
+# ----------------------------------------------------------------- benchmark configurations
 
 def config_counts(name: str, seed: int = 0, scale: int = 1) -> tuple[np.ndarray, int, dict]:
     """Count matrix, element size and tunables of one of the five benchmark configurations.

@@ -7,7 +7,7 @@
 //   - source and destination ranges lie inside their arenas,
 //   - staged bytes are read only after they were written,
 //   - within one launch no destination overlaps another destination or a source.
-// Blocks are split into the same VC_CHUNK pieces the copy kernel gets.
+// Copies are cut into the same pieces (work items) the copy kernel gets.
 // This is how indexing mistakes are found without a GPU.
 #include <algorithm>
 #include <cstdint>

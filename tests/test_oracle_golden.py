@@ -32,7 +32,7 @@ def test_digest_restatement_agrees():
 
 
 def test_c1_every_byte_of_every_recvbuf():
-    """BASELINE config 1 (P=8, r=2, int32, counts U{0..64} from seed 0, word = src*2^20 + dst*2^10 + idx):
+    """Benchmark configuration 1 (P=8, r=2, int32, counts U{0..64} from seed 0, word = src*2^20 + dst*2^10 + idx):
     the reference's complete receive buffers, byte for byte."""
     case = next(c for c in CASES if c["id"] == "C1-twophase")
     prob = problem_for_case(case)
