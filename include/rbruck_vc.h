@@ -93,6 +93,12 @@ int twophase_rbruck_alltoallv_om(int r, char *sendbuf, int *sendcounts, int *sdi
 int tuna_algorithm(int r, int b, char *sendbuf, int *sendcounts, int *sdispls, int sendtype_size, char *recvbuf,
                    int *recvcounts, int *rdispls, int recvtype_size, vc_comm_t comm);
 
+/* src/tuna2.cpp:10-239 — TuNA with the received rounds of a digit unpacked together at the end of the digit
+ * (:202-223).  On the GPU that is what a launch per batch already does, so the schedule is tuna_algorithm's.  The
+ * reference corrupts messages for b > 1 (one send buffer reused under in-flight sends, :175-185); this does not. */
+int tuna2_algorithm(int r, int b, char *sendbuf, int *sendcounts, int *sdispls, int sendtype_size, char *recvbuf,
+                    int *recvcounts, int *rdispls, int recvtype_size, vc_comm_t comm);
+
 /* src/twophase_twolayer_rbruck.cpp:237-463 — two-layer, coalesced inter-node messages, bblock groups in flight.
  * Like the reference it ignores rdispls: rank t's blocks land back to back in source-rank order. */
 int TTPL_BT_alltoallv(int n, int r, int bblock, char *sendbuf, int *sendcounts, int *sdispls, int sendtype_size,
@@ -154,6 +160,15 @@ int vc_plan_create(const char *function, int n, int r, int batch, int *sendcount
 /* Runs the planned collective; blocking.  One plan (or call) per communicator at a time. */
 int vc_plan_execute(vc_plan_t plan, char *sendbuf, char *recvbuf);
 int vc_plan_free(vc_plan_t plan);
+
+/* ---- radix choice.  The reference leaves r to the caller (its drivers sweep a list of bases,
+ * examples/rbruckv_example.cpp:33-35).  Given candidate radices this evaluates, on the device, the bytes each would
+ * move (sum over blocks of hops x bytes; hops = non-zero base-r digits of the offset inside the node, + 1 if the node
+ * differs) and returns the candidate with the smallest modelled time 2 * moved / (sustained copy rate) + launches x
+ * launch latency.  n = ranks per node for the two-layer functions, 0 or P for the one-layer ones.  `candidates` and the
+ * outputs are HOST arrays; moved_bytes_out (may be NULL) receives the moved bytes per candidate. ---- */
+int vc_suggest_radix(const int *sendcounts, int elem_size, int n, const int *candidates, int ncand, int *best_out,
+                     int64_t *moved_bytes_out, vc_comm_t comm);
 
 /* ---- measurement and inspection (the reference's global phase timers, src/rbruckv.h:13-18) ---- */
 

@@ -351,6 +351,131 @@ int ora_tuna_algorithm(int r, int b, char *sendarena, const int64_t *sbase, cons
     return lsd_compact_bruck(&c, r, w, nlpow, d, K, b, 1);
 }
 
+/* ----------------------------------------------------------------- 3b. TuNA2
+ * src/tuna2.cpp:10-239: TuNA's rounds, but the data of all rounds of a digit is received into one buffer and
+ * unpacked only after the digit's last batch (:202-223); the compact staging index comes from a table (:63-73).
+ * The reference packs every round of a batch into ONE temp_send_buffer while earlier MPI_Isends from it may still
+ * be in flight (:175-185), which corrupts messages for b > 1; a correct run is what is restated here (each round
+ * keeps its own message), so for b > 1 the pin is the alltoallv definition and not a reference run. */
+int ora_tuna2_algorithm(int r, int b, char *sendarena, const int64_t *sbase, const int *sendcounts,
+                        const int *sdispls, int esz, char *recvarena, const int64_t *rbase,
+                        const int *recvcounts, const int *rdispls, int P) {
+    if (P < 3) return -3;                       /* :19, :27 would loop forever */
+    if (r < 2) r = 2;                           /* :13 */
+    if (r > P - 1) r = P - 1;                   /* :20 */
+    if (b <= 0 || b > P) b = P;                 /* :21 */
+    ora_ctx c = make_ctx(sendarena, sbase, sendcounts, sdispls, esz, recvarena, rbase, recvcounts, rdispls, P);
+    int w, nlpow, d, K;
+    ora_radix_params_int(P, r, &w, &nlpow, &d, &K);
+    int nstage = P - K - 1;
+    int64_t stride = 0;
+    int *stage_cnt = NULL, *table = NULL;
+    char **stage = (char **)calloc((size_t)P, sizeof(char *));
+    if (K < P - 1) {
+        stride = (int64_t)global_max_count(&c) * esz;
+        stage_cnt = (int *)calloc((size_t)P * nstage, sizeof(int));
+        for (int p = 0; p < P; p++) stage[p] = (char *)malloc((size_t)(stride * nstage + 1));
+        /* table of compact indices: offsets with at least two non-zero digits, numbered in ascending order (:63-73) */
+        table = (int *)malloc(sizeof(int) * (size_t)P);
+        for (int i = 0; i < P; i++) table[i] = -1;
+        int di = 0, dist = 1;
+        for (int x = 0; x < w; x++) {
+            for (int z = 1; z < r; z++) {
+                int sp = z * dist;
+                if (sp > P) break;
+                int end = sp + dist > P ? P : sp + dist;
+                for (int i = sp + 1; i < end; i++) table[i] = di++;
+            }
+            dist *= r;
+        }
+    }
+    self_copies(&c);
+
+    int *offs = (int *)malloc(sizeof(int) * (size_t)(nlpow > 0 ? nlpow : 1));
+    ora_msg **inbox = (ora_msg **)calloc((size_t)r, sizeof(ora_msg *));     /* [z][rank]: what rank received in round z */
+    int *nbs = (int *)calloc((size_t)r, sizeof(int));
+    for (int z = 0; z < r; z++) inbox[z] = (ora_msg *)calloc((size_t)P, sizeof(ora_msg));
+    int dist = 1;
+    for (int x = 0; x < w; x++) {
+        int ze = (x == w - 1) ? r - d : r;
+        int64_t ndist = (int64_t)dist * r;
+        for (int k = 1; k < ze; k += b) {
+            int ss = ze - k < b ? ze - k : b;
+            for (int si = 0; si < ss; si++) {
+                int z = k + si, hop = z * dist;
+                int nc = (int)(P / ndist) * dist, rem = (int)(P % ndist) - hop;           /* :127-129 */
+                if (rem < 0) rem = 0;
+                int ns = rem > dist ? nc + dist : nc + rem;
+                nbs[z] = ns;
+                if (ns == 1) {                                                      /* :136-141 */
+                    for (int p = 0; p < P; p++) {
+                        int from_rank = (p + hop) % P;
+                        int64_t nbytes = (int64_t)SC(&c, from_rank, p) * esz;
+                        memcpy(rbuf(&c, p) + (int64_t)RD(&c, p, from_rank) * esz,
+                               sbuf(&c, from_rank) + (int64_t)SD(&c, from_rank, p) * esz, (size_t)nbytes);
+                        trace_msg(1, x, z, from_rank, p, 1, nbytes);
+                    }
+                    continue;
+                }
+                int nb = digit_offsets(P, dist, r, z, offs);
+                /* every rank packs (:150-185); rank p's message goes to p - hop, i.e. inbox[z][p - hop] */
+                for (int p = 0; p < P; p++) {
+                    int to = (p - hop + P) % P;
+                    ora_msg *m = &inbox[z][to];
+                    int64_t tot = 0;
+                    for (int i = 0; i < nb; i++) {
+                        int key = (p - offs[i] + P) % P;
+                        tot += (int64_t)((i % dist == 0) ? SC(&c, p, key) : stage_cnt[(int64_t)p * nstage + table[offs[i]]]) * esz;
+                    }
+                    msg_reserve(m, nb, tot);
+                    int64_t off = 0;
+                    for (int i = 0; i < nb; i++) {
+                        int key = (p - offs[i] + P) % P;
+                        int cnt; const char *from;
+                        if (i % dist == 0) { cnt = SC(&c, p, key); from = sbuf(&c, p) + (int64_t)SD(&c, p, key) * esz; }
+                        else { int ci = table[offs[i]]; cnt = stage_cnt[(int64_t)p * nstage + ci]; from = stage[p] + (int64_t)ci * stride; }
+                        m->sizes[i] = cnt;
+                        memcpy(m->bytes + off, from, (size_t)((int64_t)cnt * esz));
+                        off += (int64_t)cnt * esz;
+                    }
+                    trace_msg(0, x, z, p, to, nb, tot);
+                }
+            }
+            /* MPI_Waitall of the batch (:190) */
+        }
+        /* deferred unpack of the whole digit (:202-223) */
+        for (int z = 1; z < ze; z++) {
+            if (nbs[z] <= 1) continue;
+            int nb = digit_offsets(P, dist, r, z, offs);
+            for (int p = 0; p < P; p++) {
+                ora_msg *m = &inbox[z][p];
+                int64_t off = 0;
+                for (int i = 0; i < nb; i++) {
+                    int slot = (offs[i] + p) % P;
+                    int64_t nbytes = (int64_t)m->sizes[i] * esz;
+                    if (i < dist) {
+                        memcpy(rbuf(&c, p) + (int64_t)RD(&c, p, slot) * esz, m->bytes + off, (size_t)nbytes);
+                    } else {
+                        int ci = table[offs[i]];
+                        memcpy(stage[p] + (int64_t)ci * stride, m->bytes + off, (size_t)nbytes);
+                        stage_cnt[(int64_t)p * nstage + ci] = m->sizes[i];
+                    }
+                    off += nbytes;
+                }
+                msg_release(m);
+            }
+        }
+        dist *= r;
+    }
+    for (int z = 0; z < r; z++) free(inbox[z]);
+    for (int p = 0; p < P; p++) free(stage[p]);
+    free(inbox); free(nbs); free(offs); free(stage); free(stage_cnt); free(table);
+    return 0;
+}
+
+/* compact staging index of offset j (>= 2 non-zero digits), float form of tuna.cpp:93-97; exported for tests */
+int ora_compact_slot_float(int j, int r) { return compact_slot_float(j, r); }
+
 /* ----------------------------- 4/5. two-phase two-layer, non-uniform (TTPL) */
 
 typedef struct {

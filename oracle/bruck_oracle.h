@@ -18,7 +18,9 @@
  * textbook MPI_Alltoallv definition on brute-force inputs, against the golden
  * digests produced by the real reference under mpiexec (tests/golden/), and
  * its round structure against the closed forms for K, ns and the residency
- * invariants.  No function is "parity unpinned".
+ * invariants.  No function is "parity unpinned"; ora_tuna2_algorithm is pinned by
+ * the reference for b = 1 and by the definition for b > 1, where the reference
+ * itself is defective.
  */
 #ifndef BRUCK_ORACLE_H_
 #define BRUCK_ORACLE_H_
@@ -70,6 +72,12 @@ int ora_twophase_rbruck_alltoallv_om(int r, char *sendarena, const int64_t *sbas
 int ora_tuna_algorithm(int r, int b, char *sendarena, const int64_t *sbase, const int *sendcounts,
                        const int *sdispls, int esz, char *recvarena, const int64_t *rbase,
                        const int *recvcounts, const int *rdispls, int P);
+
+/* src/tuna2.cpp:10-239 with its send-buffer reuse (:175-185) repaired; see the note at the definition. */
+int ora_tuna2_algorithm(int r, int b, char *sendarena, const int64_t *sbase, const int *sendcounts,
+                        const int *sdispls, int esz, char *recvarena, const int64_t *rbase,
+                        const int *recvcounts, const int *rdispls, int P);
+int ora_compact_slot_float(int j, int r);
 
 /* src/twophase_twolayer_rbruck.cpp:237-463 (coalesced; ignores rdispls).
  * Returns -2 when n does not divide P, where the reference hangs. */

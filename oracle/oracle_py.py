@@ -64,6 +64,10 @@ def tuna_algorithm(r, b, prob, send, recv):
     return lib().ora_tuna_algorithm(C.c_int(r), C.c_int(b), *_v_args(prob, send, recv))
 
 
+def tuna2_algorithm(r, b, prob, send, recv):
+    return lib().ora_tuna2_algorithm(C.c_int(r), C.c_int(b), *_v_args(prob, send, recv))
+
+
 def TTPL_BT_alltoallv(n, r, bblock, prob, send, recv):
     return lib().ora_TTPL_BT_alltoallv(C.c_int(n), C.c_int(r), C.c_int(bblock), *_v_args(prob, send, recv))
 

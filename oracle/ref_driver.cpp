@@ -12,7 +12,7 @@
  * compared with MPI_Alltoallv.
  *
  * usage: mpiexec -n P ref_driver FUNC COUNTS ESZ R B N BBLOCK LAYOUT PAYLOAD SEED ITERS OUT
- *   FUNC    twophase | om | tuna | ttpl | ttpl_s1 | uniform_spreadout | uniform_isplit |
+ *   FUNC    twophase | om | tuna | tuna2 | ttpl | ttpl_s1 | uniform_spreadout | uniform_isplit |
  *           scattered | ompi_linear | ompi_pairwise | xor | spreadout | mpi_alltoallv
  *   COUNTS  file of P*P int32 (row = sender); for the uniform functions the decimal block count
  *   LAYOUT  0 packed ascending displacements, 1 reversed order with gaps
@@ -112,6 +112,7 @@ int main(int argc, char **argv) {
         if (func == "twophase") ret = twophase_rbruck_alltoallv(r, sb, sc, sd, dtype, rb, rc, rd, dtype, MPI_COMM_WORLD);
         else if (func == "om") ret = twophase_rbruck_alltoallv_om(r, sb, sc, sd, dtype, rb, rc, rd, dtype, MPI_COMM_WORLD);
         else if (func == "tuna") ret = tuna_algorithm(r, b, sb, sc, sd, dtype, rb, rc, rd, dtype, MPI_COMM_WORLD);
+        else if (func == "tuna2") ret = tuna2_algorithm(r, b, sb, sc, sd, dtype, rb, rc, rd, dtype, MPI_COMM_WORLD);
         else if (func == "ttpl") ret = TTPL_BT_alltoallv(n, r, bblock, sb, sc, sd, dtype, rb, rc, rd, dtype, MPI_COMM_WORLD);
         else if (func == "ttpl_s1") ret = TTPL_BT_alltoallv_s1(n, r, bblock, sb, sc, sd, dtype, rb, rc, rd, dtype, MPI_COMM_WORLD);
         else if (func == "uniform_spreadout") ret = uniform_spreadout_twolayer(n, r, sb, sendcounts[0], dtype, rb, recvcounts[0], dtype, MPI_COMM_WORLD);

@@ -36,6 +36,7 @@ SYMBOLS = {
     "twophase_rbruck_alltoallv": (_I, [_I] + _V_TAIL),
     "twophase_rbruck_alltoallv_om": (_I, [_I] + _V_TAIL),
     "tuna_algorithm": (_I, [_I, _I] + _V_TAIL),
+    "tuna2_algorithm": (_I, [_I, _I] + _V_TAIL),
     "TTPL_BT_alltoallv": (_I, [_I, _I, _I] + _V_TAIL),
     "TTPL_BT_alltoallv_s1": (_I, [_I, _I, _I] + _V_TAIL),
     "uniform_spreadout_twolayer": (_I, [_I, _I, _P, _I, _I, _P, _I, _I, _P]),
@@ -48,6 +49,7 @@ SYMBOLS = {
     "vc_plan_create": (_I, [C.c_char_p, _I, _I, _I, _P, _P, _I, _P, _P, _I, _P, C.POINTER(_P)]),
     "vc_plan_execute": (_I, [_P, _P, _P]),
     "vc_plan_free": (_I, [_P]),
+    "vc_suggest_radix": (_I, [_P, _I, _I, _P, _I, C.POINTER(_I), _P, _P]),
     "vc_comm_set_timing": (_I, [_P, _I]),
     "vc_comm_last_stats": (_I, [_P, C.POINTER(VcStats)]),
     "vc_comm_last_traffic": (_I, [_P, _I, _P]),

@@ -128,6 +128,11 @@ def tuna_algorithm(r: int, b: int, p: DeviceProblem, send: torch.Tensor, recv: t
     return p.comm.lib.tuna_algorithm(r, b, *_tail(p, send, recv))
 
 
+def tuna2_algorithm(r: int, b: int, p: DeviceProblem, send: torch.Tensor, recv: torch.Tensor) -> int:
+    """src/tuna2.cpp:10-239"""
+    return p.comm.lib.tuna2_algorithm(r, b, *_tail(p, send, recv))
+
+
 def TTPL_BT_alltoallv(n: int, r: int, bblock: int, p: DeviceProblem, send: torch.Tensor, recv: torch.Tensor) -> int:
     """src/twophase_twolayer_rbruck.cpp:237-463"""
     return p.comm.lib.TTPL_BT_alltoallv(n, r, bblock, *_tail(p, send, recv))
@@ -194,3 +199,13 @@ class Plan:
         if self.handle:
             self.problem.comm.lib.vc_plan_free(self.handle)
             self.handle = None
+
+
+def suggest_radix(p: DeviceProblem, candidates: list[int], n: int = 0) -> tuple[int, list[int]]:
+    """vc_suggest_radix: (best radix, bytes moved per candidate)."""
+    cand = (C.c_int * len(candidates))(*candidates)
+    moved = (C.c_int64 * len(candidates))()
+    best = C.c_int(0)
+    p.comm._check(p.comm.lib.vc_suggest_radix(p.sendcounts.data_ptr(), p.esz, n, cand, len(candidates), C.byref(best), moved,
+                                              p.comm.handle))
+    return best.value, list(moved)

@@ -338,6 +338,12 @@ extern "C" int tuna_algorithm(int r, int b, char *sendbuf, int *sendcounts, int 
     return run_v(VC_F_TUNA, 0, r, b, c, sendbuf, sendcounts, sdispls, sendtype_size, recvbuf, recvcounts, rdispls);
 }
 
+extern "C" int tuna2_algorithm(int r, int b, char *sendbuf, int *sendcounts, int *sdispls, int sendtype_size, char *recvbuf,
+                               int *recvcounts, int *rdispls, int recvtype_size, vc_comm_t c) {
+    (void)recvtype_size;
+    return run_v(VC_F_TUNA2, 0, r, b, c, sendbuf, sendcounts, sdispls, sendtype_size, recvbuf, recvcounts, rdispls);
+}
+
 extern "C" int TTPL_BT_alltoallv(int n, int r, int bblock, char *sendbuf, int *sendcounts, int *sdispls, int sendtype_size,
                                  char *recvbuf, int *recvcounts, int *rdispls, int recvtype_size, vc_comm_t c) {
     (void)recvtype_size;
@@ -423,7 +429,7 @@ struct vc_plan {
 
 static bool func_by_name(const char *name, VcFunc &f) {
     static const struct { const char *name; VcFunc f; } table[] = {
-        {"twophase_rbruck_alltoallv", VC_F_TWOPHASE}, {"twophase_rbruck_alltoallv_om", VC_F_OM}, {"tuna_algorithm", VC_F_TUNA},
+        {"twophase_rbruck_alltoallv", VC_F_TWOPHASE}, {"twophase_rbruck_alltoallv_om", VC_F_OM}, {"tuna_algorithm", VC_F_TUNA}, {"tuna2_algorithm", VC_F_TUNA2},
         {"TTPL_BT_alltoallv", VC_F_TTPL}, {"TTPL_BT_alltoallv_s1", VC_F_TTPL_S1}, {"spreadout_alltoallv", VC_F_SPREADOUT},
         {"MPICH_intra_scattered", VC_F_MPICH_SCATTERED}, {"ompi_alltoallv_intra_basic_linear", VC_F_OMPI_LINEAR},
         {"ompi_alltoallv_intra_pairwise", VC_F_OMPI_PAIRWISE}, {"exclisive_or_alltoallv", VC_F_XOR}};
@@ -467,6 +473,50 @@ extern "C" int vc_plan_free(vc_plan_t p) {
     if (p->comm->last_items == p->items.as<VcDesc>()) { p->comm->last_items = nullptr; p->comm->last_nlaunch = 0; }
     p->items.release();
     delete p;
+    return VC_OK;
+}
+
+// ------------------------------------------------------------------ radix choice
+
+// Launches a schedule of radix r needs: one per digit that has rounds, plus the inter-node launch.
+static int launches_for(int span, int r, bool inter) {
+    int w, d;
+    vc_radix_params(span, r, w, d);
+    int n = 0;
+    for (int x = 0; x < w; x++) n += ((x == w - 1) ? r - d : r) - 1 >= 1;
+    return n + (inter ? 1 : 0);
+}
+
+extern "C" int vc_suggest_radix(const int *sendcounts, int elem_size, int n, const int *candidates, int ncand, int *best_out,
+                                int64_t *moved_bytes_out, vc_comm_t c) {
+    if (!c || !sendcounts || !candidates || !best_out || elem_size < 1 || ncand < 1 || ncand > 64)
+        return fail_arg("vc_suggest_radix: bad argument (1..64 candidates)");
+    const int P = c->P;
+    if (n <= 0) n = P;
+    if (P % n != 0) return fail_arg("n must divide the number of ranks", VC_ERR_GROUP);
+    int cand[64];
+    for (int k = 0; k < ncand; k++) {
+        if (candidates[k] < 2) return fail_arg("radix must be >= 2", VC_ERR_RADIX);
+        cand[k] = std::min(candidates[k], std::max(n, 2));
+    }
+    HIP_TRY(c->scratch.reserve(sizeof(int64_t) * (size_t)P * P));
+    unsigned long long *moved_dev = c->scratch.as<unsigned long long>();
+    int *cand_dev = reinterpret_cast<int *>(moved_dev + 64);
+    HIP_TRY(hipMemsetAsync(moved_dev, 0, sizeof(unsigned long long) * 64, c->stream));
+    HIP_TRY(hipMemcpyAsync(cand_dev, cand, sizeof(int) * ncand, hipMemcpyHostToDevice, c->stream));
+    HIP_TRY(vc_launch_hop_bytes(sendcounts, elem_size, P, n, cand_dev, ncand, moved_dev, c->stream));
+    unsigned long long moved[64];
+    HIP_TRY(hipMemcpyAsync(moved, moved_dev, sizeof(unsigned long long) * ncand, hipMemcpyDeviceToHost, c->stream));
+    HIP_TRY(hipStreamSynchronize(c->stream));
+    // time model: every moved byte is read and written once at the rate the copy kernel sustains on scattered
+    // blocks, every launch costs a fixed latency
+    const double bytes_per_s = 5.2e12, launch_s = 7e-6;
+    double best = 0;
+    for (int k = 0; k < ncand; k++) {
+        const double t = 2.0 * (double)moved[k] / bytes_per_s + launch_s * launches_for(n, cand[k], n < P);
+        if (moved_bytes_out) moved_bytes_out[k] = (int64_t)moved[k];
+        if (k == 0 || t < best) { best = t; *best_out = candidates[k]; }
+    }
     return VC_OK;
 }
 

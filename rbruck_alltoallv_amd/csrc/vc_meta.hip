@@ -189,3 +189,29 @@ hipError_t vc_launch_verify(const char *sendbuf, const char *recvbuf, VcTables t
     hipLaunchKernelGGL(vc_verify_kernel, dim3(P, P), dim3(VC_THREADS), 0, st, sendbuf, recvbuf, t, esz, P, packed, mismatch);
     return hipGetLastError();
 }
+
+// ---------------------------------------------------------------------------
+// Traffic model for choosing the radix: moved[c] = sum over all blocks of hops_r(s, t) * bytes(s, t) for radix
+// r = cand[c], where hops = non-zero base-r digits of the (local) offset, plus one if the node differs, and 1 for a
+// rank's block to itself.  grid (P, ncand).
+// ---------------------------------------------------------------------------
+__global__ __launch_bounds__(VC_THREADS) void vc_hop_bytes_kernel(const int *__restrict__ sc, int esz, int P, int n,
+                                                                  const int *__restrict__ cand, unsigned long long *__restrict__ moved) {
+    __shared__ int64_t lds[VC_WAVES_PER_BLOCK];
+    const int s = blockIdx.x, r = cand[blockIdx.y];
+    int64_t acc = 0;
+    for (int t = threadIdx.x; t < P; t += VC_THREADS) {
+        int hops = (s / n != t / n) ? 1 : 0;
+        for (int j = (s % n - t % n + n) % n; j; j /= r) hops += (j % r) != 0;
+        if (s == t) hops = 1;
+        acc += (int64_t)hops * sc[(int64_t)s * P + t] * esz;
+    }
+    acc = vc_block_sum(acc, lds);
+    if (threadIdx.x == 0 && acc) atomicAdd(&moved[blockIdx.y], (unsigned long long)acc);
+}
+
+hipError_t vc_launch_hop_bytes(const int *sc, int esz, int P, int n, const int *cand_dev, int ncand, unsigned long long *moved_dev,
+                               hipStream_t st) {
+    hipLaunchKernelGGL(vc_hop_bytes_kernel, dim3(P, ncand), dim3(VC_THREADS), 0, st, sc, esz, P, n, cand_dev, moved_dev);
+    return hipGetLastError();
+}

@@ -25,7 +25,8 @@ enum VcFunc {
     VC_F_MPICH_SCATTERED,    // MPICH_intra_scattered
     VC_F_OMPI_LINEAR,        // ompi_alltoallv_intra_basic_linear
     VC_F_OMPI_PAIRWISE,      // ompi_alltoallv_intra_pairwise
-    VC_F_XOR                 // exclisive_or_alltoallv
+    VC_F_XOR,                // exclisive_or_alltoallv
+    VC_F_TUNA2               // tuna2_algorithm: TuNA's rounds with the unpack deferred to the end of each digit
 };
 
 // Digits of span-1 in base r and the number of unused values of the top digit, in
@@ -99,6 +100,8 @@ inline int vc_make_schedule(VcFunc f, int P, int n, int r, int batch, int esz, i
         vc_add_intra_launches(L, S, d, 0);
         break;
     case VC_F_TUNA:
+    case VC_F_TUNA2:                                        // src/tuna2.cpp:13-21: the same clamps; one launch per batch is already
+                                                            // "all rounds received, then unpacked together" (:202-223)
         if (P < 3) return VC_ERR_TOO_FEW_RANKS;             // src/tuna.cpp:20,28 never returns
         if (r < 2) r = 2;                                   // :13
         if (r > P - 1) r = P - 1;                           // :20

@@ -14,7 +14,7 @@ LIB = os.path.join(HERE, "_build", "libplan_emulator.so")
 CSRC = os.path.join(os.path.dirname(HERE), "rbruck_alltoallv_amd", "csrc")
 
 F_TWOPHASE, F_OM, F_TUNA, F_TTPL, F_TTPL_S1, F_UNIFORM_SPREADOUT, F_UNIFORM_ISPLIT, F_SPREADOUT, F_MPICH_SCATTERED, \
-    F_OMPI_LINEAR, F_OMPI_PAIRWISE, F_XOR = range(12)
+    F_OMPI_LINEAR, F_OMPI_PAIRWISE, F_XOR, F_TUNA2 = range(13)
 MAX_LAUNCHES = 64
 
 
@@ -113,3 +113,7 @@ def exclisive_or_alltoallv(prob, send, recv):
 
 def spreadout_alltoallv(prob, send, recv):
     return _run(F_SPREADOUT, prob, send, recv)
+
+
+def tuna2_algorithm(r, b, prob, send, recv):
+    return _run(F_TUNA2, prob, send, recv, r=r, batch=b)

@@ -103,6 +103,9 @@ def cases() -> list[dict]:
         add(f"ml-P{P}-tuna-r{r}", "tuna", ml, 1, r=r, b=0)
     add("ml-P64-ttpl-n8", "ttpl", dict(kind="ml", P=64, divide=16384), 1, r=4, n=8)
     add("ml-P128-ttpl_s1-n32", "ttpl_s1", dict(kind="ml", P=128, divide=16384), 1, r=32, n=32)
+    # TuNA2 with b = 1 (the reference reuses its send buffer under in-flight sends for b > 1, src/tuna2.cpp:175-185)
+    for P, r in ((8, 2), (12, 3), (27, 3), (32, 4), (64, 8)):
+        add(f"tuna2-P{P}-r{r}", "tuna2", dict(kind="uniform_random", P=P, hi=40, seed=P + 9, sparsify=4), 2, r=r, b=1, layout=1)
     # linear comparators
     for P in (8, 12, 32):
         cg = dict(kind="uniform_random", P=P, hi=30, seed=P + 5, sparsify=4)

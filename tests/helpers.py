@@ -60,6 +60,8 @@ def run_on(backend, case: dict, prob: W.Problem, send, recv) -> int:
         return backend.twophase_rbruck_alltoallv_om(case["r"], prob, send, recv)
     if f == "tuna":
         return backend.tuna_algorithm(case["r"], case["b"], prob, send, recv)
+    if f == "tuna2":
+        return backend.tuna2_algorithm(case["r"], case["b"], prob, send, recv)
     if f == "ttpl":
         return backend.TTPL_BT_alltoallv(case["n"], case["r"], case["bblock"], prob, send, recv)
     if f == "ttpl_s1":

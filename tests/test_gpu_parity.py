@@ -66,7 +66,8 @@ def test_flat_variants_odd_sizes(api, P):
                 for name, fn in (("twophase", lambda d: api.twophase_rbruck_alltoallv(r, dp, dsend, d)),
                                  ("om", lambda d: api.twophase_rbruck_alltoallv_om(r, dp, dsend, d)),
                                  ("tuna2", lambda d: api.tuna_algorithm(r, 2, dp, dsend, d)),
-                                 ("tunaP", lambda d: api.tuna_algorithm(r, 0, dp, dsend, d))):
+                                 ("tunaP", lambda d: api.tuna_algorithm(r, 0, dp, dsend, d)),
+                                 ("tuna2", lambda d: api.tuna2_algorithm(r, 3, dp, dsend, d))):
                     drecv = dp.new_recv_arena(0xEE)
                     rc = fn(drecv)
                     if name.startswith("tuna") and P < 3:
@@ -339,3 +340,19 @@ def test_reference_input_matrices(api):
         _device_check(api, W.make_problem(counts, 1, 0, 0), 5, lambda dp, ds: [
             (f"ML{P} twophase r=32", lambda d: api.twophase_rbruck_alltoallv(32, dp, ds, d), False),
             (f"ML{P} tuna r=8", lambda d: api.tuna_algorithm(8, 0, dp, ds, d), False)])
+
+
+def test_suggest_radix_matches_the_traffic_model(api):
+    for P, n in ((64, 0), (100, 0), (256, 0), (128, 32), (64, 8)):
+        counts = W.counts_zipf(P, 4096, 1.2, 5, P)
+        prob = W.make_problem(counts, 4, 0, 0)
+        dp = api.DeviceProblem(prob)
+        cands = [2, 3, 4, 8, 16, 32, P]
+        best, moved = api.suggest_radix(dp, cands, n)
+        for r, m in zip(cands, moved):
+            hops = W.hops_twolayer(P, n, r) if n else W.hops_flat(P, r)
+            assert 2 * m == W.algorithmic_bytes(counts, 4, hops), (P, n, r)
+        assert best in cands
+        # the model prefers fewer bytes when launch counts are equal
+        assert moved[cands.index(best)] <= moved[0]
+        dp.comm.free()

@@ -234,3 +234,40 @@ def test_linear_comparators_equal_textbook_alltoallv(P):
             assert int(rec["bytes"].sum()) == prob.payload_bytes
             pairs = set(zip(direct["src"].tolist(), direct["dst"].tolist()))
             assert len(pairs) == len(direct)
+
+
+@pytest.mark.parametrize("P", [3, 4, 5, 8, 12, 17, 27, 32, 50])
+def test_tuna2_equals_definition_and_walks_tunas_route(P):
+    """src/tuna2.cpp: same rounds as TuNA (same messages between the same ranks), unpack deferred per digit."""
+    for layout in (0, 1):
+        prob = _prob(P, layout, 2, seed=P)
+        send = W.fill_send_arena(prob, W.PAYLOAD_HASH, 5)
+        want = W.expected_recv_arena(prob, send)
+        for r in sorted({2, 3, 4, 5, 8, P, P - 1}):
+            for b in (1, 2, 0):
+                recv = np.full(prob.recv_bytes, 0xEE, dtype=np.uint8)
+                with O.trace() as t2:
+                    assert O.tuna2_algorithm(r, b, prob, send, recv) == 0
+                assert np.array_equal(recv, want), (P, layout, r, b)
+                with O.trace() as t1:
+                    assert O.tuna_algorithm(r, b, prob, send, np.empty_like(recv)) == 0
+                key = ["kind", "digit", "z", "src", "dst"]
+                assert np.array_equal(np.sort(t1.records, order=key), np.sort(t2.records, order=key))
+
+
+def test_compact_staging_index_closed_form():
+    """extra_id(j) = rank of j among the offsets with at least two non-zero digits (tuna2.cpp:63-73 builds that table;
+    tuna.cpp:93-97 evaluates j - r - (dx-1)(r-1) - dz through float logs)."""
+    lib = O.lib()
+    for P in list(range(3, 70)) + [100, 128, 243, 256, 343, 512, 1000, 1024]:
+        for r in sorted({2, 3, 4, 5, 7, 8, 16, 32, P - 1}):
+            if r < 2 or r > P - 1:
+                continue
+            w, _, _, K = W.radix_params(P, r)
+            rank = 0
+            for j in range(1, P):
+                nz = sum(1 for x in range(w) if (j // r ** x) % r)
+                if nz >= 2:
+                    assert lib.ora_compact_slot_float(j, r) == rank, (P, r, j)
+                    rank += 1
+            assert rank == P - K - 1

@@ -43,7 +43,8 @@ def test_flat_plans_all_radices(P):
                                  ("om", lambda d: E.twophase_rbruck_alltoallv_om(r, prob, send, d)),
                                  ("tuna1", lambda d: E.tuna_algorithm(r, 1, prob, send, d)),
                                  ("tuna3", lambda d: E.tuna_algorithm(r, 3, prob, send, d)),
-                                 ("tunaP", lambda d: E.tuna_algorithm(r, 0, prob, send, d))):
+                                 ("tunaP", lambda d: E.tuna_algorithm(r, 0, prob, send, d)),
+                                 ("tuna2", lambda d: E.tuna2_algorithm(r, 2, prob, send, d))):
                     recv = np.full(prob.recv_bytes, 0xEE, dtype=np.uint8)
                     rc = fn(recv)
                     if name.startswith("tuna") and P < 3:
