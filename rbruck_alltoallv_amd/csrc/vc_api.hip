@@ -499,7 +499,7 @@ extern "C" int vc_suggest_radix(const int *sendcounts, int elem_size, int n, con
         if (candidates[k] < 2) return fail_arg("radix must be >= 2", VC_ERR_RADIX);
         cand[k] = std::min(candidates[k], std::max(n, 2));
     }
-    HIP_TRY(c->scratch.reserve(sizeof(int64_t) * (size_t)P * P));
+    HIP_TRY(c->scratch.reserve(sizeof(unsigned long long) * 64 + sizeof(int) * 64));
     unsigned long long *moved_dev = c->scratch.as<unsigned long long>();
     int *cand_dev = reinterpret_cast<int *>(moved_dev + 64);
     HIP_TRY(hipMemsetAsync(moved_dev, 0, sizeof(unsigned long long) * 64, c->stream));
