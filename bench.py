@@ -45,6 +45,10 @@ def workload(name: str, seed: int):
         counts = W.counts_from_npz(os.path.join(ROOT, "tests", "golden", "inputs", f"global_comm_pattern_{P}proc.npz"))
         r = min(32, P)
         return counts, 1, "twophase_rbruck_alltoallv", dict(r=r), W.hops_flat(P, r)
+    if name.startswith("U"):
+        # equal blocks of U<bytes> bytes at configuration 4's shape: separates the cost of variable, unaligned blocks
+        counts = np.full((1024, 1024), int(name[1:]), dtype=np.int32)
+        return counts, 1, "TTPL_BT_alltoallv", dict(n=32, r=32, bblock=0), W.hops_twolayer(1024, 32, 32)
     counts, esz, tun = W.config_counts(name, seed)
     P = counts.shape[0]
     if name == "C4":
@@ -250,6 +254,7 @@ def main() -> None:
         "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "u8", "data": "synthetic",
         "config": {"workload": (f"benchmark configuration {args.workload[1:]}" if args.workload[0] == "C" else
+                                f"equal blocks of {args.workload[1:]} bytes" if args.workload[0] == "U" else
                                 f"reference input matrix inputs/{prob.P}proc") + f": {func}, P={prob.P} virtual ranks, "
                                + ", ".join(f"{k}={v}" for k, v in tun.items()) + f", {esz}-byte elements",
                    "payload_bytes": S, "algorithmic_bytes": A, "launches_per_step": int(st.n_launches),

@@ -51,9 +51,10 @@ __global__ __launch_bounds__(VC_THREADS) void vc_copy_items_kernel(const VcDesc 
     const bool has0 = t < nvec, has1 = t + VC_THREADS < nvec;
     if (has0) v0 = vc_load16(s2 + ((int64_t)t << 4));
     if (has1) v1 = vc_load16(s2 + ((int64_t)(t + VC_THREADS) << 4));
-    if (t < head) dst[t] = src[t];
+    // the < 16 head bytes (lanes 0..15) and the < 16 tail bytes (lanes 16..31) share one byte load and one byte store
     const int64_t done = head + (nvec << 4);
-    if (t < len - done) dst[done + t] = src[done + t];
+    const int64_t edge = t < 16 ? (t < head ? t : -1) : (t < 32 && done + (t - 16) < len ? done + (t - 16) : -1);
+    if (edge >= 0) dst[edge] = src[edge];
     if (has0) vc_store16(d2 + ((int64_t)t << 4), v0);
     if (has1) vc_store16(d2 + ((int64_t)(t + VC_THREADS) << 4), v1);
 }
