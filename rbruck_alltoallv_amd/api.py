@@ -187,7 +187,7 @@ class Plan:
         self.problem = p
         h = C.c_void_p()
         rc = p.comm.lib.vc_plan_create(function.encode(), n, r, batch, p.sendcounts.data_ptr(), p.sdispls.data_ptr(), p.esz,
-                                       p.recvcounts.data_ptr(), p.rdispls.data_ptr(), recv.data_ptr() & 15, p.comm.handle,
+                                       p.recvcounts.data_ptr(), p.rdispls.data_ptr(), recv.data_ptr() & 4095, p.comm.handle,
                                        C.byref(h))
         self.rc = rc
         self.handle = h if rc == 0 else None

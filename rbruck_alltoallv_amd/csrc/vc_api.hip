@@ -316,7 +316,7 @@ static int run_v(VcFunc f, int n, int r, int batch, vc_comm *c, char *sendbuf, i
     std::vector<VcLaunchInfo> L;
     rc = vc_make_schedule(f, c->P, n, r, batch, esz, 0, S, L);
     if (rc) return schedule_error(rc);
-    S.recv_lo = (int)((uintptr_t)recvbuf & 15);
+    S.recv_lo = (int)((uintptr_t)recvbuf & 4095);
     return run_schedule(c, S, L, sendbuf, recvbuf, make_tables(c, sendcounts, sdispls, recvcounts, rdispls));
 }
 
@@ -398,7 +398,7 @@ static int run_uniform(VcFunc f, int n, int r, vc_comm *c, char *sendbuf, int se
     std::vector<VcLaunchInfo> L;
     rc = vc_make_schedule(f, c->P, n, r, 0, esz, sendcount, S, L);
     if (rc) return schedule_error(rc);
-    S.recv_lo = (int)((uintptr_t)recvbuf & 15);
+    S.recv_lo = (int)((uintptr_t)recvbuf & 4095);
     const size_t PP = (size_t)c->P * c->P;
     HIP_TRY(c->uni_counts.reserve(sizeof(int) * PP));
     HIP_TRY(c->uni_displs.reserve(sizeof(int) * PP));
@@ -450,7 +450,7 @@ extern "C" int vc_plan_create(const char *function, int n, int r, int batch, int
     std::vector<VcLaunchInfo> L;
     int rc = vc_make_schedule(f, c->P, n, r, batch, elem_size, 0, S, L);
     if (rc) return schedule_error(rc);
-    S.recv_lo = recvbuf_low_bits & 15;
+    S.recv_lo = recvbuf_low_bits & 4095;
     vc_plan *p = new vc_plan();
     p->comm = c;
     rc = build_plan(c, S, L, make_tables(c, sendcounts, sdispls, recvcounts, rdispls), p->items, p->info);
@@ -462,7 +462,7 @@ extern "C" int vc_plan_create(const char *function, int n, int r, int batch, int
 
 extern "C" int vc_plan_execute(vc_plan_t p, char *sendbuf, char *recvbuf) {
     if (!p || !sendbuf || !recvbuf) return fail_arg("vc_plan_execute: null argument");
-    if ((int)((uintptr_t)recvbuf & 15) != p->info.recv_lo)
+    if ((int)((uintptr_t)recvbuf & 15) != (p->info.recv_lo & 15))
         return fail_arg("vc_plan_execute: recvbuf must have the low address bits the plan was made for");
     return run_items(p->comm, p->info, p->items.as<VcDesc>(), sendbuf, recvbuf, false);
 }

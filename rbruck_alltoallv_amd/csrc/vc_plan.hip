@@ -48,7 +48,7 @@ __global__ __launch_bounds__(VC_THREADS) void vc_plan_rows(VcSched S, const VcLa
         VcEntry e;
         if (vc_entry_block(S, info, to, id, e)) {
             const int64_t len = vc_entry_len(S, T, e);
-            items += vc_chunk_count(len, vc_entry_phase(S, T, e));
+            items += vc_chunk_count(len, vc_entry_phase(S, T, e), vc_entry_cut(S, T, e));
             bytes += len;
         }
     }
@@ -139,7 +139,7 @@ __global__ __launch_bounds__(VC_THREADS) void vc_plan_emit(VcSched S, const VcLa
     // blocks of many pieces are written by the whole workgroup, not by the lane that owns the entry
     __shared__ VcDesc big_whole[VC_THREADS];
     __shared__ int64_t big_at[VC_THREADS], big_cnt[VC_THREADS];
-    __shared__ int big_phase[VC_THREADS];
+    __shared__ int big_phase[VC_THREADS], big_cut[VC_THREADS];
     __shared__ int nbig;
     const int nent = vc_entries_per_rank(S, info);
     for (int base = 0; base < nent; base += VC_THREADS) {
@@ -147,18 +147,18 @@ __global__ __launch_bounds__(VC_THREADS) void vc_plan_emit(VcSched S, const VcLa
         VcEntry e;
         const bool active = id < nent && vc_entry_block(S, info, to, id, e);
         const int64_t len = active ? vc_entry_len(S, T, e) : 0;
-        const int phase = active ? vc_entry_phase(S, T, e) : 0;
-        const int64_t cnt = vc_chunk_count(len, phase);
+        const int phase = active ? vc_entry_phase(S, T, e) : 0, cut = active ? vc_entry_cut(S, T, e) : 0;
+        const int64_t cnt = vc_chunk_count(len, phase, cut);
         int64_t total;
         if (threadIdx.x == 0) nbig = 0;
         const int64_t at = carry + vc_block_exclusive_scan(cnt, lds, total);    // (barriers inside order the reset of nbig)
         if (cnt) {
             const VcDesc whole = vc_entry_desc(S, T, slot_off, row_base, e, to);
             if (cnt <= 4) {
-                for (int64_t c = 0; c < cnt; c++) items[at + c] = vc_chunk_of(whole, c, phase);
+                for (int64_t c = 0; c < cnt; c++) items[at + c] = vc_chunk_of(whole, c, phase, cut);
             } else {
                 const int k = atomicAdd(&nbig, 1);
-                big_whole[k] = whole; big_at[k] = at; big_cnt[k] = cnt; big_phase[k] = phase;
+                big_whole[k] = whole; big_at[k] = at; big_cnt[k] = cnt; big_phase[k] = phase; big_cut[k] = cut;
             }
         }
         __syncthreads();
@@ -166,8 +166,8 @@ __global__ __launch_bounds__(VC_THREADS) void vc_plan_emit(VcSched S, const VcLa
         for (int k = 0; k < nb; k++) {
             const VcDesc whole = big_whole[k];
             const int64_t at_k = big_at[k], cnt_k = big_cnt[k];
-            const int phase_k = big_phase[k];
-            for (int64_t c = threadIdx.x; c < cnt_k; c += VC_THREADS) items[at_k + c] = vc_chunk_of(whole, c, phase_k);
+            const int phase_k = big_phase[k], cut_k = big_cut[k];
+            for (int64_t c = threadIdx.x; c < cnt_k; c += VC_THREADS) items[at_k + c] = vc_chunk_of(whole, c, phase_k, cut_k);
         }
         carry += total;
         __syncthreads();                                  // everybody has read nbig and the list before they are reused

@@ -233,19 +233,28 @@ VC_HD VcDesc vc_entry_desc(const VcSched &S, const VcTables &T, const int64_t *s
 // the phase of the block's final address, so this holds whichever arena the copy writes to.
 VC_HD int vc_entry_phase(const VcSched &S, const VcTables &T, const VcEntry &e) { return vc_phase16(S, T, e.s, e.t); }
 
-// A copy that fits one work item (VC_CHUNK bytes from the 16-byte boundary below its destination) stays whole; a
-// longer one is cut into pieces of VC_PIECE bytes, the size at which a plain copy runs fastest on this chip
-// (one vector per lane).
-VC_HD int64_t vc_chunk_count(int64_t len, int phase) {
-    if (len <= 0) return 0;
-    return len + phase <= VC_CHUNK ? 1 : (len + phase + VC_PIECE - 1) / VC_PIECE;
+// Where a long copy is cut: pieces end where the destination address is a multiple of VC_PIECE when the destination
+// is recvbuf (whole 4 KiB-aligned pieces, no cache line shared between two workgroups), and at multiples of VC_PIECE
+// from the 16-byte boundary below the start otherwise (staging addresses are not known when pieces are counted).
+// Always congruent to the 16-byte phase.
+VC_HD int vc_entry_cut(const VcSched &S, const VcTables &T, const VcEntry &e) {
+    if (e.xdst < 0) return (int)((vc_recv_offset(S, T, e.s, e.t) + S.recv_lo) & (VC_PIECE - 1));
+    return vc_phase16(S, T, e.s, e.t);
 }
 
-VC_HD VcDesc vc_chunk_of(const VcDesc &whole, int64_t c, int phase) {
+// A copy that fits one work item (VC_CHUNK bytes from the 16-byte boundary below its destination) stays whole; a
+// longer one is cut into pieces of at most VC_PIECE bytes, the size at which a plain copy runs fastest on this chip
+// (one vector per lane).  Only the first piece has a byte-wise head and only the last one a tail.
+VC_HD int64_t vc_chunk_count(int64_t len, int phase, int cut) {
+    if (len <= 0) return 0;
+    return len + phase <= VC_CHUNK ? 1 : (len + cut + VC_PIECE - 1) / VC_PIECE;
+}
+
+VC_HD VcDesc vc_chunk_of(const VcDesc &whole, int64_t c, int phase, int cut) {
     if (whole.len + phase <= VC_CHUNK) return whole;
     VcDesc d = whole;
-    const int64_t lo = c == 0 ? 0 : c * VC_PIECE - phase;
-    int64_t hi = (c + 1) * VC_PIECE - phase;
+    const int64_t lo = c == 0 ? 0 : c * VC_PIECE - cut;
+    int64_t hi = (c + 1) * VC_PIECE - cut;
     if (hi > whole.len) hi = whole.len;
     d.src += lo; d.dst += lo; d.len = hi - lo;
     return d;

@@ -103,14 +103,18 @@ extern "C" int plan_emulate(int func, int P, int n, int r, int batch, int esz, i
                 const int phase = vc_entry_phase(S, T, e);
                 const int dst_lo = (int)(whole.dst >> VC_SPACE_SHIFT) == 1 ? recv_lo : 0;
                 if (whole.len > 0 && (int)(((whole.dst & VC_OFFSET_MASK) + dst_lo) & 15) != phase) errors++;
-                const int64_t nchunks = vc_chunk_count(whole.len, phase);
+                const int cut = vc_entry_cut(S, T, e);
+                if ((cut & 15) != phase) errors++;
+                const int64_t nchunks = vc_chunk_count(whole.len, phase, cut);
                 int64_t covered = 0;
                 items += nchunks;
                 for (int64_t c = 0; c < nchunks; c++) {
-                const VcDesc d = vc_chunk_of(whole, c, phase);
+                const VcDesc d = vc_chunk_of(whole, c, phase, cut);
                 if (d.len <= 0 || d.len > VC_CHUNK || d.src - whole.src != covered || d.dst - whole.dst != covered) { errors++; continue; }
                 // only the first piece may start off a 16-byte boundary of the destination
                 if (c > 0 && (((d.dst & VC_OFFSET_MASK) + dst_lo) & 15) != 0) errors++;
+                // ... and, in recvbuf, on a 4 KiB boundary
+                if (c > 0 && (int)(whole.dst >> VC_SPACE_SHIFT) == 1 && (((d.dst & VC_OFFSET_MASK) + dst_lo) & (VC_PIECE - 1)) != 0) errors++;
                 covered += d.len;
                 const int sspace = (int)(d.src >> VC_SPACE_SHIFT), dspace = (int)(d.dst >> VC_SPACE_SHIFT);
                 const int64_t so = d.src & VC_OFFSET_MASK, dof = d.dst & VC_OFFSET_MASK;

@@ -244,7 +244,7 @@ def test_unaligned_recvbuf_pointer_keeps_the_phase_rule():
     prob = W.make_problem(counts, 1, 1, 0)
     send = W.fill_send_arena(prob, 0, 9)
     want = W.expected_recv_arena(prob, send)
-    for recv_lo in (0, 5, 15):
+    for recv_lo in (0, 5, 15, 2048 + 7, 4095):
         for func, kw in ((E.F_TWOPHASE, dict(r=3)), (E.F_TUNA, dict(r=2, batch=1)), (E.F_TTPL, dict(n=4, r=4)),
                          (E.F_TTPL_S1, dict(n=6, r=2, batch=5)), (E.F_SPREADOUT, {})):
             recv = np.full(prob.recv_bytes, 0xEE, dtype=np.uint8)
