@@ -160,6 +160,11 @@ int vc_plan_create(const char *function, int n, int r, int batch, int *sendcount
 
 /* Runs the planned collective; blocking.  One plan (or call) per communicator at a time. */
 int vc_plan_execute(vc_plan_t plan, char *sendbuf, char *recvbuf);
+/* Only enqueues the copy kernels on the communicator's stream and returns: no synchronisation, no allocation, no
+ * host-side bookkeeping — usable while the stream is being captured into a HIP graph.  The staging arena was sized
+ * when the plan was created; a later, larger call on the same communicator may move it, after which graphs captured
+ * before are stale.  The caller orders later work after it (same stream, or an event). */
+int vc_plan_execute_async(vc_plan_t plan, char *sendbuf, char *recvbuf);
 int vc_plan_free(vc_plan_t plan);
 
 /* ---- radix choice.  The reference leaves r to the caller (its drivers sweep a list of bases,

@@ -48,6 +48,7 @@ SYMBOLS = {
     "spreadout_alltoallv": (_I, _V_TAIL),
     "vc_plan_create": (_I, [C.c_char_p, _I, _I, _I, _P, _P, _I, _P, _P, _I, _P, C.POINTER(_P)]),
     "vc_plan_execute": (_I, [_P, _P, _P]),
+    "vc_plan_execute_async": (_I, [_P, _P, _P]),
     "vc_plan_free": (_I, [_P]),
     "vc_suggest_radix": (_I, [_P, _I, _I, _P, _I, C.POINTER(_I), _P, _P]),
     "vc_comm_set_timing": (_I, [_P, _I]),

@@ -40,6 +40,10 @@ class VirtualComm:
         self._keep = [sbase, rbase]
         self._check(self.lib.vc_comm_set_bases(self.handle, sbase.data_ptr(), rbase.data_ptr()))
 
+    def use_current_stream(self) -> None:
+        """Launch on whatever stream torch has current now (e.g. the capture stream of torch.cuda.graph)."""
+        self._check(self.lib.vc_comm_set_stream(self.handle, C.c_void_p(torch.cuda.current_stream(self.device).cuda_stream)))
+
     def set_timing(self, on: bool) -> None:
         self._check(self.lib.vc_comm_set_timing(self.handle, int(on)))
 
@@ -194,6 +198,9 @@ class Plan:
 
     def execute(self, send: torch.Tensor, recv: torch.Tensor) -> int:
         return self.problem.comm.lib.vc_plan_execute(self.handle, send.data_ptr(), recv.data_ptr())
+
+    def execute_async(self, send: torch.Tensor, recv: torch.Tensor) -> int:
+        return self.problem.comm.lib.vc_plan_execute_async(self.handle, send.data_ptr(), recv.data_ptr())
 
     def free(self) -> None:
         if self.handle:

@@ -239,6 +239,14 @@ static int build_plan(vc_comm *c, VcSched S, std::vector<VcLaunchInfo> &L, VcTab
 
 // Steps 4-5: one copy kernel per launch, then the blocking synchronisation.  `planned_now` says whether events 0 and 1
 // (the planner's) belong to this call.
+// Only the launches: no allocation, no synchronisation, no host-side bookkeeping (safe under stream capture).
+static int launch_items(vc_comm *c, const PlanInfo &pi, const VcDesc *items, const char *sendbuf, char *recvbuf) {
+    if (c->stage.cap < (size_t)pi.stage_bytes + 64) return fail_arg("staging arena smaller than the plan needs");
+    for (int k = 0; k < pi.nl; k++)
+        HIP_TRY(vc_launch_copy_items(items + pi.first[k], pi.count[k], sendbuf, recvbuf, c->stage.as<char>(), c->stream));
+    return VC_OK;
+}
+
 static int run_items(vc_comm *c, const PlanInfo &pi, const VcDesc *items, const char *sendbuf, char *recvbuf, bool planned_now) {
     hipStream_t st = c->stream;
     const int nl = pi.nl;
@@ -455,6 +463,8 @@ extern "C" int vc_plan_create(const char *function, int n, int r, int batch, int
     p->comm = c;
     rc = build_plan(c, S, L, make_tables(c, sendcounts, sdispls, recvcounts, rdispls), p->items, p->info);
     if (rc == VC_OK && hipStreamSynchronize(c->stream) != hipSuccess) rc = fail_arg("vc_plan_create: stream error", VC_ERR_HIP);
+    if (rc == VC_OK && c->stage.reserve((size_t)p->info.stage_bytes + 64) != hipSuccess)       // so that executing never allocates
+        rc = fail_arg("vc_plan_create: cannot allocate the staging arena", VC_ERR_HIP);
     if (rc) { p->items.release(); delete p; return rc; }
     *plan_out = p;
     return VC_OK;
@@ -465,6 +475,13 @@ extern "C" int vc_plan_execute(vc_plan_t p, char *sendbuf, char *recvbuf) {
     if ((int)((uintptr_t)recvbuf & 15) != (p->info.recv_lo & 15))
         return fail_arg("vc_plan_execute: recvbuf must have the low address bits the plan was made for");
     return run_items(p->comm, p->info, p->items.as<VcDesc>(), sendbuf, recvbuf, false);
+}
+
+extern "C" int vc_plan_execute_async(vc_plan_t p, char *sendbuf, char *recvbuf) {
+    if (!p || !sendbuf || !recvbuf) return fail_arg("vc_plan_execute_async: null argument");
+    if ((int)((uintptr_t)recvbuf & 15) != (p->info.recv_lo & 15))
+        return fail_arg("vc_plan_execute_async: recvbuf must have the low address bits the plan was made for");
+    return launch_items(p->comm, p->info, p->items.as<VcDesc>(), sendbuf, recvbuf);
 }
 
 extern "C" int vc_plan_free(vc_plan_t p) {

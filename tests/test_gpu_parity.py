@@ -356,3 +356,34 @@ def test_suggest_radix_matches_the_traffic_model(api):
         # the model prefers fewer bytes when launch counts are equal
         assert moved[cands.index(best)] <= moved[0]
         dp.comm.free()
+
+
+def test_plan_in_a_hip_graph(api):
+    """vc_plan_execute_async only enqueues kernels, so a plan can be captured into a graph and replayed; every replay,
+    with other work and synchronisations in between, gives the eager result."""
+    import torch
+    counts = W.counts_uniform_random(64, 4096, seed=0)
+    prob = W.make_problem(counts, 1, 0, 0)
+    send = W.fill_send_arena(prob, 0, 4)
+    want = W.expected_recv_arena(prob, send, fill=0)
+    dp = api.DeviceProblem(prob)
+    ds = _to_dev(api, send)
+    dr = dp.new_recv_arena(0)
+    plan = api.Plan("twophase_rbruck_alltoallv", dp, dr, r=2)
+    assert plan.rc == 0
+    assert plan.execute(ds, dr) == 0 and np.array_equal(dr.cpu().numpy(), want)
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        dp.comm.use_current_stream()
+        assert plan.execute_async(ds, dr) == 0, dp.comm.error()
+    dp.comm.use_current_stream()
+    for rep in range(4):
+        dr.fill_(rep + 1)                                  # eager work between replays
+        torch.cuda.synchronize()
+        g.replay()
+        torch.cuda.synchronize()
+        assert np.array_equal(dr.cpu().numpy(), want), rep
+        ds2 = ds.clone()
+        assert plan.execute(ds2, dr) == 0                 # and eager calls of the library in between
+    plan.free()
+    dp.comm.free()
