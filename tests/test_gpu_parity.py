@@ -378,7 +378,8 @@ def test_plan_in_a_hip_graph(api):
         assert plan.execute_async(ds, dr) == 0, dp.comm.error()
     dp.comm.use_current_stream()
     for rep in range(4):
-        dr.fill_(rep + 1)                                  # eager work between replays
+        dr.fill_(rep + 1)                                  # eager work between replays: the stale result is wiped
+        dr.zero_()                                         # (bytes between the ranks' buffers are not written by the call)
         torch.cuda.synchronize()
         g.replay()
         torch.cuda.synchronize()
