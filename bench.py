@@ -232,6 +232,22 @@ def main() -> None:
         plan_bad = dp.verify(send, recv, packed_recv=(func == "TTPL_BT_alltoallv"))
         plan_info = {"ms_per_call": round(plan_s * 1e3, 4), "GBps_effective": round(S / plan_s / 1e9, 1),
                      "hbm_frac": round(A / plan_s / 1e9 / HBM_PEAK_GBPS, 4), "mismatched_bytes": int(plan_bad)}
+        # ... and its launches captured once into a HIP graph (what a launch-bound inner loop would replay)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            dp.comm.use_current_stream()
+            assert plan.execute_async(send, recv) == 0, dp.comm.error()
+        dp.comm.use_current_stream()
+        graph.replay()
+        torch.cuda.synchronize()
+        g0 = time.perf_counter()
+        for _ in range(args.steps):
+            graph.replay()
+            torch.cuda.synchronize()
+        graph_s = (time.perf_counter() - g0) / args.steps
+        plan_info["graph_replay_ms_per_call"] = round(graph_s * 1e3, 4)
+        plan_info["graph_mismatched_bytes"] = int(dp.verify(send, recv, packed_recv=(func == "TTPL_BT_alltoallv")))
+        del graph
         plan.free()
 
     # The linear comparator the reference drivers time beside the Bruck variants (examples/twophaseLayer_example.cpp:99-113
