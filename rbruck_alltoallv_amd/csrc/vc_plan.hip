@@ -136,11 +136,11 @@ __global__ __launch_bounds__(VC_THREADS) void vc_plan_emit(VcSched S, const VcLa
     for (int k = threadIdx.x; k < L; k += VC_THREADS) first += header[3 + 2 * nl + k];
     first = vc_block_sum(first, lds);
     int64_t carry = first + item_row_base[(int64_t)L * P + to];
-    // blocks of many pieces are written by the whole workgroup, not by the lane that owns the entry
+    // copies of many pieces are written by the whole workgroup: their pieces are numbered by a second prefix sum and
+    // every lane takes every 256th piece, finding the copy it belongs to by bisection
     __shared__ VcDesc big_whole[VC_THREADS];
-    __shared__ int64_t big_at[VC_THREADS], big_cnt[VC_THREADS];
+    __shared__ int64_t big_at[VC_THREADS], big_pre[VC_THREADS];
     __shared__ int big_phase[VC_THREADS], big_cut[VC_THREADS];
-    __shared__ int nbig;
     const int nent = vc_entries_per_rank(S, info);
     for (int base = 0; base < nent; base += VC_THREADS) {
         const int id = base + threadIdx.x;
@@ -150,27 +150,30 @@ __global__ __launch_bounds__(VC_THREADS) void vc_plan_emit(VcSched S, const VcLa
         const int phase = active ? vc_entry_phase(S, T, e) : 0, cut = active ? vc_entry_cut(S, T, e) : 0;
         const int64_t cnt = vc_chunk_count(len, phase, cut);
         int64_t total;
-        if (threadIdx.x == 0) nbig = 0;
-        const int64_t at = carry + vc_block_exclusive_scan(cnt, lds, total);    // (barriers inside order the reset of nbig)
+        const int64_t at = carry + vc_block_exclusive_scan(cnt, lds, total);
+        const bool big = cnt > 4;
         if (cnt) {
             const VcDesc whole = vc_entry_desc(S, T, slot_off, row_base, e, to);
-            if (cnt <= 4) {
+            if (!big)
                 for (int64_t c = 0; c < cnt; c++) items[at + c] = vc_chunk_of(whole, c, phase, cut);
-            } else {
-                const int k = atomicAdd(&nbig, 1);
-                big_whole[k] = whole; big_at[k] = at; big_cnt[k] = cnt; big_phase[k] = phase; big_cut[k] = cut;
-            }
+            else { big_whole[threadIdx.x] = whole; big_at[threadIdx.x] = at; big_phase[threadIdx.x] = phase; big_cut[threadIdx.x] = cut; }
         }
-        __syncthreads();
-        const int nb = nbig;
-        for (int k = 0; k < nb; k++) {
-            const VcDesc whole = big_whole[k];
-            const int64_t at_k = big_at[k], cnt_k = big_cnt[k];
-            const int phase_k = big_phase[k], cut_k = big_cut[k];
-            for (int64_t c = threadIdx.x; c < cnt_k; c += VC_THREADS) items[at_k + c] = vc_chunk_of(whole, c, phase_k, cut_k);
+        if (__syncthreads_or(big)) {
+            int64_t btotal;
+            big_pre[threadIdx.x] = vc_block_exclusive_scan(big ? cnt : 0, lds, btotal);
+            __syncthreads();
+            for (int64_t q = threadIdx.x; q < btotal; q += VC_THREADS) {
+                int lo = 0, hi = VC_THREADS - 1;              // last lane whose pieces start at or before q
+                while (lo < hi) {
+                    const int mid = (lo + hi + 1) >> 1;
+                    if (big_pre[mid] <= q) lo = mid; else hi = mid - 1;
+                }
+                const int64_t c = q - big_pre[lo];
+                items[big_at[lo] + c] = vc_chunk_of(big_whole[lo], c, big_phase[lo], big_cut[lo]);
+            }
+            __syncthreads();                              // the lists are reused by the next round
         }
         carry += total;
-        __syncthreads();                                  // everybody has read nbig and the list before they are reused
     }
 }
 
