@@ -65,7 +65,8 @@ struct vc_comm {
     bool timing = false;
     DevBuf slot_off, row_tot, row_base, org_run_base, item_row_tot, item_row_base, row_bytes, desc, header, launches, stage, rd_packed,
         uni_counts, uni_displs, scratch;
-    int64_t *h_header = nullptr;          // pinned
+    int64_t *h_header = nullptr;          // pinned, coherent: the planner writes its header straight into it
+    int64_t *h_header_dev = nullptr;      // the same memory as the device sees it
     VcLaunchInfo *h_launches = nullptr;   // pinned
     std::vector<hipEvent_t> events;
     vc_stats_t stats;
@@ -85,7 +86,8 @@ extern "C" int vc_comm_create(int nranks, vc_comm_t *comm_out) {
     c->P = nranks;
     memset(&c->stats, 0, sizeof c->stats);
     hipError_t e = hipGetDevice(&c->device);
-    if (e == hipSuccess) e = hipHostMalloc((void **)&c->h_header, sizeof(int64_t) * VC_HEADER_WORDS(VC_MAX_LAUNCHES), hipHostMallocDefault);
+    if (e == hipSuccess) e = hipHostMalloc((void **)&c->h_header, sizeof(int64_t) * VC_HEADER_WORDS(VC_MAX_LAUNCHES), hipHostMallocCoherent);
+    if (e == hipSuccess) e = hipHostGetDevicePointer((void **)&c->h_header_dev, c->h_header, 0);
     if (e == hipSuccess) e = hipHostMalloc((void **)&c->h_launches, sizeof(VcLaunchInfo) * VC_MAX_LAUNCHES, hipHostMallocDefault);
     if (e != hipSuccess) {
         (void)vc_comm_free(c);
@@ -206,8 +208,12 @@ static int build_plan(vc_comm *c, VcSched S, std::vector<VcLaunchInfo> &L, VcTab
     if (c->timing) { int rc = ensure_events(c, (size_t)nl + 4); if (rc) return rc; }
 
     if (c->timing) HIP_TRY(hipEventRecord(c->events[0], st));
-    memcpy(c->h_launches, L.data(), sizeof(VcLaunchInfo) * nl);
-    HIP_TRY(hipMemcpyAsync(c->launches.p, c->h_launches, sizeof(VcLaunchInfo) * nl, hipMemcpyHostToDevice, st));
+    if (nl <= VC_LAUNCH_PACK) {
+        HIP_TRY(vc_launch_store_launches(L.data(), nl, c->launches.as<VcLaunchInfo>(), st));
+    } else {
+        memcpy(c->h_launches, L.data(), sizeof(VcLaunchInfo) * nl);
+        HIP_TRY(hipMemcpyAsync(c->launches.p, c->h_launches, sizeof(VcLaunchInfo) * nl, hipMemcpyHostToDevice, st));
+    }
     if (S.packed_recv) {
         HIP_TRY(c->rd_packed.reserve(sizeof(int) * PP));
         HIP_TRY(vc_launch_row_scan(T.rc, c->rd_packed.as<int>(), nullptr, P, st));
@@ -215,8 +221,7 @@ static int build_plan(vc_comm *c, VcSched S, std::vector<VcLaunchInfo> &L, VcTab
     }
     HIP_TRY(vc_launch_plan_sizes(S, c->launches.as<VcLaunchInfo>(), nl, T, c->slot_off.as<int64_t>(), c->row_tot.as<int64_t>(),
                                  c->row_base.as<int64_t>(), c->org_run_base.as<int64_t>(), c->item_row_tot.as<int64_t>(),
-                                 c->item_row_base.as<int64_t>(), c->row_bytes.as<int64_t>(), c->header.as<int64_t>(), st));
-    HIP_TRY(hipMemcpyAsync(c->h_header, c->header.p, sizeof(int64_t) * VC_HEADER_WORDS(nl), hipMemcpyDeviceToHost, st));
+                                 c->item_row_base.as<int64_t>(), c->row_bytes.as<int64_t>(), c->header.as<int64_t>(), c->h_header_dev, st));
     HIP_TRY(hipStreamSynchronize(st));     // the staging arena and the item list are sized from the plan
 
     const int64_t *h = c->h_header;

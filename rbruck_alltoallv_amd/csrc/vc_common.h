@@ -64,6 +64,9 @@ struct VcLaunchInfo {
     int self;      // also performs every rank's copy to itself
 };
 
+#define VC_LAUNCH_PACK 16
+struct VcLaunchPack { VcLaunchInfo info[VC_LAUNCH_PACK]; };
+
 struct VcTables {
     const int *sc, *sd, *rc, *rd;    // [P][P] row-major, elements
     const int64_t *sbase, *rbase;    // [P] bytes
@@ -93,7 +96,9 @@ hipError_t vc_launch_uniform_tables(int *counts, int *displs, int count, int P, 
 // Passes 1 and 2: staging prefix sums and the number of work items of every launch (sizes only).
 hipError_t vc_launch_plan_sizes(const VcSched &S, const VcLaunchInfo *launches_dev, int nlaunch, VcTables T, int64_t *slot_off,
                                 int64_t *row_tot, int64_t *row_base, int64_t *org_run_base, int64_t *item_row_tot,
-                                int64_t *item_row_base, int64_t *row_bytes, int64_t *header, hipStream_t st);
+                                int64_t *item_row_base, int64_t *row_bytes, int64_t *header, int64_t *header_host, hipStream_t st);
+// Writes the first nl (<= VC_LAUNCH_PACK) launch descriptions to device memory from a kernel argument.
+hipError_t vc_launch_store_launches(const VcLaunchInfo *host, int nl, VcLaunchInfo *out, hipStream_t st);
 // Pass 3: writes the work items (needs the item buffer, sized from the header).
 hipError_t vc_launch_plan_emit(const VcSched &S, const VcLaunchInfo *launches_dev, int nlaunch, VcTables T, const int64_t *slot_off,
                                const int64_t *row_base, const int64_t *item_row_base, const int64_t *header, VcDesc *items,

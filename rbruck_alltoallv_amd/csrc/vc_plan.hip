@@ -91,7 +91,7 @@ __global__ __launch_bounds__(VC_THREADS) void vc_plan_org_rows(VcSched S, VcTabl
 __global__ __launch_bounds__(VC_THREADS) void vc_plan_bases(int P, int w, int nl, const int64_t *__restrict__ row_tot,
                                                             int64_t *__restrict__ row_base, const int64_t *__restrict__ item_row_tot,
                                                             int64_t *__restrict__ item_row_base, const int64_t *__restrict__ row_bytes,
-                                                            int64_t *__restrict__ header) {
+                                                            int64_t *__restrict__ header, int64_t *__restrict__ header_host) {
     __shared__ int64_t lds[VC_WAVES_PER_BLOCK];
     const int L = blockIdx.x;
     int64_t carry = 0, bytes = 0;
@@ -107,7 +107,10 @@ __global__ __launch_bounds__(VC_THREADS) void vc_plan_bases(int P, int w, int nl
         }
         for (int i = threadIdx.x; i < P; i += VC_THREADS) bytes += row_bytes[(int64_t)nl * P + i];
         bytes = vc_block_sum(bytes, lds);
-        if (threadIdx.x == 0) { header[0] = carry; header[1] = bytes; }
+        if (threadIdx.x == 0) {
+            header[0] = carry; header[1] = bytes;
+            if (header_host) { header_host[0] = carry; header_host[1] = bytes; }
+        }
         return;
     }
     for (int b0 = 0; b0 < P; b0 += VC_THREADS) {
@@ -120,7 +123,10 @@ __global__ __launch_bounds__(VC_THREADS) void vc_plan_bases(int P, int w, int nl
         bytes += (i < P) ? row_bytes[(int64_t)L * P + i] : 0;
     }
     bytes = vc_block_sum(bytes, lds);
-    if (threadIdx.x == 0) { header[3 + L] = bytes; header[3 + 2 * nl + L] = carry; }
+    if (threadIdx.x == 0) {
+        header[3 + L] = bytes; header[3 + 2 * nl + L] = carry;
+        if (header_host) { header_host[3 + L] = bytes; header_host[3 + 2 * nl + L] = carry; }      // pinned host memory: no copy back
+    }
 }
 
 // ---- pass 3: the work items ----
@@ -179,13 +185,13 @@ __global__ __launch_bounds__(VC_THREADS) void vc_plan_emit(VcSched S, const VcLa
 
 hipError_t vc_launch_plan_sizes(const VcSched &S, const VcLaunchInfo *launches_dev, int nlaunch, VcTables T, int64_t *slot_off,
                                 int64_t *row_tot, int64_t *row_base, int64_t *org_run_base, int64_t *item_row_tot,
-                                int64_t *item_row_base, int64_t *row_bytes, int64_t *header, hipStream_t st) {
+                                int64_t *item_row_base, int64_t *row_bytes, int64_t *header, int64_t *header_host, hipStream_t st) {
     hipLaunchKernelGGL(vc_plan_rows, dim3(S.P, S.w + nlaunch), dim3(VC_THREADS), 0, st, S, launches_dev, nlaunch, T, slot_off, row_tot,
                        item_row_tot, row_bytes);
     if (S.coalesce)
         hipLaunchKernelGGL(vc_plan_org_rows, dim3(S.P), dim3(VC_THREADS), 0, st, S, T, slot_off, row_tot, org_run_base);
     hipLaunchKernelGGL(vc_plan_bases, dim3(nlaunch + 1), dim3(VC_THREADS), 0, st, S.P, S.w + S.coalesce, nlaunch, row_tot, row_base, item_row_tot,
-                       item_row_base, row_bytes, header);
+                       item_row_base, row_bytes, header, header_host);
     return hipGetLastError();
 }
 
@@ -194,6 +200,18 @@ hipError_t vc_launch_plan_emit(const VcSched &S, const VcLaunchInfo *launches_de
                                hipStream_t st) {
     hipLaunchKernelGGL(vc_plan_emit, dim3(S.P, nlaunch), dim3(VC_THREADS), 0, st, S, launches_dev, T, slot_off, row_base, item_row_base,
                        header, nlaunch, items);
+    return hipGetLastError();
+}
+
+// ---- the launch table travels as a kernel argument when it is short (no host-to-device copy) ----
+__global__ void vc_store_launches_kernel(VcLaunchPack pack, int nl, VcLaunchInfo *__restrict__ out) {
+    if ((int)threadIdx.x < nl) out[threadIdx.x] = pack.info[threadIdx.x];
+}
+
+hipError_t vc_launch_store_launches(const VcLaunchInfo *host, int nl, VcLaunchInfo *out, hipStream_t st) {
+    VcLaunchPack pack;
+    for (int k = 0; k < nl; k++) pack.info[k] = host[k];
+    hipLaunchKernelGGL(vc_store_launches_kernel, dim3(1), dim3(VC_LAUNCH_PACK), 0, st, pack, nl, out);
     return hipGetLastError();
 }
 
