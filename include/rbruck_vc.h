@@ -139,6 +139,17 @@ int ompi_alltoallv_intra_pairwise(char *sendbuf, int *sendcounts, int *sdispls, 
 int exclisive_or_alltoallv(char *sendbuf, int *sendcounts, int *sdispls, int sendtype_size, char *recvbuf,
                            int *recvcounts, int *rdispls, int recvtype_size, vc_comm_t comm);
 
+/* src/twolayer_communicator_linear.cpp:13-88 — node-local messages (MPICH_intra_scattered on the node's ranks), then
+ * every message between nodes; returns -2 where the reference aborts (n >= P) or misbehaves (n does not divide P). */
+int twolayer_communicator_linear(int n, char *sendbuf, int *sendcounts, int *sdispls, int sendtype_size, char *recvbuf,
+                                 int *recvcounts, int *rdispls, int recvtype_size, vc_comm_t comm);
+
+/* src/twolayer_communicator_linear.cpp:92-192 — the same with bblock1 node-local and bblock2 inter-node messages in
+ * flight.  (twolayer_communicator_linear_s3, :196-318, never delivers a rank's block to itself and is not provided.) */
+int twolayer_communicator_linear_s2(int n, int bblock1, int bblock2, char *sendbuf, int *sendcounts, int *sdispls,
+                                    int sendtype_size, char *recvbuf, int *recvcounts, int *rdispls, int recvtype_size,
+                                    vc_comm_t comm);
+
 /* benchmarks/common.cpp:10-37 (declared in src/rbruckv.h:88-89; returns void there). */
 int spreadout_alltoallv(char *sendbuf, int *sendcounts, int *sdispls, int sendtype_size, char *recvbuf,
                         int *recvcounts, int *rdispls, int recvtype_size, vc_comm_t comm);

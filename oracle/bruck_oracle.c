@@ -898,6 +898,57 @@ int ora_exclisive_or_alltoallv(char *sendarena, const int64_t *sbase, const int 
     return 0;
 }
 
+/* src/twolayer_communicator_linear.cpp:13-88 and :92-192: MPICH_intra_scattered on the ranks of the own node (bblock1
+ * at a time, 0 = all), then the messages between nodes: all posted before one Waitall (plain), or bblock2 at a time
+ * over ii = 1 .. P-1 with gi = ii / n the group distance and gr = ii % n the source's local index on the receiving
+ * side (_s2; the sender posts the same message in batch gi * n + destination's local index, so on a real network it
+ * completes in the later of the two). */
+static int twolayer_linear(int n, int bblock1, int bblock2, int batched_inter, ora_ctx *c) {
+    int P = c->P;
+    if (n < 1 || n >= P || P % n != 0) return -2;                        /* :24-28 aborts (and misses n that does not divide P) */
+    int ngroup = P / n;
+    if (bblock1 <= 0 || bblock1 > n) bblock1 = n;                        /* MPICH_scattered.cpp:31 on the node communicator */
+    for (int ii = 0; ii < n; ii += bblock1) {
+        int ss = n - ii < bblock1 ? n - ii : bblock1;
+        for (int p = 0; p < P; p++)
+            for (int i = 0; i < ss; i++) {
+                int dst = p / n * n + (p % n - i - ii + 2 * n) % n;
+                if (SC(c, p, dst)) direct_message(c, p, dst, i + ii);
+            }
+    }
+    if (!batched_inter) {
+        for (int p = 0; p < P; p++)
+            for (int i = 1; i < ngroup; i++)                              /* :55-83 */
+                for (int j = 0; j < n; j++) direct_message(c, p, ((p / n + i) % ngroup) * n + j, i);
+        return 0;
+    }
+    if (bblock2 <= 0 || bblock2 > P) bblock2 = P;                        /* :132-133 */
+    for (int ii = 1; ii < P; ii += bblock2) {
+        int ss = P - ii < bblock2 ? P - ii : bblock2;
+        for (int p = 0; p < P; p++)
+            for (int i = 0; i < ss; i++) {
+                int gi = (ii + i) / n, gr = (ii + i) % n;
+                int nsrc = (p / n - gi + ngroup) % ngroup;                /* :152; a message is attributed to the batch */
+                if (nsrc == p / n) continue;                              /* in which its receive is posted            */
+                direct_message(c, nsrc * n + gr, p, ii + i);
+            }
+    }
+    return 0;
+}
+
+int ora_twolayer_communicator_linear(int n, char *sendarena, const int64_t *sbase, const int *sendcounts, const int *sdispls,
+                                     int esz, char *recvarena, const int64_t *rbase, const int *recvcounts, const int *rdispls, int P) {
+    ora_ctx c = make_ctx(sendarena, sbase, sendcounts, sdispls, esz, recvarena, rbase, recvcounts, rdispls, P);
+    return twolayer_linear(n, 0, 0, 0, &c);
+}
+
+int ora_twolayer_communicator_linear_s2(int n, int bblock1, int bblock2, char *sendarena, const int64_t *sbase, const int *sendcounts,
+                                        const int *sdispls, int esz, char *recvarena, const int64_t *rbase, const int *recvcounts,
+                                        const int *rdispls, int P) {
+    ora_ctx c = make_ctx(sendarena, sbase, sendcounts, sdispls, esz, recvarena, rbase, recvcounts, rdispls, P);
+    return twolayer_linear(n, bblock1, bblock2, 1, &c);
+}
+
 /* ------------------------------------------------------- payload + digests */
 
 void ora_fill_payload(int mode, uint64_t seed, char *sendarena, const int64_t *sbase, const int *sendcounts,

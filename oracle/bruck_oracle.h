@@ -113,6 +113,12 @@ int ora_ompi_alltoallv_intra_pairwise(char *sendarena, const int64_t *sbase, con
 int ora_exclisive_or_alltoallv(char *sendarena, const int64_t *sbase, const int *sendcounts, const int *sdispls, int esz,
                                char *recvarena, const int64_t *rbase, const int *recvcounts, const int *rdispls, int P);  /* src/exclusive_or_alltoallv.cpp:12-51 */
 
+int ora_twolayer_communicator_linear(int n, char *sendarena, const int64_t *sbase, const int *sendcounts, const int *sdispls,
+                                     int esz, char *recvarena, const int64_t *rbase, const int *recvcounts, const int *rdispls, int P); /* src/twolayer_communicator_linear.cpp:13-88 */
+int ora_twolayer_communicator_linear_s2(int n, int bblock1, int bblock2, char *sendarena, const int64_t *sbase, const int *sendcounts,
+                                        const int *sdispls, int esz, char *recvarena, const int64_t *rbase, const int *recvcounts,
+                                        const int *rdispls, int P);                                                              /* :92-192 */
+
 /* Synthetic payload (oracle/vc_synth.h) written into every rank's send blocks. */
 void ora_fill_payload(int mode, uint64_t seed, char *sendarena, const int64_t *sbase, const int *sendcounts,
                       const int *sdispls, int esz, int P);

@@ -108,6 +108,14 @@ def spreadout_alltoallv(prob, send, recv):
     return lib().ora_spreadout_alltoallv(*_v_args(prob, send, recv))
 
 
+def twolayer_communicator_linear(n, prob, send, recv):
+    return lib().ora_twolayer_communicator_linear(C.c_int(n), *_v_args(prob, send, recv))
+
+
+def twolayer_communicator_linear_s2(n, bblock1, bblock2, prob, send, recv):
+    return lib().ora_twolayer_communicator_linear_s2(C.c_int(n), C.c_int(bblock1), C.c_int(bblock2), *_v_args(prob, send, recv))
+
+
 def fill_payload(mode, seed, prob, send):
     lib().ora_fill_payload(C.c_int(mode), C.c_uint64(seed), _p(send), _p(prob.sbase), _p(prob.sendcounts),
                            _p(prob.sdispls), C.c_int(prob.esz), C.c_int(prob.P))

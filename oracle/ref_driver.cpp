@@ -13,7 +13,8 @@
  *
  * usage: mpiexec -n P ref_driver FUNC COUNTS ESZ R B N BBLOCK LAYOUT PAYLOAD SEED ITERS OUT
  *   FUNC    twophase | om | tuna | tuna2 | ttpl | ttpl_s1 | uniform_spreadout | uniform_isplit |
- *           scattered | ompi_linear | ompi_pairwise | xor | spreadout | mpi_alltoallv
+ *           scattered | ompi_linear | ompi_pairwise | xor | spreadout | tl_linear | tl_linear_s2 (B = bblock1,
+ *           BBLOCK = bblock2) | mpi_alltoallv
  *   COUNTS  file of P*P int32 (row = sender); for the uniform functions the decimal block count
  *   LAYOUT  0 packed ascending displacements, 1 reversed order with gaps
  *   OUT     prefix: OUT.digests (one hex FNV-1a per rank), OUT.recv.bin (all recv extents, rank
@@ -122,6 +123,8 @@ int main(int argc, char **argv) {
         else if (func == "ompi_pairwise") ret = ompi_alltoallv_intra_pairwise(sb, sc, sd, dtype, rb, rc, rd, dtype, MPI_COMM_WORLD);
         else if (func == "xor") ret = exclisive_or_alltoallv(sb, sc, sd, dtype, rb, rc, rd, dtype, MPI_COMM_WORLD);
         else if (func == "spreadout") spreadout_alltoallv(sb, sc, sd, dtype, rb, rc, rd, dtype, MPI_COMM_WORLD);
+        else if (func == "tl_linear") ret = twolayer_communicator_linear(n, sb, sc, sd, dtype, rb, rc, rd, dtype, MPI_COMM_WORLD);
+        else if (func == "tl_linear_s2") ret = twolayer_communicator_linear_s2(n, b, bblock, sb, sc, sd, dtype, rb, rc, rd, dtype, MPI_COMM_WORLD);
         else if (func == "mpi_alltoallv") ret = MPI_Alltoallv(sb, sc, sd, dtype, rb, rc, rd, dtype, MPI_COMM_WORLD);
         else { if (rank_ == 0) fprintf(stderr, "unknown FUNC %s\n", func.c_str()); MPI_Abort(MPI_COMM_WORLD, 2); }
         double el = MPI_Wtime() - st, mx = 0;

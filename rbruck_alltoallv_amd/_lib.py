@@ -46,6 +46,8 @@ SYMBOLS = {
     "ompi_alltoallv_intra_pairwise": (_I, _V_TAIL),
     "exclisive_or_alltoallv": (_I, _V_TAIL),
     "spreadout_alltoallv": (_I, _V_TAIL),
+    "twolayer_communicator_linear": (_I, [_I] + _V_TAIL),
+    "twolayer_communicator_linear_s2": (_I, [_I, _I, _I] + _V_TAIL),
     "vc_plan_create": (_I, [C.c_char_p, _I, _I, _I, _P, _P, _I, _P, _P, _I, _P, C.POINTER(_P)]),
     "vc_plan_execute": (_I, [_P, _P, _P]),
     "vc_plan_execute_async": (_I, [_P, _P, _P]),

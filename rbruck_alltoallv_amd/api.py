@@ -216,3 +216,13 @@ def suggest_radix(p: DeviceProblem, candidates: list[int], n: int = 0) -> tuple[
     p.comm._check(p.comm.lib.vc_suggest_radix(p.sendcounts.data_ptr(), p.esz, n, cand, len(candidates), C.byref(best), moved,
                                               p.comm.handle))
     return best.value, list(moved)
+
+
+def twolayer_communicator_linear(n: int, p: DeviceProblem, send: torch.Tensor, recv: torch.Tensor) -> int:
+    """src/twolayer_communicator_linear.cpp:13-88"""
+    return p.comm.lib.twolayer_communicator_linear(n, *_tail(p, send, recv))
+
+
+def twolayer_communicator_linear_s2(n: int, bblock1: int, bblock2: int, p: DeviceProblem, send: torch.Tensor, recv: torch.Tensor) -> int:
+    """src/twolayer_communicator_linear.cpp:92-192"""
+    return p.comm.lib.twolayer_communicator_linear_s2(n, bblock1, bblock2, *_tail(p, send, recv))

@@ -321,13 +321,13 @@ static int schedule_error(int code) {
 
 // The alltoallv-shaped functions.
 static int run_v(VcFunc f, int n, int r, int batch, vc_comm *c, char *sendbuf, int *sendcounts, int *sdispls, int esz,
-                 char *recvbuf, int *recvcounts, int *rdispls) {
+                 char *recvbuf, int *recvcounts, int *rdispls, int batch2 = 0) {
     int rc = check_common(c, sendbuf, recvbuf, esz);
     if (rc) return rc;
     if (!sendcounts || !sdispls || !recvcounts || (f != VC_F_TTPL && !rdispls)) return fail_arg("null table");
     VcSched S;
     std::vector<VcLaunchInfo> L;
-    rc = vc_make_schedule(f, c->P, n, r, batch, esz, 0, S, L);
+    rc = vc_make_schedule(f, c->P, n, r, batch, esz, 0, S, L, batch2);
     if (rc) return schedule_error(rc);
     S.recv_lo = (int)((uintptr_t)recvbuf & 4095);
     return run_schedule(c, S, L, sendbuf, recvbuf, make_tables(c, sendcounts, sdispls, recvcounts, rdispls));
@@ -399,6 +399,21 @@ extern "C" int spreadout_alltoallv(char *sendbuf, int *sendcounts, int *sdispls,
                                    int *recvcounts, int *rdispls, int recvtype_size, vc_comm_t c) {
     (void)recvtype_size;
     return run_v(VC_F_SPREADOUT, 0, 2, 0, c, sendbuf, sendcounts, sdispls, sendtype_size, recvbuf, recvcounts, rdispls);
+}
+
+// src/twolayer_communicator_linear.cpp: node-local messages first, then the messages between nodes; one hop each.
+extern "C" int twolayer_communicator_linear(int n, char *sendbuf, int *sendcounts, int *sdispls, int sendtype_size, char *recvbuf,
+                                            int *recvcounts, int *rdispls, int recvtype_size, vc_comm_t c) {
+    (void)recvtype_size;
+    return run_v(VC_F_TWOLAYER_LINEAR, n, 2, 0, c, sendbuf, sendcounts, sdispls, sendtype_size, recvbuf, recvcounts, rdispls);
+}
+
+extern "C" int twolayer_communicator_linear_s2(int n, int bblock1, int bblock2, char *sendbuf, int *sendcounts, int *sdispls,
+                                               int sendtype_size, char *recvbuf, int *recvcounts, int *rdispls, int recvtype_size,
+                                               vc_comm_t c) {
+    (void)recvtype_size;
+    return run_v(VC_F_TWOLAYER_LINEAR_S2, n, 2, bblock1, c, sendbuf, sendcounts, sdispls, sendtype_size, recvbuf, recvcounts, rdispls,
+                 bblock2);
 }
 
 // The alltoall-shaped (equal blocks) functions: the count tables are implied.

@@ -57,7 +57,7 @@ struct VcSched {
 struct VcLaunchInfo {
     int kind;      // 0: rounds of intra-node digit x with digit value in [zlo, zhi]; 1: inter-node messages, one per block;
                    // 2: direct messages; 3: inter-node messages, coalesced (entries are (source group, part) pairs)
-    int x;         // digit
+    int x;         // digit; for direct launches the scope: 0 all pairs by rank distance, 1 inside a node, 2 between nodes
     int dist;      // r^x
     int zlo, zhi;
     int qlo, qhi;  // inter-node: (group distance)*n + source local index in [qlo, qhi); direct: rank distance in [qlo, qhi)

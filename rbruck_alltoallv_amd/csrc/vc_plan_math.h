@@ -175,7 +175,16 @@ VC_HD bool vc_entry_block(const VcSched &S, const VcLaunchInfo &info, int to, in
     if (info.kind == 2) {
         // direct: `id` is the source rank; launches are batches of the distance (source - destination) mod P
         // (src/MPICH_scattered.cpp:44-45: receive from rank + i + ii)
-        const int q = (id - to + S.P) % S.P;
+        int q;
+        if (info.x == 1) {                                  // inside the node: local rank distance (twolayer_communicator_linear.cpp:45)
+            if (id / n != to / n) return false;
+            q = (id % n - to % n + n) % n;
+        } else if (info.x == 2) {                           // between nodes: (group distance)*n + source local index (:146-153)
+            if (id / n == to / n) return false;
+            q = ((to / n - id / n + S.G) % S.G) * n + id % n;
+        } else {
+            q = (id - to + S.P) % S.P;
+        }
         if (q < info.qlo || q >= info.qhi) return false;
         e.s = id; e.t = to; e.from = id; e.xprev = -1; e.id_from = to; e.xdst = -1; e.id_to = id;
         return true;

@@ -26,7 +26,9 @@ enum VcFunc {
     VC_F_OMPI_LINEAR,        // ompi_alltoallv_intra_basic_linear
     VC_F_OMPI_PAIRWISE,      // ompi_alltoallv_intra_pairwise
     VC_F_XOR,                // exclisive_or_alltoallv
-    VC_F_TUNA2               // tuna2_algorithm: TuNA's rounds with the unpack deferred to the end of each digit
+    VC_F_TUNA2,              // tuna2_algorithm: TuNA's rounds with the unpack deferred to the end of each digit
+    VC_F_TWOLAYER_LINEAR,    // twolayer_communicator_linear
+    VC_F_TWOLAYER_LINEAR_S2  // twolayer_communicator_linear_s2
 };
 
 // Digits of span-1 in base r and the number of unused values of the top digit, in
@@ -82,10 +84,23 @@ inline void vc_add_direct_launches(std::vector<VcLaunchInfo> &out, int P, int qs
     }
 }
 
-// Fills S and L for function f.  `r`, `batch` (b of tuna_algorithm, bblock of the TTPL functions) and `n`
+// Direct messages of the linear two-layer comparators: `scope` 1 = inside the node, batches of the local rank
+// distance; `scope` 2 = between nodes, batches of (group distance)*n + source local index.
+inline void vc_add_scoped_direct_launches(std::vector<VcLaunchInfo> &out, int scope, int qfirst, int qend, int qstep) {
+    if (qstep <= 0 || qstep > qend) qstep = qend;
+    for (int q = qfirst; q < qend; q += qstep) {
+        VcLaunchInfo li;
+        memset(&li, 0, sizeof li);
+        li.kind = 2; li.x = scope; li.qlo = q; li.qhi = std::min(q + qstep, qend);
+        out.push_back(li);
+    }
+}
+
+// Fills S and L for function f.  `r`, `batch` (b of tuna_algorithm, bblock of the TTPL functions; with batch2 the two
+// bblocks of twolayer_communicator_linear_s2) and `n`
 // are the caller's raw values.  Returns VC_OK or the code the entry point must return.
 inline int vc_make_schedule(VcFunc f, int P, int n, int r, int batch, int esz, int uniform_count, VcSched &S,
-                            std::vector<VcLaunchInfo> &L) {
+                            std::vector<VcLaunchInfo> &L, int batch2 = 0) {
     memset(&S, 0, sizeof S);
     L.clear();
     S.P = P; S.esz = esz; S.uniform = uniform_count;
@@ -151,6 +166,16 @@ inline int vc_make_schedule(VcFunc f, int P, int n, int r, int batch, int esz, i
     case VC_F_OMPI_PAIRWISE:                                // src/OpenMPI_pairwise.cpp:32-58: P steps; independent, so one launch
         S.n = P; S.G = 1; S.r = 2; S.msd = 0; S.w = 0;
         vc_add_direct_launches(L, P, P);
+        break;
+    case VC_F_TWOLAYER_LINEAR:                              // src/twolayer_communicator_linear.cpp:13-88
+    case VC_F_TWOLAYER_LINEAR_S2:                           // :92-192; batch = bblock1, batch2 = bblock2
+        if (n < 1 || n >= P || P % n != 0) return VC_ERR_GROUP;           // :24-28 MPI_Abort (and misses n that does not divide P)
+        S.n = n; S.G = P / n; S.r = 2; S.msd = 0; S.w = 0;
+        // intra-node: MPICH_intra_scattered on the node's communicator, all at once (:45) or bblock1 at a time (:118-123)
+        vc_add_scoped_direct_launches(L, 1, 0, n, f == VC_F_TWOLAYER_LINEAR ? n : ((batch <= 0 || batch > n) ? n : batch));
+        // inter-node: one Waitall for everything (:55-83), or bblock2 (group distance, local index) pairs at a time (:140-181)
+        vc_add_scoped_direct_launches(L, 2, f == VC_F_TWOLAYER_LINEAR ? n : 1, P,
+                                      f == VC_F_TWOLAYER_LINEAR ? P : ((batch2 <= 0 || batch2 > P) ? P : batch2));
         break;
     case VC_F_MPICH_SCATTERED:                              // src/MPICH_scattered.cpp:31-70: bblock requests in flight
         S.n = P; S.G = 1; S.r = 2; S.msd = 0; S.w = 0;

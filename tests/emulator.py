@@ -14,7 +14,7 @@ LIB = os.path.join(HERE, "_build", "libplan_emulator.so")
 CSRC = os.path.join(os.path.dirname(HERE), "rbruck_alltoallv_amd", "csrc")
 
 F_TWOPHASE, F_OM, F_TUNA, F_TTPL, F_TTPL_S1, F_UNIFORM_SPREADOUT, F_UNIFORM_ISPLIT, F_SPREADOUT, F_MPICH_SCATTERED, \
-    F_OMPI_LINEAR, F_OMPI_PAIRWISE, F_XOR, F_TUNA2 = range(13)
+    F_OMPI_LINEAR, F_OMPI_PAIRWISE, F_XOR, F_TUNA2, F_TWOLAYER_LINEAR, F_TWOLAYER_LINEAR_S2 = range(15)
 MAX_LAUNCHES = 64
 
 
@@ -41,7 +41,7 @@ class Result:
         self.traffic = traffic[: self.nlaunch] if rc == 0 else None
 
 
-def emulate(func, prob, send, recv, n=0, r=2, batch=0, uniform_count=0, recv_lo=0) -> Result:
+def emulate(func, prob, send, recv, n=0, r=2, batch=0, uniform_count=0, recv_lo=0, batch2=0) -> Result:
     global _lib
     if _lib is None:
         _lib = C.CDLL(build())
@@ -51,7 +51,7 @@ def emulate(func, prob, send, recv, n=0, r=2, batch=0, uniform_count=0, recv_lo=
     rc = _lib.plan_emulate(C.c_int(func), C.c_int(P), C.c_int(n), C.c_int(r), C.c_int(batch), C.c_int(prob.esz),
                            C.c_int(uniform_count), _p(send), C.c_int64(send.size), _p(recv), C.c_int64(recv.size),
                            _p(prob.sbase), _p(prob.rbase), _p(prob.sendcounts), _p(prob.sdispls), _p(prob.recvcounts),
-                           _p(prob.rdispls), C.c_int(recv_lo), _p(stats), _p(traffic), C.c_int(MAX_LAUNCHES))
+                           _p(prob.rdispls), C.c_int(recv_lo), _p(stats), _p(traffic), C.c_int(MAX_LAUNCHES), C.c_int(batch2))
     return Result(rc, stats, traffic)
 
 
@@ -117,3 +117,11 @@ def spreadout_alltoallv(prob, send, recv):
 
 def tuna2_algorithm(r, b, prob, send, recv):
     return _run(F_TUNA2, prob, send, recv, r=r, batch=b)
+
+
+def twolayer_communicator_linear(n, prob, send, recv):
+    return _run(F_TWOLAYER_LINEAR, prob, send, recv, n=n)
+
+
+def twolayer_communicator_linear_s2(n, bblock1, bblock2, prob, send, recv):
+    return _run(F_TWOLAYER_LINEAR_S2, prob, send, recv, n=n, batch=bblock1, batch2=bblock2)

@@ -111,6 +111,11 @@ def cases() -> list[dict]:
         cg = dict(kind="uniform_random", P=P, hi=30, seed=P + 5, sparsify=4)
         for f in ("scattered", "ompi_linear", "ompi_pairwise", "spreadout") + (("xor",) if P & (P - 1) == 0 else ()):
             add(f"cmp-P{P}-{f}", f, cg, 4, bblock=3, layout=1)
+    # linear two-layer comparators
+    for P, n in ((8, 4), (12, 3), (32, 8)):
+        cg = dict(kind="uniform_random", P=P, hi=30, seed=P + 7, sparsify=4)
+        add(f"tl-linear-P{P}-n{n}", "tl_linear", cg, 4, n=n, layout=1)
+        add(f"tl-linear-s2-P{P}-n{n}", "tl_linear_s2", cg, 4, n=n, b=2, bblock=5, layout=1)
     # uniform two-layer functions
     for P, n, r in ((16, 4, 2), (16, 4, 3), (16, 4, 4), (12, 3, 2), (64, 8, 4), (64, 16, 3)):
         add(f"uni-spread-P{P}-n{n}-r{r}", "uniform_spreadout", None, 4, r=r, n=n, count=5)

@@ -78,6 +78,10 @@ def run_on(backend, case: dict, prob: W.Problem, send, recv) -> int:
         return backend.ompi_alltoallv_intra_pairwise(prob, send, recv)
     if f == "xor":
         return backend.exclisive_or_alltoallv(prob, send, recv)
+    if f == "tl_linear":
+        return backend.twolayer_communicator_linear(case["n"], prob, send, recv)
+    if f == "tl_linear_s2":
+        return backend.twolayer_communicator_linear_s2(case["n"], case["b"], case["bblock"], prob, send, recv)
     if f == "spreadout":
         return backend.spreadout_alltoallv(prob, send, recv)
     raise ValueError(f)

@@ -35,10 +35,10 @@ static int count_overlaps(std::vector<Range> &dst, std::vector<Range> &src) {
 extern "C" int plan_emulate(int func, int P, int n, int r, int batch, int esz, int uniform_count, const char *send,
                             int64_t send_bytes, char *recv, int64_t recv_bytes, const int64_t *sbase, const int64_t *rbase,
                             const int *sc, const int *sd, const int *rc, const int *rd, int recv_lo, int64_t *stats_out,
-                            int64_t *traffic_out, int max_launches) {
+                            int64_t *traffic_out, int max_launches, int batch2) {
     VcSched S;
     std::vector<VcLaunchInfo> L;
-    int code = vc_make_schedule((VcFunc)func, P, n, r, batch, esz, uniform_count, S, L);
+    int code = vc_make_schedule((VcFunc)func, P, n, r, batch, esz, uniform_count, S, L, batch2);
     if (code) return code;
     S.recv_lo = recv_lo;
     const int64_t PP = (int64_t)P * P;

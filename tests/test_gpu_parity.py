@@ -225,6 +225,32 @@ def test_linear_comparators(api, P):
         dp.comm.free()
 
 
+@pytest.mark.parametrize("P,n", [(8, 4), (12, 3), (32, 8), (16, 1), (256, 32)])
+def test_linear_twolayer_comparators(api, P, n):
+    """twolayer_communicator_linear / _s2 (src/twolayer_communicator_linear.cpp:13-88, 92-192)."""
+    for layout in (0, 1):
+        counts = W.counts_uniform_random(P, 3000, seed=P + n)
+        counts[counts % 4 == 0] = 0
+        prob = W.make_problem(counts, 2, layout, layout)
+        send = W.fill_send_arena(prob, 0, 3)
+        want = W.expected_recv_arena(prob, send)
+        dp = api.DeviceProblem(prob)
+        ds = _to_dev(api, send)
+        for name, fn, launches in (
+                ("plain", lambda d: api.twolayer_communicator_linear(n, dp, ds, d), 2),
+                ("s2 0 0", lambda d: api.twolayer_communicator_linear_s2(n, 0, 0, dp, ds, d), 2),
+                ("s2 2 5", lambda d: api.twolayer_communicator_linear_s2(n, 2, 5, dp, ds, d), -(-n // min(2, n)) + -(-(P - 1) // 5))):
+            dr = dp.new_recv_arena(0xEE)
+            assert fn(dr) == 0, (name, dp.comm.error())
+            assert np.array_equal(dr.cpu().numpy(), want), (name, P, n, layout)
+            st = dp.comm.last_stats()
+            assert st.moved_bytes == prob.payload_bytes and st.n_launches == launches
+        dr = dp.new_recv_arena(0xEE)
+        assert api.twolayer_communicator_linear(P, dp, ds, dr) == -2
+        assert api.twolayer_communicator_linear_s2(0, 1, 1, dp, ds, dr) == -2
+        dp.comm.free()
+
+
 @pytest.mark.parametrize("shift", [(0, 0), (5, 0), (0, 7), (3, 13)])
 def test_arena_pointers_of_any_alignment(api, shift):
     """sendbuf / recvbuf need not be 16-byte aligned."""

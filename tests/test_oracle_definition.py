@@ -236,6 +236,32 @@ def test_linear_comparators_equal_textbook_alltoallv(P):
             assert len(pairs) == len(direct)
 
 
+@pytest.mark.parametrize("P,n", [(2, 1), (4, 2), (6, 3), (8, 4), (12, 3), (12, 4), (32, 8), (27, 9)])
+def test_linear_twolayer_comparators_equal_textbook_alltoallv(P, n):
+    """src/twolayer_communicator_linear.cpp:13-88, 92-192: every pair once, inside the node before between nodes."""
+    for layout in (0, 1):
+        prob = _prob(P, layout, 2, seed=P + n)
+        send = W.fill_send_arena(prob, W.PAYLOAD_HASH, 3)
+        want = W.expected_recv_arena(prob, send)
+        fns = {"plain": lambda d: O.twolayer_communicator_linear(n, prob, send, d)}
+        for b1, b2 in ((0, 0), (1, 1), (2, 5), (n + 3, P + 3)):
+            fns[f"s2-{b1}-{b2}"] = lambda d, b1=b1, b2=b2: O.twolayer_communicator_linear_s2(n, b1, b2, prob, send, d)
+        for name, fn in fns.items():
+            recv = np.full(prob.recv_bytes, 0xEE, dtype=np.uint8)
+            with O.trace() as t:
+                assert fn(recv) == 0
+            assert np.array_equal(recv, want), (name, P, n, layout)
+            rec = t.records
+            assert np.all(rec["kind"] == 5)
+            assert int(rec["bytes"].sum()) == prob.payload_bytes
+            pairs = list(zip(rec["src"].tolist(), rec["dst"].tolist()))
+            assert len(set(pairs)) == len(pairs)
+            inside = rec["src"] // n == rec["dst"] // n
+            # all messages inside the nodes come before the first one between nodes (:34 before :55 / :147)
+            if inside.any() and (~inside).any():
+                assert np.nonzero(inside)[0].max() < np.nonzero(~inside)[0].min()
+
+
 @pytest.mark.parametrize("P", [3, 4, 5, 8, 12, 17, 27, 32, 50])
 def test_tuna2_equals_definition_and_walks_tunas_route(P):
     """src/tuna2.cpp: same rounds as TuNA (same messages between the same ranks), unpack deferred per digit."""

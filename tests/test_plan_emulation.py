@@ -202,6 +202,55 @@ def test_linear_comparator_plans(P):
                     assert np.all(((src - dst) % P >= 3 * k) & ((src - dst) % P < 3 * k + 3))
 
 
+@pytest.mark.parametrize("P,n", [(4, 2), (8, 4), (12, 3), (12, 4), (32, 8), (16, 1), (27, 9)])
+def test_linear_twolayer_comparator_plans(P, n):
+    """twolayer_communicator_linear / _s2 (src/twolayer_communicator_linear.cpp:13-88, 92-192): launches inside the
+    nodes first, then between them; each launch carries the messages of one of the reference's Waitall batches."""
+    G = P // n
+    node = np.arange(P) // n
+    same = node[:, None] == node[None, :]
+    for layout in (0, 1):
+        counts = W.counts_uniform_random(P, 30, seed=P + n)
+        counts[counts % 4 == 0] = 0
+        prob = W.make_problem(counts, 2, layout, layout)
+        send = W.fill_send_arena(prob, 0, 3)
+        want = W.expected_recv_arena(prob, send)
+        for b1, b2 in ((None, None), (0, 0), (1, 1), (2, 5), (3, P + 4)):
+            recv = np.full(prob.recv_bytes, 0xEE, dtype=np.uint8)
+            if b1 is None:
+                rc = E.twolayer_communicator_linear(n, prob, send, recv)
+                e1, e2 = n, P
+            else:
+                rc = E.twolayer_communicator_linear_s2(n, b1, b2, prob, send, recv)
+                e1 = n if b1 <= 0 or b1 > n else b1
+                e2 = P if b2 <= 0 or b2 > P else b2
+            assert rc == 0 and E.last.errors == 0, (P, n, b1, b2)
+            assert np.array_equal(recv, want), (P, n, layout, b1, b2)
+            assert E.last.moved == prob.payload_bytes and E.last.stage_bytes == 0
+            n_intra = -(-n // e1)
+            first = n if b1 is None else 1
+            n_inter = -(-(P - first) // e2)
+            assert E.last.nlaunch == n_intra + n_inter
+            for k in range(E.last.nlaunch):
+                src, dst = np.nonzero(E.last.traffic[k])
+                if k < n_intra:
+                    assert np.all(same[src, dst])
+                    d = (src % n - dst % n) % n
+                    assert np.all((d >= k * e1) & (d < (k + 1) * e1))
+                else:
+                    assert not np.any(same[src, dst])
+                    q = ((dst // n - src // n) % G) * n + src % n          # ii of the receiver's loop (:150-156)
+                    lo = first + (k - n_intra) * e2
+                    assert np.all((q >= lo) & (q < lo + e2))
+    # group size that is no proper divisor of P
+    recv = np.zeros(prob.recv_bytes, dtype=np.uint8)
+    for bad in (0, P, P + 1, 5 if P % 5 else 7):
+        assert E.twolayer_communicator_linear(bad, prob, send, recv) == -2
+        assert E.twolayer_communicator_linear_s2(bad, 1, 1, prob, send, recv) == -2
+        assert O.twolayer_communicator_linear(bad, prob, send, recv) == -2
+        assert O.twolayer_communicator_linear_s2(bad, 1, 1, prob, send, recv) == -2
+
+
 @pytest.mark.parametrize("P,n,r,bblock", [(8, 4, 4, 0), (12, 4, 2, 2), (27, 9, 3, 0), (64, 16, 16, 3), (64, 32, 32, 0), (16, 2, 2, 0)])
 def test_coalesced_twolayer_route(P, n, r, bblock):
     """TTPL_BT_alltoallv: intra-node launches as in the staggered variant; every inter-node message is the coalesced
