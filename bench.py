@@ -67,6 +67,8 @@ def call(api, func, tun, dp, send, recv):
         return api.TTPL_BT_alltoallv(tun["n"], tun["r"], tun["bblock"], dp, send, recv)
     if func == "TTPL_BT_alltoallv_s1":
         return api.TTPL_BT_alltoallv_s1(tun["n"], tun["r"], tun["bblock"], dp, send, recv)
+    if func == "TTPL_rbruck_alltoallv":
+        return api.TTPL_rbruck_alltoallv(tun["n"], tun["r"], dp, send, recv)
     if func == "tuna_algorithm":
         return api.tuna_algorithm(tun["r"], tun["b"], dp, send, recv)
     if func == "twophase_rbruck_alltoallv":
@@ -172,6 +174,8 @@ def main() -> None:
         tun["r"] = args.radix
         P_ = counts.shape[0]
         hops = W.hops_twolayer(P_, tun["n"], args.radix) if "n" in tun else W.hops_flat(P_, min(args.radix, P_ - 1 if func == "tuna_algorithm" else P_))
+    if func == "TTPL_rbruck_alltoallv":
+        hops = W.hops_twolayer_bruck(counts.shape[0], tun["n"], tun["r"])
     prob = W.make_problem(counts, esz, 0, 0)
     S = prob.payload_bytes
     A = W.algorithmic_bytes(counts, esz, hops)

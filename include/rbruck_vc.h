@@ -109,6 +109,15 @@ int TTPL_BT_alltoallv(int n, int r, int bblock, char *sendbuf, int *sendcounts, 
 int TTPL_BT_alltoallv_s1(int n, int r, int bblock, char *sendbuf, int *sendcounts, int *sdispls, int sendtype_size,
                          char *recvbuf, int *recvcounts, int *rdispls, int recvtype_size, vc_comm_t comm);
 
+/* src/twophase_twolayer_rbruck.cpp:15-235 — two-layer with a radix-r Bruck over the nodes as well: after the
+ * intra-node phase (:88-168) the n blocks a rank holds per destination node travel together down the digits of the
+ * group offset, least significant first, between ranks of equal local index (:179-227).  The reference stops after
+ * exchanging those messages and never unpacks them (only blocks from the own node reach its recvbuf); this entry
+ * point completes the phase: a block whose group offset has further non-zero digits waits in staging, otherwise it
+ * lands in recvbuf at rdispls. */
+int TTPL_rbruck_alltoallv(int n, int r, char *sendbuf, int *sendcounts, int *sdispls, int sendtype_size, char *recvbuf,
+                          int *recvcounts, int *rdispls, int recvtype_size, vc_comm_t comm);
+
 /* src/twolayer_rbruck.cpp:10-134 — equal blocks of sendcount elements; rank p's buffers hold P blocks.
  * The reference scrambles sendbuf (and needs recvbuf[0..P) free of '1' bytes); this one leaves sendbuf intact. */
 int uniform_spreadout_twolayer(int n, int r, char *sendbuf, int sendcount, int sendtype_size, char *recvbuf,

@@ -684,6 +684,97 @@ int ora_TTPL_BT_alltoallv_s1(int n, int r, int bblock, char *sendarena, const in
     return 0;
 }
 
+/* src/twophase_twolayer_rbruck.cpp:15-235: the intra-node phase is the staggered variant's (:88-168: finals of the own
+ * node go to recvbuf, :151-152); then a Bruck over the nodes, least significant digit of the group offset first,
+ * between ranks of equal local index: in round (x, z) a rank sends to the rank z*r^x nodes below (:211) the n blocks
+ * of every group slot whose offset has digit x equal to z (:186-207).  The reference frees its buffers right after
+ * the exchange (:222-231); the unpack below is what its intra-node phase does at :147-161, applied to group offsets:
+ * a block whose offset has no higher non-zero digit is final, every other one waits in a slot. */
+int ora_TTPL_rbruck_alltoallv(int n, int r, char *sendarena, const int64_t *sbase, const int *sendcounts, const int *sdispls,
+                              int esz, char *recvarena, const int64_t *rbase, const int *recvcounts, const int *rdispls, int P) {
+    if (r < 2) return -1;                       /* :20 */
+    ora_ctx c = make_ctx(sendarena, sbase, sendcounts, sdispls, esz, recvarena, rbase, recvcounts, rdispls, P);
+    ttpl_state st;
+    int rc = ttpl_setup(&c, &st, n, r);         /* :26 clamps r to n */
+    if (rc) return rc;
+    int ngroup = st.ngroup;
+    r = st.r < 2 ? 2 : st.r;                    /* n == 1 would leave radix 1 (:26), which has no digits */
+    self_copies(&c);                            /* :86 */
+    ttpl_intra(&c, &st, 1);
+
+    /* slot (jg, jj) of a rank: the block of group offset jg and source local index jj while it travels */
+    char **xbuf = (char **)malloc(sizeof(char *) * (size_t)P);
+    int *xcnt = (int *)calloc((size_t)P * P, sizeof(int));
+    for (int p = 0; p < P; p++) xbuf[p] = (char *)malloc((size_t)(st.stride * P + 1));
+    int *loc = (int *)malloc(sizeof(int) * (size_t)(ngroup > 0 ? ngroup : 1));
+    ora_msg *box = (ora_msg *)calloc((size_t)P, sizeof(ora_msg));
+    int gw = 0;
+    for (int top = ngroup - 1; top; top /= r) gw++;                 /* = ceil(log(ngroup)/log(r)) of :45 */
+    int dist = 1;
+    for (int x = 0; x < gw; x++) {
+        int64_t ndist = (int64_t)dist * r;
+        for (int z = 1; z < r; z++) {
+            int hop = z * dist;
+            if (hop > ngroup - 1) break;                            /* :183 */
+            int nl = digit_offsets(ngroup, dist, r, z, loc);        /* :187-193 */
+            for (int p = 0; p < P; p++) {
+                int grank = p % n, gid = p / n;
+                int64_t tot = 0;
+                for (int pass = 0; pass < 2; pass++) {
+                    if (pass) msg_reserve(&box[p], nl * n, tot);
+                    int64_t off = 0; int k = 0;
+                    for (int i = 0; i < nl; i++)
+                        for (int jj = 0; jj < n; jj++, k++) {
+                            int jg = loc[i], cnt;
+                            const char *from;
+                            if (jg % dist == 0) {                   /* first hop between nodes: where the intra phase left it */
+                                int gt = (gid - jg + ngroup) % ngroup;          /* inter_rotate, :171-174 */
+                                int ci = gt * n + jj;
+                                int key = gt * n + (2 * grank - jj + n) % n;
+                                cnt = st.cur[(int64_t)p * P + key];
+                                from = (jj == grank) ? sbuf(&c, p) + (int64_t)SD(&c, p, ci) * esz       /* :202-205 */
+                                                     : st.extra[p] + (int64_t)ci * st.stride;
+                            } else {
+                                cnt = xcnt[(int64_t)p * P + jg * n + jj];
+                                from = xbuf[p] + (int64_t)(jg * n + jj) * st.stride;
+                            }
+                            if (!pass) { tot += (int64_t)cnt * esz; continue; }
+                            box[p].sizes[k] = cnt;
+                            memcpy(box[p].bytes + off, from, (size_t)((int64_t)cnt * esz));
+                            off += (int64_t)cnt * esz;
+                        }
+                }
+            }
+            for (int p = 0; p < P; p++) {
+                int grank = p % n, gid = p / n;
+                int from_rank = ((gid + hop) % ngroup) * n + grank;  /* :210 */
+                const ora_msg *m = &box[from_rank];
+                trace_msg(6, x, z, from_rank, p, nl * n, m->nbytes);
+                int64_t off = 0; int k = 0;
+                for (int i = 0; i < nl; i++)
+                    for (int jj = 0; jj < n; jj++, k++) {
+                        int jg = loc[i];
+                        int64_t nbytes = (int64_t)m->sizes[k] * esz;
+                        if (jg < ndist) {                            /* no higher digit: this rank is the destination */
+                            int src = ((gid + jg) % ngroup) * n + jj;
+                            memcpy(rbuf(&c, p) + (int64_t)RD(&c, p, src) * esz, m->bytes + off, (size_t)nbytes);
+                        } else {
+                            memcpy(xbuf[p] + (int64_t)(jg * n + jj) * st.stride, m->bytes + off, (size_t)nbytes);
+                            xcnt[(int64_t)p * P + jg * n + jj] = m->sizes[k];
+                        }
+                        off += nbytes;
+                    }
+            }
+            for (int p = 0; p < P; p++) msg_release(&box[p]);
+        }
+        dist *= r;
+    }
+    for (int p = 0; p < P; p++) free(xbuf[p]);
+    free(xbuf); free(xcnt); free(loc); free(box);
+    ttpl_teardown(&c, &st);
+    return 0;
+}
+
 /* ------------------------------------------------ 6/7. two-layer, uniform */
 
 /* In-place local rotation of every group's n blocks: block id swaps with

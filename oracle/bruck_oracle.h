@@ -35,9 +35,10 @@ extern "C" {
  * Isend/Irecv pair, or an inter-node message). */
 typedef struct {
     int32_t kind;    /* 0 staged Bruck round, 1 direct single-block round, 2 inter-node coalesced,
-                        3 inter-node staggered, 4 self copy, 5 direct message of a linear comparator */
-    int32_t digit;   /* x for kind 0/1, -1 otherwise */
-    int32_t z;       /* digit value of the round (kind 0/1), group distance otherwise */
+                        3 inter-node staggered, 4 self copy, 5 direct message of a linear comparator,
+                        6 round of the Bruck over the nodes */
+    int32_t digit;   /* x for kind 0/1/6, -1 otherwise */
+    int32_t z;       /* digit value of the round (kind 0/1/6), group distance otherwise */
     int32_t from, to;
     int32_t nblocks;
     int64_t bytes;
@@ -112,6 +113,13 @@ int ora_ompi_alltoallv_intra_pairwise(char *sendarena, const int64_t *sbase, con
                                       const int *rdispls, int P);                                                  /* src/OpenMPI_pairwise.cpp:14-64 */
 int ora_exclisive_or_alltoallv(char *sendarena, const int64_t *sbase, const int *sendcounts, const int *sdispls, int esz,
                                char *recvarena, const int64_t *rbase, const int *recvcounts, const int *rdispls, int P);  /* src/exclusive_or_alltoallv.cpp:12-51 */
+
+/* src/twophase_twolayer_rbruck.cpp:15-235.  The reference's inter-node Bruck (:179-227) exchanges its messages and
+ * drops them; here the received blocks are kept (per-rank slots indexed by group offset and source local index) and
+ * delivered after the last non-zero digit of their group offset.  Pinned by the reference for the blocks that stay
+ * inside a node, by the definition of alltoallv for the rest. */
+int ora_TTPL_rbruck_alltoallv(int n, int r, char *sendarena, const int64_t *sbase, const int *sendcounts, const int *sdispls,
+                              int esz, char *recvarena, const int64_t *rbase, const int *recvcounts, const int *rdispls, int P);
 
 int ora_twolayer_communicator_linear(int n, char *sendarena, const int64_t *sbase, const int *sendcounts, const int *sdispls,
                                      int esz, char *recvarena, const int64_t *rbase, const int *recvcounts, const int *rdispls, int P); /* src/twolayer_communicator_linear.cpp:13-88 */

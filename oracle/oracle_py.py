@@ -76,6 +76,10 @@ def TTPL_BT_alltoallv_s1(n, r, bblock, prob, send, recv):
     return lib().ora_TTPL_BT_alltoallv_s1(C.c_int(n), C.c_int(r), C.c_int(bblock), *_v_args(prob, send, recv))
 
 
+def TTPL_rbruck_alltoallv(n, r, prob, send, recv):
+    return lib().ora_TTPL_rbruck_alltoallv(C.c_int(n), C.c_int(r), *_v_args(prob, send, recv))
+
+
 def uniform_spreadout_twolayer(n, r, prob, count, send, recv):
     """`send` is used as scratch, as in the reference."""
     return lib().ora_uniform_spreadout_twolayer(C.c_int(n), C.c_int(r), _p(send), _p(prob.sbase), C.c_int(count),

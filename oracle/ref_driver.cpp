@@ -13,7 +13,7 @@
  *
  * usage: mpiexec -n P ref_driver FUNC COUNTS ESZ R B N BBLOCK LAYOUT PAYLOAD SEED ITERS OUT
  *   FUNC    twophase | om | tuna | tuna2 | ttpl | ttpl_s1 | uniform_spreadout | uniform_isplit |
- *           scattered | ompi_linear | ompi_pairwise | xor | spreadout | tl_linear | tl_linear_s2 (B = bblock1,
+ *           scattered | ompi_linear | ompi_pairwise | xor | spreadout | ttpl_rbruck (blocks from the own node only) | tl_linear | tl_linear_s2 (B = bblock1,
  *           BBLOCK = bblock2) | mpi_alltoallv
  *   COUNTS  file of P*P int32 (row = sender); for the uniform functions the decimal block count
  *   LAYOUT  0 packed ascending displacements, 1 reversed order with gaps
@@ -123,6 +123,7 @@ int main(int argc, char **argv) {
         else if (func == "ompi_pairwise") ret = ompi_alltoallv_intra_pairwise(sb, sc, sd, dtype, rb, rc, rd, dtype, MPI_COMM_WORLD);
         else if (func == "xor") ret = exclisive_or_alltoallv(sb, sc, sd, dtype, rb, rc, rd, dtype, MPI_COMM_WORLD);
         else if (func == "spreadout") spreadout_alltoallv(sb, sc, sd, dtype, rb, rc, rd, dtype, MPI_COMM_WORLD);
+        else if (func == "ttpl_rbruck") ret = TTPL_rbruck_alltoallv(n, r, sb, sc, sd, dtype, rb, rc, rd, dtype, MPI_COMM_WORLD);
         else if (func == "tl_linear") ret = twolayer_communicator_linear(n, sb, sc, sd, dtype, rb, rc, rd, dtype, MPI_COMM_WORLD);
         else if (func == "tl_linear_s2") ret = twolayer_communicator_linear_s2(n, b, bblock, sb, sc, sd, dtype, rb, rc, rd, dtype, MPI_COMM_WORLD);
         else if (func == "mpi_alltoallv") ret = MPI_Alltoallv(sb, sc, sd, dtype, rb, rc, rd, dtype, MPI_COMM_WORLD);
@@ -131,6 +132,12 @@ int main(int argc, char **argv) {
         MPI_Allreduce(&el, &mx, 1, MPI_DOUBLE, MPI_MAX, MPI_COMM_WORLD);
         times.push_back(mx);
     }
+
+    /* TTPL_rbruck_alltoallv never unpacks what its inter-node phase exchanges (src/twophase_twolayer_rbruck.cpp:222-231):
+     * only the blocks from the own node reach recvbuf, so only those are compared and digested */
+    if (func == "ttpl_rbruck")
+        for (int i = 0; i < P; i++)
+            if (i / n != rank_ / n) recvcounts[i] = 0;
 
     /* mismatch against MPI_Alltoallv, over the receive blocks only */
     long long bad = 0, badsum = 0;

@@ -39,6 +39,7 @@ SYMBOLS = {
     "tuna2_algorithm": (_I, [_I, _I] + _V_TAIL),
     "TTPL_BT_alltoallv": (_I, [_I, _I, _I] + _V_TAIL),
     "TTPL_BT_alltoallv_s1": (_I, [_I, _I, _I] + _V_TAIL),
+    "TTPL_rbruck_alltoallv": (_I, [_I, _I] + _V_TAIL),
     "uniform_spreadout_twolayer": (_I, [_I, _I, _P, _I, _I, _P, _I, _I, _P]),
     "uniform_inverse_isplit_r_bruck": (_I, [_I, _I, _I, _P, _I, _I, _P, _I, _I, _P]),
     "MPICH_intra_scattered": (_I, [_I] + _V_TAIL),

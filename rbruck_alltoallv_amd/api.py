@@ -147,6 +147,11 @@ def TTPL_BT_alltoallv_s1(n: int, r: int, bblock: int, p: DeviceProblem, send: to
     return p.comm.lib.TTPL_BT_alltoallv_s1(n, r, bblock, *_tail(p, send, recv))
 
 
+def TTPL_rbruck_alltoallv(n: int, r: int, p: DeviceProblem, send: torch.Tensor, recv: torch.Tensor) -> int:
+    """src/twophase_twolayer_rbruck.cpp:15-235, with the inter-node Bruck completed"""
+    return p.comm.lib.TTPL_rbruck_alltoallv(n, r, *_tail(p, send, recv))
+
+
 def uniform_spreadout_twolayer(n: int, r: int, p: DeviceProblem, count: int, send: torch.Tensor, recv: torch.Tensor) -> int:
     """src/twolayer_rbruck.cpp:10-134"""
     return p.comm.lib.uniform_spreadout_twolayer(n, r, send.data_ptr(), count, p.esz, recv.data_ptr(), count, p.esz, p.comm.handle)

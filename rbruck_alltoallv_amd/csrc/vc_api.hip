@@ -194,7 +194,7 @@ static int build_plan(vc_comm *c, VcSched S, std::vector<VcLaunchInfo> &L, VcTab
     if (nl > VC_MAX_LAUNCHES) return fail_arg("more than VC_MAX_LAUNCHES launches: raise b / bblock");
     hipStream_t st = c->stream;
     const size_t PP = (size_t)P * P;
-    const size_t wmax = (size_t)std::max(S.w, 1) + 1;      // digit regions + the organized region
+    const size_t wmax = (size_t)std::max(vc_regions(S), 1) + 1;      // staging regions
 
     HIP_TRY(c->slot_off.reserve(sizeof(int64_t) * PP * wmax));
     HIP_TRY(c->row_tot.reserve(sizeof(int64_t) * (size_t)P * wmax));
@@ -225,7 +225,7 @@ static int build_plan(vc_comm *c, VcSched S, std::vector<VcLaunchInfo> &L, VcTab
     HIP_TRY(hipStreamSynchronize(st));     // the staging arena and the item list are sized from the plan
 
     const int64_t *h = c->h_header;
-    out.nl = nl; out.n_digits = S.w; out.recv_lo = S.recv_lo;
+    out.nl = nl; out.n_digits = S.w + S.w2; out.recv_lo = S.recv_lo;
     out.stage_bytes = h[0]; out.payload_bytes = h[1];
     out.first.assign(nl, 0); out.count.assign(nl, 0); out.bytes.assign(nl, 0);
     int64_t nitems = 0;
@@ -369,6 +369,12 @@ extern "C" int TTPL_BT_alltoallv_s1(int n, int r, int bblock, char *sendbuf, int
     return run_v(VC_F_TTPL_S1, n, r, bblock, c, sendbuf, sendcounts, sdispls, sendtype_size, recvbuf, recvcounts, rdispls);
 }
 
+extern "C" int TTPL_rbruck_alltoallv(int n, int r, char *sendbuf, int *sendcounts, int *sdispls, int sendtype_size, char *recvbuf,
+                                     int *recvcounts, int *rdispls, int recvtype_size, vc_comm_t c) {
+    (void)recvtype_size;
+    return run_v(VC_F_TTPL_RBRUCK, n, r, 0, c, sendbuf, sendcounts, sdispls, sendtype_size, recvbuf, recvcounts, rdispls);
+}
+
 // The linear comparators (src/MPICH_scattered.cpp, src/OpenMPI_basic_linear.cpp, src/OpenMPI_pairwise.cpp,
 // src/exclusive_or_alltoallv.cpp, benchmarks/common.cpp): one hop per block.
 extern "C" int MPICH_intra_scattered(int bblock, char *sendbuf, int *sendcounts, int *sdispls, int sendtype_size, char *recvbuf,
@@ -458,7 +464,8 @@ struct vc_plan {
 static bool func_by_name(const char *name, VcFunc &f) {
     static const struct { const char *name; VcFunc f; } table[] = {
         {"twophase_rbruck_alltoallv", VC_F_TWOPHASE}, {"twophase_rbruck_alltoallv_om", VC_F_OM}, {"tuna_algorithm", VC_F_TUNA}, {"tuna2_algorithm", VC_F_TUNA2},
-        {"TTPL_BT_alltoallv", VC_F_TTPL}, {"TTPL_BT_alltoallv_s1", VC_F_TTPL_S1}, {"spreadout_alltoallv", VC_F_SPREADOUT},
+        {"TTPL_BT_alltoallv", VC_F_TTPL}, {"TTPL_BT_alltoallv_s1", VC_F_TTPL_S1}, {"TTPL_rbruck_alltoallv", VC_F_TTPL_RBRUCK},
+        {"twolayer_communicator_linear", VC_F_TWOLAYER_LINEAR}, {"spreadout_alltoallv", VC_F_SPREADOUT},
         {"MPICH_intra_scattered", VC_F_MPICH_SCATTERED}, {"ompi_alltoallv_intra_basic_linear", VC_F_OMPI_LINEAR},
         {"ompi_alltoallv_intra_pairwise", VC_F_OMPI_PAIRWISE}, {"exclisive_or_alltoallv", VC_F_XOR}};
     for (const auto &e : table)

@@ -41,6 +41,8 @@ struct VcSched {
     int G;            // nodes = P / n
     int r;            // radix of the intra-node digits (already clamped)
     int w;            // digits of n-1 in base r (0 when n == 1)
+    int w2;           // digits of G-1 in base r when the inter-node phase is a Bruck over the nodes too
+                      // (TTPL_rbruck_alltoallv), else 0.  Its digit x stages in region w + x.
     int msd;          // 1: most significant digit first (twophase_rbruck_alltoallv, uniform intra phase)
     int esz;          // element size in bytes
     int packed_recv;  // 1: receive side is the packed source-ordered layout (TTPL_BT_alltoallv ignores rdispls)
@@ -53,12 +55,22 @@ struct VcSched {
                       //    The organized region is staging region number w.
 };
 
+#if defined(__HIPCC__)
+#define VC_HD __host__ __device__ __forceinline__
+#else
+#define VC_HD inline
+#endif
+
+// Staging regions of a call: one per intra-node digit, one per inter-node digit, the organized region.
+VC_HD int vc_regions(const VcSched &S) { return S.w + S.w2 + S.coalesce; }
+
 // One data-moving kernel launch.
 struct VcLaunchInfo {
     int kind;      // 0: rounds of intra-node digit x with digit value in [zlo, zhi]; 1: inter-node messages, one per block;
-                   // 2: direct messages; 3: inter-node messages, coalesced (entries are (source group, part) pairs)
+                   // 2: direct messages; 3: inter-node messages, coalesced (entries are (source group, part) pairs);
+                   // 4: rounds of inter-node digit x with digit value in [zlo, zhi]
     int x;         // digit; for direct launches the scope: 0 all pairs by rank distance, 1 inside a node, 2 between nodes
-    int dist;      // r^x
+    int dist;      // r^x (ranks inside the node for kind 0, nodes for kind 4)
     int zlo, zhi;
     int qlo, qhi;  // inter-node: (group distance)*n + source local index in [qlo, qhi); direct: rank distance in [qlo, qhi)
     int self;      // also performs every rank's copy to itself

@@ -16,31 +16,30 @@
 #include "vc_plan_math.h"
 
 // ---- pass 1: row-wise prefix sums ----
-// grid (P, w + nl).  Rows y < w: staging sizes of digit y, slot_off[(y*P + to)*P + id] = offset of the
-// slot inside the row.  Rows y >= w: work-item count, moved bytes (and, for the first launch, payload)
-// of launch y - w.
+// grid (P, w + w2 + nl).  Rows y < w + w2: staging sizes of region y, slot_off[(y*P + to)*P + id] = offset of the
+// slot inside the row.  Later rows: work-item count, moved bytes (and, for the first launch, payload)
+// of launch y - w - w2.
 __global__ __launch_bounds__(VC_THREADS) void vc_plan_rows(VcSched S, const VcLaunchInfo *__restrict__ launches, int nl, VcTables T,
                                                            int64_t *__restrict__ slot_off, int64_t *__restrict__ row_tot,
                                                            int64_t *__restrict__ item_row_tot, int64_t *__restrict__ row_bytes) {
     __shared__ int64_t lds[VC_WAVES_PER_BLOCK];
     const int to = blockIdx.x, P = S.P;
-    if ((int)blockIdx.y < S.w) {
-        const int x = blockIdx.y;
-        int dist = 1;
-        for (int k = 0; k < x; k++) dist *= S.r;
+    const int nreg = S.w + S.w2;                          // the organized region is laid out by vc_plan_org_rows
+    if ((int)blockIdx.y < nreg) {
+        const int y = blockIdx.y;
         int64_t carry = 0;
         for (int base = 0; base < P; base += VC_THREADS) {
             const int id = base + threadIdx.x;
             int64_t total;
-            const int64_t v = (id < P) ? vc_stage_slot_size(S, T, x, dist, to, id) : 0;
+            const int64_t v = (id < P) ? vc_region_slot_size(S, T, y, to, id) : 0;
             const int64_t ex = vc_block_exclusive_scan(v, lds, total);
-            if (id < P) slot_off[((int64_t)x * P + to) * P + id] = carry + ex;
+            if (id < P) slot_off[((int64_t)y * P + to) * P + id] = carry + ex;
             carry += total;
         }
-        if (threadIdx.x == 0) row_tot[(int64_t)x * P + to] = carry;
+        if (threadIdx.x == 0) row_tot[(int64_t)y * P + to] = carry;
         return;
     }
-    const int L = blockIdx.y - S.w;
+    const int L = blockIdx.y - nreg;
     const VcLaunchInfo info = launches[L];
     int64_t items = 0, bytes = 0, payload = 0;
     const int nent = vc_entries_per_rank(S, info);
@@ -96,7 +95,7 @@ __global__ __launch_bounds__(VC_THREADS) void vc_plan_bases(int P, int w, int nl
     const int L = blockIdx.x;
     int64_t carry = 0, bytes = 0;
     if (L == nl) {
-        const int64_t nrows = (int64_t)w * P;                 // w counts the organized region when there is one
+        const int64_t nrows = (int64_t)w * P;                 // w = number of staging regions
         for (int64_t b0 = 0; b0 < nrows; b0 += VC_THREADS) {
             const int64_t i = b0 + threadIdx.x;
             int64_t total;
@@ -186,11 +185,11 @@ __global__ __launch_bounds__(VC_THREADS) void vc_plan_emit(VcSched S, const VcLa
 hipError_t vc_launch_plan_sizes(const VcSched &S, const VcLaunchInfo *launches_dev, int nlaunch, VcTables T, int64_t *slot_off,
                                 int64_t *row_tot, int64_t *row_base, int64_t *org_run_base, int64_t *item_row_tot,
                                 int64_t *item_row_base, int64_t *row_bytes, int64_t *header, int64_t *header_host, hipStream_t st) {
-    hipLaunchKernelGGL(vc_plan_rows, dim3(S.P, S.w + nlaunch), dim3(VC_THREADS), 0, st, S, launches_dev, nlaunch, T, slot_off, row_tot,
+    hipLaunchKernelGGL(vc_plan_rows, dim3(S.P, S.w + S.w2 + nlaunch), dim3(VC_THREADS), 0, st, S, launches_dev, nlaunch, T, slot_off, row_tot,
                        item_row_tot, row_bytes);
     if (S.coalesce)
         hipLaunchKernelGGL(vc_plan_org_rows, dim3(S.P), dim3(VC_THREADS), 0, st, S, T, slot_off, row_tot, org_run_base);
-    hipLaunchKernelGGL(vc_plan_bases, dim3(nlaunch + 1), dim3(VC_THREADS), 0, st, S.P, S.w + S.coalesce, nlaunch, row_tot, row_base, item_row_tot,
+    hipLaunchKernelGGL(vc_plan_bases, dim3(nlaunch + 1), dim3(VC_THREADS), 0, st, S.P, vc_regions(S), nlaunch, row_tot, row_base, item_row_tot,
                        item_row_base, row_bytes, header, header_host);
     return hipGetLastError();
 }

@@ -9,12 +9,6 @@
 
 #include "vc_common.h"
 
-#if defined(__HIPCC__)
-#define VC_HD __host__ __device__ __forceinline__
-#else
-#define VC_HD inline
-#endif
-
 struct VcBlock {
     int s, t;        // source and destination rank of the block
     int from;        // rank that holds it before this hop
@@ -71,6 +65,44 @@ VC_HD bool vc_intra_block(const VcSched &S, int x, int dist, int to, int id, VcB
     return true;
 }
 
+// One entry of a launch before addresses are known: which block it moves and between which arenas.
+struct VcEntry {
+    int s, t;          // the block
+    int from;          // rank that holds it before the hop
+    int xprev;         // staging region in which it waits on `from` (-1: still in sendbuf)
+    int id_from;       // its slot there
+    int xdst;          // staging region that receives it (-1: it goes to recvbuf)
+    int id_to;         // its slot on the receiver
+    int nblk;          // 1, or the number of consecutive source blocks of a coalesced inter-node message part
+};
+
+// Inter-node Bruck over the group offset jg = (source node - destination node) mod G, least significant digit
+// first, between ranks of equal local index (src/twophase_twolayer_rbruck.cpp:179-227: send to the rank
+// spoint*n below, group slots (j + gid) % ngroup, n blocks per group slot).  Entry id = jg*n + jj of rank `to`
+// is the block of source local index jj that arrives there in digit x (dist = r^x nodes), if any.
+VC_HD bool vc_inter_block(const VcSched &S, int x, int dist, int to, int id, VcEntry &e, int &z) {
+    const int n = S.n, G = S.G, r = S.r;
+    const int gto = to / n, l = to % n;
+    const int jg = id / n, jj = id % n;
+    z = (jg / dist) % r;
+    if (z == 0) return false;
+    const int low = jg % dist;                        // part of the offset travelled in earlier digits
+    const int gfrom = (gto + z * dist) % G;
+    const int gs = (gfrom + low) % G;
+    const int gt = (gs - jg + G) % G;
+    e.s = gs * n + jj; e.t = gt * n + l; e.from = gfrom * n + l; e.nblk = 1;
+    if (low) {
+        e.xprev = S.w + vc_top_digit(low, r); e.id_from = id;
+    } else {                                          // still where the intra-node phase left it
+        const int j = (jj - l + n) % n;
+        e.xprev = j == 0 ? -1 : vc_top_digit(j, r);
+        e.id_from = gt * n + jj;
+    }
+    e.xdst = jg < (int64_t)dist * r ? -1 : S.w + x;
+    e.id_to = id;
+    return true;
+}
+
 VC_HD int64_t vc_recv_offset(const VcSched &S, const VcTables &T, int s, int t) {
     const int *rd = S.packed_recv ? T.rd_packed : T.rd;
     return T.rbase[t] + (int64_t)rd[(int64_t)t * S.P + s] * S.esz;
@@ -93,8 +125,23 @@ VC_HD int64_t vc_stage_slot_size(const VcSched &S, const VcTables &T, int x, int
     return len ? ((len + vc_phase16(S, T, b.s, b.t) + 15) & ~15ll) : 0;
 }
 
+// The same for staging region y of a call: intra-node digits first, then inter-node digits.
+VC_HD int64_t vc_region_slot_size(const VcSched &S, const VcTables &T, int y, int to, int id) {
+    int dist = 1;
+    if (y < S.w) {
+        for (int k = 0; k < y; k++) dist *= S.r;
+        return vc_stage_slot_size(S, T, y, dist, to, id);
+    }
+    for (int k = S.w; k < y; k++) dist *= S.r;
+    VcEntry e;
+    int z;
+    if (!vc_inter_block(S, y - S.w, dist, to, id, e, z) || e.xdst < 0) return 0;
+    const int64_t len = (int64_t)T.sc[(int64_t)e.s * S.P + e.t] * S.esz;
+    return len ? ((len + vc_phase16(S, T, e.s, e.t) + 15) & ~15ll) : 0;
+}
+
 // Address (inside the staging arena) of the data of block (s, t) while it sits in slot `id`
-// of `holder`, having arrived there in digit x.
+// of `holder` in staging region x.
 VC_HD int64_t vc_stage_addr(const VcSched &S, const VcTables &T, const int64_t *slot_off, const int64_t *row_base,
                             int x, int holder, int id, int s, int t) {
     const int64_t row = (int64_t)x * S.P + holder;
@@ -139,16 +186,6 @@ VC_HD int64_t vc_org_slot_rel(const VcSched &S, const VcTables &T, int to, int i
     return (phase + vc_org_run_prefix(S, T, gs, t, m)) & ~15ll;
 }
 
-// One entry of a launch before addresses are known: which block it moves and between which arenas.
-struct VcEntry {
-    int s, t;          // the block
-    int from;          // rank that holds it before the hop
-    int xprev;         // digit in which it arrived in `from`'s staging area (-1: still in sendbuf)
-    int id_from;       // its slot there
-    int xdst;          // digit phase whose staging region receives it (-1: it goes to recvbuf)
-    int id_to;         // its slot on the receiver
-    int nblk;          // 1, or the number of consecutive source blocks of a coalesced inter-node message part
-};
 
 // Number of entries per receiving rank in a launch of this kind.
 VC_HD int vc_entries_per_rank(const VcSched &S, const VcLaunchInfo &info) { return info.kind == 3 ? 3 * S.G : S.P; }
@@ -193,6 +230,10 @@ VC_HD bool vc_entry_block(const VcSched &S, const VcLaunchInfo &info, int to, in
         // a rank's block to itself (src/twophase_tunable_rbruckv.cpp:63)
         e.s = e.t = e.from = to; e.xprev = -1; e.id_from = id; e.xdst = -1; e.id_to = id;
         return true;
+    }
+    if (info.kind == 4) {
+        int z;
+        return vc_inter_block(S, info.x, info.dist, to, id, e, z) && z >= info.zlo && z <= info.zhi;
     }
     if (info.kind == 0) {
         VcBlock b;

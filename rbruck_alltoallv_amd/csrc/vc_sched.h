@@ -28,7 +28,8 @@ enum VcFunc {
     VC_F_XOR,                // exclisive_or_alltoallv
     VC_F_TUNA2,              // tuna2_algorithm: TuNA's rounds with the unpack deferred to the end of each digit
     VC_F_TWOLAYER_LINEAR,    // twolayer_communicator_linear
-    VC_F_TWOLAYER_LINEAR_S2  // twolayer_communicator_linear_s2
+    VC_F_TWOLAYER_LINEAR_S2, // twolayer_communicator_linear_s2
+    VC_F_TTPL_RBRUCK         // TTPL_rbruck_alltoallv: intra-node Bruck, then a Bruck over the nodes
 };
 
 // Digits of span-1 in base r and the number of unused values of the top digit, in
@@ -58,6 +59,19 @@ inline void vc_add_intra_launches(std::vector<VcLaunchInfo> &out, const VcSched 
             li.kind = 0; li.x = x; li.dist = dist; li.zlo = zlo; li.zhi = std::min(zlo + step - 1, ze - 1);
             out.push_back(li);
         }
+    }
+}
+
+// Inter-node Bruck: one launch per digit of the group offset, least significant first.
+inline void vc_add_inter_bruck_launches(std::vector<VcLaunchInfo> &out, const VcSched &S, int d2) {
+    int dist = 1;
+    for (int x = 0; x < S.w2; x++, dist *= S.r) {
+        const int ze = (x == S.w2 - 1) ? S.r - d2 : S.r;
+        if (ze - 1 < 1) continue;
+        VcLaunchInfo li;
+        memset(&li, 0, sizeof li);
+        li.kind = 4; li.x = x; li.dist = dist; li.zlo = 1; li.zhi = ze - 1;
+        out.push_back(li);
     }
 }
 
@@ -147,6 +161,24 @@ inline int vc_make_schedule(VcFunc f, int P, int n, int r, int batch, int esz, i
             }
         }
         break;
+    case VC_F_TTPL_RBRUCK: {
+        if (r < 2) return VC_ERR_RADIX;                     // src/twophase_twolayer_rbruck.cpp:20
+        if (n < 1 || P % n != 0) return VC_ERR_GROUP;
+        if (r > n) r = n;                                   // :26
+        S.n = n; S.G = P / n; S.r = std::max(r, 2); S.msd = 0;
+        vc_radix_params(n, S.r, S.w, d);                    // :42
+        vc_add_intra_launches(L, S, d, 0);
+        if (L.empty()) {                                    // n == 1: the copies to self need a launch of their own (the
+            VcLaunchInfo li;                                // entries of an inter-node launch are not indexed by source rank)
+            memset(&li, 0, sizeof li);
+            li.kind = 0; li.dist = 1; li.zlo = 1; li.zhi = 0;
+            L.push_back(li);
+        }
+        int d2 = 0;
+        vc_radix_params(S.G, S.r, S.w2, d2);                // :45, the same radix for the digits of the group offset
+        vc_add_inter_bruck_launches(L, S, d2);
+        break;
+    }
     case VC_F_UNIFORM_SPREADOUT:
     case VC_F_UNIFORM_ISPLIT:
         if (f == VC_F_UNIFORM_SPREADOUT && r < 2) return VC_ERR_RADIX;   // src/twolayer_rbruck.cpp:12

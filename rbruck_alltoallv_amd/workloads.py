@@ -260,6 +260,16 @@ def hops_twolayer(P: int, n: int, r: int) -> np.ndarray:
     return h
 
 
+def hops_twolayer_bruck(P: int, n: int, r: int) -> np.ndarray:
+    """Two-layer with a Bruck over the nodes as well: non-zero base-r digits of the local offset plus those of the
+    group offset (r clamped to n, src/twophase_twolayer_rbruck.cpp:26)."""
+    s, t = np.meshgrid(np.arange(P), np.arange(P), indexing="ij")
+    reff = max(min(r, n), 2)
+    h = _nonzero_digits((s % n - t % n) % n, reff) + _nonzero_digits((s // n - t // n) % (P // n), reff)
+    h[s == t] = 1
+    return h
+
+
 def algorithmic_bytes(counts: np.ndarray, esz: int, hops: np.ndarray) -> int:
     """A = 2 * sum hops(s,t) * bytes(s,t): one read and one write per hop."""
     return int(2 * (hops.astype(np.int64) * counts.astype(np.int64)).sum() * esz)

@@ -14,7 +14,7 @@ LIB = os.path.join(HERE, "_build", "libplan_emulator.so")
 CSRC = os.path.join(os.path.dirname(HERE), "rbruck_alltoallv_amd", "csrc")
 
 F_TWOPHASE, F_OM, F_TUNA, F_TTPL, F_TTPL_S1, F_UNIFORM_SPREADOUT, F_UNIFORM_ISPLIT, F_SPREADOUT, F_MPICH_SCATTERED, \
-    F_OMPI_LINEAR, F_OMPI_PAIRWISE, F_XOR, F_TUNA2, F_TWOLAYER_LINEAR, F_TWOLAYER_LINEAR_S2 = range(15)
+    F_OMPI_LINEAR, F_OMPI_PAIRWISE, F_XOR, F_TUNA2, F_TWOLAYER_LINEAR, F_TWOLAYER_LINEAR_S2, F_TTPL_RBRUCK = range(16)
 MAX_LAUNCHES = 64
 
 
@@ -85,6 +85,10 @@ def TTPL_BT_alltoallv(n, r, bblock, prob, send, recv):
 
 def TTPL_BT_alltoallv_s1(n, r, bblock, prob, send, recv):
     return _run(F_TTPL_S1, prob, send, recv, n=n, r=r, batch=bblock)
+
+
+def TTPL_rbruck_alltoallv(n, r, prob, send, recv):
+    return _run(F_TTPL_RBRUCK, prob, send, recv, n=n, r=r)
 
 
 def uniform_spreadout_twolayer(n, r, prob, count, send, recv):

@@ -116,6 +116,10 @@ def cases() -> list[dict]:
         cg = dict(kind="uniform_random", P=P, hi=30, seed=P + 7, sparsify=4)
         add(f"tl-linear-P{P}-n{n}", "tl_linear", cg, 4, n=n, layout=1)
         add(f"tl-linear-s2-P{P}-n{n}", "tl_linear_s2", cg, 4, n=n, b=2, bblock=5, layout=1)
+    # TTPL_rbruck_alltoallv: the reference delivers only the blocks that stay inside a node ("scope": "node")
+    for P, n, r in ((8, 4, 2), (12, 4, 2), (12, 3, 3), (27, 9, 3), (32, 4, 2), (64, 8, 4)):
+        cg = dict(kind="uniform_random", P=P, hi=30, seed=P + 11, sparsify=4)
+        add(f"ttpl-rbruck-P{P}-n{n}-r{r}", "ttpl_rbruck", cg, 2, r=r, n=n, layout=1)
     # uniform two-layer functions
     for P, n, r in ((16, 4, 2), (16, 4, 3), (16, 4, 4), (12, 3, 2), (64, 8, 4), (64, 16, 3)):
         add(f"uni-spread-P{P}-n{n}-r{r}", "uniform_spreadout", None, 4, r=r, n=n, count=5)
@@ -144,6 +148,8 @@ def run_case(case: dict, tmp: str) -> dict:
     rec = dict(case)
     rec["P"] = P
     rec["digests"] = digests
+    if case["func"] == "ttpl_rbruck":
+        rec["scope"] = "node"
     rec["reference_says"] = line
     if case["id"] == "C1-twophase":
         os.replace(outp + ".recv.bin", os.path.join(HERE, "c1_recv.bin"))

@@ -1,6 +1,7 @@
 """Shared by the CPU and GPU tests: rebuild a golden case's inputs and run one function on the oracle."""
 from __future__ import annotations
 
+import dataclasses
 import json
 import os
 
@@ -50,6 +51,16 @@ def problem_for_case(case: dict) -> W.Problem:
     return W.make_problem(counts, case["esz"], case["layout"], recv_layout)
 
 
+def digest_problem(case: dict, prob: W.Problem) -> W.Problem:
+    """The blocks a case's digests cover: all of them, or ("scope": "node") only those whose source is on the
+    receiver's node — what the reference's TTPL_rbruck_alltoallv delivers."""
+    if case.get("scope") != "node":
+        return prob
+    node = np.arange(prob.P) // case["n"]
+    keep = node[:, None] == node[None, :]
+    return dataclasses.replace(prob, recvcounts=np.ascontiguousarray(np.where(keep, prob.recvcounts, 0).astype(np.int32)))
+
+
 def run_on(backend, case: dict, prob: W.Problem, send, recv) -> int:
     """Dispatch one golden case to a backend exposing the reference's function names
     (oracle.oracle_py on numpy arenas, or the GPU package on device arenas)."""
@@ -78,6 +89,8 @@ def run_on(backend, case: dict, prob: W.Problem, send, recv) -> int:
         return backend.ompi_alltoallv_intra_pairwise(prob, send, recv)
     if f == "xor":
         return backend.exclisive_or_alltoallv(prob, send, recv)
+    if f == "ttpl_rbruck":
+        return backend.TTPL_rbruck_alltoallv(case["n"], case["r"], prob, send, recv)
     if f == "tl_linear":
         return backend.twolayer_communicator_linear(case["n"], prob, send, recv)
     if f == "tl_linear_s2":

@@ -60,18 +60,16 @@ extern "C" int plan_emulate(int func, int P, int n, int r, int batch, int esz, i
     }
 
     // passes 1 and 2 of the planner
-    const int w = std::max(S.w, 1) + 1;                   // digit regions + the organized region
+    const int w = std::max(vc_regions(S), 1) + 1;         // staging regions
     std::vector<int64_t> slot_off(PP * w, 0), row_base((int64_t)P * w, 0);
     int64_t stage_bytes = 0;
-    for (int x = 0; x < S.w; x++) {
-        int dist = 1;
-        for (int k = 0; k < x; k++) dist *= S.r;
+    for (int x = 0; x < S.w + S.w2; x++) {
         for (int to = 0; to < P; to++) {
             row_base[(int64_t)x * P + to] = stage_bytes;
             int64_t acc = 0;
             for (int id = 0; id < P; id++) {
                 slot_off[((int64_t)x * P + to) * P + id] = acc;
-                acc += vc_stage_slot_size(S, T, x, dist, to, id);
+                acc += vc_region_slot_size(S, T, x, to, id);
             }
             stage_bytes += acc;
         }

@@ -8,7 +8,7 @@ import pytest
 
 from oracle import oracle_py as O
 from rbruck_alltoallv_amd import workloads as W
-from tests.helpers import load_golden, problem_for_case, run_on
+from tests.helpers import digest_problem, load_golden, problem_for_case, run_on
 
 pytestmark = pytest.mark.gpu
 
@@ -44,7 +44,7 @@ def test_golden_case(api, case):
     assert rc == 0, dp.comm.error()
     got = drecv.cpu().numpy()
     assert np.array_equal(got, want)
-    assert [f"{int(h):016x}" for h in O.digest_recv(prob, got)] == case["digests"]
+    assert [f"{int(h):016x}" for h in O.digest_recv(digest_problem(case, prob), got)] == case["digests"]
     assert np.array_equal(dsend.cpu().numpy(), send), "sendbuf must stay intact"
     assert dp.verify(dsend, drecv, packed_recv=(case["func"] == "ttpl")) == 0
     dp.comm.free()
@@ -248,6 +248,39 @@ def test_linear_twolayer_comparators(api, P, n):
         dr = dp.new_recv_arena(0xEE)
         assert api.twolayer_communicator_linear(P, dp, ds, dr) == -2
         assert api.twolayer_communicator_linear_s2(0, 1, 1, dp, ds, dr) == -2
+        dp.comm.free()
+
+
+@pytest.mark.parametrize("P,n,r", [(8, 4, 2), (12, 3, 3), (64, 4, 2), (64, 16, 4), (16, 1, 2), (8, 8, 2), (256, 16, 4), (243, 9, 3)])
+def test_twolayer_bruck(api, P, n, r):
+    """TTPL_rbruck_alltoallv (src/twophase_twolayer_rbruck.cpp:15-235, inter-node Bruck completed) against the oracle,
+    the definition and the oracle's per-digit traffic."""
+    for layout in (0, 1):
+        counts = W.counts_uniform_random(P, 3000 if P <= 64 else 300, seed=P + n + r)
+        counts[counts % 4 == 0] = 0
+        prob = W.make_problem(counts, 2, layout, layout)
+        send = W.fill_send_arena(prob, 0, 3)
+        want = np.full(prob.recv_bytes, 0xEE, dtype=np.uint8)
+        with O.trace() as t:
+            assert O.TTPL_rbruck_alltoallv(n, r, prob, send, want) == 0
+        assert np.array_equal(want, W.expected_recv_arena(prob, send))
+        dp = api.DeviceProblem(prob)
+        ds = _to_dev(api, send)
+        dr = dp.new_recv_arena(0xEE)
+        assert api.TTPL_rbruck_alltoallv(n, r, dp, ds, dr) == 0, dp.comm.error()
+        assert np.array_equal(dr.cpu().numpy(), want), (P, n, r, layout)
+        assert dp.verify(ds, dr) == 0
+        rec = t.records
+        st = dp.comm.last_stats()
+        assert st.moved_bytes == int(rec["bytes"].sum())
+        inter = list(dict.fromkeys(rec[rec["kind"] == 6]["digit"].tolist()))
+        if inter and P <= 64:
+            m = np.zeros((P, P), dtype=np.int64)
+            sel = rec[(rec["kind"] == 6) & (rec["digit"] == inter[-1])]
+            np.add.at(m, (sel["src"], sel["dst"]), sel["bytes"])
+            assert np.array_equal(dp.comm.last_traffic(st.n_launches - 1), m)
+        assert api.TTPL_rbruck_alltoallv(n, 1, dp, ds, dr) == -1
+        assert api.TTPL_rbruck_alltoallv(P + 1, 2, dp, ds, dr) == -2
         dp.comm.free()
 
 

@@ -262,6 +262,31 @@ def test_linear_twolayer_comparators_equal_textbook_alltoallv(P, n):
                 assert np.nonzero(inside)[0].max() < np.nonzero(~inside)[0].min()
 
 
+@pytest.mark.parametrize("P", [1, 2, 4, 6, 8, 9, 12, 16, 24, 27, 32, 36, 64])
+def test_twolayer_bruck_equals_textbook_alltoallv(P):
+    """TTPL_rbruck_alltoallv with the inter-node Bruck completed (src/twophase_twolayer_rbruck.cpp:15-235): for every
+    divisor n of P and every radix, the definition of alltoallv — the only pin the blocks that change node have,
+    since the reference drops them."""
+    for layout in (0, 1):
+        prob = _prob(P, layout, 2, seed=P + 3)
+        send = W.fill_send_arena(prob, W.PAYLOAD_HASH, 7)
+        keep = send.copy()
+        want = W.expected_recv_arena(prob, send)
+        for n in [d for d in range(1, P + 1) if P % d == 0]:
+            for r in sorted({2, 3, 4, 7, max(n, 2), P + 2}):
+                recv = np.full(prob.recv_bytes, 0xEE, dtype=np.uint8)
+                with O.trace() as t:
+                    assert O.TTPL_rbruck_alltoallv(n, r, prob, send, recv) == 0
+                assert np.array_equal(recv, want), (P, layout, n, r)
+                assert np.array_equal(send, keep)
+                rec = t.records
+                inter = rec[rec["kind"] == 6]
+                assert np.all(inter["src"] % n == inter["dst"] % n)
+                assert np.all(inter["src"] // n != inter["dst"] // n)
+                intra = rec[rec["kind"] == 0]
+                assert np.all(intra["src"] // n == intra["dst"] // n)
+
+
 @pytest.mark.parametrize("P", [3, 4, 5, 8, 12, 17, 27, 32, 50])
 def test_tuna2_equals_definition_and_walks_tunas_route(P):
     """src/tuna2.cpp: same rounds as TuNA (same messages between the same ranks), unpack deferred per digit."""

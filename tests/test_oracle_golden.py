@@ -7,7 +7,7 @@ import pytest
 
 from oracle import oracle_py as O
 from rbruck_alltoallv_amd import workloads as W
-from tests.helpers import GOLDEN_DIR, fnv1a64_blocks, load_golden, problem_for_case, run_on
+from tests.helpers import GOLDEN_DIR, digest_problem, fnv1a64_blocks, load_golden, problem_for_case, run_on
 
 CASES = load_golden()
 
@@ -18,7 +18,7 @@ def test_oracle_matches_reference_digests(case):
     send = W.fill_send_arena(prob, case["payload"], case["seed"])
     recv = np.full(prob.recv_bytes, 0xEE, dtype=np.uint8)
     assert run_on(O, case, prob, send.copy(), recv) == 0
-    got = [f"{int(h):016x}" for h in O.digest_recv(prob, recv)]
+    got = [f"{int(h):016x}" for h in O.digest_recv(digest_problem(case, prob), recv)]
     assert got == case["digests"]
 
 

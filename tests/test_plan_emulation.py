@@ -7,7 +7,7 @@ import pytest
 from oracle import oracle_py as O
 from rbruck_alltoallv_amd import workloads as W
 from tests import emulator as E
-from tests.helpers import load_golden, problem_for_case, run_on
+from tests.helpers import digest_problem, load_golden, problem_for_case, run_on
 
 CASES = load_golden()
 
@@ -20,7 +20,7 @@ def test_plan_reproduces_reference_digests(case):
     keep = send.copy()
     assert run_on(E, case, prob, send, recv) == 0
     assert E.last.errors == 0
-    assert [f"{int(h):016x}" for h in O.digest_recv(prob, recv)] == case["digests"]
+    assert [f"{int(h):016x}" for h in O.digest_recv(digest_problem(case, prob), recv)] == case["digests"]
     assert np.array_equal(recv, W.expected_recv_arena(prob, send))       # gaps between blocks stay untouched
     assert np.array_equal(send, keep)
 
@@ -155,6 +155,70 @@ def test_twolayer_route_equals_the_oracles_trace(P, n, r):
     if P > n:
         assert np.array_equal(res.traffic[len(digits)], _oracle_traffic(rec, P, rec["kind"] == 3))
     assert res.moved * 2 == W.algorithmic_bytes(prob.sendcounts, prob.esz, W.hops_twolayer(P, n, r))
+
+
+def _digits(v, r):
+    out = []
+    while v:
+        out.append(v % r)
+        v //= r
+    return out
+
+
+@pytest.mark.parametrize("P,n,r", [(8, 4, 2), (12, 4, 2), (12, 3, 3), (27, 3, 3), (64, 4, 2), (64, 16, 4), (60, 3, 3), (16, 1, 2),
+                                   (8, 8, 2), (40, 4, 5), (49, 7, 2)])
+def test_twolayer_bruck_route_equals_the_oracles_trace(P, n, r):
+    """TTPL_rbruck_alltoallv: the intra-node launches carry the reference's intra-node rounds
+    (src/twophase_twolayer_rbruck.cpp:88-168); every launch of the inter-node Bruck carries the messages of the
+    rounds of one digit of the group offset (:179-227: same rank pairs; bytes = the blocks of the group slots the
+    reference packs), and a block rides in as many inter-node launches as its group offset has non-zero digits."""
+    counts = W.counts_uniform_random(P, 20, seed=P + n + r)
+    counts[counts % 3 == 0] = 0
+    for layout in (0, 1):
+        prob = W.make_problem(counts, 1, layout, layout)
+        send = W.fill_send_arena(prob, 0, 2)
+        want = W.expected_recv_arena(prob, send)
+        recv = np.full(prob.recv_bytes, 0xEE, dtype=np.uint8)
+        with O.trace() as t:
+            assert O.TTPL_rbruck_alltoallv(n, r, prob, send, recv) == 0
+        assert np.array_equal(recv, want)
+        rec = t.records
+        recv[:] = 0xEE
+        assert E.TTPL_rbruck_alltoallv(n, r, prob, send, recv) == 0
+        res = E.last
+        assert res.errors == 0 and np.array_equal(recv, want)
+        intra = list(dict.fromkeys(rec[rec["kind"] == 0]["digit"].tolist()))
+        inter = list(dict.fromkeys(rec[rec["kind"] == 6]["digit"].tolist()))
+        assert res.nlaunch == max(len(intra), 1) + len(inter)
+        for k, x in enumerate(intra):
+            got = res.traffic[k].copy()
+            if k == 0:
+                got[np.arange(P), np.arange(P)] = 0                              # self copies
+            assert np.array_equal(got, _oracle_traffic(rec, P, (rec["digit"] == x) & (rec["kind"] == 0))), x
+        G, reff = P // n, max(min(r, n), 2)
+        for k, x in enumerate(inter):
+            got = res.traffic[max(len(intra), 1) + k]
+            assert np.array_equal(got, _oracle_traffic(rec, P, (rec["digit"] == x) & (rec["kind"] == 6))), x
+            src, dst = np.nonzero(got)
+            assert np.all(src % n == dst % n)                                    # equal local index (:210-211)
+            hop = (src // n - dst // n) % G
+            assert np.all((hop % reff ** x == 0) & (hop // reff ** x < reff) & (hop > 0))
+        # hops per block: one per non-zero digit of the local offset and of the group offset
+        s_idx, t_idx = np.meshgrid(np.arange(P), np.arange(P), indexing="ij")
+        nnz = np.vectorize(lambda v: sum(1 for dgt in _digits(int(v), reff) if dgt))
+        hops = nnz((s_idx % n - t_idx % n) % n) + nnz((s_idx // n - t_idx // n) % G)
+        hops[np.arange(P), np.arange(P)] = 1
+        assert res.moved == int((prob.sendcounts.astype(np.int64) * hops).sum()) * prob.esz
+
+
+def test_twolayer_bruck_error_codes():
+    prob = W.make_problem(W.counts_uniform_random(12, 5, seed=1), 1, 0, 0)
+    send = W.fill_send_arena(prob, 0, 2)
+    recv = np.zeros(prob.recv_bytes, dtype=np.uint8)
+    for backend in (O, E):
+        assert backend.TTPL_rbruck_alltoallv(4, 1, prob, send, recv) == -1         # src/twophase_twolayer_rbruck.cpp:20
+        assert backend.TTPL_rbruck_alltoallv(5, 2, prob, send, recv) == -2
+        assert backend.TTPL_rbruck_alltoallv(0, 2, prob, send, recv) == -2
 
 
 def test_large_blocks_split_into_pieces():
