@@ -390,6 +390,52 @@ def test_benchmark_shapes_at_reduced_size(api):
         ("uniform isplit n=32 r=3", lambda d: api.uniform_inverse_isplit_r_bruck(32, 3, 2, dp, 300, ds, d), False)])
 
 
+def _transposed(prob):
+    """The alltoallv that undoes `prob`: every rank sends back what it received, from where it landed."""
+    import dataclasses
+    return dataclasses.replace(prob, sendcounts=prob.recvcounts, sdispls=prob.rdispls, sbase=prob.rbase, send_bytes=prob.recv_bytes,
+                               recvcounts=prob.sendcounts, rdispls=prob.sdispls, rbase=prob.sbase, recv_bytes=prob.send_bytes)
+
+
+@pytest.mark.parametrize("name", ["C2", "C3", "C4", "C5"])
+def test_benchmark_configurations_at_full_size(api, name):
+    """The benchmark configurations at their real sizes (up to 17 GB of payload), where no host oracle can follow:
+    the on-device definition check, a checksum over all bytes, and the round trip — the transposed alltoallv, run by
+    a different function, must give back the send arena bit for bit."""
+    import torch
+    counts, esz, tun = W.config_counts(name, 0)
+    prob = W.make_problem(counts, esz, 0, 0)
+    P = prob.P
+    fwd = {"C2": [("twophase r=2", lambda dp, s, d: api.twophase_rbruck_alltoallv(2, dp, s, d), False),
+                  ("tuna r=8", lambda dp, s, d: api.tuna_algorithm(8, 0, dp, s, d), False)],
+           "C3": [("twophase r=16", lambda dp, s, d: api.twophase_rbruck_alltoallv(16, dp, s, d), False)],
+           "C4": [("ttpl n=32 r=32", lambda dp, s, d: api.TTPL_BT_alltoallv(32, 32, 0, dp, s, d), True),
+                  ("ttpl_rbruck n=32 r=4", lambda dp, s, d: api.TTPL_rbruck_alltoallv(32, 4, dp, s, d), False)],
+           "C5": [("tuna r=32", lambda dp, s, d: api.tuna_algorithm(32, 0, dp, s, d), False)]}[name]
+    back = {"C2": lambda dp, s, d: api.twophase_rbruck_alltoallv_om(4, dp, s, d),
+            "C3": lambda dp, s, d: api.tuna_algorithm(2, 0, dp, s, d),
+            "C4": lambda dp, s, d: api.TTPL_BT_alltoallv_s1(32, 32, 0, dp, s, d),
+            "C5": lambda dp, s, d: api.spreadout_alltoallv(dp, s, d)}[name]
+    dp = api.DeviceProblem(prob)
+    ds = dp.new_send_arena()
+    ds.zero_()
+    dp.fill_payload(0, 11, ds)
+    checksum = int(ds.sum(dtype=torch.int64))
+    for label, fn, packed in fwd:
+        print("  ", name, label, flush=True)
+        dr = dp.new_recv_arena(0)
+        assert fn(dp, ds, dr) == 0, (label, dp.comm.error())
+        assert dp.verify(ds, dr, packed_recv=packed) == 0, label
+        assert int(dr.sum(dtype=torch.int64)) == checksum, label
+        assert dp.comm.last_stats().payload_bytes == prob.payload_bytes
+    dp.comm.free()
+    tp = api.DeviceProblem(_transposed(prob))
+    dback = tp.new_recv_arena(0)
+    assert back(tp, dr, dback) == 0, tp.comm.error()
+    assert torch.equal(dback, ds), name
+    tp.comm.free()
+
+
 def test_reference_input_matrices(api):
     """The reference's own communication patterns (inputs/<P>proc), scaled down, through the function its driver uses."""
     import os
