@@ -26,5 +26,24 @@ def build_library(verbose: bool = False) -> str:
     return LIB_PATH
 
 
+EXAMPLE_SRC = os.path.join(PKG_DIR, "examples", "vc_example.cpp")
+EXAMPLE_BIN = os.path.join(PKG_DIR, "examples", "vc_example")
+
+
+def build_example(verbose: bool = False) -> str:
+    """The C++ driver above the C ABI (host code only; links the library next to it)."""
+    cmd = [HIPCC, "-O2", "-std=c++17", "-Wall", "-x", "hip", "--offload-arch=gfx950", "-Xclang", "-target-feature", "-Xclang",
+           "-packed-fp32-ops", EXAMPLE_SRC, "-L" + PKG_DIR, "-lrbruck_vc", "-Wl,-rpath,$ORIGIN/..", "-o", EXAMPLE_BIN]
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    if verbose or res.returncode != 0:
+        print(" ".join(cmd))
+        print(res.stdout)
+        print("\n".join(l for l in res.stderr.splitlines() if "packed-fp32-ops" not in l))
+    if res.returncode != 0:
+        raise RuntimeError("hipcc failed building examples/vc_example")
+    return EXAMPLE_BIN
+
+
 if __name__ == "__main__":
     print(build_library(verbose=True))
+    print(build_example(verbose=True))

@@ -1,0 +1,28 @@
+"""The C++ driver above the C ABI (rbruck_alltoallv_amd/examples/vc_example.cpp): the reference's example loops
+(examples/rbruckv_example.cpp, examples/twophaseLayer_example.cpp) with every element of every receive buffer checked
+on the host."""
+import os
+import subprocess
+
+import pytest
+
+from rbruck_alltoallv_amd.build import EXAMPLE_BIN
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("P,ncores,bases", [(64, 8, [2, 4, 8]), (12, 3, [3, 12])])
+def test_example_driver_reports_no_errors(P, ncores, bases):
+    assert os.path.exists(EXAMPLE_BIN), "build it with python -m rbruck_alltoallv_amd.build"
+    res = subprocess.run([EXAMPLE_BIN, str(P), "1", str(ncores)] + [str(b) for b in bases], capture_output=True, text=True,
+                         timeout=300)
+    assert res.returncode == 0, res.stdout[-2000:] + res.stderr[-2000:]
+    lines = res.stdout.splitlines()
+    assert lines[-1] == "errors: 0"
+    assert not any("has errors" in l or "fail!" in l for l in lines)
+    sizes = 11                                               # n = 2 .. 2048
+    assert sum(l.startswith("[Rbruckv]") for l in lines) == sizes * len(bases)
+    assert sum(l.startswith("[TTPL]") for l in lines) == sizes * len(bases)
+    assert sum(l.startswith("[TTPL_S1]") for l in lines) == sizes * len(bases)
+    assert sum(l.startswith("[Spreadout]") for l in lines) == sizes
+    assert sum(l.startswith("[ExcOr]") for l in lines) == (sizes if P & (P - 1) == 0 else 0)
