@@ -12,8 +12,9 @@
 #include <stdint.h>
 
 #define VC_THREADS 256
-// most bytes one workgroup of the copy kernel moves: 256 lanes x 2 vectors x 16 bytes
+// window of one workgroup of the copy kernel: 256 lanes x 2 vectors x 16 bytes, starting at a cache-line boundary
 #define VC_CHUNK 8192
+#define VC_LINE 128
 // piece size for copies longer than that: 256 lanes x 1 vector x 16 bytes
 #define VC_PIECE 4096
 

@@ -5,11 +5,19 @@
 // the block where the sender holds it and one write where the receiver wants it.
 //
 // Shape of the kernel, chosen by measurement on MI355X: one 256-lane workgroup per
-// work item (a piece of at most VC_CHUNK = 8 KiB of one block), every lane moving
+// work item (a piece of one block that fits a window of VC_CHUNK = 8 KiB), every lane moving
 // up to two 16-byte vectors whose loads are both issued before the stores,
 // non-temporal on both sides (the data is touched once per hop).  Many small
 // workgroups beat persistent or wider ones for a plain copy on this chip, and the
 // same holds for the scattered variable-size blocks of an alltoallv.
+//
+// Workgroups are handed to the 8 XCDs of the chip in turn (workgroup b runs on XCD
+// b mod 8) and every XCD has its own L2.  Work items that follow each other in the
+// list are neighbours in memory (pieces of one block, blocks of one run), so each
+// XCD takes a contiguous eighth of the list instead of every eighth item: cache
+// lines shared by two neighbouring items then meet in one L2, and every XCD streams
+// through its own range of addresses.  Measured: +3 % on 4 KiB blocks, +15 % on
+// 1 MiB blocks cut into pieces.
 #include "vc_common.h"
 
 typedef unsigned int vc_u32x4 __attribute__((ext_vector_type(4)));
@@ -32,38 +40,52 @@ __device__ __forceinline__ char *vc_resolve(int64_t loc, const char *sendbuf, ch
     return base + off;
 }
 
-// One workgroup per work item: byte stores up to the first 16-byte boundary of dst,
-// aligned 16-byte stores fed by (possibly unaligned) 16-byte loads, then the tail.
-__global__ __launch_bounds__(VC_THREADS) void vc_copy_items_kernel(const VcDesc *__restrict__ items, const char *__restrict__ sendbuf,
-                                                                   char *__restrict__ recvbuf, char *__restrict__ stage) {
-    const VcDesc d = items[blockIdx.x];
+// One workgroup per work item.  Lane t owns the t-th and the (t + 256)-th 16-byte vector of the window that starts at
+// the 128-byte boundary at or below dst, so every wave stores whole cache lines whatever the byte phase of the block
+// (measured: +4 % over counting vectors from the first 16-byte boundary of dst).  Vectors that lie fully inside the
+// block are moved by (possibly unaligned) 16-byte loads and aligned stores; the < 16 bytes before the first and after
+// the last of them are moved byte-wise.  The planner guarantees len + (dst & 127) <= VC_CHUNK.
+#define VC_XCDS 8
+__global__ __launch_bounds__(VC_THREADS) void vc_copy_items_kernel(const VcDesc *__restrict__ items, unsigned nitems,
+                                                                   const char *__restrict__ sendbuf, char *__restrict__ recvbuf,
+                                                                   char *__restrict__ stage) {
+    // gridDim.x is a multiple of VC_XCDS; XCD k = blockIdx.x % VC_XCDS works through items [k * per, (k + 1) * per)
+    const unsigned per = gridDim.x / VC_XCDS;
+    const unsigned idx = (blockIdx.x % VC_XCDS) * per + blockIdx.x / VC_XCDS;
+    if (idx >= nitems) return;
+    const VcDesc d = items[idx];
     const int64_t len = d.len;
     if (len <= 0) return;
     const char *src = vc_resolve(d.src, sendbuf, recvbuf, stage);
     char *dst = vc_resolve(d.dst, sendbuf, recvbuf, stage);
     const int t = threadIdx.x;
-    int64_t head = (16 - ((uintptr_t)dst & 15)) & 15;
-    if (head > len) head = len;
-    const int64_t nvec = (len - head) >> 4;                 // at most VC_CHUNK / 16 = 2 * VC_THREADS
-    const char *s2 = src + head;
-    char *d2 = dst + head;
+    const int64_t w = (int64_t)((uintptr_t)dst & (VC_LINE - 1));     // offset of the block inside the window
+    // window vector j holds block bytes [16 j - w, 16 j - w + 16)
+    const int64_t first_full = (w + 15) >> 4, end_full = (w + len) >> 4;    // at most VC_CHUNK / 16 = 2 * VC_THREADS
+    const char *sw = src - w;
+    char *dw = dst - w;
     vc_u32x4 v0, v1;
-    const bool has0 = t < nvec, has1 = t + VC_THREADS < nvec;
-    if (has0) v0 = vc_load16(s2 + ((int64_t)t << 4));
-    if (has1) v1 = vc_load16(s2 + ((int64_t)(t + VC_THREADS) << 4));
+    const bool has0 = t >= first_full && t < end_full, has1 = t + VC_THREADS < end_full;
+    if (has0) v0 = vc_load16(sw + ((int64_t)t << 4));
+    if (has1) v1 = vc_load16(sw + ((int64_t)(t + VC_THREADS) << 4));
     // the < 16 head bytes (lanes 0..15) and the < 16 tail bytes (lanes 16..31) share one byte load and one byte store
-    const int64_t done = head + (nvec << 4);
+    int64_t head = (first_full << 4) - w;
+    if (head > len) head = len;
+    int64_t done = (end_full << 4) - w;
+    if (done < head) done = head;
     const int64_t edge = t < 16 ? (t < head ? t : -1) : (t < 32 && done + (t - 16) < len ? done + (t - 16) : -1);
     if (edge >= 0) dst[edge] = src[edge];
-    if (has0) vc_store16(d2 + ((int64_t)t << 4), v0);
-    if (has1) vc_store16(d2 + ((int64_t)(t + VC_THREADS) << 4), v1);
+    if (has0) vc_store16(dw + ((int64_t)t << 4), v0);
+    if (has1) vc_store16(dw + ((int64_t)(t + VC_THREADS) << 4), v1);
 }
 
 hipError_t vc_launch_copy_items(const VcDesc *items, int64_t nitems, const char *sendbuf, char *recvbuf, char *stage, hipStream_t st) {
-    const int64_t max_grid = 0x7FFFFFFF;                  // gridDim.x limit; more items than that go in several launches
+    const int64_t max_grid = 0x7FFFFFF8;                  // gridDim.x limit; more items than that go in several launches
     for (int64_t done = 0; done < nitems; done += max_grid) {
         const int64_t now = nitems - done < max_grid ? nitems - done : max_grid;
-        hipLaunchKernelGGL(vc_copy_items_kernel, dim3((unsigned)now), dim3(VC_THREADS), 0, st, items + done, sendbuf, recvbuf, stage);
+        const int64_t grid = (now + VC_XCDS - 1) / VC_XCDS * VC_XCDS;
+        hipLaunchKernelGGL(vc_copy_items_kernel, dim3((unsigned)grid), dim3(VC_THREADS), 0, st, items + done, (unsigned)now, sendbuf,
+                           recvbuf, stage);
     }
     return hipGetLastError();
 }

@@ -292,16 +292,20 @@ VC_HD int vc_entry_cut(const VcSched &S, const VcTables &T, const VcEntry &e) {
     return vc_phase16(S, T, e.s, e.t);
 }
 
-// A copy that fits one work item (VC_CHUNK bytes from the 16-byte boundary below its destination) stays whole; a
+// A copy that fits one work item (VC_CHUNK bytes from the cache-line boundary below its destination) stays whole; a
 // longer one is cut into pieces of at most VC_PIECE bytes, the size at which a plain copy runs fastest on this chip
 // (one vector per lane).  Only the first piece has a byte-wise head and only the last one a tail.
+// The copy kernel's window starts at the cache-line boundary at or below the destination; only the 16-byte phase of
+// that address is known here (staging offsets come later), so the rest of its line offset is assumed worst.
+VC_HD bool vc_fits_one_item(int64_t len, int phase) { return len + phase + (VC_LINE - 16) <= VC_CHUNK; }
+
 VC_HD int64_t vc_chunk_count(int64_t len, int phase, int cut) {
     if (len <= 0) return 0;
-    return len + phase <= VC_CHUNK ? 1 : (len + cut + VC_PIECE - 1) / VC_PIECE;
+    return vc_fits_one_item(len, phase) ? 1 : (len + cut + VC_PIECE - 1) / VC_PIECE;
 }
 
 VC_HD VcDesc vc_chunk_of(const VcDesc &whole, int64_t c, int phase, int cut) {
-    if (whole.len + phase <= VC_CHUNK) return whole;
+    if (vc_fits_one_item(whole.len, phase)) return whole;
     VcDesc d = whole;
     const int64_t lo = c == 0 ? 0 : c * VC_PIECE - cut;
     int64_t hi = (c + 1) * VC_PIECE - cut;

@@ -108,6 +108,8 @@ extern "C" int plan_emulate(int func, int P, int n, int r, int batch, int esz, i
                 items += nchunks;
                 for (int64_t c = 0; c < nchunks; c++) {
                 const VcDesc d = vc_chunk_of(whole, c, phase, cut);
+                // the copy kernel's window: VC_CHUNK bytes from the cache-line boundary at or below the destination
+                if (d.len + (((d.dst & VC_OFFSET_MASK) + dst_lo) & (VC_LINE - 1)) > VC_CHUNK) errors++;
                 if (d.len <= 0 || d.len > VC_CHUNK || d.src - whole.src != covered || d.dst - whole.dst != covered) { errors++; continue; }
                 // only the first piece may start off a 16-byte boundary of the destination
                 if (c > 0 && (((d.dst & VC_OFFSET_MASK) + dst_lo) & 15) != 0) errors++;
