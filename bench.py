@@ -32,7 +32,7 @@ HBM_PEAK_GBPS = 8000.0
 # HBM bytes per launch of the copy kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, each scaled by what the same
 # counter reads for a plain copy of known size (profiles/vc_copy_items_kernel_C4_pmc_fetch_write.txt); counters cannot
 # be read from inside this process, so workloads that were not profiled report null.
-MEASURED_TRAFFIC_PER_LAUNCH = {("C4", "TTPL_BT_alltoallv"): 8650655758}
+MEASURED_TRAFFIC_PER_LAUNCH = {("C4", "TTPL_BT_alltoallv"): 8408923538}
 METRIC = "effective alltoallv GB/s + % HBM peak, P=64..1024 virtual ranks, 1 GPU"
 
 
