@@ -135,7 +135,13 @@ __device__ __forceinline__ uint64_t vc_hash4(uint64_t seed, uint64_t a, uint64_t
     return vc_splitmix64(h + c);
 }
 
-// One workgroup per (source, destination) pair; a thread writes 8 bytes at a time.
+// gridDim.z workgroups per (source, destination) pair, each on its own slice of the block; a thread writes 8 bytes at
+// a time.
+static unsigned vc_slices_per_block(int P) {
+    const int64_t z = (4ll << 20) / ((int64_t)P * P);      // about 4 Mi workgroups at most; many slices when P is small
+    return (unsigned)(z < 1 ? 1 : (z > 64 ? 64 : z));
+}
+
 __global__ __launch_bounds__(VC_THREADS) void vc_fill_kernel(int mode, uint64_t seed, char *__restrict__ sendbuf,
                                                              const int *__restrict__ sc, const int *__restrict__ sd,
                                                              const int64_t *__restrict__ sbase, int esz, int P) {
@@ -143,7 +149,9 @@ __global__ __launch_bounds__(VC_THREADS) void vc_fill_kernel(int mode, uint64_t 
     const int64_t len = (int64_t)sc[(int64_t)s * P + d] * esz;
     unsigned char *at = (unsigned char *)sendbuf + sbase[s] + (int64_t)sd[(int64_t)s * P + d] * esz;
     const int64_t nwords = (len + 7) >> 3;
-    for (int64_t k = threadIdx.x; k < nwords; k += VC_THREADS) {
+    const int64_t per = (nwords + gridDim.z - 1) / gridDim.z;
+    const int64_t kend = (blockIdx.z + 1) * per < nwords ? (blockIdx.z + 1) * per : nwords;
+    for (int64_t k = blockIdx.z * per + threadIdx.x; k < kend; k += VC_THREADS) {
         uint64_t word;
         if (mode == 1) {
             uint64_t lo = ((uint64_t)s << 20) + ((uint64_t)d << 10) + (uint64_t)(2 * k);
@@ -160,7 +168,7 @@ __global__ __launch_bounds__(VC_THREADS) void vc_fill_kernel(int mode, uint64_t 
 
 hipError_t vc_launch_fill_payload(int mode, uint64_t seed, char *sendbuf, const int *sc, const int *sd, const int64_t *sbase,
                                   int esz, int P, hipStream_t st) {
-    hipLaunchKernelGGL(vc_fill_kernel, dim3(P, P), dim3(VC_THREADS), 0, st, mode, seed, sendbuf, sc, sd, sbase, esz, P);
+    hipLaunchKernelGGL(vc_fill_kernel, dim3(P, P, vc_slices_per_block(P)), dim3(VC_THREADS), 0, st, mode, seed, sendbuf, sc, sd, sbase, esz, P);
     return hipGetLastError();
 }
 
@@ -175,18 +183,20 @@ __global__ __launch_bounds__(VC_THREADS) void vc_verify_kernel(const char *__res
     const int t = blockIdx.y, s = blockIdx.x;
     const int64_t len = (int64_t)T.sc[(int64_t)s * P + t] * esz;
     int64_t bad = 0;
-    if ((int64_t)T.rc[(int64_t)t * P + s] * esz != len) bad = 1;     // the count exchange itself is wrong
+    if (blockIdx.z == 0 && threadIdx.x == 0 && (int64_t)T.rc[(int64_t)t * P + s] * esz != len) bad = 1;     // the count exchange itself is wrong
     const int *rd = packed ? T.rd_packed : T.rd;
     const unsigned char *a = (const unsigned char *)sendbuf + T.sbase[s] + (int64_t)T.sd[(int64_t)s * P + t] * esz;
     const unsigned char *b = (const unsigned char *)recvbuf + T.rbase[t] + (int64_t)rd[(int64_t)t * P + s] * esz;
-    for (int64_t k = threadIdx.x; k < len; k += VC_THREADS) bad += a[k] != b[k];
+    const int64_t per = (len + gridDim.z - 1) / gridDim.z;
+    const int64_t kend = (blockIdx.z + 1) * per < len ? (blockIdx.z + 1) * per : len;
+    for (int64_t k = blockIdx.z * per + threadIdx.x; k < kend; k += VC_THREADS) bad += a[k] != b[k];
     bad = vc_block_sum(bad, lds);
     if (threadIdx.x == 0 && bad) atomicAdd(mismatch, (unsigned long long)bad);
 }
 
 hipError_t vc_launch_verify(const char *sendbuf, const char *recvbuf, VcTables t, int esz, int P, int packed,
                             unsigned long long *mismatch, hipStream_t st) {
-    hipLaunchKernelGGL(vc_verify_kernel, dim3(P, P), dim3(VC_THREADS), 0, st, sendbuf, recvbuf, t, esz, P, packed, mismatch);
+    hipLaunchKernelGGL(vc_verify_kernel, dim3(P, P, vc_slices_per_block(P)), dim3(VC_THREADS), 0, st, sendbuf, recvbuf, t, esz, P, packed, mismatch);
     return hipGetLastError();
 }
 

@@ -436,6 +436,31 @@ def test_benchmark_configurations_at_full_size(api, name):
     tp.comm.free()
 
 
+def test_blocks_beyond_two_gib(api):
+    """Counts and displacements are int32 elements, byte offsets 64-bit: a 2.4 GB block (300 M elements of 8 bytes; the
+    reference's int byte arithmetic, src/twophase_tunable_rbruckv.cpp:98, would overflow) next to empty and tiny ones."""
+    import torch
+    counts = np.array([[3, 300_000_000, 0], [1, 0, 7], [200_000_000, 5, 2]], dtype=np.int32)
+    prob = W.make_problem(counts, 8, 0, 0)
+    assert prob.payload_bytes > 2 ** 31
+    dp = api.DeviceProblem(prob)
+    ds = dp.new_send_arena()
+    dp.fill_payload(0, 5, ds)
+    checksum = int(ds.sum(dtype=torch.int64))
+    for name, fn in (("twophase r=2", lambda d: api.twophase_rbruck_alltoallv(2, dp, ds, d)),
+                     ("tuna r=2", lambda d: api.tuna_algorithm(2, 0, dp, ds, d)),
+                     ("ttpl n=1", lambda d: api.TTPL_BT_alltoallv_s1(1, 2, 0, dp, ds, d)),
+                     ("ttpl_rbruck n=1 r=2", lambda d: api.TTPL_rbruck_alltoallv(1, 2, dp, ds, d)),
+                     ("spreadout", lambda d: api.spreadout_alltoallv(dp, ds, d))):
+        print("  ", name, flush=True)
+        dr = dp.new_recv_arena(0)
+        assert fn(dr) == 0, (name, dp.comm.error())
+        assert dp.verify(ds, dr) == 0, name
+        assert int(dr.sum(dtype=torch.int64)) == checksum, name
+        del dr
+    dp.comm.free()
+
+
 def test_reference_input_matrices(api):
     """The reference's own communication patterns (inputs/<P>proc), scaled down, through the function its driver uses."""
     import os
