@@ -173,7 +173,7 @@ typedef struct vc_plan *vc_plan_t;
 /* `function` is the name of one of the alltoallv-shaped entry points above ("twophase_rbruck_alltoallv", "tuna_algorithm",
  * "TTPL_BT_alltoallv", "spreadout_alltoallv", ...); n, r and batch (b / bblock) are that function's tunables, ignored where
  * it has none.  The tables are read now and not needed afterwards; the communicator's bases are read now too.
- * recvbuf_low_bits = (address of the recvbuf that will be passed) & 4095: the low 4 bits must match at execution, the
+ * recvbuf_low_bits = (address of the recvbuf that will be passed) & 4095: the low 7 bits must match at execution, the
  * rest only decides where long copies are cut.  Same return codes as the function itself. */
 int vc_plan_create(const char *function, int n, int r, int batch, int *sendcounts, int *sdispls, int elem_size,
                    int *recvcounts, int *rdispls, int recvbuf_low_bits, vc_comm_t comm, vc_plan_t *plan_out);

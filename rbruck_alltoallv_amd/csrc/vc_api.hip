@@ -499,14 +499,14 @@ extern "C" int vc_plan_create(const char *function, int n, int r, int batch, int
 
 extern "C" int vc_plan_execute(vc_plan_t p, char *sendbuf, char *recvbuf) {
     if (!p || !sendbuf || !recvbuf) return fail_arg("vc_plan_execute: null argument");
-    if ((int)((uintptr_t)recvbuf & 15) != (p->info.recv_lo & 15))
+    if ((int)((uintptr_t)recvbuf & (VC_LINE - 1)) != (p->info.recv_lo & (VC_LINE - 1)))
         return fail_arg("vc_plan_execute: recvbuf must have the low address bits the plan was made for");
     return run_items(p->comm, p->info, p->items.as<VcDesc>(), sendbuf, recvbuf, false);
 }
 
 extern "C" int vc_plan_execute_async(vc_plan_t p, char *sendbuf, char *recvbuf) {
     if (!p || !sendbuf || !recvbuf) return fail_arg("vc_plan_execute_async: null argument");
-    if ((int)((uintptr_t)recvbuf & 15) != (p->info.recv_lo & 15))
+    if ((int)((uintptr_t)recvbuf & (VC_LINE - 1)) != (p->info.recv_lo & (VC_LINE - 1)))
         return fail_arg("vc_plan_execute_async: recvbuf must have the low address bits the plan was made for");
     return launch_items(p->comm, p->info, p->items.as<VcDesc>(), sendbuf, recvbuf);
 }

@@ -48,7 +48,7 @@ struct VcSched {
     int esz;          // element size in bytes
     int packed_recv;  // 1: receive side is the packed source-ordered layout (TTPL_BT_alltoallv ignores rdispls)
     int uniform;      // >0: equal blocks of this many elements, tables are implied (uniform_* functions)
-    int recv_lo;      // low 12 bits of the recvbuf pointer: staging slots copy the final destination's 16-byte phase,
+    int recv_lo;      // low 12 bits of the recvbuf pointer: staging slots copy the final destination's cache-line phase,
                       // long copies into recvbuf are cut at its 4 KiB boundaries
     int coalesce;     // 1: blocks that are about to leave their node wait in "organized" runs — the n blocks one rank
                       //    holds for one destination rank back to back in source order — so that an inter-node message

@@ -108,21 +108,21 @@ VC_HD int64_t vc_recv_offset(const VcSched &S, const VcTables &T, int s, int t) 
     return T.rbase[t] + (int64_t)rd[(int64_t)t * S.P + s] * S.esz;
 }
 
-// Staging slots start 16-byte aligned; the data inside starts at the 16-byte phase
+// Staging slots start cache-line (VC_LINE) aligned; the data inside starts at the line phase
 // of the block's final address in recvbuf, so that every later hop copies between
 // equally aligned addresses.
-VC_HD int vc_phase16(const VcSched &S, const VcTables &T, int s, int t) {
-    return (int)((vc_recv_offset(S, T, s, t) + S.recv_lo) & 15);
+VC_HD int vc_phase(const VcSched &S, const VcTables &T, int s, int t) {
+    return (int)((vc_recv_offset(S, T, s, t) + S.recv_lo) & (VC_LINE - 1));
 }
 
 
 // Bytes the staging slot `id` of rank `to` needs for the block that arrives in digit x
-// (0 if nothing arrives there, or if it goes to recvbuf).  Always a multiple of 16.
+// (0 if nothing arrives there, or if it goes to recvbuf).  Always a multiple of VC_LINE.
 VC_HD int64_t vc_stage_slot_size(const VcSched &S, const VcTables &T, int x, int dist, int to, int id) {
     VcBlock b;
     if (!vc_intra_block(S, x, dist, to, id, b) || !b.to_stage || b.to_org) return 0;
     const int64_t len = (int64_t)T.sc[(int64_t)b.s * S.P + b.t] * S.esz;
-    return len ? ((len + vc_phase16(S, T, b.s, b.t) + 15) & ~15ll) : 0;
+    return len ? ((len + vc_phase(S, T, b.s, b.t) + VC_LINE - 1) & ~(int64_t)(VC_LINE - 1)) : 0;
 }
 
 // The same for staging region y of a call: intra-node digits first, then inter-node digits.
@@ -137,7 +137,7 @@ VC_HD int64_t vc_region_slot_size(const VcSched &S, const VcTables &T, int y, in
     int z;
     if (!vc_inter_block(S, y - S.w, dist, to, id, e, z) || e.xdst < 0) return 0;
     const int64_t len = (int64_t)T.sc[(int64_t)e.s * S.P + e.t] * S.esz;
-    return len ? ((len + vc_phase16(S, T, e.s, e.t) + 15) & ~15ll) : 0;
+    return len ? ((len + vc_phase(S, T, e.s, e.t) + VC_LINE - 1) & ~(int64_t)(VC_LINE - 1)) : 0;
 }
 
 // Address (inside the staging arena) of the data of block (s, t) while it sits in slot `id`
@@ -145,7 +145,7 @@ VC_HD int64_t vc_region_slot_size(const VcSched &S, const VcTables &T, int y, in
 VC_HD int64_t vc_stage_addr(const VcSched &S, const VcTables &T, const int64_t *slot_off, const int64_t *row_base,
                             int x, int holder, int id, int s, int t) {
     const int64_t row = (int64_t)x * S.P + holder;
-    return row_base[row] + slot_off[row * S.P + id] + vc_phase16(S, T, s, t);
+    return row_base[row] + slot_off[row * S.P + id] + vc_phase(S, T, s, t);
 }
 
 VC_HD int64_t vc_send_offset(const VcSched &S, const VcTables &T, int s, int t) {
@@ -155,7 +155,7 @@ VC_HD int64_t vc_send_offset(const VcSched &S, const VcTables &T, int s, int t) 
 // ---- organized region (S.coalesce) ----
 // Rank `to` = (gs, l) keeps, for every other group g, a run that mirrors byte for byte the part of rank (g, l)'s
 // packed recvbuf that comes from group gs: n blocks in source order.  The block of local rank l itself never
-// moves inside the node and leaves a hole of its length.  A run starts 16-byte aligned plus the 16-byte phase of
+// moves inside the node and leaves a hole of its length.  A run starts line aligned plus the line phase of
 // its image in recvbuf, so that the inter-node copy of a run is a copy between equally aligned addresses.
 
 // byte offset, inside rank t's recvbuf, of the first block coming from group gs (packed receive layout)
@@ -170,20 +170,20 @@ VC_HD int64_t vc_org_run_prefix(const VcSched &S, const VcTables &T, int gs, int
     return (end - T.rd_packed[row + s0]) * S.esz;
 }
 
-// size of the run rank `to` keeps for group g (multiple of 16; 0 for its own group)
+// size of the run rank `to` keeps for group g (multiple of VC_LINE; 0 for its own group)
 VC_HD int64_t vc_org_run_size(const VcSched &S, const VcTables &T, int to, int g) {
     const int gs = to / S.n, t = g * S.n + to % S.n;
     if (g == gs) return 0;
-    const int64_t phase = (vc_org_run_dst(S, T, gs, t) + S.recv_lo) & 15;
-    return (phase + vc_org_run_prefix(S, T, gs, t, S.n) + 15) & ~15ll;
+    const int64_t phase = (vc_org_run_dst(S, T, gs, t) + S.recv_lo) & (VC_LINE - 1);
+    return (phase + vc_org_run_prefix(S, T, gs, t, S.n) + VC_LINE - 1) & ~(int64_t)(VC_LINE - 1);
 }
 
-// 16-byte aligned part of the offset of slot id = g*n + m inside the run (vc_stage_addr adds the block's own phase)
+// line-aligned part of the offset of slot id = g*n + m inside the run (vc_stage_addr adds the block's own phase)
 VC_HD int64_t vc_org_slot_rel(const VcSched &S, const VcTables &T, int to, int id) {
     const int gs = to / S.n, g = id / S.n, m = id % S.n, t = g * S.n + to % S.n;
     if (g == gs) return 0;
-    const int64_t phase = (vc_org_run_dst(S, T, gs, t) + S.recv_lo) & 15;
-    return (phase + vc_org_run_prefix(S, T, gs, t, m)) & ~15ll;
+    const int64_t phase = (vc_org_run_dst(S, T, gs, t) + S.recv_lo) & (VC_LINE - 1);
+    return (phase + vc_org_run_prefix(S, T, gs, t, m)) & ~(int64_t)(VC_LINE - 1);
 }
 
 
@@ -279,25 +279,24 @@ VC_HD VcDesc vc_entry_desc(const VcSched &S, const VcTables &T, const int64_t *s
 // address is a multiple of 16, so that only the first piece of a block has a byte-wise head and only the last one a
 // tail; every piece in between is whole aligned vectors.
 
-// 16-byte phase of the destination address of an entry's copy.  Staging slots and organized runs are laid out at
+// Cache-line phase of the destination address of an entry's copy.  Staging slots and organized runs are laid out at
 // the phase of the block's final address, so this holds whichever arena the copy writes to.
-VC_HD int vc_entry_phase(const VcSched &S, const VcTables &T, const VcEntry &e) { return vc_phase16(S, T, e.s, e.t); }
+VC_HD int vc_entry_phase(const VcSched &S, const VcTables &T, const VcEntry &e) { return vc_phase(S, T, e.s, e.t); }
 
 // Where a long copy is cut: pieces end where the destination address is a multiple of VC_PIECE when the destination
 // is recvbuf (whole 4 KiB-aligned pieces, no cache line shared between two workgroups), and at multiples of VC_PIECE
-// from the 16-byte boundary below the start otherwise (staging addresses are not known when pieces are counted).
-// Always congruent to the 16-byte phase.
+// from the line boundary below the start otherwise (staging addresses are not known when pieces are counted).
+// Always congruent to the line phase.
 VC_HD int vc_entry_cut(const VcSched &S, const VcTables &T, const VcEntry &e) {
     if (e.xdst < 0) return (int)((vc_recv_offset(S, T, e.s, e.t) + S.recv_lo) & (VC_PIECE - 1));
-    return vc_phase16(S, T, e.s, e.t);
+    return vc_phase(S, T, e.s, e.t);
 }
 
 // A copy that fits one work item (VC_CHUNK bytes from the cache-line boundary below its destination) stays whole; a
 // longer one is cut into pieces of at most VC_PIECE bytes, the size at which a plain copy runs fastest on this chip
 // (one vector per lane).  Only the first piece has a byte-wise head and only the last one a tail.
-// The copy kernel's window starts at the cache-line boundary at or below the destination; only the 16-byte phase of
-// that address is known here (staging offsets come later), so the rest of its line offset is assumed worst.
-VC_HD bool vc_fits_one_item(int64_t len, int phase) { return len + phase + (VC_LINE - 16) <= VC_CHUNK; }
+// The copy kernel's window starts at the cache-line boundary at or below the destination: `phase` bytes before it.
+VC_HD bool vc_fits_one_item(int64_t len, int phase) { return len + phase <= VC_CHUNK; }
 
 VC_HD int64_t vc_chunk_count(int64_t len, int phase, int cut) {
     if (len <= 0) return 0;

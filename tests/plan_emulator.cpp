@@ -100,9 +100,9 @@ extern "C" int plan_emulate(int func, int P, int n, int r, int batch, int esz, i
                 const VcDesc whole = vc_entry_desc(S, T, slot_off.data(), row_base.data(), e, to);
                 const int phase = vc_entry_phase(S, T, e);
                 const int dst_lo = (int)(whole.dst >> VC_SPACE_SHIFT) == 1 ? recv_lo : 0;
-                if (whole.len > 0 && (int)(((whole.dst & VC_OFFSET_MASK) + dst_lo) & 15) != phase) errors++;
+                if (whole.len > 0 && (int)(((whole.dst & VC_OFFSET_MASK) + dst_lo) & (VC_LINE - 1)) != phase) errors++;
                 const int cut = vc_entry_cut(S, T, e);
-                if ((cut & 15) != phase) errors++;
+                if ((cut & (VC_LINE - 1)) != phase) errors++;
                 const int64_t nchunks = vc_chunk_count(whole.len, phase, cut);
                 int64_t covered = 0;
                 items += nchunks;
@@ -111,8 +111,8 @@ extern "C" int plan_emulate(int func, int P, int n, int r, int batch, int esz, i
                 // the copy kernel's window: VC_CHUNK bytes from the cache-line boundary at or below the destination
                 if (d.len + (((d.dst & VC_OFFSET_MASK) + dst_lo) & (VC_LINE - 1)) > VC_CHUNK) errors++;
                 if (d.len <= 0 || d.len > VC_CHUNK || d.src - whole.src != covered || d.dst - whole.dst != covered) { errors++; continue; }
-                // only the first piece may start off a 16-byte boundary of the destination
-                if (c > 0 && (((d.dst & VC_OFFSET_MASK) + dst_lo) & 15) != 0) errors++;
+                // only the first piece may start off a cache-line boundary of the destination
+                if (c > 0 && (((d.dst & VC_OFFSET_MASK) + dst_lo) & (VC_LINE - 1)) != 0) errors++;
                 // ... and, in recvbuf, on a 4 KiB boundary
                 if (c > 0 && (int)(whole.dst >> VC_SPACE_SHIFT) == 1 && (((d.dst & VC_OFFSET_MASK) + dst_lo) & (VC_PIECE - 1)) != 0) errors++;
                 covered += d.len;

@@ -352,12 +352,12 @@ def test_coalesced_twolayer_route(P, n, r, bblock):
 
 def test_unaligned_recvbuf_pointer_keeps_the_phase_rule():
     """The low bits of the recvbuf pointer enter every staging phase; pieces after the first still start on a
-    16-byte boundary of the real destination address."""
+    cache-line boundary of the real destination address."""
     counts = (W.counts_uniform_random(12, 30000, seed=5) * (W.counts_uniform_random(12, 3, seed=6) > 0)).astype(np.int32)
     prob = W.make_problem(counts, 1, 1, 0)
     send = W.fill_send_arena(prob, 0, 9)
     want = W.expected_recv_arena(prob, send)
-    for recv_lo in (0, 5, 15, 2048 + 7, 4095):
+    for recv_lo in (0, 5, 15, 100, 2048 + 7, 4095):
         for func, kw in ((E.F_TWOPHASE, dict(r=3)), (E.F_TUNA, dict(r=2, batch=1)), (E.F_TTPL, dict(n=4, r=4)),
                          (E.F_TTPL_S1, dict(n=6, r=2, batch=5)), (E.F_SPREADOUT, {})):
             recv = np.full(prob.recv_bytes, 0xEE, dtype=np.uint8)
