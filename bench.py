@@ -32,7 +32,7 @@ HBM_PEAK_GBPS = 8000.0
 # HBM bytes per launch of the copy kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, each scaled by what the same
 # counter reads for a plain copy of known size (profiles/vc_copy_items_kernel_C4_pmc_fetch_write.txt); counters cannot
 # be read from inside this process, so workloads that were not profiled report null.
-MEASURED_TRAFFIC_PER_LAUNCH = {("C4", "TTPL_BT_alltoallv"): 8408923538}
+MEASURED_TRAFFIC_PER_LAUNCH = {("C4", "TTPL_BT_alltoallv", 0): 8408923538}
 METRIC = "effective alltoallv GB/s + % HBM peak, P=64..1024 virtual ranks, 1 GPU"
 
 
@@ -153,6 +153,8 @@ def main() -> None:
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="C4")
+    ap.add_argument("--forward", type=int, default=0, choices=(0, 1),
+                    help="1: forwarded execution (vc_comm_set_forwarding) is the mode that is measured; the other one is reported beside it")
     ap.add_argument("--func", default=None, help="override the function (e.g. TTPL_BT_alltoallv_s1)")
     ap.add_argument("--radix", type=int, default=0, help="override the radix r of the workload")
     ap.add_argument("--seed", type=int, default=0)
@@ -193,49 +195,49 @@ def main() -> None:
         dp.comm._check(dp.comm.lib.vc_calibration_copy(b.data_ptr(), a.data_ptr(), nb, dp.comm.handle))
         del a, b
 
-    for _ in range(args.warmup):
-        rc = call(api, func, tun, dp, send, recv)
-        assert rc == 0, dp.comm.error()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    kern_ms, kern_bytes, nkern, plan_ms = 0.0, 0, 0, 0.0
-    per_launch_ms = None
-    for _ in range(args.steps):
-        rc = call(api, func, tun, dp, send, recv)
-        assert rc == 0, dp.comm.error()
+    def timed_calls(warmup, steps):
+        for _ in range(warmup):
+            rc = call(api, func, tun, dp, send, recv)
+            assert rc == 0, dp.comm.error()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        kern_ms, kern_bytes, nkern, plan_ms = 0.0, 0, 0, 0.0
+        per_launch_ms = None
+        for _ in range(steps):
+            rc = call(api, func, tun, dp, send, recv)
+            assert rc == 0, dp.comm.error()
+            st = dp.comm.last_stats()
+            for k in range(st.n_launches):
+                kern_ms += st.launch_ms[k]
+                kern_bytes += 2 * st.launch_bytes[k]
+                nkern += 1
+            plan_ms += st.plan_ms
+            if st.n_launches <= 16:
+                now = [st.launch_ms[k] for k in range(st.n_launches)]
+                per_launch_ms = now if per_launch_ms is None else [a + b for a, b in zip(per_launch_ms, now)]
+        torch.cuda.synchronize()
+        elapsed = time.perf_counter() - t0
         st = dp.comm.last_stats()
-        for k in range(st.n_launches):
-            kern_ms += st.launch_ms[k]
-            kern_bytes += 2 * st.launch_bytes[k]
-            nkern += 1
-        plan_ms += st.plan_ms
-        if st.n_launches <= 16:
-            now = [st.launch_ms[k] for k in range(st.n_launches)]
-            per_launch_ms = now if per_launch_ms is None else [a + b for a, b in zip(per_launch_ms, now)]
-    torch.cuda.synchronize()
-    elapsed = time.perf_counter() - t0
-    st = dp.comm.last_stats()
-    assert 2 * st.moved_bytes == A, (st.moved_bytes, A)
-    assert st.payload_bytes == S
+        assert 2 * st.moved_bytes == A, (st.moved_bytes, A)
+        assert st.payload_bytes == S
+        return elapsed, kern_ms, kern_bytes, nkern, plan_ms, per_launch_ms, st
 
-    bad = dp.verify(send, recv, packed_recv=(func == "TTPL_BT_alltoallv"))
-
-    # The same collective as a persistent plan (planned once, executed many times): what the path costs when the
-    # count tables do not change between calls.  Extra information; `value` stays the full call.
-    plan_kw = {"n": tun.get("n", 0), "r": tun.get("r", 2), "batch": tun.get("b", tun.get("bblock", 0))}
-    plan = api.Plan(func, dp, recv, **plan_kw)
-    plan_info = None
-    if plan.rc == 0:
+    def plan_timing(steps):
+        """The same collective as a persistent plan (planned once, executed many times), and that plan in a HIP graph."""
+        plan_kw = {"n": tun.get("n", 0), "r": tun.get("r", 2), "batch": tun.get("b", tun.get("bblock", 0))}
+        plan = api.Plan(func, dp, recv, **plan_kw)
+        if plan.rc != 0:
+            return None
         assert plan.execute(send, recv) == 0, dp.comm.error()
         torch.cuda.synchronize()
         p0 = time.perf_counter()
-        for _ in range(args.steps):
+        for _ in range(steps):
             assert plan.execute(send, recv) == 0
         torch.cuda.synchronize()
-        plan_s = (time.perf_counter() - p0) / args.steps
-        plan_bad = dp.verify(send, recv, packed_recv=(func == "TTPL_BT_alltoallv"))
-        plan_info = {"ms_per_call": round(plan_s * 1e3, 4), "GBps_effective": round(S / plan_s / 1e9, 1),
-                     "hbm_frac": round(A / plan_s / 1e9 / HBM_PEAK_GBPS, 4), "mismatched_bytes": int(plan_bad)}
+        plan_s = (time.perf_counter() - p0) / steps
+        plan_bad = dp.verify(send, recv, packed_recv=packed)
+        info = {"ms_per_call": round(plan_s * 1e3, 4), "GBps_effective": round(S / plan_s / 1e9, 1),
+                "hbm_frac": round(A / plan_s / 1e9 / HBM_PEAK_GBPS, 4), "mismatched_bytes": int(plan_bad)}
         # ... and its launches captured once into a HIP graph (what a launch-bound inner loop would replay)
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph):
@@ -245,14 +247,39 @@ def main() -> None:
         graph.replay()
         torch.cuda.synchronize()
         g0 = time.perf_counter()
-        for _ in range(args.steps):
+        for _ in range(steps):
             graph.replay()
             torch.cuda.synchronize()
-        graph_s = (time.perf_counter() - g0) / args.steps
-        plan_info["graph_replay_ms_per_call"] = round(graph_s * 1e3, 4)
-        plan_info["graph_mismatched_bytes"] = int(dp.verify(send, recv, packed_recv=(func == "TTPL_BT_alltoallv")))
+        graph_s = (time.perf_counter() - g0) / steps
+        info["graph_replay_ms_per_call"] = round(graph_s * 1e3, 4)
+        info["graph_mismatched_bytes"] = int(dp.verify(send, recv, packed_recv=packed))
         del graph
         plan.free()
+        return info
+
+    packed = func == "TTPL_BT_alltoallv"
+    dp.comm.set_forwarding(bool(args.forward))
+    elapsed, kern_ms, kern_bytes, nkern, plan_ms, per_launch_ms, st = timed_calls(args.warmup, args.steps)
+
+    bad = dp.verify(send, recv, packed_recv=(func == "TTPL_BT_alltoallv"))
+
+    # Extra information; `value` stays the full call.
+    plan_info = plan_timing(args.steps)
+
+    # The other way of executing the same call (launch per digit phase <-> forwarded), on fewer steps.
+    dp.comm.set_forwarding(not args.forward)
+    o_steps = max(3, min(args.steps, 10))
+    o_elapsed, o_kern_ms, o_kern_bytes, o_nkern, _, _, o_st = timed_calls(2, o_steps)
+    o_bad = dp.verify(send, recv, packed_recv=packed)
+    o_plan = plan_timing(o_steps)
+    other = {"mode": "launch per digit phase" if args.forward else "forwarded (one launch, blocks carried through all hops in registers)",
+             "ms_per_call": round(o_elapsed / o_steps * 1e3, 4), "GBps_effective": round(S / (o_elapsed / o_steps) / 1e9, 1),
+             "hbm_frac_whole_call": round(A / (o_elapsed / o_steps) / 1e9 / HBM_PEAK_GBPS, 4),
+             "kernel_frac": round(o_kern_bytes / (o_kern_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4) if o_kern_ms > 0 else None,
+             "launches": int(o_st.n_launches), "mismatched_bytes": int(o_bad),
+             "plan_ms_per_call": None if o_plan is None else o_plan["ms_per_call"],
+             "plan_graph_replay_ms": None if o_plan is None else o_plan["graph_replay_ms_per_call"]}
+    dp.comm.set_forwarding(bool(args.forward))
 
     # The linear comparator the reference drivers time beside the Bruck variants (examples/twophaseLayer_example.cpp:99-113
     # times MPI_Alltoallv): on one GPU it is a single pass over the payload.  Context only, not the metric.
@@ -283,13 +310,15 @@ def main() -> None:
         "one_pass_floor_fraction": round(2 * S / (elapsed / args.steps) / 1e9 / HBM_PEAK_GBPS, 4),
         "plan_ms_per_step": round(plan_ms / args.steps, 4),
         "mismatched_bytes": int(bad),
+        "execution": "forwarded (one launch, blocks carried through all hops in registers)" if args.forward else "launch per digit phase",
         "persistent_plan": plan_info,
+        "other_execution_mode": other,
         "one_pass_comparator": {"func": "spreadout_alltoallv", "ms_per_call": round(comp_s * 1e3, 4),
                                 "GBps_effective": round(S / comp_s / 1e9, 1),
                                 "hbm_frac": round(2 * S / comp_s / 1e9 / HBM_PEAK_GBPS, 4), "mismatched_bytes": int(comp_bad)},
-        "roofline": {"bound": "hbm", "kernel": "vc_copy_items_kernel", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
+        "roofline": {"bound": "hbm", "kernel": "vc_copy_chains_kernel" if args.forward else "vc_copy_items_kernel", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
                      "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
-                     "traffic": MEASURED_TRAFFIC_PER_LAUNCH.get((args.workload, func)),
+                     "traffic": MEASURED_TRAFFIC_PER_LAUNCH.get((args.workload, func, int(bool(args.forward)))),
                      "avg_launch_ms": round(kern_ms / max(nkern, 1), 4),
                      "algorithmic_bytes_per_launch": int(kern_bytes / max(nkern, 1)),
                      "per_launch": None if per_launch_ms is None else [

@@ -47,6 +47,10 @@ class VirtualComm:
     def set_timing(self, on: bool) -> None:
         self._check(self.lib.vc_comm_set_timing(self.handle, int(on)))
 
+    def set_forwarding(self, enable: bool) -> None:
+        """vc_comm_set_forwarding: one launch per call, every block piece carried through all its hops in registers."""
+        self._check(self.lib.vc_comm_set_forwarding(self.handle, int(enable)))
+
     def last_stats(self) -> _lib.VcStats:
         s = _lib.VcStats()
         self._check(self.lib.vc_comm_last_stats(self.handle, C.byref(s)))

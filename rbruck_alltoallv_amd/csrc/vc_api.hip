@@ -18,6 +18,7 @@
 #include "../../include/rbruck_vc.h"
 #include "vc_common.h"
 #include "vc_sched.h"
+#include "vc_plan_math.h"
 
 static thread_local std::string g_last_error;
 
@@ -63,6 +64,8 @@ struct vc_comm {
     hipStream_t stream = nullptr;
     const int64_t *sbase = nullptr, *rbase = nullptr;
     bool timing = false;
+    bool forward = false;                 // forwarded execution: one launch, every block piece carried through all its hops
+    DevBuf chain_row_tot, chain_row_base, hop_src, hop_dst;
     DevBuf slot_off, row_tot, row_base, org_run_base, item_row_tot, item_row_base, row_bytes, desc, header, launches, stage, rd_packed,
         uni_counts, uni_displs, scratch;
     int64_t *h_header = nullptr;          // pinned, coherent: the planner writes its header straight into it
@@ -101,7 +104,7 @@ extern "C" int vc_comm_free(vc_comm_t c) {
     if (!c) return VC_OK;
     (void)hipStreamSynchronize(c->stream);
     for (DevBuf *b : {&c->slot_off, &c->row_tot, &c->row_base, &c->org_run_base, &c->item_row_tot, &c->item_row_base, &c->row_bytes, &c->desc, &c->header, &c->launches, &c->stage, &c->rd_packed,
-                      &c->uni_counts, &c->uni_displs, &c->scratch})
+                      &c->uni_counts, &c->uni_displs, &c->scratch, &c->chain_row_tot, &c->chain_row_base, &c->hop_src, &c->hop_dst})
         b->release();
     for (hipEvent_t e : c->events) (void)hipEventDestroy(e);
     if (c->h_header) (void)hipHostFree(c->h_header);
@@ -128,6 +131,12 @@ extern "C" int vc_comm_set_bases(vc_comm_t c, const int64_t *sbase, const int64_
 extern "C" int vc_comm_set_timing(vc_comm_t c, int enable) {
     if (!c) return fail_arg("null communicator");
     c->timing = enable != 0;
+    return VC_OK;
+}
+
+extern "C" int vc_comm_set_forwarding(vc_comm_t c, int enable) {
+    if (!c) return fail_arg("null communicator");
+    c->forward = enable != 0;
     return VC_OK;
 }
 
@@ -185,10 +194,13 @@ struct PlanInfo {
     int recv_lo = 0;
     int64_t stage_bytes = 0, payload_bytes = 0;
     std::vector<int64_t> first, count, bytes;       // per launch: first work item, item count, bytes moved
+    bool chain = false;                             // forwarded execution: `items` holds chain items instead
+    int chain_stride = 0;                           // int64 words per chain item
+    int64_t chain_items = 0;
 };
 
 // Step 3: staging prefix sums, item counts (read back to size the buffers), then the work items into `items`.
-static int build_plan(vc_comm *c, VcSched S, std::vector<VcLaunchInfo> &L, VcTables T, DevBuf &items, PlanInfo &out) {
+static int build_plan(vc_comm *c, VcSched S, std::vector<VcLaunchInfo> &L, VcTables T, DevBuf &items, PlanInfo &out, bool forward) {
     const int P = S.P;
     const int nl = (int)L.size();
     if (nl > VC_MAX_LAUNCHES) return fail_arg("more than VC_MAX_LAUNCHES launches: raise b / bblock");
@@ -205,6 +217,11 @@ static int build_plan(vc_comm *c, VcSched S, std::vector<VcLaunchInfo> &L, VcTab
     HIP_TRY(c->row_bytes.reserve(sizeof(int64_t) * (size_t)P * (nl + 1)));
     HIP_TRY(c->header.reserve(sizeof(int64_t) * VC_HEADER_WORDS(VC_MAX_LAUNCHES)));
     HIP_TRY(c->launches.reserve(sizeof(VcLaunchInfo) * VC_MAX_LAUNCHES));
+    if (forward) {
+        if (vc_hop_slots(S) > VC_MAX_HOP_SLOTS) return fail_arg("too many digits for forwarded execution");
+        HIP_TRY(c->chain_row_tot.reserve(sizeof(int64_t) * (size_t)P));
+        HIP_TRY(c->chain_row_base.reserve(sizeof(int64_t) * (size_t)P));
+    }
     if (c->timing) { int rc = ensure_events(c, (size_t)nl + 4); if (rc) return rc; }
 
     if (c->timing) HIP_TRY(hipEventRecord(c->events[0], st));
@@ -221,7 +238,8 @@ static int build_plan(vc_comm *c, VcSched S, std::vector<VcLaunchInfo> &L, VcTab
     }
     HIP_TRY(vc_launch_plan_sizes(S, c->launches.as<VcLaunchInfo>(), nl, T, c->slot_off.as<int64_t>(), c->row_tot.as<int64_t>(),
                                  c->row_base.as<int64_t>(), c->org_run_base.as<int64_t>(), c->item_row_tot.as<int64_t>(),
-                                 c->item_row_base.as<int64_t>(), c->row_bytes.as<int64_t>(), c->header.as<int64_t>(), c->h_header_dev, st));
+                                 c->item_row_base.as<int64_t>(), c->row_bytes.as<int64_t>(), forward ? c->chain_row_tot.as<int64_t>() : nullptr,
+                                 forward ? c->chain_row_base.as<int64_t>() : nullptr, c->header.as<int64_t>(), c->h_header_dev, st));
     HIP_TRY(hipStreamSynchronize(st));     // the staging arena and the item list are sized from the plan
 
     const int64_t *h = c->h_header;
@@ -235,6 +253,19 @@ static int build_plan(vc_comm *c, VcSched S, std::vector<VcLaunchInfo> &L, VcTab
         out.count[k] = h[3 + 2 * nl + k];
         nitems += out.count[k];
     }
+    if (forward) {
+        out.chain = true;
+        out.chain_stride = VC_CHAIN_HEAD + vc_hop_slots(S);
+        out.chain_items = h[2];
+        HIP_TRY(items.reserve(sizeof(int64_t) * (size_t)out.chain_stride * (size_t)std::max<int64_t>(out.chain_items, 1)));
+        HIP_TRY(c->hop_src.reserve(sizeof(int64_t) * PP));
+        HIP_TRY(c->hop_dst.reserve(sizeof(int64_t) * PP * (size_t)vc_hop_slots(S)));
+        HIP_TRY(vc_launch_chain_plan(S, c->launches.as<VcLaunchInfo>(), nl, T, c->slot_off.as<int64_t>(), c->row_base.as<int64_t>(),
+                                     c->chain_row_base.as<int64_t>(), c->hop_src.as<int64_t>(), c->hop_dst.as<int64_t>(),
+                                     items.as<int64_t>(), st));
+        if (c->timing) HIP_TRY(hipEventRecord(c->events[1], st));
+        return VC_OK;
+    }
     HIP_TRY(items.reserve(sizeof(VcDesc) * (size_t)std::max<int64_t>(nitems, 1)));
     HIP_TRY(vc_launch_plan_emit(S, c->launches.as<VcLaunchInfo>(), nl, T, c->slot_off.as<int64_t>(), c->row_base.as<int64_t>(),
                                 c->item_row_base.as<int64_t>(), c->header.as<int64_t>(), items.as<VcDesc>(), st));
@@ -245,21 +276,34 @@ static int build_plan(vc_comm *c, VcSched S, std::vector<VcLaunchInfo> &L, VcTab
 // Steps 4-5: one copy kernel per launch, then the blocking synchronisation.  `planned_now` says whether events 0 and 1
 // (the planner's) belong to this call.
 // Only the launches: no allocation, no synchronisation, no host-side bookkeeping (safe under stream capture).
-static int launch_items(vc_comm *c, const PlanInfo &pi, const VcDesc *items, const char *sendbuf, char *recvbuf) {
+static int launch_items(vc_comm *c, const PlanInfo &pi, const void *items_any, const char *sendbuf, char *recvbuf) {
     if (c->stage.cap < (size_t)pi.stage_bytes + 64) return fail_arg("staging arena smaller than the plan needs");
+    if (pi.chain) {
+        HIP_TRY(vc_launch_copy_chains(static_cast<const int64_t *>(items_any), pi.chain_stride, pi.chain_items, sendbuf, recvbuf,
+                                      c->stage.as<char>(), c->stream));
+        return VC_OK;
+    }
+    const VcDesc *items = static_cast<const VcDesc *>(items_any);
     for (int k = 0; k < pi.nl; k++)
         HIP_TRY(vc_launch_copy_items(items + pi.first[k], pi.count[k], sendbuf, recvbuf, c->stage.as<char>(), c->stream));
     return VC_OK;
 }
 
-static int run_items(vc_comm *c, const PlanInfo &pi, const VcDesc *items, const char *sendbuf, char *recvbuf, bool planned_now) {
+static int run_items(vc_comm *c, const PlanInfo &pi, const void *items_any, const char *sendbuf, char *recvbuf, bool planned_now) {
     hipStream_t st = c->stream;
-    const int nl = pi.nl;
+    const int nl = pi.chain ? 1 : pi.nl;              // kernel launches of this execution
+    const VcDesc *items = static_cast<const VcDesc *>(items_any);
     HIP_TRY(c->stage.reserve((size_t)pi.stage_bytes + 64));
     if (c->timing) { int rc = ensure_events(c, (size_t)nl + 4); if (rc) return rc; }
-    for (int k = 0; k < nl; k++) {
-        if (c->timing) HIP_TRY(hipEventRecord(c->events[2 + k], st));
-        HIP_TRY(vc_launch_copy_items(items + pi.first[k], pi.count[k], sendbuf, recvbuf, c->stage.as<char>(), st));
+    if (pi.chain) {
+        if (c->timing) HIP_TRY(hipEventRecord(c->events[2], st));
+        int rc = launch_items(c, pi, items_any, sendbuf, recvbuf);
+        if (rc) return rc;
+    } else {
+        for (int k = 0; k < nl; k++) {
+            if (c->timing) HIP_TRY(hipEventRecord(c->events[2 + k], st));
+            HIP_TRY(vc_launch_copy_items(items + pi.first[k], pi.count[k], sendbuf, recvbuf, c->stage.as<char>(), st));
+        }
     }
     if (c->timing) HIP_TRY(hipEventRecord(c->events[2 + nl], st));
     HIP_TRY(hipStreamSynchronize(st));
@@ -271,28 +315,35 @@ static int run_items(vc_comm *c, const PlanInfo &pi, const VcDesc *items, const 
     s.payload_bytes = pi.payload_bytes;
     s.moved_bytes = 0;
     s.plan_ms = s.total_ms = 0.f;
-    for (int k = 0; k < nl; k++) {
-        s.launch_bytes[k] = pi.bytes[k];
-        s.moved_bytes += pi.bytes[k];
-        s.launch_ms[k] = 0.f;
-        c->launch_first[k] = pi.first[k];
-        c->launch_items[k] = pi.count[k];
-        if (c->timing) HIP_TRY(hipEventElapsedTime(&s.launch_ms[k], c->events[2 + k], c->events[3 + k]));
+    if (pi.chain) {                                   // one launch that performs the hops of every digit
+        for (int k = 0; k < pi.nl; k++) s.moved_bytes += pi.bytes[k];
+        s.launch_bytes[0] = s.moved_bytes;
+        s.launch_ms[0] = 0.f;
+        if (c->timing) HIP_TRY(hipEventElapsedTime(&s.launch_ms[0], c->events[2], c->events[3]));
+    } else {
+        for (int k = 0; k < nl; k++) {
+            s.launch_bytes[k] = pi.bytes[k];
+            s.moved_bytes += pi.bytes[k];
+            s.launch_ms[k] = 0.f;
+            c->launch_first[k] = pi.first[k];
+            c->launch_items[k] = pi.count[k];
+            if (c->timing) HIP_TRY(hipEventElapsedTime(&s.launch_ms[k], c->events[2 + k], c->events[3 + k]));
+        }
     }
     if (c->timing) {
         if (planned_now) HIP_TRY(hipEventElapsedTime(&s.plan_ms, c->events[0], c->events[1]));
         HIP_TRY(hipEventElapsedTime(&s.total_ms, c->events[planned_now ? 0 : 2], c->events[2 + nl]));
     }
-    c->last_nlaunch = nl;
+    c->last_nlaunch = pi.chain ? 0 : nl;              // per-launch traffic can only be inspected after launch-per-digit execution
     c->last_items = items;
     return VC_OK;
 }
 
 static int run_schedule(vc_comm *c, VcSched S, std::vector<VcLaunchInfo> &L, const char *sendbuf, char *recvbuf, VcTables T) {
     PlanInfo pi;
-    int rc = build_plan(c, S, L, T, c->desc, pi);
+    int rc = build_plan(c, S, L, T, c->desc, pi, c->forward);
     if (rc) return rc;
-    return run_items(c, pi, c->desc.as<VcDesc>(), sendbuf, recvbuf, true);
+    return run_items(c, pi, c->desc.p, sendbuf, recvbuf, true);
 }
 
 static int check_common(vc_comm *c, const void *sendbuf, const void *recvbuf, int esz) {
@@ -327,7 +378,7 @@ static int run_v(VcFunc f, int n, int r, int batch, vc_comm *c, char *sendbuf, i
     if (!sendcounts || !sdispls || !recvcounts || (f != VC_F_TTPL && !rdispls)) return fail_arg("null table");
     VcSched S;
     std::vector<VcLaunchInfo> L;
-    rc = vc_make_schedule(f, c->P, n, r, batch, esz, 0, S, L, batch2);
+    rc = vc_make_schedule(f, c->P, n, r, batch, esz, 0, S, L, batch2, c->forward);
     if (rc) return schedule_error(rc);
     S.recv_lo = (int)((uintptr_t)recvbuf & 4095);
     return run_schedule(c, S, L, sendbuf, recvbuf, make_tables(c, sendcounts, sdispls, recvcounts, rdispls));
@@ -430,7 +481,7 @@ static int run_uniform(VcFunc f, int n, int r, vc_comm *c, char *sendbuf, int se
     if ((int64_t)sendcount * c->P > 0x7FFFFFFF) return fail_arg("sendcount * P must fit the reference's int displacements");
     VcSched S;
     std::vector<VcLaunchInfo> L;
-    rc = vc_make_schedule(f, c->P, n, r, 0, esz, sendcount, S, L);
+    rc = vc_make_schedule(f, c->P, n, r, 0, esz, sendcount, S, L, 0, c->forward);
     if (rc) return schedule_error(rc);
     S.recv_lo = (int)((uintptr_t)recvbuf & 4095);
     const size_t PP = (size_t)c->P * c->P;
@@ -483,12 +534,12 @@ extern "C" int vc_plan_create(const char *function, int n, int r, int batch, int
     if (!sendcounts || !sdispls || !recvcounts || (f != VC_F_TTPL && !rdispls)) return fail_arg("null table");
     VcSched S;
     std::vector<VcLaunchInfo> L;
-    int rc = vc_make_schedule(f, c->P, n, r, batch, elem_size, 0, S, L);
+    int rc = vc_make_schedule(f, c->P, n, r, batch, elem_size, 0, S, L, 0, c->forward);
     if (rc) return schedule_error(rc);
     S.recv_lo = recvbuf_low_bits & 4095;
     vc_plan *p = new vc_plan();
     p->comm = c;
-    rc = build_plan(c, S, L, make_tables(c, sendcounts, sdispls, recvcounts, rdispls), p->items, p->info);
+    rc = build_plan(c, S, L, make_tables(c, sendcounts, sdispls, recvcounts, rdispls), p->items, p->info, c->forward);
     if (rc == VC_OK && hipStreamSynchronize(c->stream) != hipSuccess) rc = fail_arg("vc_plan_create: stream error", VC_ERR_HIP);
     if (rc == VC_OK && c->stage.reserve((size_t)p->info.stage_bytes + 64) != hipSuccess)       // so that executing never allocates
         rc = fail_arg("vc_plan_create: cannot allocate the staging arena", VC_ERR_HIP);
@@ -501,14 +552,14 @@ extern "C" int vc_plan_execute(vc_plan_t p, char *sendbuf, char *recvbuf) {
     if (!p || !sendbuf || !recvbuf) return fail_arg("vc_plan_execute: null argument");
     if ((int)((uintptr_t)recvbuf & (VC_LINE - 1)) != (p->info.recv_lo & (VC_LINE - 1)))
         return fail_arg("vc_plan_execute: recvbuf must have the low address bits the plan was made for");
-    return run_items(p->comm, p->info, p->items.as<VcDesc>(), sendbuf, recvbuf, false);
+    return run_items(p->comm, p->info, p->items.p, sendbuf, recvbuf, false);
 }
 
 extern "C" int vc_plan_execute_async(vc_plan_t p, char *sendbuf, char *recvbuf) {
     if (!p || !sendbuf || !recvbuf) return fail_arg("vc_plan_execute_async: null argument");
     if ((int)((uintptr_t)recvbuf & (VC_LINE - 1)) != (p->info.recv_lo & (VC_LINE - 1)))
         return fail_arg("vc_plan_execute_async: recvbuf must have the low address bits the plan was made for");
-    return launch_items(p->comm, p->info, p->items.as<VcDesc>(), sendbuf, recvbuf);
+    return launch_items(p->comm, p->info, p->items.p, sendbuf, recvbuf);
 }
 
 extern "C" int vc_plan_free(vc_plan_t p) {
@@ -568,7 +619,8 @@ extern "C" int vc_suggest_radix(const int *sendcounts, int elem_size, int n, con
 
 extern "C" int vc_comm_last_traffic(vc_comm_t c, int launch, int64_t *matrix_out) {
     if (!c || !matrix_out) return fail_arg("vc_comm_last_traffic: null argument");
-    if (launch < 0 || launch >= c->last_nlaunch) return fail_arg("vc_comm_last_traffic: no such launch");
+    if (launch < 0 || launch >= c->last_nlaunch)
+        return fail_arg("vc_comm_last_traffic: no such launch (forwarded execution has no per-digit launches to inspect)");
     const size_t PP = (size_t)c->P * c->P;
     HIP_TRY(c->scratch.reserve(sizeof(int64_t) * PP));
     HIP_TRY(hipMemsetAsync(c->scratch.p, 0, sizeof(int64_t) * PP, c->stream));

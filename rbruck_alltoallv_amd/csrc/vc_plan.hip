@@ -16,15 +16,23 @@
 #include "vc_plan_math.h"
 
 // ---- pass 1: row-wise prefix sums ----
-// grid (P, w + w2 + nl).  Rows y < w + w2: staging sizes of region y, slot_off[(y*P + to)*P + id] = offset of the
+// grid (P, w + w2 + nl [+ 1]).  Rows y < w + w2: staging sizes of region y, slot_off[(y*P + to)*P + id] = offset of the
 // slot inside the row.  Later rows: work-item count, moved bytes (and, for the first launch, payload)
-// of launch y - w - w2.
+// of launch y - w - w2.  One more row with chain_row_tot: the chain items of forwarded execution.
 __global__ __launch_bounds__(VC_THREADS) void vc_plan_rows(VcSched S, const VcLaunchInfo *__restrict__ launches, int nl, VcTables T,
                                                            int64_t *__restrict__ slot_off, int64_t *__restrict__ row_tot,
-                                                           int64_t *__restrict__ item_row_tot, int64_t *__restrict__ row_bytes) {
+                                                           int64_t *__restrict__ item_row_tot, int64_t *__restrict__ row_bytes,
+                                                           int64_t *__restrict__ chain_row_tot) {
     __shared__ int64_t lds[VC_WAVES_PER_BLOCK];
     const int to = blockIdx.x, P = S.P;
     const int nreg = S.w + S.w2;                          // the organized region is laid out by vc_plan_org_rows
+    if ((int)blockIdx.y == nreg + nl) {                   // forwarded execution: chain items whose last hop ends on this rank
+        int64_t items = 0;
+        for (int s = threadIdx.x; s < P; s += VC_THREADS) items += vc_chain_count(S, T, s, to);
+        items = vc_block_sum(items, lds);
+        if (threadIdx.x == 0) chain_row_tot[to] = items;
+        return;
+    }
     if ((int)blockIdx.y < nreg) {
         const int y = blockIdx.y;
         int64_t carry = 0;
@@ -85,15 +93,30 @@ __global__ __launch_bounds__(VC_THREADS) void vc_plan_org_rows(VcSched S, VcTabl
 }
 
 // ---- pass 2: prefix sums over the rows ----
-// grid (nl + 1).  Workgroup L < nl: item bases of launch L's rows (relative to the launch's first item), its item
-// count and moved bytes.  Workgroup nl: staging row bases, staging bytes, payload bytes.
+// grid (nl + 1 [+ 1]).  Workgroup L < nl: item bases of launch L's rows (relative to the launch's first item), its item
+// count and moved bytes.  Workgroup nl: staging row bases, staging bytes, payload bytes.  Workgroup nl + 1: chain item bases.
 __global__ __launch_bounds__(VC_THREADS) void vc_plan_bases(int P, int w, int nl, const int64_t *__restrict__ row_tot,
                                                             int64_t *__restrict__ row_base, const int64_t *__restrict__ item_row_tot,
                                                             int64_t *__restrict__ item_row_base, const int64_t *__restrict__ row_bytes,
+                                                            const int64_t *__restrict__ chain_row_tot, int64_t *__restrict__ chain_row_base,
                                                             int64_t *__restrict__ header, int64_t *__restrict__ header_host) {
     __shared__ int64_t lds[VC_WAVES_PER_BLOCK];
     const int L = blockIdx.x;
     int64_t carry = 0, bytes = 0;
+    if (L == nl + 1) {                                    // forwarded execution: first chain item of every final receiver
+        for (int b0 = 0; b0 < P; b0 += VC_THREADS) {
+            const int i = b0 + threadIdx.x;
+            int64_t total;
+            const int64_t ex = vc_block_exclusive_scan((i < P) ? chain_row_tot[i] : 0, lds, total);
+            if (i < P) chain_row_base[i] = carry + ex;
+            carry += total;
+        }
+        if (threadIdx.x == 0) {
+            header[2] = carry;
+            if (header_host) header_host[2] = carry;
+        }
+        return;
+    }
     if (L == nl) {
         const int64_t nrows = (int64_t)w * P;                 // w = number of staging regions
         for (int64_t b0 = 0; b0 < nrows; b0 += VC_THREADS) {
@@ -184,13 +207,15 @@ __global__ __launch_bounds__(VC_THREADS) void vc_plan_emit(VcSched S, const VcLa
 
 hipError_t vc_launch_plan_sizes(const VcSched &S, const VcLaunchInfo *launches_dev, int nlaunch, VcTables T, int64_t *slot_off,
                                 int64_t *row_tot, int64_t *row_base, int64_t *org_run_base, int64_t *item_row_tot,
-                                int64_t *item_row_base, int64_t *row_bytes, int64_t *header, int64_t *header_host, hipStream_t st) {
-    hipLaunchKernelGGL(vc_plan_rows, dim3(S.P, S.w + S.w2 + nlaunch), dim3(VC_THREADS), 0, st, S, launches_dev, nlaunch, T, slot_off, row_tot,
-                       item_row_tot, row_bytes);
+                                int64_t *item_row_base, int64_t *row_bytes, int64_t *chain_row_tot, int64_t *chain_row_base,
+                                int64_t *header, int64_t *header_host, hipStream_t st) {
+    const int chain = chain_row_tot ? 1 : 0;
+    hipLaunchKernelGGL(vc_plan_rows, dim3(S.P, S.w + S.w2 + nlaunch + chain), dim3(VC_THREADS), 0, st, S, launches_dev, nlaunch, T, slot_off,
+                       row_tot, item_row_tot, row_bytes, chain_row_tot);
     if (S.coalesce)
         hipLaunchKernelGGL(vc_plan_org_rows, dim3(S.P), dim3(VC_THREADS), 0, st, S, T, slot_off, row_tot, org_run_base);
-    hipLaunchKernelGGL(vc_plan_bases, dim3(nlaunch + 1), dim3(VC_THREADS), 0, st, S.P, vc_regions(S), nlaunch, row_tot, row_base, item_row_tot,
-                       item_row_base, row_bytes, header, header_host);
+    hipLaunchKernelGGL(vc_plan_bases, dim3(nlaunch + 1 + chain), dim3(VC_THREADS), 0, st, S.P, vc_regions(S), nlaunch, row_tot, row_base,
+                       item_row_tot, item_row_base, row_bytes, chain_row_tot, chain_row_base, header, header_host);
     return hipGetLastError();
 }
 
@@ -199,6 +224,78 @@ hipError_t vc_launch_plan_emit(const VcSched &S, const VcLaunchInfo *launches_de
                                hipStream_t st) {
     hipLaunchKernelGGL(vc_plan_emit, dim3(S.P, nlaunch), dim3(VC_THREADS), 0, st, S, launches_dev, T, slot_off, row_base, item_row_base,
                        header, nlaunch, items);
+    return hipGetLastError();
+}
+
+// ---- forwarded execution ----
+// grid (P, nl): every entry of every launch leaves the destination of its hop (and, for a block's first hop, its
+// source in sendbuf) in the per-block hop tables.
+__global__ __launch_bounds__(VC_THREADS) void vc_chain_hops(VcSched S, const VcLaunchInfo *__restrict__ launches, VcTables T,
+                                                            const int64_t *__restrict__ slot_off, const int64_t *__restrict__ row_base,
+                                                            int64_t *__restrict__ hop_src, int64_t *__restrict__ hop_dst) {
+    const int to = blockIdx.x, P = S.P;
+    const VcLaunchInfo info = launches[blockIdx.y];
+    const int nent = vc_entries_per_rank(S, info);
+    for (int id = threadIdx.x; id < nent; id += VC_THREADS) {
+        VcEntry e;
+        if (!vc_entry_block(S, info, to, id, e)) continue;
+        const VcDesc d = vc_entry_desc(S, T, slot_off, row_base, e, to);
+        const int64_t key = (int64_t)e.t * P + e.s;
+        hop_dst[(int64_t)vc_hop_slot(S, info, e) * P * P + key] = d.dst;
+        if (e.xprev < 0) hop_src[key] = d.src;
+    }
+}
+
+__global__ __launch_bounds__(VC_THREADS) void vc_fill64_kernel(int64_t *__restrict__ p, int64_t n, int64_t value) {
+    const int64_t i = (int64_t)blockIdx.x * VC_THREADS + threadIdx.x;
+    if (i < n) p[i] = value;
+}
+
+// grid (P): the chain items of the blocks that end on rank t, in source order; big blocks are written by the whole
+// workgroup as in vc_plan_emit.
+__global__ __launch_bounds__(VC_THREADS) void vc_chain_emit(VcSched S, VcTables T, const int64_t *__restrict__ chain_row_base,
+                                                            const int64_t *__restrict__ hop_src, const int64_t *__restrict__ hop_dst,
+                                                            int64_t *__restrict__ items) {
+    __shared__ int64_t lds[VC_WAVES_PER_BLOCK];
+    __shared__ int64_t big_at[VC_THREADS], big_pre[VC_THREADS];
+    const int t = blockIdx.x, P = S.P;
+    const int stride = VC_CHAIN_HEAD + vc_hop_slots(S);
+    int64_t carry = chain_row_base[t];
+    for (int base = 0; base < P; base += VC_THREADS) {
+        const int s = base + threadIdx.x;
+        const int64_t cnt = s < P ? vc_chain_count(S, T, s, t) : 0;
+        int64_t total;
+        const int64_t at = carry + vc_block_exclusive_scan(cnt, lds, total);
+        const bool big = cnt > 4;
+        if (!big)
+            for (int64_t c = 0; c < cnt; c++) vc_chain_item(S, T, hop_src, hop_dst, s, t, c, items + (at + c) * stride);
+        else big_at[threadIdx.x] = at;
+        if (__syncthreads_or(big)) {
+            int64_t btotal;
+            big_pre[threadIdx.x] = vc_block_exclusive_scan(big ? cnt : 0, lds, btotal);
+            __syncthreads();
+            for (int64_t q = threadIdx.x; q < btotal; q += VC_THREADS) {
+                int lo = 0, hi = VC_THREADS - 1;              // last lane whose pieces start at or before q
+                while (lo < hi) {
+                    const int mid = (lo + hi + 1) >> 1;
+                    if (big_pre[mid] <= q) lo = mid; else hi = mid - 1;
+                }
+                const int64_t c = q - big_pre[lo];
+                vc_chain_item(S, T, hop_src, hop_dst, base + lo, t, c, items + (big_at[lo] + c) * stride);
+            }
+            __syncthreads();
+        }
+        carry += total;
+    }
+}
+
+hipError_t vc_launch_chain_plan(const VcSched &S, const VcLaunchInfo *launches_dev, int nlaunch, VcTables T, const int64_t *slot_off,
+                                const int64_t *row_base, const int64_t *chain_row_base, int64_t *hop_src, int64_t *hop_dst,
+                                int64_t *items, hipStream_t st) {
+    const int64_t n = (int64_t)vc_hop_slots(S) * S.P * S.P;
+    hipLaunchKernelGGL(vc_fill64_kernel, dim3((unsigned)((n + VC_THREADS - 1) / VC_THREADS)), dim3(VC_THREADS), 0, st, hop_dst, n, (int64_t)-1);
+    hipLaunchKernelGGL(vc_chain_hops, dim3(S.P, nlaunch), dim3(VC_THREADS), 0, st, S, launches_dev, T, slot_off, row_base, hop_src, hop_dst);
+    hipLaunchKernelGGL(vc_chain_emit, dim3(S.P), dim3(VC_THREADS), 0, st, S, T, chain_row_base, hop_src, hop_dst, items);
     return hipGetLastError();
 }
 

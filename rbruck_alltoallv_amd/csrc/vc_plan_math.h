@@ -312,3 +312,58 @@ VC_HD VcDesc vc_chunk_of(const VcDesc &whole, int64_t c, int phase, int cut) {
     d.src += lo; d.dst += lo; d.len = hi - lo;
     return d;
 }
+
+// ---- forwarded execution: one work item carries a piece of a block through all its hops ----
+// The hops of one block depend only on each other: hop k + 1 reads what hop k wrote.  When one workgroup performs all
+// of them it keeps the piece in registers between the hops: the data is read once (from sendbuf) and written once per
+// hop (to the staging slot of every intermediate holder, then to recvbuf).  Memory ends up exactly as after the
+// launch-per-digit execution.
+//
+// A block moves at most once per digit, so its hops are indexed by "hop slots": intra-node digit x, inter-node digit
+// S.w + x, and one last slot for what goes straight to recvbuf by an inter-node or direct message (or stays on its rank).
+#define VC_MAX_HOP_SLOTS 32
+
+VC_HD int vc_hop_slots(const VcSched &S) { return S.w + S.w2 + 1; }
+
+VC_HD int vc_hop_slot(const VcSched &S, const VcLaunchInfo &info, const VcEntry &e) {
+    if (e.s == e.t) return S.w + S.w2;
+    return info.kind == 0 ? info.x : (info.kind == 4 ? S.w + info.x : S.w + S.w2);
+}
+
+// All hops of a block cut it at the same places: where its image in recvbuf crosses a multiple of VC_PIECE.
+VC_HD int vc_chain_cut(const VcSched &S, const VcTables &T, int s, int t) {
+    return (int)((vc_recv_offset(S, T, s, t) + S.recv_lo) & (VC_PIECE - 1));
+}
+
+VC_HD int64_t vc_chain_count(const VcSched &S, const VcTables &T, int s, int t) {
+    const int64_t len = (int64_t)T.sc[(int64_t)s * S.P + t] * S.esz;
+    return vc_chunk_count(len, vc_phase(S, T, s, t), vc_chain_cut(S, T, s, t));
+}
+
+// Layout of a chain item, in int64 words; `stride` = VC_CHAIN_HEAD + hop slots of the call.
+#define VC_CHAIN_SRC 0    // space-tagged source offset of the piece (always in sendbuf)
+#define VC_CHAIN_LEN 1
+#define VC_CHAIN_NHOP 2
+#define VC_CHAIN_HEAD 3   // followed by the space-tagged destination of the piece at every hop
+
+// Writes piece c of block (s, t) to `item`.  hop_src[key] and hop_dst[slot * P * P + key] (key = t * P + s) hold the
+// whole block's source and its destination per hop slot (-1: does not move in that slot).
+VC_HD void vc_chain_item(const VcSched &S, const VcTables &T, const int64_t *hop_src, const int64_t *hop_dst, int s, int t, int64_t c,
+                         int64_t *item) {
+    const int64_t PP = (int64_t)S.P * S.P, key = (int64_t)t * S.P + s;
+    const int64_t len = (int64_t)T.sc[(int64_t)s * S.P + t] * S.esz;
+    const int phase = vc_phase(S, T, s, t), cut = vc_chain_cut(S, T, s, t);
+    VcDesc whole;
+    whole.src = hop_src[key]; whole.dst = 0; whole.len = len; whole.from = s; whole.to = t;
+    const VcDesc piece = vc_chunk_of(whole, c, phase, cut);
+    const int64_t lo = piece.dst;                      // offset of the piece inside the block
+    item[VC_CHAIN_SRC] = piece.src;
+    item[VC_CHAIN_LEN] = piece.len;
+    int nhop = 0;
+    const int nslots = vc_hop_slots(S);
+    for (int k = 0; k < nslots; k++) {
+        const int64_t d = hop_dst[(int64_t)k * PP + key];
+        if (d >= 0) item[VC_CHAIN_HEAD + nhop++] = d + lo;
+    }
+    item[VC_CHAIN_NHOP] = nhop;
+}

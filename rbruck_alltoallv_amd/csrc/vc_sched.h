@@ -112,9 +112,10 @@ inline void vc_add_scoped_direct_launches(std::vector<VcLaunchInfo> &out, int sc
 
 // Fills S and L for function f.  `r`, `batch` (b of tuna_algorithm, bblock of the TTPL functions; with batch2 the two
 // bblocks of twolayer_communicator_linear_s2) and `n`
-// are the caller's raw values.  Returns VC_OK or the code the entry point must return.
+// are the caller's raw values; `forward`: the schedule is for forwarded execution (one work item per block piece
+// through all hops).  Returns VC_OK or the code the entry point must return.
 inline int vc_make_schedule(VcFunc f, int P, int n, int r, int batch, int esz, int uniform_count, VcSched &S,
-                            std::vector<VcLaunchInfo> &L, int batch2 = 0) {
+                            std::vector<VcLaunchInfo> &L, int batch2 = 0, bool forward = false) {
     memset(&S, 0, sizeof S);
     L.clear();
     S.P = P; S.esz = esz; S.uniform = uniform_count;
@@ -154,8 +155,9 @@ inline int vc_make_schedule(VcFunc f, int P, int n, int r, int batch, int esz, i
             const int groups = (batch <= 0 || batch > S.G) ? S.G : batch;                      // :421
             const size_t first_inter = L.size();
             vc_add_inter_launches(L, S, groups * n);
-            // coalesced messages need the organized region, which the intra-node launches fill
-            if (S.w > 0 && S.G > 1) {
+            // coalesced messages need the organized region, which the intra-node launches fill; forwarded execution
+            // carries every block on its own and keeps the per-block inter-node messages
+            if (S.w > 0 && S.G > 1 && !forward) {
                 S.coalesce = 1;
                 for (size_t k = first_inter; k < L.size(); k++) L[k].kind = 3;
             }

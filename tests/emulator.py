@@ -41,7 +41,7 @@ class Result:
         self.traffic = traffic[: self.nlaunch] if rc == 0 else None
 
 
-def emulate(func, prob, send, recv, n=0, r=2, batch=0, uniform_count=0, recv_lo=0, batch2=0) -> Result:
+def emulate(func, prob, send, recv, n=0, r=2, batch=0, uniform_count=0, recv_lo=0, batch2=0, forward=None) -> Result:
     global _lib
     if _lib is None:
         _lib = C.CDLL(build())
@@ -51,12 +51,15 @@ def emulate(func, prob, send, recv, n=0, r=2, batch=0, uniform_count=0, recv_lo=
     rc = _lib.plan_emulate(C.c_int(func), C.c_int(P), C.c_int(n), C.c_int(r), C.c_int(batch), C.c_int(prob.esz),
                            C.c_int(uniform_count), _p(send), C.c_int64(send.size), _p(recv), C.c_int64(recv.size),
                            _p(prob.sbase), _p(prob.rbase), _p(prob.sendcounts), _p(prob.sdispls), _p(prob.recvcounts),
-                           _p(prob.rdispls), C.c_int(recv_lo), _p(stats), _p(traffic), C.c_int(MAX_LAUNCHES), C.c_int(batch2))
+                           _p(prob.rdispls), C.c_int(recv_lo), _p(stats), _p(traffic), C.c_int(MAX_LAUNCHES), C.c_int(batch2),
+                           C.c_int(int(FORWARD if forward is None else forward)))
     return Result(rc, stats, traffic)
 
 
 # the reference's names, returning the return code and remembering the last Result
 last = None
+# module-wide switch: emulate forwarded execution (and check it against the launch-per-digit execution)
+FORWARD = False
 
 
 def _run(*a, **k):

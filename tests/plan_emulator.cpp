@@ -35,10 +35,10 @@ static int count_overlaps(std::vector<Range> &dst, std::vector<Range> &src) {
 extern "C" int plan_emulate(int func, int P, int n, int r, int batch, int esz, int uniform_count, const char *send,
                             int64_t send_bytes, char *recv, int64_t recv_bytes, const int64_t *sbase, const int64_t *rbase,
                             const int *sc, const int *sd, const int *rc, const int *rd, int recv_lo, int64_t *stats_out,
-                            int64_t *traffic_out, int max_launches, int batch2) {
+                            int64_t *traffic_out, int max_launches, int batch2, int forward) {
     VcSched S;
     std::vector<VcLaunchInfo> L;
-    int code = vc_make_schedule((VcFunc)func, P, n, r, batch, esz, uniform_count, S, L, batch2);
+    int code = vc_make_schedule((VcFunc)func, P, n, r, batch, esz, uniform_count, S, L, batch2, forward != 0);
     if (code) return code;
     S.recv_lo = recv_lo;
     const int64_t PP = (int64_t)P * P;
@@ -86,6 +86,11 @@ extern "C" int plan_emulate(int func, int P, int n, int r, int batch, int esz, i
         }
     std::vector<char> stage((size_t)stage_bytes + 64, (char)0xCD);
     std::vector<char> written((size_t)stage_bytes + 64, 0);
+    // forwarded execution is checked against the launch-per-digit execution of the same schedule: that one runs first,
+    // into copies of the arenas
+    char *const recv_final = recv;
+    std::vector<char> recv_steps;
+    if (forward) { recv_steps.assign(recv, recv + recv_bytes); recv = recv_steps.data(); }
 
     int64_t errors = 0, moved = 0, items = 0;
     const int nl = (int)L.size();
@@ -140,6 +145,74 @@ extern "C" int plan_emulate(int func, int P, int n, int r, int batch, int esz, i
             if (dspace == 2) memset(written.data() + (d.dst & VC_OFFSET_MASK), 1, (size_t)d.len);
             moved += d.len;
         }
+    }
+    if (forward) {
+        const int nslots = vc_hop_slots(S), stride = VC_CHAIN_HEAD + nslots;
+        if (nslots > VC_MAX_HOP_SLOTS) errors++;
+        std::vector<int64_t> hop_src(PP, -1), hop_dst((size_t)nslots * PP, -1);
+        for (int k = 0; k < nl; k++) {                    // vc_chain_hops
+            const int nent = vc_entries_per_rank(S, L[k]);
+            for (int to = 0; to < P; to++)
+                for (int id = 0; id < nent; id++) {
+                    VcEntry e;
+                    if (!vc_entry_block(S, L[k], to, id, e)) continue;
+                    if (e.nblk != 1) { errors++; continue; }
+                    const VcDesc d = vc_entry_desc(S, T, slot_off.data(), row_base.data(), e, to);
+                    const int64_t key = (int64_t)e.t * P + e.s;
+                    int64_t &cell = hop_dst[(int64_t)vc_hop_slot(S, L[k], e) * PP + key];
+                    if (cell != -1) errors++;             // a block moves at most once per hop slot
+                    cell = d.dst;
+                    if (e.xprev < 0) { if (hop_src[key] != -1) errors++; hop_src[key] = d.src; }
+                }
+        }
+        std::vector<char> stage2((size_t)stage_bytes + 64, (char)0xCD);
+        std::vector<Range> dst_ranges, none;
+        std::vector<int64_t> item(stride);
+        int64_t chain_items = 0, chain_moved = 0;
+        for (int t = 0; t < P; t++)                       // vc_chain_emit + vc_copy_chains_kernel
+            for (int s0 = 0; s0 < P; s0++) {
+                const int64_t len = (int64_t)T.sc[(int64_t)s0 * P + t] * esz;
+                const int64_t cnt = vc_chain_count(S, T, s0, t);
+                if ((len > 0) != (cnt > 0)) errors++;
+                if (len > 0 && hop_src[(int64_t)t * P + s0] < 0) { errors++; continue; }
+                int64_t covered = 0;
+                for (int64_t c = 0; c < cnt; c++) {
+                    vc_chain_item(S, T, hop_src.data(), hop_dst.data(), s0, t, c, item.data());
+                    const int64_t src = item[VC_CHAIN_SRC], plen = item[VC_CHAIN_LEN], nhop = item[VC_CHAIN_NHOP];
+                    chain_items++;
+                    if ((int)(src >> VC_SPACE_SHIFT) != 0 || plen <= 0 || nhop < 1) { errors++; continue; }
+                    const int64_t so = src & VC_OFFSET_MASK;
+                    if (so + plen > send_bytes) { errors++; continue; }
+                    if (so - (hop_src[(int64_t)t * P + s0] & VC_OFFSET_MASK) != covered) errors++;
+                    int line = -1;
+                    bool reaches_recv = false;
+                    for (int64_t k = 0; k < nhop; k++) {
+                        const int64_t d = item[VC_CHAIN_HEAD + k];
+                        const int dspace = (int)(d >> VC_SPACE_SHIFT);
+                        const int64_t dof = d & VC_OFFSET_MASK;
+                        const int64_t dlim = dspace == 1 ? recv_bytes : (dspace == 2 ? stage_bytes : -1);
+                        if (dof < 0 || dof + plen > dlim) { errors++; continue; }
+                        const int ph = (int)((dof + (dspace == 1 ? recv_lo : 0)) & (VC_LINE - 1));
+                        if (line >= 0 && ph != line) errors++;        // one lane mapping serves every hop
+                        line = ph;
+                        if (plen + ph > VC_CHUNK) errors++;
+                        if (c > 0 && ph != 0) errors++;
+                        dst_ranges.push_back({dof, dof + plen, dspace});
+                        memcpy((dspace == 1 ? recv_final : stage2.data()) + dof, send + so, (size_t)plen);
+                        chain_moved += plen;
+                        reaches_recv |= dspace == 1;
+                    }
+                    if (!reaches_recv) errors++;
+                    covered += plen;
+                }
+                if (covered != len) errors++;
+            }
+        errors += count_overlaps(dst_ranges, none);
+        // same memory as after the launch-per-digit execution
+        if (chain_moved != moved) errors++;
+        if (memcmp(stage.data(), stage2.data(), (size_t)stage_bytes) != 0) errors++;
+        if (memcmp(recv_steps.data(), recv_final, (size_t)recv_bytes) != 0) errors++;
+        items = chain_items;
     }
     stats_out[0] = nl; stats_out[1] = stage_bytes; stats_out[2] = moved; stats_out[3] = errors; stats_out[4] = items;
     return 0;

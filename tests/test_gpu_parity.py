@@ -518,3 +518,96 @@ def test_plan_in_a_hip_graph(api):
         assert plan.execute(ds2, dr) == 0                 # and eager calls of the library in between
     plan.free()
     dp.comm.free()
+
+
+# ---- forwarded execution (vc_comm_set_forwarding): one launch, every block piece carried through all its hops ----
+
+@pytest.mark.parametrize("case", CASES, ids=[c["id"] for c in CASES])
+def test_golden_case_forwarded(api, case):
+    print("case", case["id"], flush=True)
+    prob = problem_for_case(case)
+    send = W.fill_send_arena(prob, case["payload"], case["seed"])
+    want = np.full(prob.recv_bytes, 0xEE, dtype=np.uint8)
+    assert run_on(O, case, prob, send.copy(), want) == 0
+    dp = api.DeviceProblem(prob)
+    dp.comm.set_forwarding(True)
+    dsend = _to_dev(api, send)
+    drecv = dp.new_recv_arena(0xEE)
+    rc = run_on(api, case, dp, dsend, drecv)
+    assert rc == 0, dp.comm.error()
+    got = drecv.cpu().numpy()
+    assert np.array_equal(got, want)
+    assert [f"{int(h):016x}" for h in O.digest_recv(digest_problem(case, prob), got)] == case["digests"]
+    assert np.array_equal(dsend.cpu().numpy(), send), "sendbuf must stay intact"
+    st = dp.comm.last_stats()
+    assert st.n_launches == 1
+    # same hops as the launch-per-digit execution: every hop of every block is written once
+    dp.comm.set_forwarding(False)
+    drecv2 = dp.new_recv_arena(0xEE)
+    assert run_on(api, case, dp, dsend, drecv2) == 0
+    if case["func"] != "ttpl":                       # (the coalesced variant also counts nothing more: same hops per block)
+        assert dp.comm.last_stats().moved_bytes == st.moved_bytes
+    assert st.payload_bytes == prob.payload_bytes
+    dp.comm.free()
+
+
+def test_forwarded_shapes_plans_and_graphs(api):
+    """Forwarded execution on the benchmark shapes (reduced), unaligned arenas, as a persistent plan and inside a HIP graph."""
+    import torch
+    c4 = W.counts_normal(1024, 256.0, 64.0, 0, 1024, 0)
+    c3 = W.counts_zipf(256, 4096, 1.2, 5, 0)
+    c5 = W.counts_fft_rows(512, 32, 4096)
+    for prob, calls in (
+            (W.make_problem(c4, 1, 0, 0), [("ttpl", lambda dp, s, d: api.TTPL_BT_alltoallv(32, 32, 0, dp, s, d), True),
+                                          ("s1 r=2", lambda dp, s, d: api.TTPL_BT_alltoallv_s1(32, 2, 7, dp, s, d), False),
+                                          ("ttpl_rbruck r=4", lambda dp, s, d: api.TTPL_rbruck_alltoallv(32, 4, dp, s, d), False),
+                                          ("twophase r=2", lambda dp, s, d: api.twophase_rbruck_alltoallv(2, dp, s, d), False)]),
+            (W.make_problem(c3, 4, 1, 1), [("twophase r=16", lambda dp, s, d: api.twophase_rbruck_alltoallv(16, dp, s, d), False),
+                                          ("tuna r=3 b=1", lambda dp, s, d: api.tuna_algorithm(3, 1, dp, s, d), False)]),
+            (W.make_problem(c5, 8, 0, 0), [("tuna r=32", lambda dp, s, d: api.tuna_algorithm(32, 0, dp, s, d), False),
+                                          ("spreadout", lambda dp, s, d: api.spreadout_alltoallv(dp, s, d), False)])):
+        dp = api.DeviceProblem(prob)
+        dp.comm.set_forwarding(True)
+        ds = dp.new_send_arena()
+        dp.fill_payload(0, 3, ds)
+        for name, fn, packed in calls:
+            print("  ", name, flush=True)
+            dr = dp.new_recv_arena(0xEE)
+            assert fn(dp, ds, dr) == 0, (name, dp.comm.error())
+            assert dp.verify(ds, dr, packed_recv=packed) == 0, name
+            assert dp.comm.last_stats().n_launches == 1
+        dp.comm.free()
+    # unaligned arenas, a plan, a graph
+    counts = (W.counts_uniform_random(12, 30000, seed=5) * (W.counts_uniform_random(12, 3, seed=6) > 0)).astype(np.int32)
+    prob = W.make_problem(counts, 1, 1, 0)
+    send = W.fill_send_arena(prob, 0, 9)
+    want = W.expected_recv_arena(prob, send)
+    dp = api.DeviceProblem(prob)
+    dp.comm.set_forwarding(True)
+    sbig = torch.zeros(prob.send_bytes + 64, dtype=torch.uint8, device="cuda:0")
+    ds = sbig[5:5 + prob.send_bytes]
+    ds.copy_(torch.from_numpy(send))
+    rbig = torch.full((prob.recv_bytes + 256,), 0xEE, dtype=torch.uint8, device="cuda:0")
+    dr = rbig[77:77 + prob.recv_bytes]
+    assert api.twophase_rbruck_alltoallv(3, dp, ds, dr) == 0, dp.comm.error()
+    assert np.array_equal(dr.cpu().numpy(), want)
+    assert bool((rbig[:77] == 0xEE).all()) and bool((rbig[77 + prob.recv_bytes:] == 0xEE).all())
+    plan = api.Plan("tuna_algorithm", dp, dr, r=2, batch=0)
+    assert plan.rc == 0, dp.comm.error()
+    for _ in range(3):
+        dr.fill_(0xEE)
+        assert plan.execute(ds, dr) == 0, dp.comm.error()
+        assert np.array_equal(dr.cpu().numpy(), want)
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        dp.comm.use_current_stream()
+        assert plan.execute_async(ds, dr) == 0, dp.comm.error()
+    dp.comm.use_current_stream()
+    for _ in range(3):
+        dr.fill_(0xEE)
+        torch.cuda.synchronize()
+        g.replay()
+        torch.cuda.synchronize()
+        assert np.array_equal(dr.cpu().numpy(), want)
+    plan.free()
+    dp.comm.free()

@@ -364,3 +364,83 @@ def test_unaligned_recvbuf_pointer_keeps_the_phase_rule():
             res = E.emulate(func, prob, send, recv, recv_lo=recv_lo, **kw)
             assert res.rc == 0 and res.errors == 0, (func, recv_lo, res.errors)
             assert np.array_equal(recv, want)
+
+
+# ---- forwarded execution: one work item carries a block piece through all its hops ----
+
+@pytest.fixture
+def forwarded():
+    E.FORWARD = True
+    yield
+    E.FORWARD = False
+
+
+@pytest.mark.parametrize("case", CASES, ids=[c["id"] for c in CASES])
+def test_forwarded_plan_reproduces_reference_digests(case, forwarded):
+    """The chain items write the same bytes to the same staging slots and receive buffers as the launch-per-digit
+    execution (the emulator runs both and compares the arenas), and the result has the reference's digests."""
+    prob = problem_for_case(case)
+    send = W.fill_send_arena(prob, case["payload"], case["seed"])
+    recv = np.full(prob.recv_bytes, 0xEE, dtype=np.uint8)
+    keep = send.copy()
+    assert run_on(E, case, prob, send, recv) == 0
+    assert E.last.errors == 0
+    assert [f"{int(h):016x}" for h in O.digest_recv(digest_problem(case, prob), recv)] == case["digests"]
+    assert np.array_equal(recv, W.expected_recv_arena(prob, send))
+    assert np.array_equal(send, keep)
+
+
+@pytest.mark.parametrize("P", [1, 2, 3, 5, 8, 12, 17, 27, 32, 50])
+def test_forwarded_flat_plans_all_radices(P, forwarded):
+    for layout in (0, 1):
+        prob = _prob(P, layout, 2, seed=P + 60)
+        send = W.fill_send_arena(prob, 0, 3)
+        want = W.expected_recv_arena(prob, send)
+        for r in sorted({2, 3, 4, 5, 8, P, P + 3} - {1}):
+            calls = [lambda d: E.twophase_rbruck_alltoallv(r, prob, send, d), lambda d: E.twophase_rbruck_alltoallv_om(r, prob, send, d)]
+            if P >= 3:
+                calls += [lambda d: E.tuna_algorithm(r, 2, prob, send, d), lambda d: E.tuna2_algorithm(r, 0, prob, send, d)]
+            for fn in calls:
+                recv = np.full(prob.recv_bytes, 0xEE, dtype=np.uint8)
+                assert fn(recv) == 0 and E.last.errors == 0, (P, r)
+                assert np.array_equal(recv, want)
+                # hops: the chain writes every block once per non-zero digit
+                assert E.last.moved * 2 == W.algorithmic_bytes(prob.sendcounts, prob.esz, W.hops_flat(P, min(r, P - 1) if fn in calls[2:] else min(r, P)))
+
+
+@pytest.mark.parametrize("P,n", [(4, 2), (6, 3), (8, 4), (12, 4), (16, 8), (32, 8), (8, 8), (8, 1), (27, 9), (64, 4)])
+def test_forwarded_twolayer_plans(P, n, forwarded):
+    for layout in (0, 1):
+        prob = _prob(P, layout, 1, seed=P + n, recv_layout=0)
+        send = W.fill_send_arena(prob, 0, 3)
+        want = W.expected_recv_arena(prob, send)
+        for r in sorted({2, 3, max(n, 2)}):
+            for fn in (lambda d: E.TTPL_BT_alltoallv(n, r, 3, prob, send, d), lambda d: E.TTPL_BT_alltoallv_s1(n, r, 5, prob, send, d),
+                       lambda d: E.TTPL_rbruck_alltoallv(n, r, prob, send, d)):
+                recv = np.full(prob.recv_bytes, 0xEE, dtype=np.uint8)
+                assert fn(recv) == 0 and E.last.errors == 0, (P, n, r)
+                assert np.array_equal(recv, want)
+    if 2 <= n < P:
+        up = W.make_uniform_problem(P, 7, 4)
+        us = W.fill_send_arena(up, 0, 1)
+        uw = W.expected_recv_arena(up, us)
+        for fn in (lambda d: E.uniform_spreadout_twolayer(n, 2, up, 7, us.copy(), d), lambda d: E.uniform_inverse_isplit_r_bruck(n, 3, 2, up, 7, us.copy(), d),
+                   lambda d: E.twolayer_communicator_linear_s2(n, 2, 5, up, us, d)):
+            ur = np.full(up.recv_bytes, 0xEE, dtype=np.uint8)
+            assert fn(ur) == 0 and E.last.errors == 0
+            assert np.array_equal(ur, uw)
+
+
+def test_forwarded_large_blocks_and_unaligned_recvbuf(forwarded):
+    counts = (W.counts_uniform_random(12, 30000, seed=5) * (W.counts_uniform_random(12, 3, seed=6) > 0)).astype(np.int32)
+    prob = W.make_problem(counts, 1, 1, 0)
+    send = W.fill_send_arena(prob, 0, 9)
+    want = W.expected_recv_arena(prob, send)
+    for recv_lo in (0, 5, 100, 2048 + 7, 4095):
+        for func, kw in ((E.F_TWOPHASE, dict(r=3)), (E.F_TUNA, dict(r=2, batch=1)), (E.F_TTPL, dict(n=4, r=4)),
+                         (E.F_TTPL_S1, dict(n=6, r=2, batch=5)), (E.F_TTPL_RBRUCK, dict(n=2, r=2)), (E.F_SPREADOUT, {})):
+            recv = np.full(prob.recv_bytes, 0xEE, dtype=np.uint8)
+            res = E.emulate(func, prob, send, recv, recv_lo=recv_lo, **kw)
+            assert res.rc == 0 and res.errors == 0, (func, recv_lo, res.errors)
+            assert np.array_equal(recv, want)
+            assert res.items > 12 * 12
