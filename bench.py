@@ -153,8 +153,9 @@ def main() -> None:
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="C4")
-    ap.add_argument("--forward", type=int, default=0, choices=(0, 1),
-                    help="1: forwarded execution (vc_comm_set_forwarding) is the mode that is measured; the other one is reported beside it")
+    ap.add_argument("--forward", type=int, default=1, choices=(0, 1),
+                    help="1 (the library's default): forwarded execution is the mode that is measured; 0: one launch per digit "
+                         "phase (vc_comm_set_forwarding(comm, 0)); the other one is reported beside it")
     ap.add_argument("--func", default=None, help="override the function (e.g. TTPL_BT_alltoallv_s1)")
     ap.add_argument("--radix", type=int, default=0, help="override the radix r of the workload")
     ap.add_argument("--seed", type=int, default=0)

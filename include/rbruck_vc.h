@@ -56,14 +56,16 @@ int vc_comm_set_stream(vc_comm_t comm, void *hip_stream);
 int vc_comm_set_bases(vc_comm_t comm, const int64_t *sbase_bytes, const int64_t *rbase_bytes);
 
 /* How the collectives execute (no counterpart in the reference, whose ranks are separate processes).
- * 0 (default): one kernel launch per digit phase (or per batch of its rounds); every hop reads the block where the
- *    previous hop left it.
- * 1: forwarded execution.  One launch for the whole call; the workgroup that moves a piece of a block performs all
- *    the hops of that block one after the other and keeps the piece in registers in between, so the data is read once
- *    (from sendbuf) and written once per hop (into the staging slot of every intermediate holder, then into recvbuf).
- *    Results, and the staging contents, are the same; the batching tunables (b, bblock) then have no effect, and
- *    TTPL_BT_alltoallv sends its inter-node data per block instead of coalesced.  Applies to calls and to plans
- *    created afterwards. */
+ * 1 (default): forwarded execution.  One launch for the whole call; the workgroup that moves a piece of a block performs
+ *    all the hops of that block one after the other and keeps the piece in registers in between, so the data is read
+ *    once (from sendbuf) and written once per hop (into the staging slot of every intermediate holder, then into
+ *    recvbuf).  The batching tunables (b, bblock) then have no effect, and TTPL_BT_alltoallv sends its inter-node data
+ *    per block instead of coalesced.  Calls on more than 4096 ranks fall back to mode 0 (the per-block hop table
+ *    would grow to gigabytes).
+ * 0: one kernel launch per digit phase (or per batch of its rounds, as b / bblock say); every hop reads the block
+ *    where the previous hop left it.  This is the mode whose launches vc_comm_last_stats and vc_comm_last_traffic
+ *    describe one by one.
+ * Results, and the staging contents, are the same in both.  Applies to calls and to plans created afterwards. */
 int vc_comm_set_forwarding(vc_comm_t comm, int enable);
 
 /* Text of the most recent failure on this thread ("" if none). */

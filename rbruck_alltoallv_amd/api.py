@@ -80,6 +80,11 @@ class VirtualComm:
             pass
 
 
+# None: the library's default execution mode (forwarded); True / False: every new DeviceProblem sets this mode on its
+# communicator (the tests run both)
+DEFAULT_FORWARDING = None
+
+
 class DeviceProblem:
     """Rank-major tables and arena bases of a Problem, resident in HBM, plus its communicator."""
 
@@ -95,6 +100,8 @@ class DeviceProblem:
         self.rbase = torch.from_numpy(prob.rbase).to(dev)
         self.comm = comm or VirtualComm(prob.P, device)
         self.comm.set_bases(self.sbase, self.rbase)
+        if DEFAULT_FORWARDING is not None:
+            self.comm.set_forwarding(DEFAULT_FORWARDING)
 
     def new_send_arena(self) -> torch.Tensor:
         return torch.zeros(self.host.send_bytes, dtype=torch.uint8, device=self.sbase.device)

@@ -64,7 +64,7 @@ struct vc_comm {
     hipStream_t stream = nullptr;
     const int64_t *sbase = nullptr, *rbase = nullptr;
     bool timing = false;
-    bool forward = false;                 // forwarded execution: one launch, every block piece carried through all its hops
+    bool forward = true;                  // forwarded execution: one launch, every block piece carried through all its hops
     DevBuf chain_row_tot, chain_row_base, hop_src, hop_dst;
     DevBuf slot_off, row_tot, row_base, org_run_base, item_row_tot, item_row_base, row_bytes, desc, header, launches, stage, rd_packed,
         uni_counts, uni_displs, scratch;
@@ -339,9 +339,9 @@ static int run_items(vc_comm *c, const PlanInfo &pi, const void *items_any, cons
     return VC_OK;
 }
 
-static int run_schedule(vc_comm *c, VcSched S, std::vector<VcLaunchInfo> &L, const char *sendbuf, char *recvbuf, VcTables T) {
+static int run_schedule(vc_comm *c, VcSched S, std::vector<VcLaunchInfo> &L, const char *sendbuf, char *recvbuf, VcTables T, bool forward) {
     PlanInfo pi;
-    int rc = build_plan(c, S, L, T, c->desc, pi, c->forward);
+    int rc = build_plan(c, S, L, T, c->desc, pi, forward);
     if (rc) return rc;
     return run_items(c, pi, c->desc.p, sendbuf, recvbuf, true);
 }
@@ -370,6 +370,13 @@ static int schedule_error(int code) {
     return code;
 }
 
+// Forwarded execution keeps one int64 per block and hop slot (at most 2 * log2(P) + 1 slots); beyond 4096 ranks a call
+// falls back to one launch per digit.
+static bool use_forwarding(const vc_comm *c, int P, int r_hint) {
+    (void)r_hint;
+    return c->forward && P <= 4096;
+}
+
 // The alltoallv-shaped functions.
 static int run_v(VcFunc f, int n, int r, int batch, vc_comm *c, char *sendbuf, int *sendcounts, int *sdispls, int esz,
                  char *recvbuf, int *recvcounts, int *rdispls, int batch2 = 0) {
@@ -378,10 +385,11 @@ static int run_v(VcFunc f, int n, int r, int batch, vc_comm *c, char *sendbuf, i
     if (!sendcounts || !sdispls || !recvcounts || (f != VC_F_TTPL && !rdispls)) return fail_arg("null table");
     VcSched S;
     std::vector<VcLaunchInfo> L;
-    rc = vc_make_schedule(f, c->P, n, r, batch, esz, 0, S, L, batch2, c->forward);
+    const bool forward = use_forwarding(c, c->P, r);
+    rc = vc_make_schedule(f, c->P, n, r, batch, esz, 0, S, L, batch2, forward);
     if (rc) return schedule_error(rc);
     S.recv_lo = (int)((uintptr_t)recvbuf & 4095);
-    return run_schedule(c, S, L, sendbuf, recvbuf, make_tables(c, sendcounts, sdispls, recvcounts, rdispls));
+    return run_schedule(c, S, L, sendbuf, recvbuf, make_tables(c, sendcounts, sdispls, recvcounts, rdispls), forward);
 }
 
 extern "C" int twophase_rbruck_alltoallv(int r, char *sendbuf, int *sendcounts, int *sdispls, int sendtype_size, char *recvbuf,
@@ -481,7 +489,8 @@ static int run_uniform(VcFunc f, int n, int r, vc_comm *c, char *sendbuf, int se
     if ((int64_t)sendcount * c->P > 0x7FFFFFFF) return fail_arg("sendcount * P must fit the reference's int displacements");
     VcSched S;
     std::vector<VcLaunchInfo> L;
-    rc = vc_make_schedule(f, c->P, n, r, 0, esz, sendcount, S, L, 0, c->forward);
+    const bool forward = use_forwarding(c, c->P, r);
+    rc = vc_make_schedule(f, c->P, n, r, 0, esz, sendcount, S, L, 0, forward);
     if (rc) return schedule_error(rc);
     S.recv_lo = (int)((uintptr_t)recvbuf & 4095);
     const size_t PP = (size_t)c->P * c->P;
@@ -489,7 +498,7 @@ static int run_uniform(VcFunc f, int n, int r, vc_comm *c, char *sendbuf, int se
     HIP_TRY(c->uni_displs.reserve(sizeof(int) * PP));
     HIP_TRY(vc_launch_uniform_tables(c->uni_counts.as<int>(), c->uni_displs.as<int>(), sendcount, c->P, c->stream));
     const int *cnt = c->uni_counts.as<int>(), *dsp = c->uni_displs.as<int>();
-    return run_schedule(c, S, L, sendbuf, recvbuf, make_tables(c, cnt, dsp, cnt, dsp));
+    return run_schedule(c, S, L, sendbuf, recvbuf, make_tables(c, cnt, dsp, cnt, dsp), forward);
 }
 
 extern "C" int uniform_spreadout_twolayer(int n, int r, char *sendbuf, int sendcount, int sendtype_size, char *recvbuf,
@@ -534,12 +543,13 @@ extern "C" int vc_plan_create(const char *function, int n, int r, int batch, int
     if (!sendcounts || !sdispls || !recvcounts || (f != VC_F_TTPL && !rdispls)) return fail_arg("null table");
     VcSched S;
     std::vector<VcLaunchInfo> L;
-    int rc = vc_make_schedule(f, c->P, n, r, batch, elem_size, 0, S, L, 0, c->forward);
+    const bool forward = use_forwarding(c, c->P, r);
+    int rc = vc_make_schedule(f, c->P, n, r, batch, elem_size, 0, S, L, 0, forward);
     if (rc) return schedule_error(rc);
     S.recv_lo = recvbuf_low_bits & 4095;
     vc_plan *p = new vc_plan();
     p->comm = c;
-    rc = build_plan(c, S, L, make_tables(c, sendcounts, sdispls, recvcounts, rdispls), p->items, p->info, c->forward);
+    rc = build_plan(c, S, L, make_tables(c, sendcounts, sdispls, recvcounts, rdispls), p->items, p->info, forward);
     if (rc == VC_OK && hipStreamSynchronize(c->stream) != hipSuccess) rc = fail_arg("vc_plan_create: stream error", VC_ERR_HIP);
     if (rc == VC_OK && c->stage.reserve((size_t)p->info.stage_bytes + 64) != hipSuccess)       // so that executing never allocates
         rc = fail_arg("vc_plan_create: cannot allocate the staging arena", VC_ERR_HIP);

@@ -15,12 +15,15 @@ pytestmark = pytest.mark.gpu
 CASES = load_golden()
 
 
-@pytest.fixture(scope="module")
-def api():
+@pytest.fixture(scope="module", params=["forwarded", "launch-per-digit"])
+def api(request):
+    """The package's API with one of the two execution modes set on every communicator the tests create."""
     import torch
     assert torch.cuda.is_available(), "these tests need the GPU"
     from rbruck_alltoallv_amd import api as A
-    return A
+    A.DEFAULT_FORWARDING = request.param == "forwarded"
+    yield A
+    A.DEFAULT_FORWARDING = None
 
 
 def _to_dev(api, arr):
@@ -112,6 +115,8 @@ def _oracle_traffic(rec, P, select):
 @pytest.mark.parametrize("func,P,r", [("twophase", 27, 3), ("om", 64, 4), ("tuna", 30, 29), ("tuna", 17, 5)])
 def test_route_on_gpu_equals_oracle_trace(api, func, P, r):
     """The launches of the GPU call carry, rank to rank, the bytes of the reference's rounds digit by digit."""
+    if api.DEFAULT_FORWARDING:
+        pytest.skip("launches can be inspected one by one only in the launch-per-digit mode")
     counts = W.counts_uniform_random(P, 20, seed=P * 7 + r)
     counts[counts % 3 == 0] = 0
     prob = W.make_problem(counts, 2, 0, 0)
@@ -244,7 +249,7 @@ def test_linear_twolayer_comparators(api, P, n):
             assert fn(dr) == 0, (name, dp.comm.error())
             assert np.array_equal(dr.cpu().numpy(), want), (name, P, n, layout)
             st = dp.comm.last_stats()
-            assert st.moved_bytes == prob.payload_bytes and st.n_launches == launches
+            assert st.moved_bytes == prob.payload_bytes and st.n_launches == (1 if api.DEFAULT_FORWARDING else launches)
         dr = dp.new_recv_arena(0xEE)
         assert api.twolayer_communicator_linear(P, dp, ds, dr) == -2
         assert api.twolayer_communicator_linear_s2(0, 1, 1, dp, ds, dr) == -2
@@ -274,7 +279,7 @@ def test_twolayer_bruck(api, P, n, r):
         st = dp.comm.last_stats()
         assert st.moved_bytes == int(rec["bytes"].sum())
         inter = list(dict.fromkeys(rec[rec["kind"] == 6]["digit"].tolist()))
-        if inter and P <= 64:
+        if inter and P <= 64 and not api.DEFAULT_FORWARDING:
             m = np.zeros((P, P), dtype=np.int64)
             sel = rec[(rec["kind"] == 6) & (rec["digit"] == inter[-1])]
             np.add.at(m, (sel["src"], sel["dst"]), sel["bytes"])
@@ -331,7 +336,8 @@ def test_persistent_plans(api):
         plan = api.Plan(function, dp, dr, **kw)
         assert plan.rc == 0, dp.comm.error()
         assert direct(dr) == 0
-        traffic_direct = [dp.comm.last_traffic(k) for k in range(dp.comm.last_stats().n_launches)]
+        per_digit = not api.DEFAULT_FORWARDING
+        traffic_direct = [dp.comm.last_traffic(k) for k in range(dp.comm.last_stats().n_launches)] if per_digit else [None]
         for rep in range(3):
             dr2 = dp.new_recv_arena(0xEE)
             ds2 = ds.clone()
@@ -339,7 +345,7 @@ def test_persistent_plans(api):
             assert np.array_equal(dr2.cpu().numpy(), want), (function, rep)
         st = dp.comm.last_stats()
         assert st.n_launches == len(traffic_direct) and st.payload_bytes == prob.payload_bytes
-        for k, m in enumerate(traffic_direct):
+        for k, m in enumerate(traffic_direct if per_digit else []):
             assert np.array_equal(dp.comm.last_traffic(k), m)
         # a receive arena with other low address bits is refused, not mis-copied
         rbig = torch.full((prob.recv_bytes + 16,), 0xEE, dtype=torch.uint8, device="cuda:0")
