@@ -30,9 +30,11 @@ from rbruck_alltoallv_amd import workloads as W  # noqa: E402
 
 HBM_PEAK_GBPS = 8000.0
 # HBM bytes per launch of the copy kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, each scaled by what the same
-# counter reads for a plain copy of known size (profiles/vc_copy_items_kernel_C4_pmc_fetch_write.txt); counters cannot
-# be read from inside this process, so workloads that were not profiled report null.
-MEASURED_TRAFFIC_PER_LAUNCH = {("C4", "TTPL_BT_alltoallv", 0): 8408923538}
+# counter reads for a plain copy of known size (profiles/vc_copy_chains_kernel_C4_pmc_fetch_write.txt for forwarded
+# execution, profiles/vc_copy_items_kernel_C4_pmc_fetch_write.txt for one launch per digit); counters cannot be read
+# from inside this process, so workloads that were not profiled report null.  Forwarded execution reads every block
+# once and writes it once per hop, so its traffic is below the algorithmic bytes (one read + one write per hop).
+MEASURED_TRAFFIC_PER_LAUNCH = {("C4", "TTPL_BT_alltoallv", 1): 12780833548, ("C4", "TTPL_BT_alltoallv", 0): 8409189840}
 METRIC = "effective alltoallv GB/s + % HBM peak, P=64..1024 virtual ranks, 1 GPU"
 
 
@@ -326,6 +328,11 @@ def main() -> None:
                          {"ms": round(m / args.steps, 4), "GBps": round(2 * st.launch_bytes[k] / (m / args.steps) / 1e6, 1) if m > 0 else 0.0}
                          for k, m in enumerate(per_launch_ms)]},
     }
+    tr = out["roofline"]["traffic"]
+    if tr and kern_ms > 0:
+        # measured HBM bytes per launch over the same launch duration: what the memory system actually sustained
+        out["roofline"]["traffic_GBps"] = round(tr / (kern_ms / max(nkern, 1) * 1e-3) / 1e9, 1)
+        out["roofline"]["traffic_over_algorithmic"] = round(tr / (kern_bytes / max(nkern, 1)), 4)
     if not args.no_cpu_baseline:
         del send, recv
         torch.cuda.empty_cache()
