@@ -467,6 +467,24 @@ def test_blocks_beyond_two_gib(api):
     dp.comm.free()
 
 
+def test_more_than_4096_ranks(api):
+    """Above 4096 ranks forwarded execution is not used (its hop table would take gigabytes): the call runs one launch per
+    digit whatever the mode."""
+    P = 4100
+    rng = np.random.default_rng(3)
+    counts = np.where(rng.random((P, P)) < 0.01, rng.integers(1, 400, (P, P)), 0).astype(np.int32)
+    prob = W.make_problem(counts, 2, 0, 0)
+    dp = api.DeviceProblem(prob)
+    ds = dp.new_send_arena()
+    dp.fill_payload(0, 2, ds)
+    dr = dp.new_recv_arena(0xEE)
+    assert api.twophase_rbruck_alltoallv(65, dp, ds, dr) == 0, dp.comm.error()
+    assert dp.verify(ds, dr) == 0
+    st = dp.comm.last_stats()
+    assert st.n_launches == 2 and st.payload_bytes == prob.payload_bytes
+    dp.comm.free()
+
+
 def test_reference_input_matrices(api):
     """The reference's own communication patterns (inputs/<P>proc), scaled down, through the function its driver uses."""
     import os
