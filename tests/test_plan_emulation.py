@@ -211,6 +211,25 @@ def test_twolayer_bruck_route_equals_the_oracles_trace(P, n, r):
         assert res.moved == int((prob.sendcounts.astype(np.int64) * hops).sum()) * prob.esz
 
 
+@pytest.mark.parametrize("esz", [3, 5, 12, 24])
+def test_element_sizes_that_are_no_power_of_two(esz):
+    """The reference multiplies counts and displacements by MPI_Type_size (src/twophase_tunable_rbruckv.cpp:28, 63); any
+    contiguous type size must work."""
+    counts = W.counts_uniform_random(12, 700, seed=esz)
+    counts[counts % 3 == 0] = 0
+    prob = W.make_problem(counts, esz, 1, 1)
+    send = W.fill_send_arena(prob, 0, 3)
+    want = W.expected_recv_arena(prob, send)
+    for forward in (False, True):
+        for func, kw in ((E.F_TWOPHASE, dict(r=3)), (E.F_TUNA, dict(r=2)), (E.F_TTPL_S1, dict(n=4, r=2)), (E.F_TTPL_RBRUCK, dict(n=3, r=2))):
+            recv = np.full(prob.recv_bytes, 0xEE, dtype=np.uint8)
+            res = E.emulate(func, prob, send, recv, forward=forward, **kw)
+            assert res.rc == 0 and res.errors == 0, (esz, func, forward)
+            assert np.array_equal(recv, want)
+            ref = np.full(prob.recv_bytes, 0xEE, dtype=np.uint8)
+            assert O.twophase_rbruck_alltoallv(3, prob, send, ref) == 0 and np.array_equal(ref, want)
+
+
 def test_twolayer_bruck_error_codes():
     prob = W.make_problem(W.counts_uniform_random(12, 5, seed=1), 1, 0, 0)
     send = W.fill_send_arena(prob, 0, 2)
