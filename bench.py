@@ -177,10 +177,16 @@ def main() -> None:
         func = args.func
     if args.radix:
         tun["r"] = args.radix
+    if args.func or args.radix:
+        # the hop model follows the function that is actually called
         P_ = counts.shape[0]
-        hops = W.hops_twolayer(P_, tun["n"], args.radix) if "n" in tun else W.hops_flat(P_, min(args.radix, P_ - 1 if func == "tuna_algorithm" else P_))
-    if func == "TTPL_rbruck_alltoallv":
-        hops = W.hops_twolayer_bruck(counts.shape[0], tun["n"], tun["r"])
+        if func in ("twophase_rbruck_alltoallv", "twophase_rbruck_alltoallv_om", "tuna_algorithm"):
+            tun.setdefault("b", 0)
+            hops = W.hops_flat(P_, min(tun["r"], P_ - 1 if func == "tuna_algorithm" else P_))
+        else:
+            tun.setdefault("n", 32)
+            tun.setdefault("bblock", 0)
+            hops = W.hops_twolayer_bruck(P_, tun["n"], tun["r"]) if func == "TTPL_rbruck_alltoallv" else W.hops_twolayer(P_, tun["n"], tun["r"])
     prob = W.make_problem(counts, esz, 0, 0)
     S = prob.payload_bytes
     A = W.algorithmic_bytes(counts, esz, hops)
