@@ -119,6 +119,8 @@ inline int vc_make_schedule(VcFunc f, int P, int n, int r, int batch, int esz, i
     memset(&S, 0, sizeof S);
     L.clear();
     S.P = P; S.esz = esz; S.uniform = uniform_count;
+    if (forward) batch = batch2 = 0;                        // one kernel performs every hop: batches of rounds mean nothing
+
     int d = 0;
     switch (f) {
     case VC_F_TWOPHASE:
