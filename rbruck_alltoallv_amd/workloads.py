@@ -181,14 +181,30 @@ def make_uniform_problem(P: int, count: int, esz: int, align: int = 256) -> Prob
 
 
 def fill_send_arena(prob: Problem, mode: int, seed: int) -> np.ndarray:
-    """Host-side payload for small problems (the GPU harness has its own fill kernel for big ones)."""
+    """Host-side payload (the GPU harness has its own fill kernel for big problems): block (s, d) holds
+    block_payload(mode, seed, s, d, nbytes).  One vectorised pass per source rank."""
     arena = np.zeros(prob.send_bytes, dtype=np.uint8)
-    for s in range(prob.P):
-        for d in range(prob.P):
-            nb = int(prob.sendcounts[s, d]) * prob.esz
-            if nb:
-                at = int(prob.sbase[s]) + int(prob.sdispls[s, d]) * prob.esz
-                arena[at:at + nb] = block_payload(mode, seed, s, d, nb)
+    P, esz = prob.P, prob.esz
+    unit = 4 if mode == PAYLOAD_SELFDESC32 else 8
+    ranks = np.arange(P)
+    lane = np.arange(unit, dtype=np.int64)[None, :]
+    for s in range(P):
+        nb = prob.sendcounts[s].astype(np.int64) * esz
+        nw = (nb + unit - 1) // unit
+        tot = int(nw.sum())
+        if tot == 0:
+            continue
+        d_idx = np.repeat(ranks, nw)
+        k_idx = np.arange(tot, dtype=np.int64) - np.repeat(np.cumsum(nw) - nw, nw)
+        if mode == PAYLOAD_SELFDESC32:
+            words = ((np.uint32(s) << np.uint32(20)) + (d_idx.astype(np.uint32) << np.uint32(10)) + k_idx.astype(np.uint32)).astype("<u4")
+        else:
+            words = hash4(seed, s, d_idx.astype(np.uint64), k_idx.astype(np.uint64)).astype("<u8")
+        data = words.view(np.uint8).reshape(tot, unit)
+        pos = k_idx[:, None] * unit + lane                       # byte position inside the block
+        valid = pos < nb[d_idx][:, None]
+        dest = (int(prob.sbase[s]) + prob.sdispls[s].astype(np.int64)[d_idx] * esz)[:, None] + pos
+        arena[dest[valid]] = data[valid]
     return arena
 
 

@@ -120,6 +120,13 @@ def cases() -> list[dict]:
     for P, n, r in ((8, 4, 2), (12, 4, 2), (12, 3, 3), (27, 9, 3), (32, 4, 2), (64, 8, 4)):
         cg = dict(kind="uniform_random", P=P, hi=30, seed=P + 11, sparsify=4)
         add(f"ttpl-rbruck-P{P}-n{n}-r{r}", "ttpl_rbruck", cg, 2, r=r, n=n, layout=1)
+    # the benchmark configurations at their REAL rank counts, with small blocks (minutes of mpiexec each)
+    add("C3p-twophase-r16", "twophase", dict(kind="zipf", P=256, max=512, seed=0), 4, r=16)
+    add("C3p-tuna-r16", "tuna", dict(kind="zipf", P=256, max=512, seed=0), 4, r=16, b=0)
+    c4p = dict(kind="normal", P=1024, mean=64.0, sd=16.0, hi=256, seed=0)
+    add("C4p-ttpl", "ttpl", c4p, 1, r=32, n=32, bblock=0)
+    add("C4p-ttpl_s1", "ttpl_s1", c4p, 1, r=32, n=32, bblock=0)
+    add("C5p-tuna-r32", "tuna", dict(kind="fft", P=512, row_len=32, count=8), 8, r=32, b=0)
     # uniform two-layer functions
     for P, n, r in ((16, 4, 2), (16, 4, 3), (16, 4, 4), (12, 3, 2), (64, 8, 4), (64, 16, 3)):
         add(f"uni-spread-P{P}-n{n}-r{r}", "uniform_spreadout", None, 4, r=r, n=n, count=5)
@@ -140,7 +147,7 @@ def run_case(case: dict, tmp: str) -> dict:
     outp = os.path.join(tmp, "out")
     cmd = [MPIEXEC, "-n", str(P), DRIVER, case["func"], counts_arg, str(case["esz"]), str(case["r"]), str(case["b"]),
            str(case["n"]), str(case["bblock"]), str(case["layout"]), str(case["payload"]), str(case["seed"]), "1", outp]
-    res = subprocess.run(cmd, capture_output=True, text=True, timeout=600)
+    res = subprocess.run(cmd, capture_output=True, text=True, timeout=1800)
     line = res.stdout.strip().splitlines()[-1] if res.stdout.strip() else ""
     if res.returncode != 0:
         raise RuntimeError(f"{case['id']}: reference run failed ({res.returncode}): {line} {res.stderr[-400:]}")
@@ -157,15 +164,27 @@ def run_case(case: dict, tmp: str) -> dict:
 
 
 def main() -> None:
+    """Without arguments every case is run again; `--only TEXT` runs the cases whose id contains TEXT and replaces just
+    those in the existing golden.json."""
     if not os.path.exists(DRIVER):
         raise SystemExit("build the reference driver first: make -C oracle ref")
+    only = sys.argv[sys.argv.index("--only") + 1] if "--only" in sys.argv else None
+    path = os.path.join(HERE, "golden.json")
+    todo = [c for c in cases() if only is None or only in c["id"]]
     recs = []
     with tempfile.TemporaryDirectory() as tmp:
-        for case in cases():
+        for case in todo:
             rec = run_case(case, tmp)
             print(rec["id"], rec["reference_says"], flush=True)
             recs.append(rec)
-    with open(os.path.join(HERE, "golden.json"), "w") as f:
+    if only is not None:
+        new = {r["id"]: r for r in recs}
+        old = json.load(open(path))["cases"]
+        order = [c["id"] for c in cases()]
+        merged = {r["id"]: r for r in old}
+        merged.update(new)
+        recs = [merged[i] for i in order if i in merged]
+    with open(path, "w") as f:
         json.dump({"made_by": "tests/golden/make_golden.py", "mpi": "MPICH 3.3.2 (/opt/conda), mpiexec -n P, oversubscribed on 8 cores",
                    "cases": recs}, f, indent=1)
     print(f"{len(recs)} cases written")

@@ -26,9 +26,15 @@ static int count_overlaps(std::vector<Range> &dst, std::vector<Range> &src) {
     std::sort(dst.begin(), dst.end(), key);
     for (size_t i = 1; i < dst.size(); i++)
         if (dst[i].space == dst[i - 1].space && dst[i].lo < dst[i - 1].hi) bad++;
-    for (const Range &s : src)
-        for (const Range &d : dst)
-            if (d.space == s.space && d.lo < s.hi && s.lo < d.hi) { bad++; break; }
+    // a source against the sorted destinations: only the last destination that starts below the source's end can reach
+    // into it once the destinations do not overlap each other
+    for (const Range &s : src) {
+        const Range probe{s.hi, 0, s.space};
+        auto it = std::lower_bound(dst.begin(), dst.end(), probe, key);      // first destination with lo >= s.hi
+        if (it == dst.begin()) continue;
+        --it;
+        if (it->space == s.space && it->lo < s.hi && s.lo < it->hi) bad++;
+    }
     return bad;
 }
 
