@@ -214,14 +214,14 @@ int vc_suggest_radix(const int *sendcounts, int elem_size, int n, const int *can
 #define VC_MAX_LAUNCHES 1024
 
 typedef struct {
-    int32_t n_launches;          /* data-moving kernel launches of the last call */
+    int32_t n_launches;          /* data-moving kernel launches of the last call (1 in forwarded execution) */
     int32_t n_digits;            /* digit phases among them */
     int64_t payload_bytes;       /* S: sum of all blocks */
-    int64_t moved_bytes;         /* sum over launches of the bytes copied (each counted once) */
+    int64_t moved_bytes;         /* sum over all hops of the bytes copied (each hop counted once) */
     int64_t staging_bytes;       /* staging arena the call needed */
     float plan_ms;               /* metadata kernels (valid when timing is on) */
     float total_ms;              /* whole call on the stream (valid when timing is on) */
-    int64_t launch_bytes[VC_MAX_LAUNCHES];
+    int64_t launch_bytes[VC_MAX_LAUNCHES];   /* bytes the hops of a launch copy (forwarded execution: [0] = moved_bytes) */
     float launch_ms[VC_MAX_LAUNCHES];  /* per data-moving launch, HIP events on the comm's stream */
 } vc_stats_t;
 
@@ -230,7 +230,8 @@ int vc_comm_set_timing(vc_comm_t comm, int enable);
 int vc_comm_last_stats(vc_comm_t comm, vc_stats_t *out);
 
 /* Route of the last call: for launch `launch`, the bytes sent from every rank to every rank, as a HOST
- * [P][P] int64 matrix (row = sender).  For tests that pin the route against the oracle's message trace. */
+ * [P][P] int64 matrix (row = sender).  For tests that pin the route against the oracle's message trace.  Only after a
+ * call in the launch-per-digit mode (vc_comm_set_forwarding(comm, 0)). */
 int vc_comm_last_traffic(vc_comm_t comm, int launch, int64_t *matrix_out);
 
 /* ---- harness utilities (payload of the reference drivers, examples/rbruckv_example.cpp:88-92, and a
