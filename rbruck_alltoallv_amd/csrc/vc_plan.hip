@@ -152,7 +152,8 @@ __global__ __launch_bounds__(VC_THREADS) void vc_plan_bases(int P, int w, int nl
 }
 
 // ---- pass 3: the work items ----
-// grid (P, nl).  Repeats the row scan of pass 1 to place every block's pieces.
+// grid (P, nl, Z).  Repeats the row scan of pass 1 to place every block's pieces; Z workgroups share a receiver's entries
+// when there are few ranks (their blocks are then huge and have many pieces).
 __global__ __launch_bounds__(VC_THREADS) void vc_plan_emit(VcSched S, const VcLaunchInfo *__restrict__ launches, VcTables T,
                                                            const int64_t *__restrict__ slot_off, const int64_t *__restrict__ row_base,
                                                            const int64_t *__restrict__ item_row_base, const int64_t *__restrict__ header,
@@ -169,8 +170,19 @@ __global__ __launch_bounds__(VC_THREADS) void vc_plan_emit(VcSched S, const VcLa
     __shared__ VcDesc big_whole[VC_THREADS];
     __shared__ int64_t big_at[VC_THREADS], big_pre[VC_THREADS];
     __shared__ int big_phase[VC_THREADS], big_cut[VC_THREADS];
-    const int nent = vc_entries_per_rank(S, info);
-    for (int base = 0; base < nent; base += VC_THREADS) {
+    const int nent_all = vc_entries_per_rank(S, info);
+    // workgroup (to, L, z) writes the z-th slice of the receiver's entries; the items of the slices before it come first
+    const int per = (nent_all + (int)gridDim.z - 1) / (int)gridDim.z;
+    const int e_lo = (int)blockIdx.z * per < nent_all ? (int)blockIdx.z * per : nent_all;
+    const int nent = e_lo + per < nent_all ? e_lo + per : nent_all;
+    int64_t before = 0;
+    for (int id = threadIdx.x; id < e_lo; id += VC_THREADS) {
+        VcEntry e;
+        if (vc_entry_block(S, info, to, id, e))
+            before += vc_chunk_count(vc_entry_len(S, T, e), vc_entry_phase(S, T, e), vc_entry_cut(S, T, e));
+    }
+    carry += vc_block_sum(before, lds);
+    for (int base = e_lo; base < nent; base += VC_THREADS) {
         const int id = base + threadIdx.x;
         VcEntry e;
         const bool active = id < nent && vc_entry_block(S, info, to, id, e);
@@ -222,8 +234,9 @@ hipError_t vc_launch_plan_sizes(const VcSched &S, const VcLaunchInfo *launches_d
 hipError_t vc_launch_plan_emit(const VcSched &S, const VcLaunchInfo *launches_dev, int nlaunch, VcTables T, const int64_t *slot_off,
                                const int64_t *row_base, const int64_t *item_row_base, const int64_t *header, VcDesc *items,
                                hipStream_t st) {
-    hipLaunchKernelGGL(vc_plan_emit, dim3(S.P, nlaunch), dim3(VC_THREADS), 0, st, S, launches_dev, T, slot_off, row_base, item_row_base,
-                       header, nlaunch, items);
+    const int slices = S.P >= 1024 ? 1 : (S.P >= 64 ? 1024 / S.P : 16);
+    hipLaunchKernelGGL(vc_plan_emit, dim3(S.P, nlaunch, slices), dim3(VC_THREADS), 0, st, S, launches_dev, T, slot_off, row_base,
+                       item_row_base, header, nlaunch, items);
     return hipGetLastError();
 }
 
@@ -251,8 +264,9 @@ __global__ __launch_bounds__(VC_THREADS) void vc_fill64_kernel(int64_t *__restri
     if (i < n) p[i] = value;
 }
 
-// grid (P): the chain items of the blocks that end on rank t, in source order; big blocks are written by the whole
-// workgroup as in vc_plan_emit.
+// grid (P, Z): the chain items of the blocks that end on rank t, in source order; workgroup (t, z) writes those of the
+// z-th slice of the sources (few ranks with huge blocks would otherwise leave most of the chip idle); big blocks are
+// written by the whole workgroup as in vc_plan_emit.
 __global__ __launch_bounds__(VC_THREADS) void vc_chain_emit(VcSched S, VcTables T, const int64_t *__restrict__ chain_row_base,
                                                             const int64_t *__restrict__ hop_src, const int64_t *__restrict__ hop_dst,
                                                             int64_t *__restrict__ items) {
@@ -260,10 +274,14 @@ __global__ __launch_bounds__(VC_THREADS) void vc_chain_emit(VcSched S, VcTables 
     __shared__ int64_t big_at[VC_THREADS], big_pre[VC_THREADS];
     const int t = blockIdx.x, P = S.P;
     const int stride = VC_CHAIN_HEAD + vc_hop_slots(S);
-    int64_t carry = chain_row_base[t];
-    for (int base = 0; base < P; base += VC_THREADS) {
+    const int per = (P + (int)gridDim.y - 1) / (int)gridDim.y;
+    const int s_lo = (int)blockIdx.y * per < P ? (int)blockIdx.y * per : P, s_hi = s_lo + per < P ? s_lo + per : P;
+    int64_t before = 0;                                   // items of this receiver's earlier sources
+    for (int s = threadIdx.x; s < s_lo; s += VC_THREADS) before += vc_chain_count(S, T, s, t);
+    int64_t carry = chain_row_base[t] + vc_block_sum(before, lds);
+    for (int base = s_lo; base < s_hi; base += VC_THREADS) {
         const int s = base + threadIdx.x;
-        const int64_t cnt = s < P ? vc_chain_count(S, T, s, t) : 0;
+        const int64_t cnt = s < s_hi ? vc_chain_count(S, T, s, t) : 0;
         int64_t total;
         const int64_t at = carry + vc_block_exclusive_scan(cnt, lds, total);
         const bool big = cnt > 4;
@@ -295,7 +313,8 @@ hipError_t vc_launch_chain_plan(const VcSched &S, const VcLaunchInfo *launches_d
     const int64_t n = (int64_t)vc_hop_slots(S) * S.P * S.P;
     hipLaunchKernelGGL(vc_fill64_kernel, dim3((unsigned)((n + VC_THREADS - 1) / VC_THREADS)), dim3(VC_THREADS), 0, st, hop_dst, n, (int64_t)-1);
     hipLaunchKernelGGL(vc_chain_hops, dim3(S.P, nlaunch), dim3(VC_THREADS), 0, st, S, launches_dev, T, slot_off, row_base, hop_src, hop_dst);
-    hipLaunchKernelGGL(vc_chain_emit, dim3(S.P), dim3(VC_THREADS), 0, st, S, T, chain_row_base, hop_src, hop_dst, items);
+    const int slices = S.P >= 1024 ? 1 : (S.P >= 64 ? 1024 / S.P : 16);      // about a thousand workgroups at least
+    hipLaunchKernelGGL(vc_chain_emit, dim3(S.P, slices), dim3(VC_THREADS), 0, st, S, T, chain_row_base, hop_src, hop_dst, items);
     return hipGetLastError();
 }
 
