@@ -60,8 +60,7 @@ int vc_comm_set_bases(vc_comm_t comm, const int64_t *sbase_bytes, const int64_t 
  *    all the hops of that block one after the other and keeps the piece in registers in between, so the data is read
  *    once (from sendbuf) and written once per hop (into the staging slot of every intermediate holder, then into
  *    recvbuf).  The batching tunables (b, bblock) then have no effect, and TTPL_BT_alltoallv sends its inter-node data
- *    per block instead of coalesced.  Calls on more than 4096 ranks fall back to mode 0 (the per-block hop table
- *    would grow to gigabytes).
+ *    per block instead of coalesced.
  * 0: one kernel launch per digit phase (or per batch of its rounds, as b / bblock say); every hop reads the block
  *    where the previous hop left it.  This is the mode whose launches vc_comm_last_stats and vc_comm_last_traffic
  *    describe one by one.

@@ -65,7 +65,7 @@ struct vc_comm {
     const int64_t *sbase = nullptr, *rbase = nullptr;
     bool timing = false;
     bool forward = true;                  // forwarded execution: one launch, every block piece carried through all its hops
-    DevBuf chain_row_tot, chain_row_base, hop_src, hop_dst;
+    DevBuf chain_row_tot, chain_row_base;
     DevBuf slot_off, row_tot, row_base, org_run_base, item_row_tot, item_row_base, row_bytes, desc, header, launches, stage, rd_packed,
         uni_counts, uni_displs, scratch;
     int64_t *h_header = nullptr;          // pinned, coherent: the planner writes its header straight into it
@@ -104,7 +104,7 @@ extern "C" int vc_comm_free(vc_comm_t c) {
     if (!c) return VC_OK;
     (void)hipStreamSynchronize(c->stream);
     for (DevBuf *b : {&c->slot_off, &c->row_tot, &c->row_base, &c->org_run_base, &c->item_row_tot, &c->item_row_base, &c->row_bytes, &c->desc, &c->header, &c->launches, &c->stage, &c->rd_packed,
-                      &c->uni_counts, &c->uni_displs, &c->scratch, &c->chain_row_tot, &c->chain_row_base, &c->hop_src, &c->hop_dst})
+                      &c->uni_counts, &c->uni_displs, &c->scratch, &c->chain_row_tot, &c->chain_row_base})
         b->release();
     for (hipEvent_t e : c->events) (void)hipEventDestroy(e);
     if (c->h_header) (void)hipHostFree(c->h_header);
@@ -258,10 +258,7 @@ static int build_plan(vc_comm *c, VcSched S, std::vector<VcLaunchInfo> &L, VcTab
         out.chain_stride = VC_CHAIN_HEAD + vc_hop_slots(S);
         out.chain_items = h[2];
         HIP_TRY(items.reserve(sizeof(int64_t) * (size_t)out.chain_stride * (size_t)std::max<int64_t>(out.chain_items, 1)));
-        HIP_TRY(c->hop_src.reserve(sizeof(int64_t) * PP));
-        HIP_TRY(c->hop_dst.reserve(sizeof(int64_t) * PP * (size_t)vc_hop_slots(S)));
-        HIP_TRY(vc_launch_chain_plan(S, c->launches.as<VcLaunchInfo>(), nl, T, c->slot_off.as<int64_t>(), c->row_base.as<int64_t>(),
-                                     c->chain_row_base.as<int64_t>(), c->hop_src.as<int64_t>(), c->hop_dst.as<int64_t>(),
+        HIP_TRY(vc_launch_chain_plan(S, T, c->slot_off.as<int64_t>(), c->row_base.as<int64_t>(), c->chain_row_base.as<int64_t>(),
                                      items.as<int64_t>(), st));
         if (c->timing) HIP_TRY(hipEventRecord(c->events[1], st));
         return VC_OK;
@@ -370,11 +367,9 @@ static int schedule_error(int code) {
     return code;
 }
 
-// Forwarded execution keeps one int64 per block and hop slot (at most 2 * log2(P) + 1 slots); beyond 4096 ranks a call
-// falls back to one launch per digit.
 static bool use_forwarding(const vc_comm *c, int P, int r_hint) {
-    (void)r_hint;
-    return c->forward && P <= 4096;
+    (void)P; (void)r_hint;
+    return c->forward;
 }
 
 // The alltoallv-shaped functions.

@@ -50,6 +50,9 @@ struct VcSched {
     int uniform;      // >0: equal blocks of this many elements, tables are implied (uniform_* functions)
     int recv_lo;      // low 12 bits of the recvbuf pointer: staging slots copy the final destination's cache-line phase,
                       // long copies into recvbuf are cut at its 4 KiB boundaries
+    int last_hop;     // which blocks make a hop that is no digit round and ends in recvbuf, besides every rank's block to
+                      // itself: 0 none (one-layer Bruck; Bruck over the nodes), 1 those that change node (inter-node
+                      // messages), 2 all (direct one-hop functions)
     int coalesce;     // 1: blocks that are about to leave their node wait in "organized" runs — the n blocks one rank
                       //    holds for one destination rank back to back in source order — so that an inter-node message
                       //    is a contiguous copy (TTPL_BT_alltoallv, src/twophase_twolayer_rbruck.cpp:388-398, 430-453).
@@ -112,10 +115,9 @@ hipError_t vc_launch_plan_sizes(const VcSched &S, const VcLaunchInfo *launches_d
                                 int64_t *row_tot, int64_t *row_base, int64_t *org_run_base, int64_t *item_row_tot,
                                 int64_t *item_row_base, int64_t *row_bytes, int64_t *chain_row_tot, int64_t *chain_row_base,
                                 int64_t *header, int64_t *header_host, hipStream_t st);
-// Forwarded execution: per-block hop tables (hop_src: P*P, hop_dst: hop slots * P*P int64), then the chain items.
-hipError_t vc_launch_chain_plan(const VcSched &S, const VcLaunchInfo *launches_dev, int nlaunch, VcTables T, const int64_t *slot_off,
-                                const int64_t *row_base, const int64_t *chain_row_base, int64_t *hop_src, int64_t *hop_dst,
-                                int64_t *items, hipStream_t st);
+// Forwarded execution: the chain items (every block's route in closed form, staging addresses from the plan tables).
+hipError_t vc_launch_chain_plan(const VcSched &S, VcTables T, const int64_t *slot_off, const int64_t *row_base,
+                                const int64_t *chain_row_base, int64_t *items, hipStream_t st);
 // Writes the first nl (<= VC_LAUNCH_PACK) launch descriptions to device memory from a kernel argument.
 hipError_t vc_launch_store_launches(const VcLaunchInfo *host, int nl, VcLaunchInfo *out, hipStream_t st);
 // Pass 3: writes the work items (needs the item buffer, sized from the header).

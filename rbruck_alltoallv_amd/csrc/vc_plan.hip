@@ -241,39 +241,22 @@ hipError_t vc_launch_plan_emit(const VcSched &S, const VcLaunchInfo *launches_de
 }
 
 // ---- forwarded execution ----
-// grid (P, nl): every entry of every launch leaves the destination of its hop (and, for a block's first hop, its
-// source in sendbuf) in the per-block hop tables.
-__global__ __launch_bounds__(VC_THREADS) void vc_chain_hops(VcSched S, const VcLaunchInfo *__restrict__ launches, VcTables T,
-                                                            const int64_t *__restrict__ slot_off, const int64_t *__restrict__ row_base,
-                                                            int64_t *__restrict__ hop_src, int64_t *__restrict__ hop_dst) {
-    const int to = blockIdx.x, P = S.P;
-    const VcLaunchInfo info = launches[blockIdx.y];
-    const int nent = vc_entries_per_rank(S, info);
-    for (int id = threadIdx.x; id < nent; id += VC_THREADS) {
-        VcEntry e;
-        if (!vc_entry_block(S, info, to, id, e)) continue;
-        const VcDesc d = vc_entry_desc(S, T, slot_off, row_base, e, to);
-        const int64_t key = (int64_t)e.t * P + e.s;
-        hop_dst[(int64_t)vc_hop_slot(S, info, e) * P * P + key] = d.dst;
-        if (e.xprev < 0) hop_src[key] = d.src;
-    }
-}
-
-__global__ __launch_bounds__(VC_THREADS) void vc_fill64_kernel(int64_t *__restrict__ p, int64_t n, int64_t value) {
-    const int64_t i = (int64_t)blockIdx.x * VC_THREADS + threadIdx.x;
-    if (i < n) p[i] = value;
-}
-
 // grid (P, Z): the chain items of the blocks that end on rank t, in source order; workgroup (t, z) writes those of the
 // z-th slice of the sources (few ranks with huge blocks would otherwise leave most of the chip idle); big blocks are
 // written by the whole workgroup as in vc_plan_emit.
-__global__ __launch_bounds__(VC_THREADS) void vc_chain_emit(VcSched S, VcTables T, const int64_t *__restrict__ chain_row_base,
-                                                            const int64_t *__restrict__ hop_src, const int64_t *__restrict__ hop_dst,
-                                                            int64_t *__restrict__ items) {
+__global__ __launch_bounds__(VC_THREADS) void vc_chain_emit(VcSched S, VcTables T, const int64_t *__restrict__ slot_off,
+                                                            const int64_t *__restrict__ row_base,
+                                                            const int64_t *__restrict__ chain_row_base, int64_t *__restrict__ items) {
     __shared__ int64_t lds[VC_WAVES_PER_BLOCK];
     __shared__ int64_t big_at[VC_THREADS], big_pre[VC_THREADS];
+    // a block of many pieces keeps its route here while the whole workgroup writes its items (routes of more hops than
+    // fit are evaluated again for every piece)
+    const int VC_ROUTE_CACHE = 6;
+    __shared__ int64_t big_dst[VC_THREADS][VC_ROUTE_CACHE];
+    __shared__ int big_nhop[VC_THREADS];
     const int t = blockIdx.x, P = S.P;
     const int stride = VC_CHAIN_HEAD + vc_hop_slots(S);
+    const bool cached = vc_hop_slots(S) <= VC_ROUTE_CACHE;
     const int per = (P + (int)gridDim.y - 1) / (int)gridDim.y;
     const int s_lo = (int)blockIdx.y * per < P ? (int)blockIdx.y * per : P, s_hi = s_lo + per < P ? s_lo + per : P;
     int64_t before = 0;                                   // items of this receiver's earlier sources
@@ -286,8 +269,11 @@ __global__ __launch_bounds__(VC_THREADS) void vc_chain_emit(VcSched S, VcTables 
         const int64_t at = carry + vc_block_exclusive_scan(cnt, lds, total);
         const bool big = cnt > 4;
         if (!big)
-            for (int64_t c = 0; c < cnt; c++) vc_chain_item(S, T, hop_src, hop_dst, s, t, c, items + (at + c) * stride);
-        else big_at[threadIdx.x] = at;
+            for (int64_t c = 0; c < cnt; c++) vc_chain_item(S, T, slot_off, row_base, s, t, c, items + (at + c) * stride);
+        else {
+            big_at[threadIdx.x] = at;
+            if (cached) big_nhop[threadIdx.x] = vc_chain_route(S, T, slot_off, row_base, s, t, big_dst[threadIdx.x]);
+        }
         if (__syncthreads_or(big)) {
             int64_t btotal;
             big_pre[threadIdx.x] = vc_block_exclusive_scan(big ? cnt : 0, lds, btotal);
@@ -299,7 +285,12 @@ __global__ __launch_bounds__(VC_THREADS) void vc_chain_emit(VcSched S, VcTables 
                     if (big_pre[mid] <= q) lo = mid; else hi = mid - 1;
                 }
                 const int64_t c = q - big_pre[lo];
-                vc_chain_item(S, T, hop_src, hop_dst, base + lo, t, c, items + (big_at[lo] + c) * stride);
+                const int sb = base + lo;
+                if (cached)
+                    vc_chain_piece(VC_SPACE_SEND | vc_send_offset(S, T, sb, t), (int64_t)T.sc[(int64_t)sb * P + t] * S.esz, vc_phase(S, T, sb, t),
+                                   vc_chain_cut(S, T, sb, t), c, big_dst[lo], big_nhop[lo], items + (big_at[lo] + c) * stride);
+                else
+                    vc_chain_item(S, T, slot_off, row_base, sb, t, c, items + (big_at[lo] + c) * stride);
             }
             __syncthreads();
         }
@@ -307,14 +298,10 @@ __global__ __launch_bounds__(VC_THREADS) void vc_chain_emit(VcSched S, VcTables 
     }
 }
 
-hipError_t vc_launch_chain_plan(const VcSched &S, const VcLaunchInfo *launches_dev, int nlaunch, VcTables T, const int64_t *slot_off,
-                                const int64_t *row_base, const int64_t *chain_row_base, int64_t *hop_src, int64_t *hop_dst,
-                                int64_t *items, hipStream_t st) {
-    const int64_t n = (int64_t)vc_hop_slots(S) * S.P * S.P;
-    hipLaunchKernelGGL(vc_fill64_kernel, dim3((unsigned)((n + VC_THREADS - 1) / VC_THREADS)), dim3(VC_THREADS), 0, st, hop_dst, n, (int64_t)-1);
-    hipLaunchKernelGGL(vc_chain_hops, dim3(S.P, nlaunch), dim3(VC_THREADS), 0, st, S, launches_dev, T, slot_off, row_base, hop_src, hop_dst);
+hipError_t vc_launch_chain_plan(const VcSched &S, VcTables T, const int64_t *slot_off, const int64_t *row_base,
+                                const int64_t *chain_row_base, int64_t *items, hipStream_t st) {
     const int slices = S.P >= 1024 ? 1 : (S.P >= 64 ? 1024 / S.P : 16);      // about a thousand workgroups at least
-    hipLaunchKernelGGL(vc_chain_emit, dim3(S.P, slices), dim3(VC_THREADS), 0, st, S, T, chain_row_base, hop_src, hop_dst, items);
+    hipLaunchKernelGGL(vc_chain_emit, dim3(S.P, slices), dim3(VC_THREADS), 0, st, S, T, slot_off, row_base, chain_row_base, items);
     return hipGetLastError();
 }
 

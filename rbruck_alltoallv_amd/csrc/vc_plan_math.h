@@ -346,24 +346,64 @@ VC_HD int64_t vc_chain_count(const VcSched &S, const VcTables &T, int s, int t) 
 #define VC_CHAIN_NHOP 2
 #define VC_CHAIN_HEAD 3   // followed by the space-tagged destination of the piece at every hop
 
-// Writes piece c of block (s, t) to `item`.  hop_src[key] and hop_dst[slot * P * P + key] (key = t * P + s) hold the
-// whole block's source and its destination per hop slot (-1: does not move in that slot).
-VC_HD void vc_chain_item(const VcSched &S, const VcTables &T, const int64_t *hop_src, const int64_t *hop_dst, int s, int t, int64_t c,
-                         int64_t *item) {
-    const int64_t PP = (int64_t)S.P * S.P, key = (int64_t)t * S.P + s;
-    const int64_t len = (int64_t)T.sc[(int64_t)s * S.P + t] * S.esz;
-    const int phase = vc_phase(S, T, s, t), cut = vc_chain_cut(S, T, s, t);
+// The route of block (s, t) in closed form: does it move in hop slot k, and where to?  After digit x of a Bruck that
+// runs least significant digit first a block has travelled (offset mod r^(x+1)) ranks down from its source, most
+// significant first (offset div r^x) * r^x; it sits in slot (destination group) * n + (local offset + local rank) % n
+// of its holder (src/twophase_twolayer_rbruck.cpp:322), and lands in recvbuf when no digit is left and it is on its
+// destination's node.  The CPU check of the plan compares this with what the launches' entries say, block by block.
+VC_HD bool vc_block_hop(const VcSched &S, const VcTables &T, const int64_t *slot_off, const int64_t *row_base, int s, int t, int k,
+                        int64_t &dst) {
+    const int n = S.n, G = S.G, r = S.r, final_slot = S.w + S.w2;
+    const int64_t to_recv = VC_SPACE_RECV | vc_recv_offset(S, T, s, t);
+    if (s == t) { dst = to_recv; return k == final_slot; }
+    const int gs = s / n, gt = t / n, ls = s % n, lt = t % n;
+    if (k == final_slot) { dst = to_recv; return S.last_hop == 2 || (S.last_hop == 1 && gs != gt); }
+    const bool intra = k < S.w;
+    const int x = intra ? k : k - S.w;
+    const int span = intra ? n : G;
+    const int j = intra ? (ls - lt + n) % n : (gs - gt + G) % G;       // offset inside the node / between the nodes
+    int64_t dist = 1;
+    for (int i = 0; i < x; i++) dist *= r;
+    if (dist >= span || (j / dist) % r == 0) return false;
+    const int64_t nd = dist * r;
+    const bool msd = intra && S.msd;
+    const int64_t travelled = msd ? (j / dist) * dist : j % nd;
+    const bool last = msd ? j % dist == 0 : j < nd;
+    const int pos = (int)((((intra ? ls : gs) - travelled) % span + span) % span);   // local rank / node of the holder after the hop
+    const int to = intra ? gs * n + pos : pos * n + lt;
+    const int id = intra ? gt * n + (j + pos) % n : j * n + ls;
+    dst = (last && (intra ? gs == gt : true)) ? to_recv : (VC_SPACE_STAGE | vc_stage_addr(S, T, slot_off, row_base, k, to, id, s, t));
+    return true;
+}
+
+// Piece c of a block whose source and hop destinations (whole block) are known.
+VC_HD void vc_chain_piece(int64_t src, int64_t len, int phase, int cut, int64_t c, const int64_t *dst, int nhop, int64_t *item) {
     VcDesc whole;
-    whole.src = hop_src[key]; whole.dst = 0; whole.len = len; whole.from = s; whole.to = t;
-    const VcDesc piece = vc_chunk_of(whole, c, phase, cut);
-    const int64_t lo = piece.dst;                      // offset of the piece inside the block
+    whole.src = src; whole.dst = 0; whole.len = len; whole.from = 0; whole.to = 0;
+    const VcDesc piece = vc_chunk_of(whole, c, phase, cut);      // piece.dst = offset of the piece inside the block
     item[VC_CHAIN_SRC] = piece.src;
     item[VC_CHAIN_LEN] = piece.len;
+    item[VC_CHAIN_NHOP] = nhop;
+    for (int k = 0; k < nhop; k++) item[VC_CHAIN_HEAD + k] = dst[k] + piece.dst;
+}
+
+// Hop destinations of block (s, t) in slot order; returns their number.
+VC_HD int vc_chain_route(const VcSched &S, const VcTables &T, const int64_t *slot_off, const int64_t *row_base, int s, int t,
+                         int64_t *dst) {
     int nhop = 0;
     const int nslots = vc_hop_slots(S);
     for (int k = 0; k < nslots; k++) {
-        const int64_t d = hop_dst[(int64_t)k * PP + key];
-        if (d >= 0) item[VC_CHAIN_HEAD + nhop++] = d + lo;
+        int64_t d;
+        if (vc_block_hop(S, T, slot_off, row_base, s, t, k, d)) dst[nhop++] = d;
     }
-    item[VC_CHAIN_NHOP] = nhop;
+    return nhop;
+}
+
+// Writes piece c of block (s, t) to `item`.
+VC_HD void vc_chain_item(const VcSched &S, const VcTables &T, const int64_t *slot_off, const int64_t *row_base, int s, int t, int64_t c,
+                         int64_t *item) {
+    const int64_t len = (int64_t)T.sc[(int64_t)s * S.P + t] * S.esz;
+    const int nhop = vc_chain_route(S, T, slot_off, row_base, s, t, item + VC_CHAIN_HEAD);   // whole-block destinations first
+    vc_chain_piece(VC_SPACE_SEND | vc_send_offset(S, T, s, t), len, vc_phase(S, T, s, t), vc_chain_cut(S, T, s, t), c,
+                   item + VC_CHAIN_HEAD, nhop, item);
 }

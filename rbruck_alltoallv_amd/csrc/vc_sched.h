@@ -127,7 +127,7 @@ inline int vc_make_schedule(VcFunc f, int P, int n, int r, int batch, int esz, i
     case VC_F_OM:
         if (r < 2) return VC_ERR_RADIX;                     // src/twophase_tunable_rbruckv.cpp:16, -om.cpp:13
         if (r > P) r = P;                                   // :22, :19
-        S.n = P; S.G = 1; S.r = r; S.msd = (f == VC_F_TWOPHASE);
+        S.n = P; S.G = 1; S.r = r; S.msd = (f == VC_F_TWOPHASE); S.last_hop = 0;
         vc_radix_params(P, S.r, S.w, d);
         vc_add_intra_launches(L, S, d, 0);
         break;
@@ -138,7 +138,7 @@ inline int vc_make_schedule(VcFunc f, int P, int n, int r, int batch, int esz, i
         if (r < 2) r = 2;                                   // :13
         if (r > P - 1) r = P - 1;                           // :20
         if (batch <= 0 || batch > P) batch = P;             // :21
-        S.n = P; S.G = 1; S.r = r; S.msd = 0;
+        S.n = P; S.G = 1; S.r = r; S.msd = 0; S.last_hop = 0;
         vc_radix_params(P, S.r, S.w, d);
         vc_add_intra_launches(L, S, d, batch);
         break;
@@ -147,7 +147,7 @@ inline int vc_make_schedule(VcFunc f, int P, int n, int r, int batch, int esz, i
         if (r < 2) return VC_ERR_RADIX;                     // src/twophase_twolayer_rbruck.cpp:242, :472
         if (n < 1 || P % n != 0) return VC_ERR_GROUP;       // the reference truncates P/n (:260) and hangs
         if (r > n) r = n;                                   // :248
-        S.n = n; S.G = P / n; S.r = std::max(r, 2); S.msd = 0;
+        S.n = n; S.G = P / n; S.r = std::max(r, 2); S.msd = 0; S.last_hop = 1;
         S.packed_recv = (f == VC_F_TTPL);                   // the coalesced variant never reads rdispls
         vc_radix_params(n, S.r, S.w, d);
         vc_add_intra_launches(L, S, d, 0);
@@ -169,7 +169,7 @@ inline int vc_make_schedule(VcFunc f, int P, int n, int r, int batch, int esz, i
         if (r < 2) return VC_ERR_RADIX;                     // src/twophase_twolayer_rbruck.cpp:20
         if (n < 1 || P % n != 0) return VC_ERR_GROUP;
         if (r > n) r = n;                                   // :26
-        S.n = n; S.G = P / n; S.r = std::max(r, 2); S.msd = 0;
+        S.n = n; S.G = P / n; S.r = std::max(r, 2); S.msd = 0; S.last_hop = 0;
         vc_radix_params(n, S.r, S.w, d);                    // :42
         vc_add_intra_launches(L, S, d, 0);
         if (L.empty()) {                                    // n == 1: the copies to self need a launch of their own (the
@@ -189,7 +189,7 @@ inline int vc_make_schedule(VcFunc f, int P, int n, int r, int batch, int esz, i
         if (r < 2) r = 2;                                                // :143
         if (n < 2 || n >= P || P % n != 0) return VC_ERR_GROUP;          // :18-22, :145-149 MPI_Abort
         if (r > n) r = n;
-        S.n = n; S.G = P / n; S.r = r; S.msd = 1;           // intra-node phase is most significant digit first (:69)
+        S.n = n; S.G = P / n; S.r = r; S.msd = 1; S.last_hop = 1;   // intra-node phase is most significant digit first (:69)
         vc_radix_params(n, S.r, S.w, d);
         vc_add_intra_launches(L, S, d, 0);
         vc_add_inter_launches(L, S, P);                     // every group at once (:107-128; :243-274 with r2 = ngroup)
@@ -200,13 +200,13 @@ inline int vc_make_schedule(VcFunc f, int P, int n, int r, int batch, int esz, i
     case VC_F_SPREADOUT:                                    // benchmarks/common.cpp:10-37: all 2P requests, one Waitall
     case VC_F_OMPI_LINEAR:                                  // src/OpenMPI_basic_linear.cpp:10-77: self copy, then everything at once
     case VC_F_OMPI_PAIRWISE:                                // src/OpenMPI_pairwise.cpp:32-58: P steps; independent, so one launch
-        S.n = P; S.G = 1; S.r = 2; S.msd = 0; S.w = 0;
+        S.n = P; S.G = 1; S.r = 2; S.msd = 0; S.w = 0; S.last_hop = 2;
         vc_add_direct_launches(L, P, P);
         break;
     case VC_F_TWOLAYER_LINEAR:                              // src/twolayer_communicator_linear.cpp:13-88
     case VC_F_TWOLAYER_LINEAR_S2:                           // :92-192; batch = bblock1, batch2 = bblock2
         if (n < 1 || n >= P || P % n != 0) return VC_ERR_GROUP;           // :24-28 MPI_Abort (and misses n that does not divide P)
-        S.n = n; S.G = P / n; S.r = 2; S.msd = 0; S.w = 0;
+        S.n = n; S.G = P / n; S.r = 2; S.msd = 0; S.w = 0; S.last_hop = 2;
         // intra-node: MPICH_intra_scattered on the node's communicator, all at once (:45) or bblock1 at a time (:118-123)
         vc_add_scoped_direct_launches(L, 1, 0, n, f == VC_F_TWOLAYER_LINEAR ? n : ((batch <= 0 || batch > n) ? n : batch));
         // inter-node: one Waitall for everything (:55-83), or bblock2 (group distance, local index) pairs at a time (:140-181)
@@ -214,7 +214,7 @@ inline int vc_make_schedule(VcFunc f, int P, int n, int r, int batch, int esz, i
                                       f == VC_F_TWOLAYER_LINEAR ? P : ((batch2 <= 0 || batch2 > P) ? P : batch2));
         break;
     case VC_F_MPICH_SCATTERED:                              // src/MPICH_scattered.cpp:31-70: bblock requests in flight
-        S.n = P; S.G = 1; S.r = 2; S.msd = 0; S.w = 0;
+        S.n = P; S.G = 1; S.r = 2; S.msd = 0; S.w = 0; S.last_hop = 2;
         vc_add_direct_launches(L, P, (batch <= 0 || batch > P) ? P : batch);
         break;
     }

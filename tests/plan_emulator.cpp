@@ -182,8 +182,17 @@ extern "C" int plan_emulate(int func, int P, int n, int r, int batch, int esz, i
                 if ((len > 0) != (cnt > 0)) errors++;
                 if (len > 0 && hop_src[(int64_t)t * P + s0] < 0) { errors++; continue; }
                 int64_t covered = 0;
+                // the closed-form route of the block against what the launches' entries say, hop slot by hop slot
+                const int64_t key0 = (int64_t)t * P + s0;
+                for (int k = 0; k < nslots; k++) {
+                    int64_t d;
+                    const bool moves = vc_block_hop(S, T, slot_off.data(), row_base.data(), s0, t, k, d);
+                    const int64_t cell = hop_dst[(int64_t)k * PP + key0];
+                    if (moves ? cell != d : cell != -1) errors++;
+                }
+                if (hop_src[key0] != (VC_SPACE_SEND | vc_send_offset(S, T, s0, t))) errors++;
                 for (int64_t c = 0; c < cnt; c++) {
-                    vc_chain_item(S, T, hop_src.data(), hop_dst.data(), s0, t, c, item.data());
+                    vc_chain_item(S, T, slot_off.data(), row_base.data(), s0, t, c, item.data());
                     const int64_t src = item[VC_CHAIN_SRC], plen = item[VC_CHAIN_LEN], nhop = item[VC_CHAIN_NHOP];
                     chain_items++;
                     if ((int)(src >> VC_SPACE_SHIFT) != 0 || plen <= 0 || nhop < 1) { errors++; continue; }
