@@ -225,9 +225,7 @@ static int build_plan(vc_comm *c, VcSched S, std::vector<VcLaunchInfo> &L, VcTab
     if (c->timing) { int rc = ensure_events(c, (size_t)nl + 4); if (rc) return rc; }
 
     if (c->timing) HIP_TRY(hipEventRecord(c->events[0], st));
-    if (nl <= VC_LAUNCH_PACK) {
-        HIP_TRY(vc_launch_store_launches(L.data(), nl, c->launches.as<VcLaunchInfo>(), st));
-    } else {
+    if (nl > VC_LAUNCH_PACK) {                             // a short launch table travels as a kernel argument instead
         memcpy(c->h_launches, L.data(), sizeof(VcLaunchInfo) * nl);
         HIP_TRY(hipMemcpyAsync(c->launches.p, c->h_launches, sizeof(VcLaunchInfo) * nl, hipMemcpyHostToDevice, st));
     }
@@ -236,7 +234,7 @@ static int build_plan(vc_comm *c, VcSched S, std::vector<VcLaunchInfo> &L, VcTab
         HIP_TRY(vc_launch_row_scan(T.rc, c->rd_packed.as<int>(), nullptr, P, st));
         T.rd_packed = c->rd_packed.as<int>();
     }
-    HIP_TRY(vc_launch_plan_sizes(S, c->launches.as<VcLaunchInfo>(), nl, T, c->slot_off.as<int64_t>(), c->row_tot.as<int64_t>(),
+    HIP_TRY(vc_launch_plan_sizes(S, L.data(), c->launches.as<VcLaunchInfo>(), nl, T, c->slot_off.as<int64_t>(), c->row_tot.as<int64_t>(),
                                  c->row_base.as<int64_t>(), c->org_run_base.as<int64_t>(), c->item_row_tot.as<int64_t>(),
                                  c->item_row_base.as<int64_t>(), c->row_bytes.as<int64_t>(), forward ? c->chain_row_tot.as<int64_t>() : nullptr,
                                  forward ? c->chain_row_base.as<int64_t>() : nullptr, c->header.as<int64_t>(), c->h_header_dev, st));
@@ -259,13 +257,13 @@ static int build_plan(vc_comm *c, VcSched S, std::vector<VcLaunchInfo> &L, VcTab
         out.chain_items = h[2];
         HIP_TRY(items.reserve(sizeof(int64_t) * (size_t)out.chain_stride * (size_t)std::max<int64_t>(out.chain_items, 1)));
         HIP_TRY(vc_launch_chain_plan(S, T, c->slot_off.as<int64_t>(), c->row_base.as<int64_t>(), c->chain_row_base.as<int64_t>(),
-                                     items.as<int64_t>(), st));
+                                     items.as<int64_t>(), out.chain_items, st));
         if (c->timing) HIP_TRY(hipEventRecord(c->events[1], st));
         return VC_OK;
     }
     HIP_TRY(items.reserve(sizeof(VcDesc) * (size_t)std::max<int64_t>(nitems, 1)));
-    HIP_TRY(vc_launch_plan_emit(S, c->launches.as<VcLaunchInfo>(), nl, T, c->slot_off.as<int64_t>(), c->row_base.as<int64_t>(),
-                                c->item_row_base.as<int64_t>(), c->header.as<int64_t>(), items.as<VcDesc>(), st));
+    HIP_TRY(vc_launch_plan_emit(S, L.data(), c->launches.as<VcLaunchInfo>(), nl, T, c->slot_off.as<int64_t>(), c->row_base.as<int64_t>(),
+                                c->item_row_base.as<int64_t>(), c->header.as<int64_t>(), items.as<VcDesc>(), nitems, st));
     if (c->timing) HIP_TRY(hipEventRecord(c->events[1], st));
     return VC_OK;
 }

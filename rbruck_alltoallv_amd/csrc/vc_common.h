@@ -109,21 +109,22 @@ hipError_t vc_launch_uniform_tables(int *counts, int *displs, int count, int P, 
 //   [0] staging bytes   [1] payload bytes   [2] chain items (forwarded execution)
 //   [3 + L] bytes moved by launch L   [3 + nl + L] unused on the device   [3 + 2 nl + L] work items of launch L
 #define VC_HEADER_WORDS(nl) (3 + 3 * (nl))
-// Passes 1 and 2: staging prefix sums and the number of work items of every launch (sizes only).  With chain_row_tot /
+// Passes 1 and 2: staging prefix sums and the number of work items of every launch (sizes only).  The launch table
+// travels as a kernel argument when it has at most VC_LAUNCH_PACK entries (launches_dev is then not read).  With chain_row_tot /
 // chain_row_base (P int64 each, or null) also the chain items per final receiver and their total in header[2].
-hipError_t vc_launch_plan_sizes(const VcSched &S, const VcLaunchInfo *launches_dev, int nlaunch, VcTables T, int64_t *slot_off,
+hipError_t vc_launch_plan_sizes(const VcSched &S, const VcLaunchInfo *launches_host, const VcLaunchInfo *launches_dev, int nlaunch,
+                                VcTables T, int64_t *slot_off,
                                 int64_t *row_tot, int64_t *row_base, int64_t *org_run_base, int64_t *item_row_tot,
                                 int64_t *item_row_base, int64_t *row_bytes, int64_t *chain_row_tot, int64_t *chain_row_base,
                                 int64_t *header, int64_t *header_host, hipStream_t st);
 // Forwarded execution: the chain items (every block's route in closed form, staging addresses from the plan tables).
 hipError_t vc_launch_chain_plan(const VcSched &S, VcTables T, const int64_t *slot_off, const int64_t *row_base,
-                                const int64_t *chain_row_base, int64_t *items, hipStream_t st);
-// Writes the first nl (<= VC_LAUNCH_PACK) launch descriptions to device memory from a kernel argument.
-hipError_t vc_launch_store_launches(const VcLaunchInfo *host, int nl, VcLaunchInfo *out, hipStream_t st);
+                                const int64_t *chain_row_base, int64_t *items, int64_t nitems, hipStream_t st);
 // Pass 3: writes the work items (needs the item buffer, sized from the header).
-hipError_t vc_launch_plan_emit(const VcSched &S, const VcLaunchInfo *launches_dev, int nlaunch, VcTables T, const int64_t *slot_off,
+hipError_t vc_launch_plan_emit(const VcSched &S, const VcLaunchInfo *launches_host, const VcLaunchInfo *launches_dev, int nlaunch,
+                               VcTables T, const int64_t *slot_off,
                                const int64_t *row_base, const int64_t *item_row_base, const int64_t *header, VcDesc *items,
-                               hipStream_t st);
+                               int64_t nitems, hipStream_t st);
 hipError_t vc_launch_traffic(const VcDesc *desc, int64_t ndesc, int64_t *matrix, int P, hipStream_t st);
 
 // vc_copy.hip

@@ -10,6 +10,8 @@
 // staging arena is compact; a second family of prefix sums numbers the work
 // items (block pieces of at most VC_CHUNK bytes) so that every launch gets a
 // dense list with no empty entries.
+#include <cstring>
+
 #include "vc_common.h"
 #include "vc_scan.h"
 
@@ -19,7 +21,7 @@
 // grid (P, w + w2 + nl [+ 1]).  Rows y < w + w2: staging sizes of region y, slot_off[(y*P + to)*P + id] = offset of the
 // slot inside the row.  Later rows: work-item count, moved bytes (and, for the first launch, payload)
 // of launch y - w - w2.  One more row with chain_row_tot: the chain items of forwarded execution.
-__global__ __launch_bounds__(VC_THREADS) void vc_plan_rows(VcSched S, const VcLaunchInfo *__restrict__ launches, int nl, VcTables T,
+__global__ __launch_bounds__(VC_THREADS) void vc_plan_rows(VcSched S, VcLaunchPack pack, const VcLaunchInfo *__restrict__ launches, int nl, VcTables T,
                                                            int64_t *__restrict__ slot_off, int64_t *__restrict__ row_tot,
                                                            int64_t *__restrict__ item_row_tot, int64_t *__restrict__ row_bytes,
                                                            int64_t *__restrict__ chain_row_tot) {
@@ -48,7 +50,7 @@ __global__ __launch_bounds__(VC_THREADS) void vc_plan_rows(VcSched S, const VcLa
         return;
     }
     const int L = blockIdx.y - nreg;
-    const VcLaunchInfo info = launches[L];
+    const VcLaunchInfo info = launches ? launches[L] : pack.info[L];     // a short launch table travels as a kernel argument
     int64_t items = 0, bytes = 0, payload = 0;
     const int nent = vc_entries_per_rank(S, info);
     for (int id = threadIdx.x; id < nent; id += VC_THREADS) {
@@ -154,13 +156,13 @@ __global__ __launch_bounds__(VC_THREADS) void vc_plan_bases(int P, int w, int nl
 // ---- pass 3: the work items ----
 // grid (P, nl, Z).  Repeats the row scan of pass 1 to place every block's pieces; Z workgroups share a receiver's entries
 // when there are few ranks (their blocks are then huge and have many pieces).
-__global__ __launch_bounds__(VC_THREADS) void vc_plan_emit(VcSched S, const VcLaunchInfo *__restrict__ launches, VcTables T,
+__global__ __launch_bounds__(VC_THREADS) void vc_plan_emit(VcSched S, VcLaunchPack pack, const VcLaunchInfo *__restrict__ launches, VcTables T,
                                                            const int64_t *__restrict__ slot_off, const int64_t *__restrict__ row_base,
                                                            const int64_t *__restrict__ item_row_base, const int64_t *__restrict__ header,
                                                            int nl, VcDesc *__restrict__ items) {
     __shared__ int64_t lds[VC_WAVES_PER_BLOCK];
     const int to = blockIdx.x, L = blockIdx.y, P = S.P;
-    const VcLaunchInfo info = launches[L];
+    const VcLaunchInfo info = launches ? launches[L] : pack.info[L];
     int64_t first = 0;                                    // items of the launches before this one
     for (int k = threadIdx.x; k < L; k += VC_THREADS) first += header[3 + 2 * nl + k];
     first = vc_block_sum(first, lds);
@@ -217,12 +219,29 @@ __global__ __launch_bounds__(VC_THREADS) void vc_plan_emit(VcSched S, const VcLa
     }
 }
 
-hipError_t vc_launch_plan_sizes(const VcSched &S, const VcLaunchInfo *launches_dev, int nlaunch, VcTables T, int64_t *slot_off,
+// Workgroups that share one receiver's entries when items are emitted: one per ~2048 items of an average row, so that
+// a few ranks with huge blocks (many pieces each) still fill the chip, and small problems stay one workgroup per row.
+static int vc_emit_slices(int64_t nitems, int64_t rows) {
+    const int64_t per_row = nitems / (rows > 0 ? rows : 1);
+    const int64_t z = (per_row + 2047) / 2048;
+    return (int)(z < 1 ? 1 : (z > 16 ? 16 : z));
+}
+
+static VcLaunchPack vc_pack_launches(const VcLaunchInfo *host, int nl) {
+    VcLaunchPack pack;
+    memset(&pack, 0, sizeof pack);
+    for (int k = 0; k < nl && k < VC_LAUNCH_PACK; k++) pack.info[k] = host[k];
+    return pack;
+}
+
+hipError_t vc_launch_plan_sizes(const VcSched &S, const VcLaunchInfo *launches_host, const VcLaunchInfo *launches_dev, int nlaunch,
+                                VcTables T, int64_t *slot_off,
                                 int64_t *row_tot, int64_t *row_base, int64_t *org_run_base, int64_t *item_row_tot,
                                 int64_t *item_row_base, int64_t *row_bytes, int64_t *chain_row_tot, int64_t *chain_row_base,
                                 int64_t *header, int64_t *header_host, hipStream_t st) {
     const int chain = chain_row_tot ? 1 : 0;
-    hipLaunchKernelGGL(vc_plan_rows, dim3(S.P, S.w + S.w2 + nlaunch + chain), dim3(VC_THREADS), 0, st, S, launches_dev, nlaunch, T, slot_off,
+    hipLaunchKernelGGL(vc_plan_rows, dim3(S.P, S.w + S.w2 + nlaunch + chain), dim3(VC_THREADS), 0, st, S,
+                       vc_pack_launches(launches_host, nlaunch), nlaunch <= VC_LAUNCH_PACK ? nullptr : launches_dev, nlaunch, T, slot_off,
                        row_tot, item_row_tot, row_bytes, chain_row_tot);
     if (S.coalesce)
         hipLaunchKernelGGL(vc_plan_org_rows, dim3(S.P), dim3(VC_THREADS), 0, st, S, T, slot_off, row_tot, org_run_base);
@@ -231,12 +250,13 @@ hipError_t vc_launch_plan_sizes(const VcSched &S, const VcLaunchInfo *launches_d
     return hipGetLastError();
 }
 
-hipError_t vc_launch_plan_emit(const VcSched &S, const VcLaunchInfo *launches_dev, int nlaunch, VcTables T, const int64_t *slot_off,
+hipError_t vc_launch_plan_emit(const VcSched &S, const VcLaunchInfo *launches_host, const VcLaunchInfo *launches_dev, int nlaunch,
+                               VcTables T, const int64_t *slot_off,
                                const int64_t *row_base, const int64_t *item_row_base, const int64_t *header, VcDesc *items,
-                               hipStream_t st) {
-    const int slices = S.P >= 1024 ? 1 : (S.P >= 64 ? 1024 / S.P : 16);
-    hipLaunchKernelGGL(vc_plan_emit, dim3(S.P, nlaunch, slices), dim3(VC_THREADS), 0, st, S, launches_dev, T, slot_off, row_base,
-                       item_row_base, header, nlaunch, items);
+                               int64_t nitems, hipStream_t st) {
+    const int slices = vc_emit_slices(nitems, (int64_t)S.P * nlaunch);
+    hipLaunchKernelGGL(vc_plan_emit, dim3(S.P, nlaunch, slices), dim3(VC_THREADS), 0, st, S, vc_pack_launches(launches_host, nlaunch),
+                       nlaunch <= VC_LAUNCH_PACK ? nullptr : launches_dev, T, slot_off, row_base, item_row_base, header, nlaunch, items);
     return hipGetLastError();
 }
 
@@ -299,21 +319,9 @@ __global__ __launch_bounds__(VC_THREADS) void vc_chain_emit(VcSched S, VcTables 
 }
 
 hipError_t vc_launch_chain_plan(const VcSched &S, VcTables T, const int64_t *slot_off, const int64_t *row_base,
-                                const int64_t *chain_row_base, int64_t *items, hipStream_t st) {
-    const int slices = S.P >= 1024 ? 1 : (S.P >= 64 ? 1024 / S.P : 16);      // about a thousand workgroups at least
+                                const int64_t *chain_row_base, int64_t *items, int64_t nitems, hipStream_t st) {
+    const int slices = vc_emit_slices(nitems, S.P);
     hipLaunchKernelGGL(vc_chain_emit, dim3(S.P, slices), dim3(VC_THREADS), 0, st, S, T, slot_off, row_base, chain_row_base, items);
-    return hipGetLastError();
-}
-
-// ---- the launch table travels as a kernel argument when it is short (no host-to-device copy) ----
-__global__ void vc_store_launches_kernel(VcLaunchPack pack, int nl, VcLaunchInfo *__restrict__ out) {
-    if ((int)threadIdx.x < nl) out[threadIdx.x] = pack.info[threadIdx.x];
-}
-
-hipError_t vc_launch_store_launches(const VcLaunchInfo *host, int nl, VcLaunchInfo *out, hipStream_t st) {
-    VcLaunchPack pack;
-    for (int k = 0; k < nl; k++) pack.info[k] = host[k];
-    hipLaunchKernelGGL(vc_store_launches_kernel, dim3(1), dim3(VC_LAUNCH_PACK), 0, st, pack, nl, out);
     return hipGetLastError();
 }
 
