@@ -202,8 +202,8 @@ int vc_plan_free(vc_plan_t plan);
 /* ---- radix choice.  The reference leaves r to the caller (its drivers sweep a list of bases,
  * examples/rbruckv_example.cpp:33-35).  Given candidate radices this evaluates, on the device, the bytes each would
  * move (sum over blocks of hops x bytes; hops = non-zero base-r digits of the offset inside the node, + 1 if the node
- * differs) and returns the candidate with the smallest modelled time 2 * moved / (sustained copy rate) + launches x
- * launch latency.  n = ranks per node for the two-layer functions, 0 or P for the one-layer ones.  `candidates` and the
+ * differs) and returns the candidate with the smallest modelled time: 2 * moved / (sustained copy rate) + launches x
+ * launch latency for one launch per digit, moved / rate (one write per hop, one launch) for forwarded execution.  n = ranks per node for the two-layer functions, 0 or P for the one-layer ones.  `candidates` and the
  * outputs are HOST arrays; moved_bytes_out (may be NULL) receives the moved bytes per candidate. ---- */
 int vc_suggest_radix(const int *sendcounts, int elem_size, int n, const int *candidates, int ncand, int *best_out,
                      int64_t *moved_bytes_out, vc_comm_t comm);

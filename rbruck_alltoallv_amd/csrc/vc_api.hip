@@ -365,11 +365,6 @@ static int schedule_error(int code) {
     return code;
 }
 
-static bool use_forwarding(const vc_comm *c, int P, int r_hint) {
-    (void)P; (void)r_hint;
-    return c->forward;
-}
-
 // The alltoallv-shaped functions.
 static int run_v(VcFunc f, int n, int r, int batch, vc_comm *c, char *sendbuf, int *sendcounts, int *sdispls, int esz,
                  char *recvbuf, int *recvcounts, int *rdispls, int batch2 = 0) {
@@ -378,7 +373,7 @@ static int run_v(VcFunc f, int n, int r, int batch, vc_comm *c, char *sendbuf, i
     if (!sendcounts || !sdispls || !recvcounts || (f != VC_F_TTPL && !rdispls)) return fail_arg("null table");
     VcSched S;
     std::vector<VcLaunchInfo> L;
-    const bool forward = use_forwarding(c, c->P, r);
+    const bool forward = c->forward;
     rc = vc_make_schedule(f, c->P, n, r, batch, esz, 0, S, L, batch2, forward);
     if (rc) return schedule_error(rc);
     S.recv_lo = (int)((uintptr_t)recvbuf & 4095);
@@ -482,7 +477,7 @@ static int run_uniform(VcFunc f, int n, int r, vc_comm *c, char *sendbuf, int se
     if ((int64_t)sendcount * c->P > 0x7FFFFFFF) return fail_arg("sendcount * P must fit the reference's int displacements");
     VcSched S;
     std::vector<VcLaunchInfo> L;
-    const bool forward = use_forwarding(c, c->P, r);
+    const bool forward = c->forward;
     rc = vc_make_schedule(f, c->P, n, r, 0, esz, sendcount, S, L, 0, forward);
     if (rc) return schedule_error(rc);
     S.recv_lo = (int)((uintptr_t)recvbuf & 4095);
@@ -536,7 +531,7 @@ extern "C" int vc_plan_create(const char *function, int n, int r, int batch, int
     if (!sendcounts || !sdispls || !recvcounts || (f != VC_F_TTPL && !rdispls)) return fail_arg("null table");
     VcSched S;
     std::vector<VcLaunchInfo> L;
-    const bool forward = use_forwarding(c, c->P, r);
+    const bool forward = c->forward;
     int rc = vc_make_schedule(f, c->P, n, r, batch, elem_size, 0, S, L, 0, forward);
     if (rc) return schedule_error(rc);
     S.recv_lo = recvbuf_low_bits & 4095;
@@ -606,12 +601,15 @@ extern "C" int vc_suggest_radix(const int *sendcounts, int elem_size, int n, con
     unsigned long long moved[64];
     HIP_TRY(hipMemcpyAsync(moved, moved_dev, sizeof(unsigned long long) * ncand, hipMemcpyDeviceToHost, c->stream));
     HIP_TRY(hipStreamSynchronize(c->stream));
-    // time model: every moved byte is read and written once at the rate the copy kernel sustains on scattered
-    // blocks, every launch costs a fixed latency
+    // time model, at the rate the copy kernels sustain on scattered blocks.  One launch per digit: every moved byte is
+    // read and written once and every launch costs a fixed latency.  Forwarded execution: one launch; every byte is
+    // written once per hop, and read only once (moved[k] counts one payload for every hop, so the payload itself is the
+    // same for all candidates and drops out of the comparison).
     const double bytes_per_s = 5.2e12, launch_s = 7e-6;
     double best = 0;
     for (int k = 0; k < ncand; k++) {
-        const double t = 2.0 * (double)moved[k] / bytes_per_s + launch_s * launches_for(n, cand[k], n < P);
+        const double t = c->forward ? (double)moved[k] / bytes_per_s
+                                    : 2.0 * (double)moved[k] / bytes_per_s + launch_s * launches_for(n, cand[k], n < P);
         if (moved_bytes_out) moved_bytes_out[k] = (int64_t)moved[k];
         if (k == 0 || t < best) { best = t; *best_out = candidates[k]; }
     }
