@@ -22,8 +22,10 @@ def build() -> str:
     deps = [SRC] + [os.path.join(CSRC, f) for f in ("vc_plan_math.h", "vc_sched.h", "vc_common.h")]
     if not os.path.exists(LIB) or os.path.getmtime(LIB) < max(os.path.getmtime(d) for d in deps):
         os.makedirs(os.path.dirname(LIB), exist_ok=True)
-        subprocess.run(["/opt/rocm/bin/hipcc", "-O1", "-g", "-std=c++17", "-fPIC", "-shared", "-o", LIB, SRC],
+        tmp = f"{LIB}.{os.getpid()}.tmp"                      # parallel test workers may build at the same time
+        subprocess.run(["/opt/rocm/bin/hipcc", "-O1", "-g", "-std=c++17", "-fPIC", "-shared", "-o", tmp, SRC],
                        check=True, capture_output=True)
+        os.replace(tmp, LIB)
     return LIB
 
 
