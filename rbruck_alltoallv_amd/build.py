@@ -26,22 +26,27 @@ def build_library(verbose: bool = False) -> str:
     return LIB_PATH
 
 
-EXAMPLE_SRC = os.path.join(PKG_DIR, "examples", "vc_example.cpp")
+EXAMPLES = ("vc_example", "vc_mlinputs_example")
 EXAMPLE_BIN = os.path.join(PKG_DIR, "examples", "vc_example")
+MLINPUTS_EXAMPLE_BIN = os.path.join(PKG_DIR, "examples", "vc_mlinputs_example")
 
 
-def build_example(verbose: bool = False) -> str:
-    """The C++ driver above the C ABI (host code only; links the library next to it)."""
-    cmd = [HIPCC, "-O2", "-std=c++17", "-Wall", "-x", "hip", "--offload-arch=gfx950", "-Xclang", "-target-feature", "-Xclang",
-           "-packed-fp32-ops", EXAMPLE_SRC, "-L" + PKG_DIR, "-lrbruck_vc", "-Wl,-rpath,$ORIGIN/..", "-o", EXAMPLE_BIN]
-    res = subprocess.run(cmd, capture_output=True, text=True)
-    if verbose or res.returncode != 0:
-        print(" ".join(cmd))
-        print(res.stdout)
-        print("\n".join(l for l in res.stderr.splitlines() if "packed-fp32-ops" not in l))
-    if res.returncode != 0:
-        raise RuntimeError("hipcc failed building examples/vc_example")
-    return EXAMPLE_BIN
+def build_example(verbose: bool = False) -> list[str]:
+    """The C++ drivers above the C ABI (host code only; they link the library next to them)."""
+    built = []
+    for name in EXAMPLES:
+        src, out = os.path.join(PKG_DIR, "examples", name + ".cpp"), os.path.join(PKG_DIR, "examples", name)
+        cmd = [HIPCC, "-O2", "-std=c++17", "-Wall", "-x", "hip", "--offload-arch=gfx950", "-Xclang", "-target-feature", "-Xclang",
+               "-packed-fp32-ops", src, "-L" + PKG_DIR, "-lrbruck_vc", "-Wl,-rpath,$ORIGIN/..", "-o", out]
+        res = subprocess.run(cmd, capture_output=True, text=True)
+        if verbose or res.returncode != 0:
+            print(" ".join(cmd))
+            print(res.stdout)
+            print("\n".join(l for l in res.stderr.splitlines() if "packed-fp32-ops" not in l))
+        if res.returncode != 0:
+            raise RuntimeError(f"hipcc failed building examples/{name}")
+        built.append(out)
+    return built
 
 
 if __name__ == "__main__":
