@@ -346,6 +346,9 @@ static int check_common(vc_comm *c, const void *sendbuf, const void *recvbuf, in
     if (!sendbuf || !recvbuf) return fail_arg("null buffer");
     if (esz < 1) return fail_arg("element size must be >= 1");
     if (!c->sbase || !c->rbase) return fail_arg("vc_comm_set_bases has not been called");
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev != c->device)
+        return fail_arg("the communicator was created on another HIP device than the current one");
     return VC_OK;
 }
 
