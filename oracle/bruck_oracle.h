@@ -20,7 +20,9 @@
  * its round structure against the closed forms for K, ns and the residency
  * invariants.  No function is "parity unpinned"; ora_tuna2_algorithm is pinned by
  * the reference for b = 1 and by the definition for b > 1, where the reference
- * itself is defective.
+ * itself is defective; ora_TTPL_rbruck_alltoallv is pinned by the reference for
+ * the blocks that stay inside a node (the reference drops the others after
+ * exchanging them) and by the definition for all of them.
  */
 #ifndef BRUCK_ORACLE_H_
 #define BRUCK_ORACLE_H_
