@@ -316,8 +316,8 @@ VC_HD VcDesc vc_chunk_of(const VcDesc &whole, int64_t c, int phase, int cut) {
 // ---- forwarded execution: one work item carries a piece of a block through all its hops ----
 // The hops of one block depend only on each other: hop k + 1 reads what hop k wrote.  When one workgroup performs all
 // of them it keeps the piece in registers between the hops: the data is read once (from sendbuf) and written once per
-// hop (to the staging slot of every intermediate holder, then to recvbuf).  Memory ends up exactly as after the
-// launch-per-digit execution.
+// hop (to the staging slot of every intermediate holder, then to recvbuf).  Every block ends up in the same places as
+// after the launch-per-digit execution.
 //
 // A block moves at most once per digit, so its hops are indexed by "hop slots": intra-node digit x, inter-node digit
 // S.w + x, and one last slot for what goes straight to recvbuf by an inter-node or direct message (or stays on its rank).
@@ -325,6 +325,8 @@ VC_HD VcDesc vc_chunk_of(const VcDesc &whole, int64_t c, int phase, int cut) {
 
 VC_HD int vc_hop_slots(const VcSched &S) { return S.w + S.w2 + 1; }
 
+// Hop slot of an entry of a launch (the CPU check of the plan derives every block's route from the launches' entries
+// this way and compares it with vc_block_hop).
 VC_HD int vc_hop_slot(const VcSched &S, const VcLaunchInfo &info, const VcEntry &e) {
     if (e.s == e.t) return S.w + S.w2;
     return info.kind == 0 ? info.x : (info.kind == 4 ? S.w + info.x : S.w + S.w2);
