@@ -38,3 +38,22 @@ def test_stats_struct_layout_matches_header():
     text = open(os.path.join(ROOT, "include", "rbruck_vc.h")).read()
     assert f"#define VC_MAX_LAUNCHES {_lib.VC_MAX_LAUNCHES}" in text
     assert ctypes.sizeof(_lib.VcStats) == 8 + 3 * 8 + 2 * 4 + _lib.VC_MAX_LAUNCHES * (8 + 4)
+
+
+def test_argument_errors_need_no_gpu():
+    """Entry points reject bad arguments before touching the device; without a HIP device vc_comm_create says so."""
+    lib = _lib.load()
+    handle = ctypes.c_void_p()
+    assert lib.vc_comm_create(0, ctypes.byref(handle)) == -5                 # VC_ERR_ARG: nranks < 1
+    assert b"nranks" in lib.vc_last_error_string()
+    rc = lib.vc_comm_create(4, ctypes.byref(handle))
+    assert rc in (0, -6)                                                      # VC_OK on a GPU box, VC_ERR_NO_DEVICE here
+    if rc == 0:
+        assert lib.vc_comm_size(handle) == 4
+        assert lib.vc_comm_free(handle) == 0
+    else:
+        assert b"no HIP device" in lib.vc_last_error_string()
+    assert lib.vc_comm_size(None) == -5
+    assert lib.vc_comm_set_forwarding(None, 1) == -5
+    assert lib.twophase_rbruck_alltoallv(2, None, None, None, 1, None, None, None, 1, None) == -5
+    assert lib.vc_plan_execute(None, None, None) == -5
