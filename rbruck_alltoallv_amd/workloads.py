@@ -94,6 +94,53 @@ def counts_fft_rows(P: int, row_len: int, count: int) -> np.ndarray:
     return np.where(row[:, None] == row[None, :], count, 0).astype(np.int32)
 
 
+def _row_shuffle(rows: np.ndarray, seed: int) -> np.ndarray:
+    """Every row shuffled on its own (the reference's drivers std::shuffle each rank's sendcounts with a time seed;
+    here the order comes from the hash)."""
+    P = rows.shape[0]
+    s, d = np.meshgrid(np.arange(P, dtype=np.uint64), np.arange(rows.shape[1], dtype=np.uint64), indexing="ij")
+    order = np.argsort(hash4(seed, s, d, 7), axis=1, kind="stable")
+    return np.take_along_axis(rows, order, axis=1)
+
+
+def counts_truncated_normal_rows(P: int, mean: float, deviation: float, max_value: int, seed: int = 0) -> np.ndarray:
+    """examples/other_distributions.cpp:70-88 (dist 0): every rank draws P counts from Normal(mean, deviation), redrawing
+    values outside [0, max_value], then shuffles them."""
+    s, d = np.meshgrid(np.arange(P, dtype=np.uint64), np.arange(P, dtype=np.uint64), indexing="ij")
+    out = np.full((P, P), -1.0)
+    for attempt in range(64):
+        todo = (out < 0) | (out > max_value)
+        if not todo.any():
+            break
+        u1 = ((hash4(seed + 2 * attempt, s, d, 1) >> np.uint64(11)).astype(np.float64) + 1.0) / 9007199254740992.0
+        u2 = (hash4(seed + 2 * attempt + 1, s, d, 2) >> np.uint64(11)).astype(np.float64) / 9007199254740992.0
+        z = np.sqrt(-2.0 * np.log(u1)) * np.cos(2.0 * np.pi * u2)
+        out = np.where(todo, mean + deviation * z, out)
+    out = np.clip(out, 0, max_value)
+    return _row_shuffle(out.astype(np.int32), seed)
+
+
+def counts_power_law_rows(P: int, x: float, max_value: int, seed: int = 0) -> np.ndarray:
+    """examples/other_distributions.cpp:91-103 (dist 1): counts max_value * x^k, k = 0 .. P-1, shuffled per rank."""
+    row = (max_value * np.power(float(x), np.arange(P))).astype(np.int32)
+    return _row_shuffle(np.tile(row, (P, 1)), seed)
+
+
+def counts_sparse_blocks(P: int, xzero: float, yzero: float, number: int, last: int = 0) -> np.ndarray:
+    """examples/FFT_distribution.cpp:68-87: the first ranks send `number` elements to the first destinations, a share
+    xzero of the destinations and yzero of the ranks stays empty; with last > 0 every rank sends `number` to all but
+    the last destination, which gets `last`."""
+    counts = np.zeros((P, P), dtype=np.int32)
+    if last == 0:
+        number_count = P - int(np.ceil(P * xzero))
+        rank_count = P - int(np.ceil(P * yzero))
+        counts[:rank_count, :number_count] = number
+    else:
+        counts[:, :P - 1] = number
+        counts[:, P - 1] = last
+    return counts
+
+
 def counts_from_text(path: str) -> np.ndarray:
     """Whitespace-separated P x P matrix, row = sender (the layout of the reference's
     inputs/<P>proc/global_comm_pattern_<P>proc.txt, read by examples/MLinputs_example.cpp:119-145)."""

@@ -484,6 +484,19 @@ def test_more_than_4096_ranks(api):
     dp.comm.free()
 
 
+def test_distributions_of_the_reference_drivers(api):
+    """examples/other_distributions.cpp (truncated normal, power law) and examples/FFT_distribution.cpp (sparse blocks) at
+    256 ranks, 8-byte elements, through the functions those drivers call."""
+    for name, counts in (("truncated normal", W.counts_truncated_normal_rows(256, 600.0, 250.0, 1500, seed=1)),
+                         ("power law", W.counts_power_law_rows(256, 0.98, 4000, seed=2)),
+                         ("sparse blocks", W.counts_sparse_blocks(256, 0.4, 0.25, 777)),
+                         ("last block differs", W.counts_sparse_blocks(256, 0.0, 0.0, 50, last=90001))):
+        _device_check(api, W.make_problem(counts, 8, 0, 0), 6, lambda dp, ds: [
+            (f"{name}: twophase r=16", lambda d: api.twophase_rbruck_alltoallv(16, dp, ds, d), False),
+            (f"{name}: s1 n=16 r=4", lambda d: api.TTPL_BT_alltoallv_s1(16, 4, 0, dp, ds, d), False),
+            (f"{name}: ttpl n=32 r=32", lambda d: api.TTPL_BT_alltoallv(32, 32, 0, dp, ds, d), True)])
+
+
 def test_reference_input_matrices(api):
     """The reference's own communication patterns (inputs/<P>proc), scaled down, through the function its driver uses."""
     import os

@@ -463,3 +463,28 @@ def test_forwarded_large_blocks_and_unaligned_recvbuf(forwarded):
             assert res.rc == 0 and res.errors == 0, (func, recv_lo, res.errors)
             assert np.array_equal(recv, want)
             assert res.items > 12 * 12
+
+
+@pytest.mark.parametrize("name,counts", [
+    ("truncated normal", lambda: W.counts_truncated_normal_rows(24, 300.0, 120.0, 700, seed=1)),
+    ("power law", lambda: W.counts_power_law_rows(24, 0.8, 900, seed=2)),
+    ("sparse blocks", lambda: W.counts_sparse_blocks(24, 0.4, 0.25, 37)),
+    ("last block differs", lambda: W.counts_sparse_blocks(24, 0.0, 0.0, 5, last=401))])
+def test_distributions_of_the_reference_drivers(name, counts):
+    """The count distributions of examples/other_distributions.cpp and examples/FFT_distribution.cpp, 8-byte elements as
+    there, through the functions those drivers call — in both execution modes, against the oracle and the definition."""
+    c = counts()
+    assert c.shape == (24, 24) and c.min() >= 0
+    prob = W.make_problem(c, 8, 0, 0)
+    send = W.fill_send_arena(prob, 0, 3)
+    want = W.expected_recv_arena(prob, send)
+    for forward in (False, True):
+        for func, kw, ofn in ((E.F_TWOPHASE, dict(r=4), lambda d: O.twophase_rbruck_alltoallv(4, prob, send, d)),
+                              (E.F_TTPL_S1, dict(n=6, r=3, batch=4), lambda d: O.TTPL_BT_alltoallv_s1(6, 3, 4, prob, send, d)),
+                              (E.F_TTPL, dict(n=4, r=2, batch=0), lambda d: O.TTPL_BT_alltoallv(4, 2, 0, prob, send, d))):
+            recv = np.full(prob.recv_bytes, 0xEE, dtype=np.uint8)
+            res = E.emulate(func, prob, send, recv, forward=forward, **kw)
+            assert res.rc == 0 and res.errors == 0, (name, func, forward)
+            assert np.array_equal(recv, want)
+            ref = np.full(prob.recv_bytes, 0xEE, dtype=np.uint8)
+            assert ofn(ref) == 0 and np.array_equal(ref, want)
