@@ -2,7 +2,8 @@
 //
 // One process plays all ranks.  The loop structure, the payload (element = destination + 10 * source), the sweep
 // over block sizes (n = 2 .. 2048 elements of 8 bytes, a random share of n per pair) and the result lines follow
-// examples/rbruckv_example.cpp:49-131 and examples/twophaseLayer_example.cpp:48-225 of the reference; where those
+// examples/rbruckv_example.cpp:49-131, examples/twophaseLayer_example.cpp:48-225 and, for the equal-block functions,
+// examples/twolayer_example.cpp:49-140 of the reference; where those
 // call MPI_Alltoall / the displacement loops / a collective, this calls the function of librbruck_vc that replaces it.
 // The error check compares every received element with the value its sender wrote (the reference's check_errors,
 // src/utils.cpp:31-46, only tests the last decimal digit).
@@ -135,6 +136,45 @@ int main(int argc, char **argv) {
             }
         }
         CHECK_HIP(hipFree(sendbuf)); CHECK_HIP(hipFree(recvbuf));
+
+        // examples/twolayer_example.cpp:49-140: the equal-block functions, n elements per pair
+        if (ncores >= 2 && ncores < P && P % ncores == 0 && (long long)n * P <= 0x7FFFFFFF) {
+            std::vector<int64_t> h_ext((size_t)P, (int64_t)P * n);
+            CHECK_HIP(hipMemcpy(ext, h_ext.data(), sizeof(int64_t) * P, hipMemcpyHostToDevice));
+            CHECK_VC(vc_bases_from_extents(ext, esz, 256, sbase, total, comm));
+            CHECK_VC(vc_bases_from_extents(ext, esz, 256, rbase, total + 1, comm));
+            CHECK_HIP(hipMemcpy(h_total, total, sizeof h_total, hipMemcpyDeviceToHost));
+            CHECK_HIP(hipMemcpy(h_sbase.data(), sbase, sizeof(int64_t) * P, hipMemcpyDeviceToHost));
+            CHECK_VC(vc_comm_set_bases(comm, sbase, rbase));            // same layout on both sides
+            std::vector<elem_t> u_send((size_t)h_total[0] / esz + 1, 0), u_recv((size_t)h_total[1] / esz + 1);
+            for (int s = 0; s < P; s++)
+                for (int d = 0; d < P; d++)
+                    for (int k = 0; k < n; k++) u_send[h_sbase[s] / esz + (size_t)d * n + k] = (elem_t)d + (elem_t)s * 10;
+            char *usend, *urecv;
+            CHECK_HIP(hipMalloc(&usend, h_total[0] + 16)); CHECK_HIP(hipMalloc(&urecv, h_total[1] + 16));
+            CHECK_HIP(hipMemcpy(usend, u_send.data(), h_total[0], hipMemcpyHostToDevice));
+            auto timed_uniform = [&](const char *tag, int base, const std::function<int()> &call) {
+                for (int it = 0; it < loopcount; it++) {
+                    CHECK_HIP(hipMemset(urecv, 0, h_total[1]));
+                    const auto st = std::chrono::steady_clock::now();
+                    const int rcode = call();
+                    const double t = std::chrono::duration<double>(std::chrono::steady_clock::now() - st).count();
+                    if (rcode != 0) { printf("%s fail! (%d: %s)\n", tag, rcode, vc_last_error_string()); errors++; continue; }
+                    CHECK_HIP(hipMemcpy(u_recv.data(), urecv, h_total[1], hipMemcpyDeviceToHost));
+                    long long bad = 0;
+                    for (int t_ = 0; t_ < P; t_++)
+                        for (int s = 0; s < P; s++)
+                            for (int k = 0; k < n; k++) bad += u_recv[h_sbase[t_] / esz + (size_t)s * n + k] != (elem_t)t_ + (elem_t)s * 10;
+                    if (bad) { printf("[%s] %d has errors %lld\n", tag, base, bad); errors += bad; }
+                    printf("[%s] %d, %d, %d, %g\n", tag, P, n, base, t);
+                }
+            };
+            for (int base : bases) {
+                timed_uniform("SOR_alltoall", base, [&] { return uniform_spreadout_twolayer(ncores, base, usend, n, esz, urecv, n, esz, comm); });
+                timed_uniform("BR_alltoall", base, [&] { return uniform_inverse_isplit_r_bruck(ncores, base, base, usend, n, esz, urecv, n, esz, comm); });
+            }
+            CHECK_HIP(hipFree(usend)); CHECK_HIP(hipFree(urecv));
+        }
     }
     printf("errors: %lld\n", errors);
     vc_comm_free(comm);

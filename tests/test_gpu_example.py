@@ -26,6 +26,8 @@ def test_example_driver_reports_no_errors(P, ncores, bases):
     assert sum(l.startswith("[TTPL_S1]") for l in lines) == sizes * len(bases)
     assert sum(l.startswith("[Spreadout]") for l in lines) == sizes
     assert sum(l.startswith("[ExcOr]") for l in lines) == (sizes if P & (P - 1) == 0 else 0)
+    assert sum(l.startswith("[SOR_alltoall]") for l in lines) == sizes * len(bases)      # the equal-block functions
+    assert sum(l.startswith("[BR_alltoall]") for l in lines) == sizes * len(bases)
 
 
 def test_mlinputs_driver_reads_the_reference_text_format(tmp_path):
