@@ -40,6 +40,9 @@ typedef struct vc_comm *vc_comm_t;
 #define VC_ERR_HIP (-4)        /* a HIP runtime call failed; vc_last_error_string() says which */
 #define VC_ERR_ARG (-5)        /* null handle / pointer, element size < 1, bases not set */
 #define VC_ERR_NO_DEVICE (-6)  /* no HIP device */
+#define VC_ERR_TABLES (-7)     /* a negative count or displacement in the tables (found on the device before anything is copied) */
+#define VC_ERR_OVERFLOW (-8)   /* vc_displs_from_counts: a rank's counts sum past INT_MAX elements, where the reference's int
+                                  displacements wrap (examples/rbruckv_example.cpp:69-72) */
 
 /* ---- communicator (replaces MPI_Comm; MPI_Comm_size/MPI_Comm_rank have no per-rank analogue) ---- */
 
@@ -77,7 +80,8 @@ const char *vc_last_error_string(void);
 int vc_alltoall_counts(const int *sendcounts, int *recvcounts, vc_comm_t comm);
 
 /* Exclusive prefix sum of every rank's counts (examples/rbruckv_example.cpp:69-72,77-82): displs[p][i] =
- * sum_{k<i} counts[p][k].  extent_out (may be NULL) receives each rank's total, P int64 elements. */
+ * sum_{k<i} counts[p][k].  extent_out (may be NULL) receives each rank's total, P int64 elements.  Returns VC_ERR_TABLES
+ * for a negative count and VC_ERR_OVERFLOW when a total does not fit an int (displs and extent_out are written anyway). */
 int vc_displs_from_counts(const int *counts, int *displs, int64_t *extent_out, vc_comm_t comm);
 
 /* Packed arena bases: base[p] = sum_{q<p} roundup(extent[q] * elem_size, align); total_out (device, 1 int64,

@@ -157,8 +157,14 @@ extern "C" int vc_alltoall_counts(const int *sendcounts, int *recvcounts, vc_com
 
 extern "C" int vc_displs_from_counts(const int *counts, int *displs, int64_t *extent_out, vc_comm_t c) {
     if (!c || !counts || !displs) return fail_arg("vc_displs_from_counts: null argument");
-    HIP_TRY(vc_launch_row_scan(counts, displs, extent_out, c->P, c->stream));
+    HIP_TRY(c->scratch.reserve(2 * sizeof(int)));
+    int flags[2] = {0, 0};
+    HIP_TRY(hipMemsetAsync(c->scratch.p, 0, sizeof flags, c->stream));
+    HIP_TRY(vc_launch_row_scan(counts, displs, extent_out, c->scratch.as<int>(), c->P, c->stream));
+    HIP_TRY(hipMemcpyAsync(flags, c->scratch.p, sizeof flags, hipMemcpyDeviceToHost, c->stream));
     HIP_TRY(hipStreamSynchronize(c->stream));
+    if (flags[1]) return fail_arg("vc_displs_from_counts: negative count", VC_ERR_TABLES);
+    if (flags[0]) return fail_arg("vc_displs_from_counts: a rank's counts sum past INT_MAX elements", VC_ERR_OVERFLOW);
     return VC_OK;
 }
 
@@ -214,7 +220,7 @@ static int build_plan(vc_comm *c, VcSched S, std::vector<VcLaunchInfo> &L, VcTab
     HIP_TRY(c->org_run_base.reserve(sizeof(int64_t) * (size_t)P * std::max(S.G, 1)));
     HIP_TRY(c->item_row_tot.reserve(sizeof(int64_t) * (size_t)P * nl));
     HIP_TRY(c->item_row_base.reserve(sizeof(int64_t) * (size_t)P * nl));
-    HIP_TRY(c->row_bytes.reserve(sizeof(int64_t) * (size_t)P * (nl + 1)));
+    HIP_TRY(c->row_bytes.reserve(sizeof(int64_t) * (size_t)P * (nl + 2)));
     HIP_TRY(c->header.reserve(sizeof(int64_t) * VC_HEADER_WORDS(VC_MAX_LAUNCHES)));
     HIP_TRY(c->launches.reserve(sizeof(VcLaunchInfo) * VC_MAX_LAUNCHES));
     if (forward) {
@@ -231,7 +237,7 @@ static int build_plan(vc_comm *c, VcSched S, std::vector<VcLaunchInfo> &L, VcTab
     }
     if (S.packed_recv) {
         HIP_TRY(c->rd_packed.reserve(sizeof(int) * PP));
-        HIP_TRY(vc_launch_row_scan(T.rc, c->rd_packed.as<int>(), nullptr, P, st));
+        HIP_TRY(vc_launch_row_scan(T.rc, c->rd_packed.as<int>(), nullptr, nullptr, P, st));
         T.rd_packed = c->rd_packed.as<int>();
     }
     HIP_TRY(vc_launch_plan_sizes(S, L.data(), c->launches.as<VcLaunchInfo>(), nl, T, c->slot_off.as<int64_t>(), c->row_tot.as<int64_t>(),
@@ -241,6 +247,8 @@ static int build_plan(vc_comm *c, VcSched S, std::vector<VcLaunchInfo> &L, VcTab
     HIP_TRY(hipStreamSynchronize(st));     // the staging arena and the item list are sized from the plan
 
     const int64_t *h = c->h_header;
+    if (h[3 + nl] != 0)       // nothing has been copied yet: such tables would send the copy kernels outside the arenas
+        return fail_arg("negative entries in sendcounts / sdispls / recvcounts / rdispls", VC_ERR_TABLES);
     out.nl = nl; out.n_digits = S.w + S.w2; out.recv_lo = S.recv_lo;
     out.stage_bytes = h[0]; out.payload_bytes = h[1];
     out.first.assign(nl, 0); out.count.assign(nl, 0); out.bytes.assign(nl, 0);
@@ -655,7 +663,7 @@ extern "C" int vc_verify_alltoallv(const char *sendbuf, const int *sendcounts, c
     VcTables T = make_tables(c, sendcounts, sdispls, recvcounts, rdispls);
     if (packed_recv) {
         HIP_TRY(c->rd_packed.reserve(sizeof(int) * PP));
-        HIP_TRY(vc_launch_row_scan(recvcounts, c->rd_packed.as<int>(), nullptr, c->P, c->stream));
+        HIP_TRY(vc_launch_row_scan(recvcounts, c->rd_packed.as<int>(), nullptr, nullptr, c->P, c->stream));
         T.rd_packed = c->rd_packed.as<int>();
     }
     HIP_TRY(c->scratch.reserve(sizeof(int64_t) * PP));

@@ -93,7 +93,8 @@ struct VcTables {
 
 // vc_meta.hip
 hipError_t vc_launch_transpose(const int *in, int *out, int P, hipStream_t st);
-hipError_t vc_launch_row_scan(const int *counts, int *displs, int64_t *extent, int P, hipStream_t st);
+// flags (device, 2 ints the caller has zeroed, or null): [0] set when a row's total passes INT_MAX, [1] when a count is negative
+hipError_t vc_launch_row_scan(const int *counts, int *displs, int64_t *extent, int *flags, int P, hipStream_t st);
 hipError_t vc_launch_bases(const int64_t *extent, int esz, int64_t align, int64_t *base, int64_t *total, int P, hipStream_t st);
 hipError_t vc_launch_max(const int *counts, int *out, int64_t nelem, hipStream_t st);
 hipError_t vc_launch_fill_payload(int mode, uint64_t seed, char *sendbuf, const int *sc, const int *sd, const int64_t *sbase,
@@ -107,7 +108,8 @@ hipError_t vc_launch_uniform_tables(int *counts, int *displs, int count, int P, 
 // vc_plan.hip
 // header layout (int64), nl = number of launches:
 //   [0] staging bytes   [1] payload bytes   [2] chain items (forwarded execution)
-//   [3 + L] bytes moved by launch L   [3 + nl + L] unused on the device   [3 + 2 nl + L] work items of launch L
+//   [3 + L] bytes moved by launch L   [3 + nl] negative entries found in the count / displacement tables
+//   [3 + 2 nl + L] work items of launch L
 #define VC_HEADER_WORDS(nl) (3 + 3 * (nl))
 // Passes 1 and 2: staging prefix sums and the number of work items of every launch (sizes only).  The launch table
 // travels as a kernel argument when it has at most VC_LAUNCH_PACK entries (launches_dev is then not read).  With chain_row_tot /

@@ -41,7 +41,7 @@ hipError_t vc_launch_transpose(const int *in, int *out, int P, hipStream_t st) {
 // rows longer than the workgroup.
 // ---------------------------------------------------------------------------
 __global__ __launch_bounds__(VC_THREADS) void vc_row_scan_kernel(const int *__restrict__ counts, int *__restrict__ displs,
-                                                                 int64_t *__restrict__ extent, int P) {
+                                                                 int64_t *__restrict__ extent, int *__restrict__ flags, int P) {
     __shared__ int64_t lds[VC_WAVES_PER_BLOCK];
     const int p = blockIdx.x;
     int64_t carry = 0;
@@ -50,13 +50,16 @@ __global__ __launch_bounds__(VC_THREADS) void vc_row_scan_kernel(const int *__re
         int64_t v = (i < P) ? counts[(int64_t)p * P + i] : 0, total;
         int64_t ex = vc_block_exclusive_scan(v, lds, total);
         if (i < P) displs[(int64_t)p * P + i] = (int)(carry + ex);
+        if (flags && v < 0) flags[1] = 1;                 // a negative count
         carry += total;
     }
     if (extent && threadIdx.x == 0) extent[p] = carry;
+    // the last displacement is the largest when no count is negative
+    if (flags && threadIdx.x == 0 && carry > 0x7FFFFFFFll) flags[0] = 1;
 }
 
-hipError_t vc_launch_row_scan(const int *counts, int *displs, int64_t *extent, int P, hipStream_t st) {
-    hipLaunchKernelGGL(vc_row_scan_kernel, dim3(P), dim3(VC_THREADS), 0, st, counts, displs, extent, P);
+hipError_t vc_launch_row_scan(const int *counts, int *displs, int64_t *extent, int *flags, int P, hipStream_t st) {
+    hipLaunchKernelGGL(vc_row_scan_kernel, dim3(P), dim3(VC_THREADS), 0, st, counts, displs, extent, flags, P);
     return hipGetLastError();
 }
 

@@ -19,8 +19,8 @@
 
 // ---- pass 1: row-wise prefix sums ----
 // grid (P, w + w2 + nl [+ 1]).  Rows y < w + w2: staging sizes of region y, slot_off[(y*P + to)*P + id] = offset of the
-// slot inside the row.  Later rows: work-item count, moved bytes (and, for the first launch, payload)
-// of launch y - w - w2.  One more row with chain_row_tot: the chain items of forwarded execution.
+// slot inside the row.  Later rows: work-item count, moved bytes (and, for the first launch, payload and the number of
+// negative table entries) of launch y - w - w2.  One more row with chain_row_tot: the chain items of forwarded execution.
 __global__ __launch_bounds__(VC_THREADS) void vc_plan_rows(VcSched S, VcLaunchPack pack, const VcLaunchInfo *__restrict__ launches, int nl, VcTables T,
                                                            int64_t *__restrict__ slot_off, int64_t *__restrict__ row_tot,
                                                            int64_t *__restrict__ item_row_tot, int64_t *__restrict__ row_bytes,
@@ -61,15 +61,20 @@ __global__ __launch_bounds__(VC_THREADS) void vc_plan_rows(VcSched S, VcLaunchPa
             bytes += len;
         }
     }
+    int64_t bad = 0;                                      // entries of this rank's rows no rank could have passed
     if (L == 0)
-        for (int id = threadIdx.x; id < P; id += VC_THREADS) payload += (int64_t)T.rc[(int64_t)to * P + id] * S.esz;
+        for (int id = threadIdx.x; id < P; id += VC_THREADS) {
+            const int64_t i = (int64_t)to * P + id;
+            payload += (int64_t)T.rc[i] * S.esz;
+            bad += (T.sc[i] < 0) | (T.sd[i] < 0) | (T.rc[i] < 0) | (!S.packed_recv && T.rd[i] < 0);
+        }
     items = vc_block_sum(items, lds);
     bytes = vc_block_sum(bytes, lds);
-    if (L == 0) payload = vc_block_sum(payload, lds);
+    if (L == 0) { payload = vc_block_sum(payload, lds); bad = vc_block_sum(bad, lds); }
     if (threadIdx.x == 0) {
         item_row_tot[(int64_t)L * P + to] = items;
         row_bytes[(int64_t)L * P + to] = bytes;
-        if (L == 0) row_bytes[(int64_t)nl * P + to] = payload;
+        if (L == 0) { row_bytes[(int64_t)nl * P + to] = payload; row_bytes[(int64_t)(nl + 1) * P + to] = bad; }
     }
 }
 
@@ -129,11 +134,13 @@ __global__ __launch_bounds__(VC_THREADS) void vc_plan_bases(int P, int w, int nl
             if (i < nrows) row_base[i] = carry + ex;
             carry += total;
         }
-        for (int i = threadIdx.x; i < P; i += VC_THREADS) bytes += row_bytes[(int64_t)nl * P + i];
+        int64_t bad = 0;
+        for (int i = threadIdx.x; i < P; i += VC_THREADS) { bytes += row_bytes[(int64_t)nl * P + i]; bad += row_bytes[(int64_t)(nl + 1) * P + i]; }
         bytes = vc_block_sum(bytes, lds);
+        bad = vc_block_sum(bad, lds);
         if (threadIdx.x == 0) {
-            header[0] = carry; header[1] = bytes;
-            if (header_host) { header_host[0] = carry; header_host[1] = bytes; }
+            header[0] = carry; header[1] = bytes; header[3 + nl] = bad;
+            if (header_host) { header_host[0] = carry; header_host[1] = bytes; header_host[3 + nl] = bad; }
         }
         return;
     }

@@ -105,6 +105,38 @@ def test_error_codes(api):
     dp.comm.free()
 
 
+def test_tables_are_validated_before_anything_moves(api):
+    """A negative count or displacement would send the copy kernels outside the arenas: the planner finds it on the
+    device and the call returns VC_ERR_TABLES (-7) with recvbuf untouched; the communicator stays usable."""
+    import torch
+    counts = W.counts_uniform_random(12, 40, seed=5)
+    prob = W.make_problem(counts, 4, 0, 0)
+    dp = api.DeviceProblem(prob)
+    s, d = dp.new_send_arena(), dp.new_recv_arena()
+    dp.fill_payload(0, 1, s)
+    for name in ("sendcounts", "sdispls", "recvcounts", "rdispls"):
+        table = getattr(dp, name)
+        keep = int(table[7, 3].item())
+        table[7, 3] = -1
+        for call in (lambda: api.twophase_rbruck_alltoallv(3, dp, s, d), lambda: api.tuna_algorithm(2, 1, dp, s, d),
+                     lambda: api.TTPL_BT_alltoallv_s1(4, 2, 0, dp, s, d), lambda: api.spreadout_alltoallv(dp, s, d)):
+            assert call() == -7 and "negative" in dp.comm.error()
+        assert bool((d == 0xEE).all())
+        table[7, 3] = keep
+    assert api.twophase_rbruck_alltoallv(3, dp, s, d) == 0 and dp.verify(s, d) == 0
+    # the displacement scan reports what the reference's int arithmetic would silently wrap
+    big = torch.full((2, 2), 2 ** 30, dtype=torch.int32, device="cuda:0")
+    displs = torch.zeros_like(big)
+    ext = torch.zeros(2, dtype=torch.int64, device="cuda:0")
+    c2 = api.VirtualComm(2)
+    assert c2.lib.vc_displs_from_counts(big.data_ptr(), displs.data_ptr(), ext.data_ptr(), c2.handle) == -8
+    assert ext.tolist() == [2 ** 31, 2 ** 31]
+    big[1, 0] = -4
+    assert c2.lib.vc_displs_from_counts(big.data_ptr(), displs.data_ptr(), ext.data_ptr(), c2.handle) == -7
+    c2.free()
+    dp.comm.free()
+
+
 def _oracle_traffic(rec, P, select):
     m = np.zeros((P, P), dtype=np.int64)
     for t in rec[select]:
