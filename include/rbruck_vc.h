@@ -237,6 +237,11 @@ int vc_comm_last_stats(vc_comm_t comm, vc_stats_t *out);
  * call in the launch-per-digit mode (vc_comm_set_forwarding(comm, 0)). */
 int vc_comm_last_traffic(vc_comm_t comm, int launch, int64_t *matrix_out);
 
+/* The staging arena as the last call left it: DEVICE pointer and the bytes that call used (what the reference keeps in
+ * extra_buffer / temp_recv_buffer between rounds, src/twophase_tunable_rbruckv.cpp:59-61).  Both execution modes leave
+ * the same bytes there; tests compare them.  The pointer is valid until a call on this communicator needs more. */
+int vc_comm_staging(vc_comm_t comm, void **ptr_out, int64_t *bytes_out);
+
 /* ---- harness utilities (payload of the reference drivers, examples/rbruckv_example.cpp:88-92, and a
  * receiver-side check in the spirit of src/utils.cpp:31-46, but exact) ---- */
 

@@ -59,6 +59,7 @@ SYMBOLS = {
     "vc_comm_set_timing": (_I, [_P, _I]),
     "vc_comm_last_stats": (_I, [_P, C.POINTER(VcStats)]),
     "vc_comm_last_traffic": (_I, [_P, _I, _P]),
+    "vc_comm_staging": (_I, [_P, C.POINTER(_P), C.POINTER(_I64)]),
     "vc_fill_payload": (_I, [_I, _U64, _P, _P, _P, _I, _P]),
     "vc_verify_alltoallv": (_I, [_P, _P, _P, _I, _P, _P, _P, _I, C.POINTER(_I64), _P]),
     "vc_calibration_copy": (_I, [_P, _P, _I64, _P]),

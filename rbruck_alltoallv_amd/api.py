@@ -61,6 +61,12 @@ class VirtualComm:
         self._check(self.lib.vc_comm_last_traffic(self.handle, launch, m.ctypes.data_as(C.c_void_p)))
         return m
 
+    def staging(self) -> tuple[int, int]:
+        """(device address, bytes used by the last call) of the staging arena."""
+        ptr, size = C.c_void_p(), C.c_int64()
+        self._check(self.lib.vc_comm_staging(self.handle, C.byref(ptr), C.byref(size)))
+        return ptr.value or 0, size.value
+
     def error(self) -> str:
         return self.lib.vc_last_error_string().decode()
 

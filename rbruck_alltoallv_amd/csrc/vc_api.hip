@@ -643,6 +643,13 @@ extern "C" int vc_comm_last_traffic(vc_comm_t c, int launch, int64_t *matrix_out
     return VC_OK;
 }
 
+extern "C" int vc_comm_staging(vc_comm_t c, void **ptr_out, int64_t *bytes_out) {
+    if (!c || !ptr_out || !bytes_out) return fail_arg("vc_comm_staging: null argument");
+    *ptr_out = c->stage.p;
+    *bytes_out = c->stats.staging_bytes;
+    return VC_OK;
+}
+
 // ------------------------------------------------------------ harness utilities
 
 extern "C" int vc_fill_payload(int mode, uint64_t seed, char *sendbuf, const int *sendcounts, const int *sdispls, int elem_size,

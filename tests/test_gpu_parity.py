@@ -619,6 +619,49 @@ def test_golden_case_forwarded(api, case):
     dp.comm.free()
 
 
+def test_both_execution_modes_leave_the_same_staging(api):
+    """The route on the GPU, forwarded execution included: after a call the staging arena holds every block in every
+    slot it waited in on the way, byte for byte what the launch-per-digit execution (whose launches are pinned against
+    the oracle's message trace) leaves there; bytes between the slots are not touched by either."""
+    import torch
+    c4 = W.counts_normal(256, 300.0, 120.0, 0, 1500, 0)
+    c3 = W.counts_zipf(60, 9000, 1.2, 5, 0)
+    for prob, calls in (
+            (W.make_problem(c4, 1, 0, 0), [("s1 r=2", lambda dp, s, d: api.TTPL_BT_alltoallv_s1(16, 2, 0, dp, s, d)),
+                                          ("s1 r=16", lambda dp, s, d: api.TTPL_BT_alltoallv_s1(16, 16, 0, dp, s, d)),
+                                          ("ttpl_rbruck r=3", lambda dp, s, d: api.TTPL_rbruck_alltoallv(16, 3, dp, s, d)),
+                                          ("om r=4", lambda dp, s, d: api.twophase_rbruck_alltoallv_om(4, dp, s, d))]),
+            (W.make_problem(c3, 4, 1, 1), [("twophase r=2", lambda dp, s, d: api.twophase_rbruck_alltoallv(2, dp, s, d)),
+                                          ("twophase r=7", lambda dp, s, d: api.twophase_rbruck_alltoallv(7, dp, s, d)),
+                                          ("tuna r=3", lambda dp, s, d: api.tuna_algorithm(3, 2, dp, s, d))])):
+        dp = api.DeviceProblem(prob)
+        ds = dp.new_send_arena()
+        dp.fill_payload(0, 11, ds)
+        lib, h = dp.comm.lib, dp.comm.handle
+        for name, fn in calls:
+            print("  ", name, flush=True)
+            snaps, sizes = [], []
+            for forward in (False, True):
+                dp.comm.set_forwarding(forward)
+                dr = dp.new_recv_arena(0xEE)
+                assert fn(dp, ds, dr) == 0, (name, dp.comm.error())          # sizes the arena
+                ptr, size = dp.comm.staging()
+                n = (size + 15) // 16 * 16
+                assert size > 0 and ptr
+                pattern = torch.full((n,), 0xAB, dtype=torch.uint8, device="cuda:0")
+                assert lib.vc_calibration_copy(ptr, pattern.data_ptr(), n, h) == 0
+                assert fn(dp, ds, dr) == 0 and dp.verify(ds, dr) == 0
+                assert dp.comm.staging() == (ptr, size)
+                snap = torch.empty(n, dtype=torch.uint8, device="cuda:0")
+                assert lib.vc_calibration_copy(snap.data_ptr(), ptr, n, h) == 0
+                snaps.append(snap.cpu().numpy())
+                sizes.append(size)
+            assert sizes[0] == sizes[1], name
+            assert np.array_equal(snaps[0], snaps[1]), name
+            assert np.count_nonzero(snaps[0] != 0xAB) > sizes[0] // 4, name        # the slots were written
+        dp.comm.free()
+
+
 def test_forwarded_shapes_plans_and_graphs(api):
     """Forwarded execution on the benchmark shapes (reduced), unaligned arenas, as a persistent plan and inside a HIP graph."""
     import torch
