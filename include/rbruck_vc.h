@@ -224,6 +224,10 @@ typedef struct {
     int64_t staging_bytes;       /* staging arena the call needed */
     float plan_ms;               /* metadata kernels (valid when timing is on) */
     float total_ms;              /* whole call on the stream (valid when timing is on) */
+    float intra_ms;              /* launches inside the nodes: the digit rounds (the reference's getBlock_time ... replace_time) */
+    float inter_ms;              /* launches between the nodes (orgData_time, prepSP_time, SP_time; intra_time / iteration_time of
+                                    src/twolayer_communicator_linear.cpp:10-11 likewise).  Forwarded execution has one launch
+                                    for both: its time is in intra_ms and inter_ms is 0. */
     int64_t launch_bytes[VC_MAX_LAUNCHES];   /* bytes the hops of a launch copy (forwarded execution: [0] = moved_bytes) */
     float launch_ms[VC_MAX_LAUNCHES];  /* per data-moving launch, HIP events on the comm's stream */
 } vc_stats_t;

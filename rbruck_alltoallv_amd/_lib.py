@@ -16,7 +16,8 @@ VC_ERR_TABLES, VC_ERR_OVERFLOW = -7, -8
 class VcStats(C.Structure):
     _fields_ = [("n_launches", C.c_int32), ("n_digits", C.c_int32), ("payload_bytes", C.c_int64),
                 ("moved_bytes", C.c_int64), ("staging_bytes", C.c_int64), ("plan_ms", C.c_float),
-                ("total_ms", C.c_float), ("launch_bytes", C.c_int64 * VC_MAX_LAUNCHES),
+                ("total_ms", C.c_float), ("intra_ms", C.c_float), ("inter_ms", C.c_float),
+                ("launch_bytes", C.c_int64 * VC_MAX_LAUNCHES),
                 ("launch_ms", C.c_float * VC_MAX_LAUNCHES)]
 
 

@@ -200,6 +200,7 @@ struct PlanInfo {
     int recv_lo = 0;
     int64_t stage_bytes = 0, payload_bytes = 0;
     std::vector<int64_t> first, count, bytes;       // per launch: first work item, item count, bytes moved
+    std::vector<char> inter;                        // per launch: its messages cross nodes
     bool chain = false;                             // forwarded execution: `items` holds chain items instead
     int chain_stride = 0;                           // int64 words per chain item
     int64_t chain_items = 0;
@@ -251,9 +252,10 @@ static int build_plan(vc_comm *c, VcSched S, std::vector<VcLaunchInfo> &L, VcTab
         return fail_arg("negative entries in sendcounts / sdispls / recvcounts / rdispls", VC_ERR_TABLES);
     out.nl = nl; out.n_digits = S.w + S.w2; out.recv_lo = S.recv_lo;
     out.stage_bytes = h[0]; out.payload_bytes = h[1];
-    out.first.assign(nl, 0); out.count.assign(nl, 0); out.bytes.assign(nl, 0);
+    out.first.assign(nl, 0); out.count.assign(nl, 0); out.bytes.assign(nl, 0); out.inter.assign(nl, 0);
     int64_t nitems = 0;
     for (int k = 0; k < nl; k++) {
+        out.inter[k] = L[k].kind == 1 || L[k].kind == 3 || L[k].kind == 4 || (L[k].kind == 2 && L[k].x == 2);
         out.bytes[k] = h[3 + k];
         out.first[k] = nitems;
         out.count[k] = h[3 + 2 * nl + k];
@@ -317,12 +319,13 @@ static int run_items(vc_comm *c, const PlanInfo &pi, const void *items_any, cons
     s.staging_bytes = pi.stage_bytes;
     s.payload_bytes = pi.payload_bytes;
     s.moved_bytes = 0;
-    s.plan_ms = s.total_ms = 0.f;
+    s.plan_ms = s.total_ms = s.intra_ms = s.inter_ms = 0.f;
     if (pi.chain) {                                   // one launch that performs the hops of every digit
         for (int k = 0; k < pi.nl; k++) s.moved_bytes += pi.bytes[k];
         s.launch_bytes[0] = s.moved_bytes;
         s.launch_ms[0] = 0.f;
         if (c->timing) HIP_TRY(hipEventElapsedTime(&s.launch_ms[0], c->events[2], c->events[3]));
+        s.intra_ms = s.launch_ms[0];
     } else {
         for (int k = 0; k < nl; k++) {
             s.launch_bytes[k] = pi.bytes[k];
@@ -331,6 +334,7 @@ static int run_items(vc_comm *c, const PlanInfo &pi, const void *items_any, cons
             c->launch_first[k] = pi.first[k];
             c->launch_items[k] = pi.count[k];
             if (c->timing) HIP_TRY(hipEventElapsedTime(&s.launch_ms[k], c->events[2 + k], c->events[3 + k]));
+            (pi.inter[k] ? s.inter_ms : s.intra_ms) += s.launch_ms[k];
         }
     }
     if (c->timing) {

@@ -619,6 +619,31 @@ def test_golden_case_forwarded(api, case):
     dp.comm.free()
 
 
+def test_phase_times(api):
+    """With timing on, the statistics split the launches as the reference's phase timers do (src/rbruckv.h:13-18):
+    inside the nodes and between them."""
+    prob = W.make_problem(W.counts_normal(64, 300.0, 100.0, 0, 1000, 0), 1, 0, 0)
+    dp = api.DeviceProblem(prob)
+    ds, dr = dp.new_send_arena(), dp.new_recv_arena()
+    dp.fill_payload(0, 2, ds)
+    dp.comm.set_timing(True)
+    for forward in (False, True):
+        dp.comm.set_forwarding(forward)
+        for name, fn, two_layer in (("ttpl", lambda: api.TTPL_BT_alltoallv_s1(8, 2, 0, dp, ds, dr), True),
+                                    ("twophase", lambda: api.twophase_rbruck_alltoallv(4, dp, ds, dr), False)):
+            assert fn() == 0
+            st = dp.comm.last_stats()
+            launches = sum(st.launch_ms[k] for k in range(st.n_launches))
+            assert st.intra_ms > 0 and abs(st.intra_ms + st.inter_ms - launches) < 1e-3 * max(launches, 1e-3), name
+            assert (st.inter_ms > 0) == (two_layer and not forward), name
+            assert st.total_ms >= launches and st.plan_ms > 0, name
+    dp.comm.set_timing(False)
+    assert api.twophase_rbruck_alltoallv(4, dp, ds, dr) == 0
+    st = dp.comm.last_stats()
+    assert st.total_ms == 0 and st.intra_ms == 0 and st.inter_ms == 0
+    dp.comm.free()
+
+
 def test_both_execution_modes_leave_the_same_staging(api):
     """The route on the GPU, forwarded execution included: after a call the staging arena holds every block in every
     slot it waited in on the way, byte for byte what the launch-per-digit execution (whose launches are pinned against
