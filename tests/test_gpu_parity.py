@@ -619,6 +619,54 @@ def test_golden_case_forwarded(api, case):
     dp.comm.free()
 
 
+def test_seeded_random_sweep(api):
+    """Random rank counts, radices, node sizes, batches, element sizes, count ranges (with zeros and a few huge blocks),
+    displacement layouts and recvbuf alignments; three of the entry points per case, checked against the definition
+    on the device, and the bytes around recvbuf must stay untouched."""
+    import random
+    import torch
+    rnd = random.Random(2024)
+    for it in range(60):
+        P = rnd.choice([2, 3, 4, 6, 7, 8, 12, 16, 24, 27, 30, 36, 48, 64, 81, 96, 100, 128])
+        esz = rnd.choice([1, 1, 2, 3, 4, 8, 12])
+        hi = rnd.choice([0, 1, 5, 60, 700, 5000, 20000])
+        layout = rnd.choice([0, 1])
+        counts = W.counts_uniform_random(P, hi, seed=it)
+        if rnd.random() < 0.5:
+            counts[counts % rnd.choice([2, 3, 5]) == 0] = 0
+        if rnd.random() < 0.2 and P >= 4:
+            counts[rnd.randrange(P), rnd.randrange(P)] = rnd.choice([100000, 300000])
+        n = rnd.choice([d for d in range(1, P + 1) if P % d == 0])
+        r = rnd.choice([2, 3, 4, 5, 8, 16, 31, P, P + 1])
+        b = rnd.choice([0, 1, 2, 7])
+        prob = W.make_problem(counts, esz, layout, layout)
+        dp = api.DeviceProblem(prob)
+        ds = dp.new_send_arena()
+        dp.fill_payload(0, it, ds)
+        shift = rnd.choice([0, 0, 1, 7, 64, 100])
+        rbig = torch.full((prob.recv_bytes + 256,), 0xEE, dtype=torch.uint8, device="cuda:0")
+        dr = rbig[shift:shift + prob.recv_bytes]
+        calls = [("twophase", lambda: api.twophase_rbruck_alltoallv(r, dp, ds, dr), False),
+                 ("om", lambda: api.twophase_rbruck_alltoallv_om(r, dp, ds, dr), False),
+                 ("s1", lambda: api.TTPL_BT_alltoallv_s1(n, r, b, dp, ds, dr), False),
+                 ("rbruck", lambda: api.TTPL_rbruck_alltoallv(n, r, dp, ds, dr), False),
+                 ("scattered", lambda: api.MPICH_intra_scattered(b, dp, ds, dr), False)]
+        if P >= 3:
+            calls += [("tuna", lambda: api.tuna_algorithm(r, b, dp, ds, dr), False),
+                      ("tuna2", lambda: api.tuna2_algorithm(r, b, dp, ds, dr), False)]
+        if layout == 0:
+            calls.append(("ttpl", lambda: api.TTPL_BT_alltoallv(n, r, b, dp, ds, dr), True))
+        if 1 <= n < P:
+            calls.append(("tl_s2", lambda: api.twolayer_communicator_linear_s2(n, b, b + 1, dp, ds, dr), False))
+        for name, fn, packed in rnd.sample(calls, 3):
+            what = f"case {it} {name}: P={P} n={n} r={r} b={b} esz={esz} hi={hi} layout={layout} shift={shift}"
+            rbig.fill_(0xEE)
+            assert fn() == 0, (what, dp.comm.error())
+            assert dp.verify(ds, dr, packed_recv=packed) == 0, what
+            assert bool((rbig[:shift] == 0xEE).all()) and bool((rbig[shift + prob.recv_bytes:] == 0xEE).all()), what
+        dp.comm.free()
+
+
 def test_phase_times(api):
     """With timing on, the statistics split the launches as the reference's phase timers do (src/rbruckv.h:13-18):
     inside the nodes and between them."""
