@@ -149,6 +149,13 @@ def cpu_baseline(name: str, seed: int, budget_s: float) -> dict:
             "seconds": t}
 
 
+# vc_stats_t.execution of the timed calls (the library's default mode picks between the two forwarded kernels)
+EXECUTION_NAMES = {0: "launch per digit phase",
+                   1: "forwarded (one launch, blocks carried through all hops in registers)",
+                   2: "forwarded, without a work-item list (one workgroup per pair of ranks; one host synchronisation per call)"}
+EXECUTION_KERNELS = {0: "vc_copy_items_kernel", 1: "vc_copy_chains_kernel", 2: "vc_copy_blocks_kernel"}
+
+
 def main() -> None:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -281,7 +288,7 @@ def main() -> None:
     o_elapsed, o_kern_ms, o_kern_bytes, o_nkern, _, _, o_st = timed_calls(2, o_steps)
     o_bad = dp.verify(send, recv, packed_recv=packed)
     o_plan = plan_timing(o_steps)
-    other = {"mode": "launch per digit phase" if args.forward else "forwarded (one launch, blocks carried through all hops in registers)",
+    other = {"mode": EXECUTION_NAMES[int(o_st.execution)],
              "ms_per_call": round(o_elapsed / o_steps * 1e3, 4), "GBps_effective": round(S / (o_elapsed / o_steps) / 1e9, 1),
              "hbm_frac_whole_call": round(A / (o_elapsed / o_steps) / 1e9 / HBM_PEAK_GBPS, 4),
              "kernel_frac": round(o_kern_bytes / (o_kern_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4) if o_kern_ms > 0 else None,
@@ -319,13 +326,13 @@ def main() -> None:
         "one_pass_floor_fraction": round(2 * S / (elapsed / args.steps) / 1e9 / HBM_PEAK_GBPS, 4),
         "plan_ms_per_step": round(plan_ms / args.steps, 4),
         "mismatched_bytes": int(bad),
-        "execution": "forwarded (one launch, blocks carried through all hops in registers)" if args.forward else "launch per digit phase",
+        "execution": EXECUTION_NAMES[int(st.execution)],
         "persistent_plan": plan_info,
         "other_execution_mode": other,
         "one_pass_comparator": {"func": "spreadout_alltoallv", "ms_per_call": round(comp_s * 1e3, 4),
                                 "GBps_effective": round(S / comp_s / 1e9, 1),
                                 "hbm_frac": round(2 * S / comp_s / 1e9 / HBM_PEAK_GBPS, 4), "mismatched_bytes": int(comp_bad)},
-        "roofline": {"bound": "hbm", "kernel": "vc_copy_chains_kernel" if args.forward else "vc_copy_items_kernel", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
+        "roofline": {"bound": "hbm", "kernel": EXECUTION_KERNELS[int(st.execution)], "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
                      "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
                      "traffic": MEASURED_TRAFFIC_PER_LAUNCH.get((args.workload, func, int(bool(args.forward)))),
                      "avg_launch_ms": round(kern_ms / max(nkern, 1), 4),

@@ -63,11 +63,17 @@ int vc_comm_set_bases(vc_comm_t comm, const int64_t *sbase_bytes, const int64_t 
  *    all the hops of that block one after the other and keeps the piece in registers in between, so the data is read
  *    once (from sendbuf) and written once per hop (into the staging slot of every intermediate holder, then into
  *    recvbuf).  The batching tunables (b, bblock) then have no effect, and TTPL_BT_alltoallv sends its inter-node data
- *    per block instead of coalesced.
+ *    per block instead of coalesced.  The copy kernel normally works through a list of block pieces that a planning
+ *    kernel writes first (after the host has learnt its size).  On communicators of at most 128 ranks, when the last
+ *    call consisted of few, short blocks, the next one goes without the list: one workgroup per pair of ranks derives
+ *    its block's route itself, the kernel is enqueued right behind the size computation, and the call needs one host
+ *    synchronisation instead of two (24 - 35 us instead of 37 - 47 us per call of 16 - 64 ranks on MI355X).
+ * 2: forwarded, always through the list.   3: forwarded, always without it (any size; slower beyond ~128 ranks).
  * 0: one kernel launch per digit phase (or per batch of its rounds, as b / bblock say); every hop reads the block
  *    where the previous hop left it.  This is the mode whose launches vc_comm_last_stats and vc_comm_last_traffic
  *    describe one by one.
- * Results, and the staging contents, are the same in both.  Applies to calls and to plans created afterwards. */
+ * Results, and the staging contents, are the same in all of them.  Applies to calls and to plans created afterwards
+ * (plans always hold a list). */
 int vc_comm_set_forwarding(vc_comm_t comm, int enable);
 
 /* Text of the most recent failure on this thread ("" if none). */
@@ -230,6 +236,8 @@ typedef struct {
                                     for both: its time is in intra_ms and inter_ms is 0. */
     int64_t launch_bytes[VC_MAX_LAUNCHES];   /* bytes the hops of a launch copy (forwarded execution: [0] = moved_bytes) */
     float launch_ms[VC_MAX_LAUNCHES];  /* per data-moving launch, HIP events on the comm's stream */
+    int32_t execution;           /* how the call ran: 0 launch per digit, 1 forwarded through a work-item list, 2 forwarded
+                                    without one (see vc_comm_set_forwarding) */
 } vc_stats_t;
 
 /* Per-launch HIP-event timing of the following calls (0 = off, default). */

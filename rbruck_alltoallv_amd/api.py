@@ -47,8 +47,10 @@ class VirtualComm:
     def set_timing(self, on: bool) -> None:
         self._check(self.lib.vc_comm_set_timing(self.handle, int(on)))
 
-    def set_forwarding(self, enable: bool) -> None:
-        """vc_comm_set_forwarding: one launch per call, every block piece carried through all its hops in registers."""
+    def set_forwarding(self, enable: bool | int) -> None:
+        """vc_comm_set_forwarding: 0 / False one launch per digit phase; 1 / True forwarded (one launch per call, every
+        block piece carried through all its hops in registers; the library picks list or listless); 2 forwarded through
+        a work-item list; 3 forwarded without one."""
         self._check(self.lib.vc_comm_set_forwarding(self.handle, int(enable)))
 
     def last_stats(self) -> _lib.VcStats:

@@ -29,6 +29,12 @@ static int fail_hip(hipError_t e, const char *what, int line) {
     return VC_ERR_HIP;
 }
 
+// The default mode goes without a work-item list only where that was measured to win: at most this many pairs of ranks
+// (128 ranks) and block pieces, no block of more than VC_LISTLESS_MAX_PIECES pieces (one workgroup moves them in turn).
+// 16 - 64 ranks: 24 - 35 us per call against 37 - 47 us; 128 ranks: even; 256 ranks and more: the list wins.
+#define VC_LISTLESS_MAX_ITEMS 16384
+#define VC_LISTLESS_MAX_PIECES 8
+
 #define HIP_TRY(expr)                                                   \
     do {                                                                \
         hipError_t e_ = (expr);                                         \
@@ -64,7 +70,10 @@ struct vc_comm {
     hipStream_t stream = nullptr;
     const int64_t *sbase = nullptr, *rbase = nullptr;
     bool timing = false;
-    bool forward = true;                  // forwarded execution: one launch, every block piece carried through all its hops
+    int forward = 1;                      // vc_comm_set_forwarding: 0 launch per digit, 1 forwarded (list or listless as the last
+                                          // call suggests), 2 forwarded through a work-item list, 3 forwarded, listless if possible
+    bool hint_valid = false;              // what the last forwarded call on this communicator looked like
+    int64_t hint_items = 0, hint_max_pieces = 0;
     DevBuf chain_row_tot, chain_row_base;
     DevBuf slot_off, row_tot, row_base, org_run_base, item_row_tot, item_row_base, row_bytes, desc, header, launches, stage, rd_packed,
         uni_counts, uni_displs, scratch;
@@ -136,7 +145,8 @@ extern "C" int vc_comm_set_timing(vc_comm_t c, int enable) {
 
 extern "C" int vc_comm_set_forwarding(vc_comm_t c, int enable) {
     if (!c) return fail_arg("null communicator");
-    c->forward = enable != 0;
+    if (enable < 0 || enable > 3) return fail_arg("vc_comm_set_forwarding: 0, 1, 2 or 3");
+    c->forward = enable;
     return VC_OK;
 }
 
@@ -201,13 +211,16 @@ struct PlanInfo {
     int64_t stage_bytes = 0, payload_bytes = 0;
     std::vector<int64_t> first, count, bytes;       // per launch: first work item, item count, bytes moved
     std::vector<char> inter;                        // per launch: its messages cross nodes
+    int64_t items_total = 0;                        // work items of all launches
     bool chain = false;                             // forwarded execution: `items` holds chain items instead
     int chain_stride = 0;                           // int64 words per chain item
-    int64_t chain_items = 0;
+    int64_t chain_items = 0, max_pieces = 0;        // (max_pieces: the most pieces any block is cut into)
+    bool listless = false;                          // forwarded execution that went without the item list
 };
 
-// Step 3: staging prefix sums, item counts (read back to size the buffers), then the work items into `items`.
-static int build_plan(vc_comm *c, VcSched S, std::vector<VcLaunchInfo> &L, VcTables T, DevBuf &items, PlanInfo &out, bool forward) {
+// Step 3a: enqueues the planning kernels that size everything (staging prefix sums, item counts, table check); their
+// result lands in the pinned header.
+static int plan_sizes(vc_comm *c, const VcSched &S, std::vector<VcLaunchInfo> &L, VcTables &T, bool forward) {
     const int P = S.P;
     const int nl = (int)L.size();
     if (nl > VC_MAX_LAUNCHES) return fail_arg("more than VC_MAX_LAUNCHES launches: raise b / bblock");
@@ -226,7 +239,7 @@ static int build_plan(vc_comm *c, VcSched S, std::vector<VcLaunchInfo> &L, VcTab
     HIP_TRY(c->launches.reserve(sizeof(VcLaunchInfo) * VC_MAX_LAUNCHES));
     if (forward) {
         if (vc_hop_slots(S) > VC_MAX_HOP_SLOTS) return fail_arg("too many digits for forwarded execution");
-        HIP_TRY(c->chain_row_tot.reserve(sizeof(int64_t) * (size_t)P));
+        HIP_TRY(c->chain_row_tot.reserve(sizeof(int64_t) * 2 * (size_t)P));
         HIP_TRY(c->chain_row_base.reserve(sizeof(int64_t) * (size_t)P));
     }
     if (c->timing) { int rc = ensure_events(c, (size_t)nl + 4); if (rc) return rc; }
@@ -245,10 +258,14 @@ static int build_plan(vc_comm *c, VcSched S, std::vector<VcLaunchInfo> &L, VcTab
                                  c->row_base.as<int64_t>(), c->org_run_base.as<int64_t>(), c->item_row_tot.as<int64_t>(),
                                  c->item_row_base.as<int64_t>(), c->row_bytes.as<int64_t>(), forward ? c->chain_row_tot.as<int64_t>() : nullptr,
                                  forward ? c->chain_row_base.as<int64_t>() : nullptr, c->header.as<int64_t>(), c->h_header_dev, st));
-    HIP_TRY(hipStreamSynchronize(st));     // the staging arena and the item list are sized from the plan
+    return VC_OK;
+}
 
+// Step 3b, after the stream has been synchronised: what the planning kernels found.
+static int plan_read(vc_comm *c, const VcSched &S, const std::vector<VcLaunchInfo> &L, PlanInfo &out, bool forward) {
+    const int nl = (int)L.size();
     const int64_t *h = c->h_header;
-    if (h[3 + nl] != 0)       // nothing has been copied yet: such tables would send the copy kernels outside the arenas
+    if (h[VC_HEADER_BAD] != 0)    // such tables would send the copy kernels outside the arenas
         return fail_arg("negative entries in sendcounts / sdispls / recvcounts / rdispls", VC_ERR_TABLES);
     out.nl = nl; out.n_digits = S.w + S.w2; out.recv_lo = S.recv_lo;
     out.stage_bytes = h[0]; out.payload_bytes = h[1];
@@ -256,26 +273,44 @@ static int build_plan(vc_comm *c, VcSched S, std::vector<VcLaunchInfo> &L, VcTab
     int64_t nitems = 0;
     for (int k = 0; k < nl; k++) {
         out.inter[k] = L[k].kind == 1 || L[k].kind == 3 || L[k].kind == 4 || (L[k].kind == 2 && L[k].x == 2);
-        out.bytes[k] = h[3 + k];
+        out.bytes[k] = h[VC_HEADER_FIXED + k];
         out.first[k] = nitems;
-        out.count[k] = h[3 + 2 * nl + k];
+        out.count[k] = h[VC_HEADER_FIXED + nl + k];
         nitems += out.count[k];
     }
+    out.items_total = nitems;
     if (forward) {
         out.chain = true;
         out.chain_stride = VC_CHAIN_HEAD + vc_hop_slots(S);
         out.chain_items = h[2];
-        HIP_TRY(items.reserve(sizeof(int64_t) * (size_t)out.chain_stride * (size_t)std::max<int64_t>(out.chain_items, 1)));
-        HIP_TRY(vc_launch_chain_plan(S, T, c->slot_off.as<int64_t>(), c->row_base.as<int64_t>(), c->chain_row_base.as<int64_t>(),
-                                     items.as<int64_t>(), out.chain_items, st));
-        if (c->timing) HIP_TRY(hipEventRecord(c->events[1], st));
-        return VC_OK;
+        out.max_pieces = h[VC_HEADER_MAX_PIECES];
     }
-    HIP_TRY(items.reserve(sizeof(VcDesc) * (size_t)std::max<int64_t>(nitems, 1)));
-    HIP_TRY(vc_launch_plan_emit(S, L.data(), c->launches.as<VcLaunchInfo>(), nl, T, c->slot_off.as<int64_t>(), c->row_base.as<int64_t>(),
-                                c->item_row_base.as<int64_t>(), c->header.as<int64_t>(), items.as<VcDesc>(), nitems, st));
+    return VC_OK;
+}
+
+// Step 3c: the work items into `items` (sized from the plan).
+static int plan_emit(vc_comm *c, const VcSched &S, std::vector<VcLaunchInfo> &L, const VcTables &T, DevBuf &items, const PlanInfo &pi) {
+    hipStream_t st = c->stream;
+    if (pi.chain) {
+        HIP_TRY(items.reserve(sizeof(int64_t) * (size_t)pi.chain_stride * (size_t)std::max<int64_t>(pi.chain_items, 1)));
+        HIP_TRY(vc_launch_chain_plan(S, T, c->slot_off.as<int64_t>(), c->row_base.as<int64_t>(), c->chain_row_base.as<int64_t>(),
+                                     items.as<int64_t>(), pi.chain_items, st));
+    } else {
+        HIP_TRY(items.reserve(sizeof(VcDesc) * (size_t)std::max<int64_t>(pi.items_total, 1)));
+        HIP_TRY(vc_launch_plan_emit(S, L.data(), c->launches.as<VcLaunchInfo>(), pi.nl, T, c->slot_off.as<int64_t>(), c->row_base.as<int64_t>(),
+                                    c->item_row_base.as<int64_t>(), c->header.as<int64_t>(), items.as<VcDesc>(), pi.items_total, st));
+    }
     if (c->timing) HIP_TRY(hipEventRecord(c->events[1], st));
     return VC_OK;
+}
+
+static int build_plan(vc_comm *c, VcSched S, std::vector<VcLaunchInfo> &L, VcTables T, DevBuf &items, PlanInfo &out, bool forward) {
+    int rc = plan_sizes(c, S, L, T, forward);
+    if (rc) return rc;
+    HIP_TRY(hipStreamSynchronize(c->stream));     // the staging arena and the item list are sized from the plan
+    rc = plan_read(c, S, L, out, forward);
+    if (rc) return rc;
+    return plan_emit(c, S, L, T, items, out);
 }
 
 // Steps 4-5: one copy kernel per launch, then the blocking synchronisation.  `planned_now` says whether events 0 and 1
@@ -291,6 +326,46 @@ static int launch_items(vc_comm *c, const PlanInfo &pi, const void *items_any, c
     const VcDesc *items = static_cast<const VcDesc *>(items_any);
     for (int k = 0; k < pi.nl; k++)
         HIP_TRY(vc_launch_copy_items(items + pi.first[k], pi.count[k], sendbuf, recvbuf, c->stage.as<char>(), c->stream));
+    return VC_OK;
+}
+
+// After the final synchronisation: the statistics of the call.
+static int finish_stats(vc_comm *c, const PlanInfo &pi, const void *items_any, bool planned_now) {
+    const int nl = pi.chain ? 1 : pi.nl;              // kernel launches of this execution
+    vc_stats_t &s = c->stats;
+    s.n_launches = nl;
+    s.n_digits = pi.n_digits;
+    s.staging_bytes = pi.stage_bytes;
+    s.payload_bytes = pi.payload_bytes;
+    s.moved_bytes = 0;
+    s.execution = pi.chain ? (pi.listless ? 2 : 1) : 0;
+    s.plan_ms = s.total_ms = s.intra_ms = s.inter_ms = 0.f;
+    if (pi.chain) {                                   // one launch that performs the hops of every digit
+        for (int k = 0; k < pi.nl; k++) s.moved_bytes += pi.bytes[k];
+        s.launch_bytes[0] = s.moved_bytes;
+        s.launch_ms[0] = 0.f;
+        if (c->timing) HIP_TRY(hipEventElapsedTime(&s.launch_ms[0], c->events[2], c->events[3]));
+        s.intra_ms = s.launch_ms[0];
+        c->hint_valid = true;
+        c->hint_items = pi.chain_items;
+        c->hint_max_pieces = pi.max_pieces;
+    } else {
+        for (int k = 0; k < nl; k++) {
+            s.launch_bytes[k] = pi.bytes[k];
+            s.moved_bytes += pi.bytes[k];
+            s.launch_ms[k] = 0.f;
+            c->launch_first[k] = pi.first[k];
+            c->launch_items[k] = pi.count[k];
+            if (c->timing) HIP_TRY(hipEventElapsedTime(&s.launch_ms[k], c->events[2 + k], c->events[3 + k]));
+            (pi.inter[k] ? s.inter_ms : s.intra_ms) += s.launch_ms[k];
+        }
+    }
+    if (c->timing) {
+        if (planned_now) HIP_TRY(hipEventElapsedTime(&s.plan_ms, c->events[0], c->events[1]));
+        HIP_TRY(hipEventElapsedTime(&s.total_ms, c->events[planned_now ? 0 : 2], c->events[2 + nl]));
+    }
+    c->last_nlaunch = pi.chain ? 0 : nl;              // per-launch traffic can only be inspected after launch-per-digit execution
+    c->last_items = static_cast<const VcDesc *>(items_any);
     return VC_OK;
 }
 
@@ -312,43 +387,49 @@ static int run_items(vc_comm *c, const PlanInfo &pi, const void *items_any, cons
     }
     if (c->timing) HIP_TRY(hipEventRecord(c->events[2 + nl], st));
     HIP_TRY(hipStreamSynchronize(st));
+    return finish_stats(c, pi, items_any, planned_now);
+}
 
-    vc_stats_t &s = c->stats;
-    s.n_launches = nl;
-    s.n_digits = pi.n_digits;
-    s.staging_bytes = pi.stage_bytes;
-    s.payload_bytes = pi.payload_bytes;
-    s.moved_bytes = 0;
-    s.plan_ms = s.total_ms = s.intra_ms = s.inter_ms = 0.f;
-    if (pi.chain) {                                   // one launch that performs the hops of every digit
-        for (int k = 0; k < pi.nl; k++) s.moved_bytes += pi.bytes[k];
-        s.launch_bytes[0] = s.moved_bytes;
-        s.launch_ms[0] = 0.f;
-        if (c->timing) HIP_TRY(hipEventElapsedTime(&s.launch_ms[0], c->events[2], c->events[3]));
-        s.intra_ms = s.launch_ms[0];
-    } else {
-        for (int k = 0; k < nl; k++) {
-            s.launch_bytes[k] = pi.bytes[k];
-            s.moved_bytes += pi.bytes[k];
-            s.launch_ms[k] = 0.f;
-            c->launch_first[k] = pi.first[k];
-            c->launch_items[k] = pi.count[k];
-            if (c->timing) HIP_TRY(hipEventElapsedTime(&s.launch_ms[k], c->events[2 + k], c->events[3 + k]));
-            (pi.inter[k] ? s.inter_ms : s.intra_ms) += s.launch_ms[k];
-        }
-    }
-    if (c->timing) {
-        if (planned_now) HIP_TRY(hipEventElapsedTime(&s.plan_ms, c->events[0], c->events[1]));
-        HIP_TRY(hipEventElapsedTime(&s.total_ms, c->events[planned_now ? 0 : 2], c->events[2 + nl]));
-    }
-    c->last_nlaunch = pi.chain ? 0 : nl;              // per-launch traffic can only be inspected after launch-per-digit execution
-    c->last_items = items;
-    return VC_OK;
+// Whether a forwarded call should try to go without the work-item list: worth it when writing the list (and waiting for
+// its size before that) costs more than the slower per-block kernel loses, i.e. for calls of few, short blocks.  The
+// last forwarded call on the communicator is the guide (mode 1), or the caller says so (mode 3).
+static bool want_listless(const vc_comm *c, const VcSched &S) {
+    if (c->forward == 3) return true;
+    if (c->forward != 1 || !c->hint_valid) return false;
+    return (int64_t)S.P * S.P <= VC_LISTLESS_MAX_ITEMS && c->hint_items <= VC_LISTLESS_MAX_ITEMS &&
+           c->hint_max_pieces <= VC_LISTLESS_MAX_PIECES;
 }
 
 static int run_schedule(vc_comm *c, VcSched S, std::vector<VcLaunchInfo> &L, const char *sendbuf, char *recvbuf, VcTables T, bool forward) {
     PlanInfo pi;
-    int rc = build_plan(c, S, L, T, c->desc, pi, forward);
+    hipStream_t st = c->stream;
+    int rc = plan_sizes(c, S, L, T, forward);
+    if (rc) return rc;
+    if (forward && want_listless(c, S)) {
+        // the copy kernel goes out right behind the planning kernels and checks their verdict on the device; when the
+        // staging arena turns out too small it has touched nothing, and goes out once more behind a larger arena
+        for (int attempt = 0; attempt < 2; attempt++) {
+            const int64_t stage_cap = c->stage.cap >= 64 ? (int64_t)c->stage.cap - 64 : 0;
+            if (c->timing) {
+                if (attempt == 0) HIP_TRY(hipEventRecord(c->events[1], st));
+                HIP_TRY(hipEventRecord(c->events[2], st));
+            }
+            HIP_TRY(vc_launch_copy_blocks(S, T, c->slot_off.as<int64_t>(), c->row_base.as<int64_t>(), c->header.as<int64_t>(), stage_cap,
+                                          sendbuf, recvbuf, c->stage.as<char>(), st));
+            if (c->timing) HIP_TRY(hipEventRecord(c->events[3], st));
+            HIP_TRY(hipStreamSynchronize(st));
+            rc = plan_read(c, S, L, pi, true);
+            if (rc) return rc;
+            if (pi.stage_bytes <= stage_cap) { pi.listless = true; break; }
+            HIP_TRY(c->stage.reserve((size_t)pi.stage_bytes + 64));
+        }
+        if (!pi.listless) return fail_arg("the plan changed between two launches of one call", VC_ERR_HIP);
+        return finish_stats(c, pi, nullptr, true);
+    }
+    HIP_TRY(hipStreamSynchronize(st));             // the staging arena and the item list are sized from the plan
+    rc = plan_read(c, S, L, pi, forward);
+    if (rc) return rc;
+    rc = plan_emit(c, S, L, T, c->desc, pi);
     if (rc) return rc;
     return run_items(c, pi, c->desc.p, sendbuf, recvbuf, true);
 }
@@ -388,7 +469,7 @@ static int run_v(VcFunc f, int n, int r, int batch, vc_comm *c, char *sendbuf, i
     if (!sendcounts || !sdispls || !recvcounts || (f != VC_F_TTPL && !rdispls)) return fail_arg("null table");
     VcSched S;
     std::vector<VcLaunchInfo> L;
-    const bool forward = c->forward;
+    const bool forward = c->forward != 0;
     rc = vc_make_schedule(f, c->P, n, r, batch, esz, 0, S, L, batch2, forward);
     if (rc) return schedule_error(rc);
     S.recv_lo = (int)((uintptr_t)recvbuf & 4095);
@@ -492,7 +573,7 @@ static int run_uniform(VcFunc f, int n, int r, vc_comm *c, char *sendbuf, int se
     if ((int64_t)sendcount * c->P > 0x7FFFFFFF) return fail_arg("sendcount * P must fit the reference's int displacements");
     VcSched S;
     std::vector<VcLaunchInfo> L;
-    const bool forward = c->forward;
+    const bool forward = c->forward != 0;
     rc = vc_make_schedule(f, c->P, n, r, 0, esz, sendcount, S, L, 0, forward);
     if (rc) return schedule_error(rc);
     S.recv_lo = (int)((uintptr_t)recvbuf & 4095);
@@ -546,7 +627,7 @@ extern "C" int vc_plan_create(const char *function, int n, int r, int batch, int
     if (!sendcounts || !sdispls || !recvcounts || (f != VC_F_TTPL && !rdispls)) return fail_arg("null table");
     VcSched S;
     std::vector<VcLaunchInfo> L;
-    const bool forward = c->forward;
+    const bool forward = c->forward != 0;
     int rc = vc_make_schedule(f, c->P, n, r, batch, elem_size, 0, S, L, 0, forward);
     if (rc) return schedule_error(rc);
     S.recv_lo = recvbuf_low_bits & 4095;
@@ -623,7 +704,7 @@ extern "C" int vc_suggest_radix(const int *sendcounts, int elem_size, int n, con
     const double bytes_per_s = 5.2e12, launch_s = 7e-6;
     double best = 0;
     for (int k = 0; k < ncand; k++) {
-        const double t = c->forward ? (double)moved[k] / bytes_per_s
+        const double t = c->forward != 0 ? (double)moved[k] / bytes_per_s
                                     : 2.0 * (double)moved[k] / bytes_per_s + launch_s * launches_for(n, cand[k], n < P);
         if (moved_bytes_out) moved_bytes_out[k] = (int64_t)moved[k];
         if (k == 0 || t < best) { best = t; *best_out = candidates[k]; }

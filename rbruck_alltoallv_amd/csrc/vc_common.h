@@ -108,12 +108,17 @@ hipError_t vc_launch_uniform_tables(int *counts, int *displs, int count, int P, 
 // vc_plan.hip
 // header layout (int64), nl = number of launches:
 //   [0] staging bytes   [1] payload bytes   [2] chain items (forwarded execution)
-//   [3 + L] bytes moved by launch L   [3 + nl] negative entries found in the count / displacement tables
-//   [3 + 2 nl + L] work items of launch L
-#define VC_HEADER_WORDS(nl) (3 + 3 * (nl))
+//   [3] negative entries found in the count / displacement tables
+//   [4] the most pieces any block is cut into (forwarded execution)
+//   [5 + L] bytes moved by launch L   [5 + nl + L] work items of launch L
+#define VC_HEADER_FIXED 5
+#define VC_HEADER_BAD 3
+#define VC_HEADER_MAX_PIECES 4
+#define VC_HEADER_WORDS(nl) (VC_HEADER_FIXED + 2 * (nl))
 // Passes 1 and 2: staging prefix sums and the number of work items of every launch (sizes only).  The launch table
 // travels as a kernel argument when it has at most VC_LAUNCH_PACK entries (launches_dev is then not read).  With chain_row_tot /
-// chain_row_base (P int64 each, or null) also the chain items per final receiver and their total in header[2].
+// chain_row_base (2 P and P int64, or null) also the chain items per final receiver, their total in header[2] and the most
+// pieces of any block in header[4].
 hipError_t vc_launch_plan_sizes(const VcSched &S, const VcLaunchInfo *launches_host, const VcLaunchInfo *launches_dev, int nlaunch,
                                 VcTables T, int64_t *slot_off,
                                 int64_t *row_tot, int64_t *row_base, int64_t *org_run_base, int64_t *item_row_tot,
@@ -133,4 +138,9 @@ hipError_t vc_launch_traffic(const VcDesc *desc, int64_t ndesc, int64_t *matrix,
 hipError_t vc_launch_copy_items(const VcDesc *items, int64_t nitems, const char *sendbuf, char *recvbuf, char *stage, hipStream_t st);
 hipError_t vc_launch_copy_chains(const int64_t *items, int stride, int64_t nitems, const char *sendbuf, char *recvbuf, char *stage,
                                  hipStream_t st);
+// Forwarded execution without a work-item list: one workgroup per (source, destination) pair works out the route of its
+// block from the plan tables and carries it through.  Reads the device `header` the planning kernels before it on the
+// stream have written and does nothing when the plan needs more than stage_cap bytes of staging or found bad tables.
+hipError_t vc_launch_copy_blocks(const VcSched &S, VcTables T, const int64_t *slot_off, const int64_t *row_base, const int64_t *header,
+                                 int64_t stage_cap, const char *sendbuf, char *recvbuf, char *stage, hipStream_t st);
 hipError_t vc_launch_calibration_copy(const char *src, char *dst, int64_t nbytes, hipStream_t st);

@@ -20,6 +20,7 @@
 // 1 MiB blocks cut into pieces.
 #include "vc_common.h"
 #include "vc_plan_math.h"
+#include "vc_scan.h"
 
 typedef unsigned int vc_u32x4 __attribute__((ext_vector_type(4)));
 struct __attribute__((packed, aligned(1))) VcU128 { vc_u32x4 v; };
@@ -47,6 +48,10 @@ __device__ __forceinline__ char *vc_resolve(int64_t loc, const char *sendbuf, ch
 // block are moved by (possibly unaligned) 16-byte loads and aligned stores; the < 16 bytes before the first and after
 // the last of them are moved byte-wise.  The planner guarantees len + (dst & 127) <= VC_CHUNK.
 #define VC_XCDS 8
+// Workgroups of one launch: a dispatch counts its grid in work-items in 32 bits, so gridDim.x * VC_THREADS must stay
+// below 2^32 (a larger grid is not refused: it runs truncated); longer lists go out in several launches.  A multiple of
+// VC_XCDS.
+#define VC_MAX_GRID ((int64_t)((1ull << 32) / VC_THREADS) - VC_XCDS)
 __global__ __launch_bounds__(VC_THREADS) void vc_copy_items_kernel(const VcDesc *__restrict__ items, unsigned nitems,
                                                                    const char *__restrict__ sendbuf, char *__restrict__ recvbuf,
                                                                    char *__restrict__ stage) {
@@ -82,19 +87,10 @@ __global__ __launch_bounds__(VC_THREADS) void vc_copy_items_kernel(const VcDesc 
 
 // Forwarded execution: one workgroup carries a piece through all the hops of its block.  The piece is read once, from
 // sendbuf; every hop stores the same registers (all destinations of a block share the offset inside their cache line,
-// so one mapping of lanes to window vectors serves them all).
-__global__ __launch_bounds__(VC_THREADS) void vc_copy_chains_kernel(const int64_t *__restrict__ items, int stride, unsigned nitems,
-                                                                    const char *__restrict__ sendbuf, char *__restrict__ recvbuf,
-                                                                    char *__restrict__ stage) {
-    const unsigned per = gridDim.x / VC_XCDS;
-    const unsigned idx = (blockIdx.x % VC_XCDS) * per + blockIdx.x / VC_XCDS;
-    if (idx >= nitems) return;
-    const int64_t *it = items + (int64_t)idx * stride;
-    const int64_t len = it[VC_CHAIN_LEN];
-    const int nhop = (int)it[VC_CHAIN_NHOP];
-    if (len <= 0 || nhop <= 0) return;
-    const char *src = vc_resolve(it[VC_CHAIN_SRC], sendbuf, recvbuf, stage);
-    char *dst = vc_resolve(it[VC_CHAIN_HEAD], sendbuf, recvbuf, stage);
+// so one mapping of lanes to window vectors serves them all).  dst_of(k) is where hop k puts the piece.
+template <class DstOf>
+__device__ __forceinline__ void vc_forward_piece(const char *src, int64_t len, int nhop, DstOf dst_of) {
+    char *dst = dst_of(0);
     const int t = threadIdx.x;
     const int64_t w = (int64_t)((uintptr_t)dst & (VC_LINE - 1));
     const int64_t first_full = (w + 15) >> 4, end_full = (w + len) >> 4;
@@ -111,7 +107,7 @@ __global__ __launch_bounds__(VC_THREADS) void vc_copy_chains_kernel(const int64_
     char edge_byte = 0;
     if (edge >= 0) edge_byte = src[edge];
     for (int k = 0; k < nhop; k++) {
-        if (k) dst = vc_resolve(it[VC_CHAIN_HEAD + k], sendbuf, recvbuf, stage);
+        if (k) dst = dst_of(k);
         char *dw = dst - w;
         if (edge >= 0) dst[edge] = edge_byte;
         if (has0) vc_store16(dw + ((int64_t)t << 4), v0);
@@ -119,11 +115,81 @@ __global__ __launch_bounds__(VC_THREADS) void vc_copy_chains_kernel(const int64_
     }
 }
 
+__global__ __launch_bounds__(VC_THREADS) void vc_copy_chains_kernel(const int64_t *__restrict__ items, int stride, unsigned nitems,
+                                                                    const char *__restrict__ sendbuf, char *__restrict__ recvbuf,
+                                                                    char *__restrict__ stage) {
+    const unsigned per = gridDim.x / VC_XCDS;
+    const unsigned idx = (blockIdx.x % VC_XCDS) * per + blockIdx.x / VC_XCDS;
+    if (idx >= nitems) return;
+    const int64_t *it = items + (int64_t)idx * stride;
+    const int64_t len = it[VC_CHAIN_LEN];
+    const int nhop = (int)it[VC_CHAIN_NHOP];
+    if (len <= 0 || nhop <= 0) return;
+    vc_forward_piece(vc_resolve(it[VC_CHAIN_SRC], sendbuf, recvbuf, stage), len, nhop,
+                     [&](int k) { return vc_resolve(it[VC_CHAIN_HEAD + k], sendbuf, recvbuf, stage); });
+}
+
+// Forwarded execution without a work-item list, for calls whose planning would otherwise cost more than their copying:
+// one workgroup per (source, destination) pair, in the order of the chain items (by destination, then source, an eighth
+// of the pairs per XCD).  The workgroup works out the route of its block in closed form from the plan tables (lane k
+// evaluates hop slot k), then carries the block through it piece by piece.  The kernel is enqueued right behind the
+// planning kernels, before the host has seen their result, so it checks that result itself: nothing is touched when the
+// plan needs more staging than there is or the tables hold negative entries (the host then takes the other path).
+__global__ __launch_bounds__(VC_THREADS) void vc_copy_blocks_kernel(VcSched S, VcTables T, const int64_t *__restrict__ slot_off,
+                                                                    const int64_t *__restrict__ row_base,
+                                                                    const int64_t *__restrict__ header, int64_t stage_cap,
+                                                                    int64_t first_pair, const char *__restrict__ sendbuf,
+                                                                    char *__restrict__ recvbuf, char *__restrict__ stage) {
+    if (header[0] > stage_cap || header[VC_HEADER_BAD] != 0) return;
+    __shared__ int64_t route[VC_MAX_HOP_SLOTS];
+    __shared__ int route_len;
+    const int64_t per = gridDim.x / VC_XCDS;
+    const int64_t idx = first_pair + (int64_t)(blockIdx.x % VC_XCDS) * per + blockIdx.x / VC_XCDS;
+    if (idx >= (int64_t)S.P * S.P) return;
+    const int t = (int)(idx / S.P), s = (int)(idx % S.P);
+    const int64_t len = (int64_t)T.sc[(int64_t)s * S.P + t] * S.esz;
+    if (len <= 0) return;
+    if (threadIdx.x < VC_WAVE) {                          // hop slots <= VC_MAX_HOP_SLOTS < lanes of the first wavefront
+        int64_t dst = 0;
+        const bool moves = (int)threadIdx.x < vc_hop_slots(S) && vc_block_hop(S, T, slot_off, row_base, s, t, threadIdx.x, dst);
+        const unsigned long long mask = __ballot(moves);
+        if (moves) route[__popcll(mask & ((1ull << threadIdx.x) - 1))] = dst;
+        if (threadIdx.x == 0) route_len = __popcll(mask);
+    }
+    __syncthreads();
+    const int nhop = route_len;
+    if (nhop <= 0) return;
+    const char *src = sendbuf + vc_send_offset(S, T, s, t);
+    const int phase = vc_phase(S, T, s, t), cut = vc_chain_cut(S, T, s, t);
+    if (vc_fits_one_item(len, phase)) {
+        vc_forward_piece(src, len, nhop, [&](int k) { return vc_resolve(route[k], sendbuf, recvbuf, stage); });
+        return;
+    }
+    const int64_t pieces = vc_chunk_count(len, phase, cut);
+    for (int64_t c = 0; c < pieces; c++) {                // the same cuts as the chain items of this block
+        const int64_t lo = c == 0 ? 0 : c * VC_PIECE - cut;
+        int64_t hi = (c + 1) * VC_PIECE - cut;
+        if (hi > len) hi = len;
+        vc_forward_piece(src + lo, hi - lo, nhop, [&](int k) { return vc_resolve(route[k] + lo, sendbuf, recvbuf, stage); });
+    }
+}
+
+hipError_t vc_launch_copy_blocks(const VcSched &S, VcTables T, const int64_t *slot_off, const int64_t *row_base, const int64_t *header,
+                                 int64_t stage_cap, const char *sendbuf, char *recvbuf, char *stage, hipStream_t st) {
+    const int64_t npairs = (int64_t)S.P * S.P;
+    for (int64_t done = 0; done < npairs; done += VC_MAX_GRID) {
+        const int64_t now = npairs - done < VC_MAX_GRID ? npairs - done : VC_MAX_GRID;
+        const int64_t grid = (now + VC_XCDS - 1) / VC_XCDS * VC_XCDS;
+        hipLaunchKernelGGL(vc_copy_blocks_kernel, dim3((unsigned)grid), dim3(VC_THREADS), 0, st, S, T, slot_off, row_base, header, stage_cap,
+                           done, sendbuf, recvbuf, stage);
+    }
+    return hipGetLastError();
+}
+
 hipError_t vc_launch_copy_chains(const int64_t *items, int stride, int64_t nitems, const char *sendbuf, char *recvbuf, char *stage,
                                  hipStream_t st) {
-    const int64_t max_grid = 0x7FFFFFF8;
-    for (int64_t done = 0; done < nitems; done += max_grid) {
-        const int64_t now = nitems - done < max_grid ? nitems - done : max_grid;
+    for (int64_t done = 0; done < nitems; done += VC_MAX_GRID) {
+        const int64_t now = nitems - done < VC_MAX_GRID ? nitems - done : VC_MAX_GRID;
         const int64_t grid = (now + VC_XCDS - 1) / VC_XCDS * VC_XCDS;
         hipLaunchKernelGGL(vc_copy_chains_kernel, dim3((unsigned)grid), dim3(VC_THREADS), 0, st, items + done * stride, stride, (unsigned)now,
                            sendbuf, recvbuf, stage);
@@ -132,9 +198,8 @@ hipError_t vc_launch_copy_chains(const int64_t *items, int stride, int64_t nitem
 }
 
 hipError_t vc_launch_copy_items(const VcDesc *items, int64_t nitems, const char *sendbuf, char *recvbuf, char *stage, hipStream_t st) {
-    const int64_t max_grid = 0x7FFFFFF8;                  // gridDim.x limit; more items than that go in several launches
-    for (int64_t done = 0; done < nitems; done += max_grid) {
-        const int64_t now = nitems - done < max_grid ? nitems - done : max_grid;
+    for (int64_t done = 0; done < nitems; done += VC_MAX_GRID) {
+        const int64_t now = nitems - done < VC_MAX_GRID ? nitems - done : VC_MAX_GRID;
         const int64_t grid = (now + VC_XCDS - 1) / VC_XCDS * VC_XCDS;
         hipLaunchKernelGGL(vc_copy_items_kernel, dim3((unsigned)grid), dim3(VC_THREADS), 0, st, items + done, (unsigned)now, sendbuf,
                            recvbuf, stage);
@@ -151,8 +216,10 @@ __global__ __launch_bounds__(VC_THREADS) void vc_calibration_copy_kernel(const v
 
 hipError_t vc_launch_calibration_copy(const char *src, char *dst, int64_t nbytes, hipStream_t st) {
     const int64_t nvec = nbytes / 16;
-    if (nvec <= 0) return hipSuccess;
-    hipLaunchKernelGGL(vc_calibration_copy_kernel, dim3((unsigned)((nvec + VC_THREADS - 1) / VC_THREADS)), dim3(VC_THREADS), 0, st,
-                       reinterpret_cast<const vc_u32x4 *>(src), reinterpret_cast<vc_u32x4 *>(dst), nvec);
+    for (int64_t done = 0; done < nvec; done += VC_MAX_GRID * VC_THREADS) {
+        const int64_t now = nvec - done < VC_MAX_GRID * VC_THREADS ? nvec - done : VC_MAX_GRID * VC_THREADS;
+        hipLaunchKernelGGL(vc_calibration_copy_kernel, dim3((unsigned)((now + VC_THREADS - 1) / VC_THREADS)), dim3(VC_THREADS), 0, st,
+                           reinterpret_cast<const vc_u32x4 *>(src) + done, reinterpret_cast<vc_u32x4 *>(dst) + done, now);
+    }
     return hipGetLastError();
 }

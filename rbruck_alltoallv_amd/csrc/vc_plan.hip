@@ -29,10 +29,15 @@ __global__ __launch_bounds__(VC_THREADS) void vc_plan_rows(VcSched S, VcLaunchPa
     const int to = blockIdx.x, P = S.P;
     const int nreg = S.w + S.w2;                          // the organized region is laid out by vc_plan_org_rows
     if ((int)blockIdx.y == nreg + nl) {                   // forwarded execution: chain items whose last hop ends on this rank
-        int64_t items = 0;
-        for (int s = threadIdx.x; s < P; s += VC_THREADS) items += vc_chain_count(S, T, s, to);
+        int64_t items = 0, most = 0;
+        for (int s = threadIdx.x; s < P; s += VC_THREADS) {
+            const int64_t cnt = vc_chain_count(S, T, s, to);
+            items += cnt;
+            most = cnt > most ? cnt : most;
+        }
         items = vc_block_sum(items, lds);
-        if (threadIdx.x == 0) chain_row_tot[to] = items;
+        most = vc_block_max(most, lds);
+        if (threadIdx.x == 0) { chain_row_tot[to] = items; chain_row_tot[P + to] = most; }
         return;
     }
     if ((int)blockIdx.y < nreg) {
@@ -111,16 +116,18 @@ __global__ __launch_bounds__(VC_THREADS) void vc_plan_bases(int P, int w, int nl
     const int L = blockIdx.x;
     int64_t carry = 0, bytes = 0;
     if (L == nl + 1) {                                    // forwarded execution: first chain item of every final receiver
+        int64_t most = 0;
         for (int b0 = 0; b0 < P; b0 += VC_THREADS) {
             const int i = b0 + threadIdx.x;
             int64_t total;
             const int64_t ex = vc_block_exclusive_scan((i < P) ? chain_row_tot[i] : 0, lds, total);
-            if (i < P) chain_row_base[i] = carry + ex;
+            if (i < P) { chain_row_base[i] = carry + ex; most = chain_row_tot[P + i] > most ? chain_row_tot[P + i] : most; }
             carry += total;
         }
+        most = vc_block_max(most, lds);
         if (threadIdx.x == 0) {
-            header[2] = carry;
-            if (header_host) header_host[2] = carry;
+            header[2] = carry; header[VC_HEADER_MAX_PIECES] = most;
+            if (header_host) { header_host[2] = carry; header_host[VC_HEADER_MAX_PIECES] = most; }
         }
         return;
     }
@@ -139,8 +146,8 @@ __global__ __launch_bounds__(VC_THREADS) void vc_plan_bases(int P, int w, int nl
         bytes = vc_block_sum(bytes, lds);
         bad = vc_block_sum(bad, lds);
         if (threadIdx.x == 0) {
-            header[0] = carry; header[1] = bytes; header[3 + nl] = bad;
-            if (header_host) { header_host[0] = carry; header_host[1] = bytes; header_host[3 + nl] = bad; }
+            header[0] = carry; header[1] = bytes; header[VC_HEADER_BAD] = bad;
+            if (header_host) { header_host[0] = carry; header_host[1] = bytes; header_host[VC_HEADER_BAD] = bad; }
         }
         return;
     }
@@ -155,8 +162,8 @@ __global__ __launch_bounds__(VC_THREADS) void vc_plan_bases(int P, int w, int nl
     }
     bytes = vc_block_sum(bytes, lds);
     if (threadIdx.x == 0) {
-        header[3 + L] = bytes; header[3 + 2 * nl + L] = carry;
-        if (header_host) { header_host[3 + L] = bytes; header_host[3 + 2 * nl + L] = carry; }      // pinned host memory: no copy back
+        header[VC_HEADER_FIXED + L] = bytes; header[VC_HEADER_FIXED + nl + L] = carry;
+        if (header_host) { header_host[VC_HEADER_FIXED + L] = bytes; header_host[VC_HEADER_FIXED + nl + L] = carry; }      // pinned host memory: no copy back
     }
 }
 
@@ -171,7 +178,7 @@ __global__ __launch_bounds__(VC_THREADS) void vc_plan_emit(VcSched S, VcLaunchPa
     const int to = blockIdx.x, L = blockIdx.y, P = S.P;
     const VcLaunchInfo info = launches ? launches[L] : pack.info[L];
     int64_t first = 0;                                    // items of the launches before this one
-    for (int k = threadIdx.x; k < L; k += VC_THREADS) first += header[3 + 2 * nl + k];
+    for (int k = threadIdx.x; k < L; k += VC_THREADS) first += header[VC_HEADER_FIXED + nl + k];
     first = vc_block_sum(first, lds);
     int64_t carry = first + item_row_base[(int64_t)L * P + to];
     // copies of many pieces are written by the whole workgroup: their pieces are numbered by a second prefix sum and

@@ -46,3 +46,19 @@ __device__ __forceinline__ int64_t vc_block_sum(int64_t v, int64_t *lds) {
     (void)vc_block_exclusive_scan(v, lds, total);
     return total;
 }
+
+// Maximum across a 256-thread workgroup (every thread gets the result).
+__device__ __forceinline__ int64_t vc_block_max(int64_t v, int64_t *lds) {
+#pragma unroll
+    for (int o = VC_WAVE / 2; o > 0; o >>= 1) {
+        const int64_t u = __shfl_xor(v, o, VC_WAVE);
+        v = u > v ? u : v;
+    }
+    __syncthreads();                       // protects lds from the previous use
+    if ((threadIdx.x & (VC_WAVE - 1)) == 0) lds[threadIdx.x / VC_WAVE] = v;
+    __syncthreads();
+    int64_t m = lds[0];
+#pragma unroll
+    for (int k = 1; k < VC_WAVES_PER_BLOCK; k++) m = lds[k] > m ? lds[k] : m;
+    return m;
+}

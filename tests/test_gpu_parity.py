@@ -15,13 +15,17 @@ pytestmark = pytest.mark.gpu
 CASES = load_golden()
 
 
-@pytest.fixture(scope="module", params=["forwarded", "launch-per-digit"])
+# vc_comm_set_forwarding: 2 forwarded through a work-item list, 3 forwarded without one, 0 one launch per digit phase
+MODES = {"forwarded": 2, "forwarded-listless": 3, "launch-per-digit": 0}
+
+
+@pytest.fixture(scope="module", params=list(MODES))
 def api(request):
-    """The package's API with one of the two execution modes set on every communicator the tests create."""
+    """The package's API with one of the execution modes set on every communicator the tests create."""
     import torch
     assert torch.cuda.is_available(), "these tests need the GPU"
     from rbruck_alltoallv_amd import api as A
-    A.DEFAULT_FORWARDING = request.param == "forwarded"
+    A.DEFAULT_FORWARDING = MODES[request.param]
     yield A
     A.DEFAULT_FORWARDING = None
 
@@ -516,6 +520,26 @@ def test_more_than_4096_ranks(api):
     dp.comm.free()
 
 
+def test_more_work_items_than_one_launch_holds(api):
+    """4100 x 4100 non-empty pairs are 16.81 M work items; one dispatch holds 2^32 / 256 - 8 workgroups (its grid is
+    counted in work-items, in 32 bits), so the list goes out in two launches."""
+    P = 4100
+    rng = np.random.default_rng(8)
+    counts = rng.integers(1, 4, (P, P)).astype(np.int32)
+    prob = W.make_problem(counts, 1, 0, 0)
+    dp = api.DeviceProblem(prob)
+    ds = dp.new_send_arena()
+    dp.fill_payload(0, 6, ds)
+    for name, fn in (("spreadout", lambda dr: api.spreadout_alltoallv(dp, ds, dr)),
+                     ("twophase r=65", lambda dr: api.twophase_rbruck_alltoallv(65, dp, ds, dr))):
+        print("  ", name, flush=True)
+        dr = dp.new_recv_arena(0xEE)
+        assert fn(dr) == 0, (name, dp.comm.error())
+        assert dp.verify(ds, dr) == 0, name
+        assert dp.comm.last_stats().payload_bytes == prob.payload_bytes
+    dp.comm.free()
+
+
 def test_distributions_of_the_reference_drivers(api):
     """examples/other_distributions.cpp (truncated normal, power law) and examples/FFT_distribution.cpp (sparse blocks) at
     256 ranks, 8-byte elements, through the functions those drivers call."""
@@ -598,7 +622,7 @@ def test_golden_case_forwarded(api, case):
     want = np.full(prob.recv_bytes, 0xEE, dtype=np.uint8)
     assert run_on(O, case, prob, send.copy(), want) == 0
     dp = api.DeviceProblem(prob)
-    dp.comm.set_forwarding(True)
+    dp.comm.set_forwarding(api.DEFAULT_FORWARDING or 2)
     dsend = _to_dev(api, send)
     drecv = dp.new_recv_arena(0xEE)
     rc = run_on(api, case, dp, dsend, drecv)
@@ -667,6 +691,30 @@ def test_seeded_random_sweep(api):
         dp.comm.free()
 
 
+def test_default_mode_picks_the_listless_kernel_for_small_calls(api):
+    """Mode 1 (the library's default): forwarded, and after a call of few short blocks the next one goes without the
+    work-item list; after one with long blocks the list comes back.  Every call is exact whichever way it went."""
+    small = W.make_problem(W.counts_uniform_random(64, 4096, seed=0), 1, 0, 0)
+    big_counts = W.counts_uniform_random(64, 4096, seed=1)
+    big_counts[5, 9] = 200000                          # 49 pieces
+    big = W.make_problem(big_counts, 1, 0, 0)
+    comm = api.VirtualComm(64)
+    comm.set_forwarding(1)
+    seen = []
+    for prob in (small, small, small, big, big, small, small):
+        dp = api.DeviceProblem(prob, comm=comm)
+        comm.set_forwarding(1)
+        ds, dr = dp.new_send_arena(), dp.new_recv_arena()
+        dp.fill_payload(0, 4, ds)
+        assert api.twophase_rbruck_alltoallv(2, dp, ds, dr) == 0, comm.error()
+        assert dp.verify(ds, dr) == 0
+        st = comm.last_stats()
+        assert st.n_launches == 1 and st.payload_bytes == prob.payload_bytes
+        seen.append(st.execution)
+    assert seen == [1, 2, 2, 2, 1, 1, 2]
+    comm.free()
+
+
 def test_phase_times(api):
     """With timing on, the statistics split the launches as the reference's phase timers do (src/rbruckv.h:13-18):
     inside the nodes and between them."""
@@ -714,8 +762,8 @@ def test_both_execution_modes_leave_the_same_staging(api):
         for name, fn in calls:
             print("  ", name, flush=True)
             snaps, sizes = [], []
-            for forward in (False, True):
-                dp.comm.set_forwarding(forward)
+            for mode in (0, 2, 3):
+                dp.comm.set_forwarding(mode)
                 dr = dp.new_recv_arena(0xEE)
                 assert fn(dp, ds, dr) == 0, (name, dp.comm.error())          # sizes the arena
                 ptr, size = dp.comm.staging()
@@ -727,10 +775,11 @@ def test_both_execution_modes_leave_the_same_staging(api):
                 assert dp.comm.staging() == (ptr, size)
                 snap = torch.empty(n, dtype=torch.uint8, device="cuda:0")
                 assert lib.vc_calibration_copy(snap.data_ptr(), ptr, n, h) == 0
+                assert dp.comm.last_stats().execution == {0: 0, 2: 1, 3: 2}[mode]
                 snaps.append(snap.cpu().numpy())
                 sizes.append(size)
-            assert sizes[0] == sizes[1], name
-            assert np.array_equal(snaps[0], snaps[1]), name
+            assert sizes[0] == sizes[1] == sizes[2], name
+            assert np.array_equal(snaps[0], snaps[1]) and np.array_equal(snaps[0], snaps[2]), name
             assert np.count_nonzero(snaps[0] != 0xAB) > sizes[0] // 4, name        # the slots were written
         dp.comm.free()
 
@@ -751,7 +800,7 @@ def test_forwarded_shapes_plans_and_graphs(api):
             (W.make_problem(c5, 8, 0, 0), [("tuna r=32", lambda dp, s, d: api.tuna_algorithm(32, 0, dp, s, d), False),
                                           ("spreadout", lambda dp, s, d: api.spreadout_alltoallv(dp, s, d), False)])):
         dp = api.DeviceProblem(prob)
-        dp.comm.set_forwarding(True)
+        dp.comm.set_forwarding(api.DEFAULT_FORWARDING or 2)
         ds = dp.new_send_arena()
         dp.fill_payload(0, 3, ds)
         for name, fn, packed in calls:
@@ -767,7 +816,7 @@ def test_forwarded_shapes_plans_and_graphs(api):
     send = W.fill_send_arena(prob, 0, 9)
     want = W.expected_recv_arena(prob, send)
     dp = api.DeviceProblem(prob)
-    dp.comm.set_forwarding(True)
+    dp.comm.set_forwarding(api.DEFAULT_FORWARDING or 2)
     sbig = torch.zeros(prob.send_bytes + 64, dtype=torch.uint8, device="cuda:0")
     ds = sbig[5:5 + prob.send_bytes]
     ds.copy_(torch.from_numpy(send))
