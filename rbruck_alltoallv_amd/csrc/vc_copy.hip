@@ -161,15 +161,10 @@ __global__ __launch_bounds__(VC_THREADS) void vc_copy_blocks_kernel(VcSched S, V
     if (nhop <= 0) return;
     const char *src = sendbuf + vc_send_offset(S, T, s, t);
     const int phase = vc_phase(S, T, s, t), cut = vc_chain_cut(S, T, s, t);
-    if (vc_fits_one_item(len, phase)) {
-        vc_forward_piece(src, len, nhop, [&](int k) { return vc_resolve(route[k], sendbuf, recvbuf, stage); });
-        return;
-    }
     const int64_t pieces = vc_chunk_count(len, phase, cut);
     for (int64_t c = 0; c < pieces; c++) {                // the same cuts as the chain items of this block
-        const int64_t lo = c == 0 ? 0 : c * VC_PIECE - cut;
-        int64_t hi = (c + 1) * VC_PIECE - cut;
-        if (hi > len) hi = len;
+        int64_t lo, hi;
+        vc_piece_range(len, phase, cut, c, lo, hi);
         vc_forward_piece(src + lo, hi - lo, nhop, [&](int k) { return vc_resolve(route[k] + lo, sendbuf, recvbuf, stage); });
     }
 }

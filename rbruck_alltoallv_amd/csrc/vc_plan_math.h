@@ -303,12 +303,18 @@ VC_HD int64_t vc_chunk_count(int64_t len, int phase, int cut) {
     return vc_fits_one_item(len, phase) ? 1 : (len + cut + VC_PIECE - 1) / VC_PIECE;
 }
 
+// Bytes [lo, hi) of a copy of `len` bytes that piece c of its vc_chunk_count(len, phase, cut) pieces moves.
+VC_HD void vc_piece_range(int64_t len, int phase, int cut, int64_t c, int64_t &lo, int64_t &hi) {
+    if (vc_fits_one_item(len, phase)) { lo = 0; hi = len; return; }
+    lo = c == 0 ? 0 : c * VC_PIECE - cut;
+    hi = (c + 1) * VC_PIECE - cut;
+    if (hi > len) hi = len;
+}
+
 VC_HD VcDesc vc_chunk_of(const VcDesc &whole, int64_t c, int phase, int cut) {
-    if (vc_fits_one_item(whole.len, phase)) return whole;
+    int64_t lo, hi;
+    vc_piece_range(whole.len, phase, cut, c, lo, hi);
     VcDesc d = whole;
-    const int64_t lo = c == 0 ? 0 : c * VC_PIECE - cut;
-    int64_t hi = (c + 1) * VC_PIECE - cut;
-    if (hi > whole.len) hi = whole.len;
     d.src += lo; d.dst += lo; d.len = hi - lo;
     return d;
 }
