@@ -332,7 +332,7 @@ def main() -> None:
         "one_pass_comparator": {"func": "spreadout_alltoallv", "ms_per_call": round(comp_s * 1e3, 4),
                                 "GBps_effective": round(S / comp_s / 1e9, 1),
                                 "hbm_frac": round(2 * S / comp_s / 1e9 / HBM_PEAK_GBPS, 4), "mismatched_bytes": int(comp_bad)},
-        "roofline": {"bound": "hbm", "kernel": EXECUTION_KERNELS[int(st.execution)], "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
+        "roofline": {"bound": "hbm", "kernel": EXECUTION_KERNELS[int(st.execution)] + ("" if st.execution == 2 else f"<{int(st.lanes_per_item)}>"), "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
                      "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
                      "traffic": MEASURED_TRAFFIC_PER_LAUNCH.get((args.workload, func, int(bool(args.forward)))),
                      "avg_launch_ms": round(kern_ms / max(nkern, 1), 4),

@@ -135,9 +135,11 @@ hipError_t vc_launch_plan_emit(const VcSched &S, const VcLaunchInfo *launches_ho
 hipError_t vc_launch_traffic(const VcDesc *desc, int64_t ndesc, int64_t *matrix, int P, hipStream_t st);
 
 // vc_copy.hip
-hipError_t vc_launch_copy_items(const VcDesc *items, int64_t nitems, const char *sendbuf, char *recvbuf, char *stage, hipStream_t st);
-hipError_t vc_launch_copy_chains(const int64_t *items, int stride, int64_t nitems, const char *sendbuf, char *recvbuf, char *stage,
-                                 hipStream_t st);
+// lanes: VC_THREADS (a workgroup per item) or VC_WAVE (a wavefront per item, for lists of short pieces)
+hipError_t vc_launch_copy_items(const VcDesc *items, int64_t nitems, int lanes, const char *sendbuf, char *recvbuf, char *stage,
+                                hipStream_t st);
+hipError_t vc_launch_copy_chains(const int64_t *items, int stride, int64_t nitems, int lanes, const char *sendbuf, char *recvbuf,
+                                 char *stage, hipStream_t st);
 // Forwarded execution without a work-item list: one workgroup per (source, destination) pair works out the route of its
 // block from the plan tables and carries it through.  Reads the device `header` the planning kernels before it on the
 // stream have written and does nothing when the plan needs more than stage_cap bytes of staging or found bad tables.

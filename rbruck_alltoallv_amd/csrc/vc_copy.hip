@@ -42,63 +42,36 @@ __device__ __forceinline__ char *vc_resolve(int64_t loc, const char *sendbuf, ch
     return base + off;
 }
 
-// One workgroup per work item.  Lane t owns the t-th and the (t + 256)-th 16-byte vector of the window that starts at
-// the 128-byte boundary at or below dst, so every wave stores whole cache lines whatever the byte phase of the block
-// (measured: +4 % over counting vectors from the first 16-byte boundary of dst).  Vectors that lie fully inside the
-// block are moved by (possibly unaligned) 16-byte loads and aligned stores; the < 16 bytes before the first and after
-// the last of them are moved byte-wise.  The planner guarantees len + (dst & 127) <= VC_CHUNK.
+// One workgroup (or one wavefront) of LANES lanes per work item.  Lane t owns the t-th, (t + LANES)-th, ... 16-byte vector
+// of the window that starts at the 128-byte boundary at or below dst, so every wave stores whole cache lines whatever
+// the byte phase of the block (measured: +4 % over counting vectors from the first 16-byte boundary of dst).  Vectors
+// that lie fully inside the block are moved by (possibly unaligned) 16-byte loads and aligned stores; the < 16 bytes
+// before the first and after the last of them are moved byte-wise (lanes 0..15 the head, lanes 16..31 the tail: one byte
+// load and one byte store each).  The planner guarantees len + (dst & 127) <= VC_CHUNK.
 #define VC_XCDS 8
 // Workgroups of one launch: a dispatch counts its grid in work-items in 32 bits, so gridDim.x * VC_THREADS must stay
 // below 2^32 (a larger grid is not refused: it runs truncated); longer lists go out in several launches.  A multiple of
 // VC_XCDS.
 #define VC_MAX_GRID ((int64_t)((1ull << 32) / VC_THREADS) - VC_XCDS)
-__global__ __launch_bounds__(VC_THREADS) void vc_copy_items_kernel(const VcDesc *__restrict__ items, unsigned nitems,
-                                                                   const char *__restrict__ sendbuf, char *__restrict__ recvbuf,
-                                                                   char *__restrict__ stage) {
-    // gridDim.x is a multiple of VC_XCDS; XCD k = blockIdx.x % VC_XCDS works through items [k * per, (k + 1) * per)
-    const unsigned per = gridDim.x / VC_XCDS;
-    const unsigned idx = (blockIdx.x % VC_XCDS) * per + blockIdx.x / VC_XCDS;
-    if (idx >= nitems) return;
-    const VcDesc d = items[idx];
-    const int64_t len = d.len;
-    if (len <= 0) return;
-    const char *src = vc_resolve(d.src, sendbuf, recvbuf, stage);
-    char *dst = vc_resolve(d.dst, sendbuf, recvbuf, stage);
-    const int t = threadIdx.x;
-    const int64_t w = (int64_t)((uintptr_t)dst & (VC_LINE - 1));     // offset of the block inside the window
-    // window vector j holds block bytes [16 j - w, 16 j - w + 16)
-    const int64_t first_full = (w + 15) >> 4, end_full = (w + len) >> 4;    // at most VC_CHUNK / 16 = 2 * VC_THREADS
-    const char *sw = src - w;
-    char *dw = dst - w;
-    vc_u32x4 v0, v1;
-    const bool has0 = t >= first_full && t < end_full, has1 = t + VC_THREADS < end_full;
-    if (has0) v0 = vc_load16(sw + ((int64_t)t << 4));
-    if (has1) v1 = vc_load16(sw + ((int64_t)(t + VC_THREADS) << 4));
-    // the < 16 head bytes (lanes 0..15) and the < 16 tail bytes (lanes 16..31) share one byte load and one byte store
-    int64_t head = (first_full << 4) - w;
-    if (head > len) head = len;
-    int64_t done = (end_full << 4) - w;
-    if (done < head) done = head;
-    const int64_t edge = t < 16 ? (t < head ? t : -1) : (t < 32 && done + (t - 16) < len ? done + (t - 16) : -1);
-    if (edge >= 0) dst[edge] = src[edge];
-    if (has0) vc_store16(dw + ((int64_t)t << 4), v0);
-    if (has1) vc_store16(dw + ((int64_t)(t + VC_THREADS) << 4), v1);
-}
-
 // Forwarded execution: one workgroup carries a piece through all the hops of its block.  The piece is read once, from
 // sendbuf; every hop stores the same registers (all destinations of a block share the offset inside their cache line,
 // so one mapping of lanes to window vectors serves them all).  dst_of(k) is where hop k puts the piece.
-template <class DstOf>
+template <int LANES, class DstOf>
 __device__ __forceinline__ void vc_forward_piece(const char *src, int64_t len, int nhop, DstOf dst_of) {
+    constexpr int VECS = VC_CHUNK / 16 / LANES;           // window vectors per lane: 2 for a workgroup of 256, 8 for one wavefront
     char *dst = dst_of(0);
     const int t = threadIdx.x;
     const int64_t w = (int64_t)((uintptr_t)dst & (VC_LINE - 1));
     const int64_t first_full = (w + 15) >> 4, end_full = (w + len) >> 4;
     const char *sw = src - w;
-    vc_u32x4 v0, v1;
-    const bool has0 = t >= first_full && t < end_full, has1 = t + VC_THREADS < end_full;
-    if (has0) v0 = vc_load16(sw + ((int64_t)t << 4));
-    if (has1) v1 = vc_load16(sw + ((int64_t)(t + VC_THREADS) << 4));
+    vc_u32x4 v[VECS];
+    bool has[VECS];
+#pragma unroll
+    for (int i = 0; i < VECS; i++) {
+        const int64_t j = t + i * LANES;
+        has[i] = (i > 0 || j >= first_full) && j < end_full;
+        if (has[i]) v[i] = vc_load16(sw + (j << 4));
+    }
     int64_t head = (first_full << 4) - w;
     if (head > len) head = len;
     int64_t done = (end_full << 4) - w;
@@ -110,14 +83,19 @@ __device__ __forceinline__ void vc_forward_piece(const char *src, int64_t len, i
         if (k) dst = dst_of(k);
         char *dw = dst - w;
         if (edge >= 0) dst[edge] = edge_byte;
-        if (has0) vc_store16(dw + ((int64_t)t << 4), v0);
-        if (has1) vc_store16(dw + ((int64_t)(t + VC_THREADS) << 4), v1);
+#pragma unroll
+        for (int i = 0; i < VECS; i++)
+            if (has[i]) vc_store16(dw + ((int64_t)(t + i * LANES) << 4), v[i]);
     }
 }
 
-__global__ __launch_bounds__(VC_THREADS) void vc_copy_chains_kernel(const int64_t *__restrict__ items, int stride, unsigned nitems,
-                                                                    const char *__restrict__ sendbuf, char *__restrict__ recvbuf,
-                                                                    char *__restrict__ stage) {
+// LANES = VC_THREADS: one workgroup of four wavefronts per item, the shape that moves blocks of several KiB fastest.
+// LANES = VC_WAVE: one wavefront per item, for lists of short pieces: four times as many items in flight per compute
+// unit, and no wavefronts that start only to find nothing left for them in a piece of a few hundred bytes.
+template <int LANES>
+__global__ __launch_bounds__(LANES) void vc_copy_chains_kernel(const int64_t *__restrict__ items, int stride, unsigned nitems,
+                                                               const char *__restrict__ sendbuf, char *__restrict__ recvbuf,
+                                                               char *__restrict__ stage) {
     const unsigned per = gridDim.x / VC_XCDS;
     const unsigned idx = (blockIdx.x % VC_XCDS) * per + blockIdx.x / VC_XCDS;
     if (idx >= nitems) return;
@@ -125,8 +103,23 @@ __global__ __launch_bounds__(VC_THREADS) void vc_copy_chains_kernel(const int64_
     const int64_t len = it[VC_CHAIN_LEN];
     const int nhop = (int)it[VC_CHAIN_NHOP];
     if (len <= 0 || nhop <= 0) return;
-    vc_forward_piece(vc_resolve(it[VC_CHAIN_SRC], sendbuf, recvbuf, stage), len, nhop,
-                     [&](int k) { return vc_resolve(it[VC_CHAIN_HEAD + k], sendbuf, recvbuf, stage); });
+    vc_forward_piece<LANES>(vc_resolve(it[VC_CHAIN_SRC], sendbuf, recvbuf, stage), len, nhop,
+                            [&](int k) { return vc_resolve(it[VC_CHAIN_HEAD + k], sendbuf, recvbuf, stage); });
+}
+
+// Launch-per-digit execution: one hop of one piece per item.
+template <int LANES>
+__global__ __launch_bounds__(LANES) void vc_copy_items_kernel(const VcDesc *__restrict__ items, unsigned nitems,
+                                                              const char *__restrict__ sendbuf, char *__restrict__ recvbuf,
+                                                              char *__restrict__ stage) {
+    // gridDim.x is a multiple of VC_XCDS; XCD k = blockIdx.x % VC_XCDS works through items [k * per, (k + 1) * per)
+    const unsigned per = gridDim.x / VC_XCDS;
+    const unsigned idx = (blockIdx.x % VC_XCDS) * per + blockIdx.x / VC_XCDS;
+    if (idx >= nitems) return;
+    const VcDesc d = items[idx];
+    if (d.len <= 0) return;
+    char *dst = vc_resolve(d.dst, sendbuf, recvbuf, stage);
+    vc_forward_piece<LANES>(vc_resolve(d.src, sendbuf, recvbuf, stage), d.len, 1, [&](int) { return dst; });
 }
 
 // Forwarded execution without a work-item list, for calls whose planning would otherwise cost more than their copying:
@@ -165,7 +158,7 @@ __global__ __launch_bounds__(VC_THREADS) void vc_copy_blocks_kernel(VcSched S, V
     for (int64_t c = 0; c < pieces; c++) {                // the same cuts as the chain items of this block
         int64_t lo, hi;
         vc_piece_range(len, phase, cut, c, lo, hi);
-        vc_forward_piece(src + lo, hi - lo, nhop, [&](int k) { return vc_resolve(route[k] + lo, sendbuf, recvbuf, stage); });
+        vc_forward_piece<VC_THREADS>(src + lo, hi - lo, nhop, [&](int k) { return vc_resolve(route[k] + lo, sendbuf, recvbuf, stage); });
     }
 }
 
@@ -181,23 +174,32 @@ hipError_t vc_launch_copy_blocks(const VcSched &S, VcTables T, const int64_t *sl
     return hipGetLastError();
 }
 
-hipError_t vc_launch_copy_chains(const int64_t *items, int stride, int64_t nitems, const char *sendbuf, char *recvbuf, char *stage,
-                                 hipStream_t st) {
+hipError_t vc_launch_copy_chains(const int64_t *items, int stride, int64_t nitems, int lanes, const char *sendbuf, char *recvbuf,
+                                 char *stage, hipStream_t st) {
     for (int64_t done = 0; done < nitems; done += VC_MAX_GRID) {
         const int64_t now = nitems - done < VC_MAX_GRID ? nitems - done : VC_MAX_GRID;
         const int64_t grid = (now + VC_XCDS - 1) / VC_XCDS * VC_XCDS;
-        hipLaunchKernelGGL(vc_copy_chains_kernel, dim3((unsigned)grid), dim3(VC_THREADS), 0, st, items + done * stride, stride, (unsigned)now,
-                           sendbuf, recvbuf, stage);
+        if (lanes == VC_WAVE)
+            hipLaunchKernelGGL(vc_copy_chains_kernel<VC_WAVE>, dim3((unsigned)grid), dim3(VC_WAVE), 0, st, items + done * stride, stride,
+                               (unsigned)now, sendbuf, recvbuf, stage);
+        else
+            hipLaunchKernelGGL(vc_copy_chains_kernel<VC_THREADS>, dim3((unsigned)grid), dim3(VC_THREADS), 0, st, items + done * stride,
+                               stride, (unsigned)now, sendbuf, recvbuf, stage);
     }
     return hipGetLastError();
 }
 
-hipError_t vc_launch_copy_items(const VcDesc *items, int64_t nitems, const char *sendbuf, char *recvbuf, char *stage, hipStream_t st) {
+hipError_t vc_launch_copy_items(const VcDesc *items, int64_t nitems, int lanes, const char *sendbuf, char *recvbuf, char *stage,
+                                hipStream_t st) {
     for (int64_t done = 0; done < nitems; done += VC_MAX_GRID) {
         const int64_t now = nitems - done < VC_MAX_GRID ? nitems - done : VC_MAX_GRID;
         const int64_t grid = (now + VC_XCDS - 1) / VC_XCDS * VC_XCDS;
-        hipLaunchKernelGGL(vc_copy_items_kernel, dim3((unsigned)grid), dim3(VC_THREADS), 0, st, items + done, (unsigned)now, sendbuf,
-                           recvbuf, stage);
+        if (lanes == VC_WAVE)
+            hipLaunchKernelGGL(vc_copy_items_kernel<VC_WAVE>, dim3((unsigned)grid), dim3(VC_WAVE), 0, st, items + done, (unsigned)now,
+                               sendbuf, recvbuf, stage);
+        else
+            hipLaunchKernelGGL(vc_copy_items_kernel<VC_THREADS>, dim3((unsigned)grid), dim3(VC_THREADS), 0, st, items + done,
+                               (unsigned)now, sendbuf, recvbuf, stage);
     }
     return hipGetLastError();
 }
