@@ -239,7 +239,8 @@ typedef struct {
     int32_t execution;           /* how the call ran: 0 launch per digit, 1 forwarded through a work-item list, 2 forwarded
                                     without one (see vc_comm_set_forwarding) */
     int32_t lanes_per_item;      /* 256: the copy kernel gave every work item a workgroup; 64: a wavefront (lists of short
-                                    pieces).  Launch-per-digit execution: of the launch that moved the most bytes. */
+                                    pieces); 16: a quarter of one (pieces of a few hundred bytes).  Launch-per-digit
+                                    execution: of the launch that moved the most bytes. */
 } vc_stats_t;
 
 /* Per-launch HIP-event timing of the following calls (0 = off, default). */

@@ -264,10 +264,17 @@ static int plan_sizes(vc_comm *c, const VcSched &S, std::vector<VcLaunchInfo> &L
     return VC_OK;
 }
 
-// Lanes per work item.  A list of short pieces goes to the wavefront-per-item kernel: four times as many items in flight
-// per compute unit.  Measured on 1 Mi items: pieces of 0..128 B take 0.37 of the workgroup-per-item kernel's time,
-// 0..1 KiB 0.5, 0..4 KiB 0.8 - 0.95, pieces around 4 KiB 1.0 - 1.08.  The average piece decides.
-static int lanes_for(int64_t bytes, int64_t items) { return items > 0 && bytes / items < 3072 ? VC_WAVE : VC_THREADS; }
+// Lanes per work item, from the average piece of the list.  Short pieces leave most of a workgroup idle, and what bounds
+// the launch is then the number of items in flight: a wavefront per item keeps four times as many as a workgroup, a
+// quarter of a wavefront sixteen times.  Measured on 1 Mi items (P = 1024, times of the copy kernel, workgroup /
+// wavefront / quarter): pieces uniform in 0..16 B 832 / 269 / 86 us, 0..256 B 883 / 350 / 213, 0..1 KiB 922 / 456 / 445,
+// 0..2 KiB 1105 / 695 / 783, 0..4 KiB 1450 / 1318 / 1479; around 4 KiB and above the workgroup is 5 - 8 % faster than the
+// wavefront.
+static int lanes_for(int64_t bytes, int64_t items) {
+    if (items <= 0) return VC_THREADS;
+    const int64_t average = bytes / items;
+    return average < 448 ? 16 : (average < 3072 ? VC_WAVE : VC_THREADS);
+}
 
 // Step 3b, after the stream has been synchronised: what the planning kernels found.
 static int plan_read(vc_comm *c, const VcSched &S, const std::vector<VcLaunchInfo> &L, PlanInfo &out, bool forward) {

@@ -135,7 +135,8 @@ hipError_t vc_launch_plan_emit(const VcSched &S, const VcLaunchInfo *launches_ho
 hipError_t vc_launch_traffic(const VcDesc *desc, int64_t ndesc, int64_t *matrix, int P, hipStream_t st);
 
 // vc_copy.hip
-// lanes: VC_THREADS (a workgroup per item) or VC_WAVE (a wavefront per item, for lists of short pieces)
+// lanes: VC_THREADS (a workgroup per item), VC_WAVE (a wavefront per item, for lists of short pieces) or 16 (a quarter of
+// a wavefront, for lists of pieces of a few hundred bytes)
 hipError_t vc_launch_copy_items(const VcDesc *items, int64_t nitems, int lanes, const char *sendbuf, char *recvbuf, char *stage,
                                 hipStream_t st);
 hipError_t vc_launch_copy_chains(const int64_t *items, int stride, int64_t nitems, int lanes, const char *sendbuf, char *recvbuf,

@@ -122,6 +122,75 @@ __global__ __launch_bounds__(LANES) void vc_copy_items_kernel(const VcDesc *__re
     vc_forward_piece<LANES>(vc_resolve(d.src, sendbuf, recvbuf, stage), d.len, 1, [&](int) { return dst; });
 }
 
+// A quarter of a wavefront (16 lanes) per item, four items per wavefront, for lists of pieces of a few hundred bytes:
+// such a launch is bound by how many items are in flight, not by HBM, and a piece of 100 bytes has work for 7 lanes.
+// Every group of 16 lanes reads its own item; lane t of the group owns window vectors t, t + 16 of every 512-byte pass
+// (most items need one pass; longer ones loop), and moves head byte t and tail byte t.
+template <class DstOf>
+__device__ __forceinline__ void vc_forward_piece_quarter(const char *src, int64_t len, int nhop, DstOf dst_of) {
+    const int t = threadIdx.x & 15;
+    char *dst = dst_of(0);
+    const int64_t w = (int64_t)((uintptr_t)dst & (VC_LINE - 1));
+    const int64_t first_full = (w + 15) >> 4, end_full = (w + len) >> 4;
+    int64_t head = (first_full << 4) - w;
+    if (head > len) head = len;
+    int64_t done = (end_full << 4) - w;
+    if (done < head) done = head;
+    const bool has_head = t < head, has_tail = done + t < len;
+    char head_byte = 0, tail_byte = 0;
+    if (has_head) head_byte = src[t];
+    if (has_tail) tail_byte = src[done + t];
+    for (int k = 0; k < nhop; k++) {
+        if (k) dst = dst_of(k);
+        if (has_head) dst[t] = head_byte;
+        if (has_tail) dst[done + t] = tail_byte;
+    }
+    const char *sw = src - w;
+    for (int64_t j = t; j < end_full; j += 32) {
+        const bool has0 = j >= first_full, has1 = j + 16 >= first_full && j + 16 < end_full;
+        vc_u32x4 v0, v1;
+        if (has0) v0 = vc_load16(sw + (j << 4));
+        if (has1) v1 = vc_load16(sw + ((j + 16) << 4));
+        for (int k = 0; k < nhop; k++) {
+            char *dw = dst_of(k) - w;
+            if (has0) vc_store16(dw + (j << 4), v0);
+            if (has1) vc_store16(dw + ((j + 16) << 4), v1);
+        }
+    }
+}
+
+#define VC_QUARTER 16                                     // lanes per item of the kernels below
+#define VC_ITEMS_PER_WAVE (VC_WAVE / VC_QUARTER)
+
+// gridDim.x wavefronts, a multiple of VC_XCDS; XCD k works through the k-th eighth of them, each taking four items in a row
+__global__ __launch_bounds__(VC_WAVE) void vc_copy_chains_quarter_kernel(const int64_t *__restrict__ items, int stride, unsigned nitems,
+                                                                         const char *__restrict__ sendbuf, char *__restrict__ recvbuf,
+                                                                         char *__restrict__ stage) {
+    const unsigned per = gridDim.x / VC_XCDS;
+    const unsigned wave = (blockIdx.x % VC_XCDS) * per + blockIdx.x / VC_XCDS;
+    const int64_t idx = (int64_t)wave * VC_ITEMS_PER_WAVE + threadIdx.x / VC_QUARTER;
+    if (idx >= nitems) return;
+    const int64_t *it = items + idx * stride;
+    const int64_t len = it[VC_CHAIN_LEN];
+    const int nhop = (int)it[VC_CHAIN_NHOP];
+    if (len <= 0 || nhop <= 0) return;
+    vc_forward_piece_quarter(vc_resolve(it[VC_CHAIN_SRC], sendbuf, recvbuf, stage), len, nhop,
+                             [&](int k) { return vc_resolve(it[VC_CHAIN_HEAD + k], sendbuf, recvbuf, stage); });
+}
+
+__global__ __launch_bounds__(VC_WAVE) void vc_copy_items_quarter_kernel(const VcDesc *__restrict__ items, unsigned nitems,
+                                                                        const char *__restrict__ sendbuf, char *__restrict__ recvbuf,
+                                                                        char *__restrict__ stage) {
+    const unsigned per = gridDim.x / VC_XCDS;
+    const unsigned wave = (blockIdx.x % VC_XCDS) * per + blockIdx.x / VC_XCDS;
+    const int64_t idx = (int64_t)wave * VC_ITEMS_PER_WAVE + threadIdx.x / VC_QUARTER;
+    if (idx >= nitems) return;
+    const VcDesc d = items[idx];
+    if (d.len <= 0) return;
+    char *dst = vc_resolve(d.dst, sendbuf, recvbuf, stage);
+    vc_forward_piece_quarter(vc_resolve(d.src, sendbuf, recvbuf, stage), d.len, 1, [&](int) { return dst; });
+}
+
 // Forwarded execution without a work-item list, for calls whose planning would otherwise cost more than their copying:
 // one workgroup per (source, destination) pair, in the order of the chain items (by destination, then source, an eighth
 // of the pairs per XCD).  The workgroup works out the route of its block in closed form from the plan tables (lane k
@@ -174,32 +243,45 @@ hipError_t vc_launch_copy_blocks(const VcSched &S, VcTables T, const int64_t *sl
     return hipGetLastError();
 }
 
+// Items of one launch: as many as VC_MAX_GRID workgroups or wavefronts take.
+static int64_t vc_items_per_launch(int lanes) { return lanes == VC_QUARTER ? VC_MAX_GRID * VC_ITEMS_PER_WAVE : VC_MAX_GRID; }
+
+static unsigned vc_grid_for(int64_t items, int lanes) {
+    const int64_t units = lanes == VC_QUARTER ? (items + VC_ITEMS_PER_WAVE - 1) / VC_ITEMS_PER_WAVE : items;
+    return (unsigned)((units + VC_XCDS - 1) / VC_XCDS * VC_XCDS);
+}
+
 hipError_t vc_launch_copy_chains(const int64_t *items, int stride, int64_t nitems, int lanes, const char *sendbuf, char *recvbuf,
                                  char *stage, hipStream_t st) {
-    for (int64_t done = 0; done < nitems; done += VC_MAX_GRID) {
-        const int64_t now = nitems - done < VC_MAX_GRID ? nitems - done : VC_MAX_GRID;
-        const int64_t grid = (now + VC_XCDS - 1) / VC_XCDS * VC_XCDS;
-        if (lanes == VC_WAVE)
-            hipLaunchKernelGGL(vc_copy_chains_kernel<VC_WAVE>, dim3((unsigned)grid), dim3(VC_WAVE), 0, st, items + done * stride, stride,
-                               (unsigned)now, sendbuf, recvbuf, stage);
+    const int64_t step = vc_items_per_launch(lanes);
+    for (int64_t done = 0; done < nitems; done += step) {
+        const int64_t now = nitems - done < step ? nitems - done : step;
+        const dim3 grid(vc_grid_for(now, lanes));
+        const int64_t *first = items + done * stride;
+        if (lanes == VC_QUARTER)
+            hipLaunchKernelGGL(vc_copy_chains_quarter_kernel, grid, dim3(VC_WAVE), 0, st, first, stride, (unsigned)now, sendbuf, recvbuf, stage);
+        else if (lanes == VC_WAVE)
+            hipLaunchKernelGGL(vc_copy_chains_kernel<VC_WAVE>, grid, dim3(VC_WAVE), 0, st, first, stride, (unsigned)now, sendbuf, recvbuf, stage);
         else
-            hipLaunchKernelGGL(vc_copy_chains_kernel<VC_THREADS>, dim3((unsigned)grid), dim3(VC_THREADS), 0, st, items + done * stride,
-                               stride, (unsigned)now, sendbuf, recvbuf, stage);
+            hipLaunchKernelGGL(vc_copy_chains_kernel<VC_THREADS>, grid, dim3(VC_THREADS), 0, st, first, stride, (unsigned)now, sendbuf, recvbuf,
+                               stage);
     }
     return hipGetLastError();
 }
 
 hipError_t vc_launch_copy_items(const VcDesc *items, int64_t nitems, int lanes, const char *sendbuf, char *recvbuf, char *stage,
                                 hipStream_t st) {
-    for (int64_t done = 0; done < nitems; done += VC_MAX_GRID) {
-        const int64_t now = nitems - done < VC_MAX_GRID ? nitems - done : VC_MAX_GRID;
-        const int64_t grid = (now + VC_XCDS - 1) / VC_XCDS * VC_XCDS;
-        if (lanes == VC_WAVE)
-            hipLaunchKernelGGL(vc_copy_items_kernel<VC_WAVE>, dim3((unsigned)grid), dim3(VC_WAVE), 0, st, items + done, (unsigned)now,
-                               sendbuf, recvbuf, stage);
+    const int64_t step = vc_items_per_launch(lanes);
+    for (int64_t done = 0; done < nitems; done += step) {
+        const int64_t now = nitems - done < step ? nitems - done : step;
+        const dim3 grid(vc_grid_for(now, lanes));
+        if (lanes == VC_QUARTER)
+            hipLaunchKernelGGL(vc_copy_items_quarter_kernel, grid, dim3(VC_WAVE), 0, st, items + done, (unsigned)now, sendbuf, recvbuf, stage);
+        else if (lanes == VC_WAVE)
+            hipLaunchKernelGGL(vc_copy_items_kernel<VC_WAVE>, grid, dim3(VC_WAVE), 0, st, items + done, (unsigned)now, sendbuf, recvbuf, stage);
         else
-            hipLaunchKernelGGL(vc_copy_items_kernel<VC_THREADS>, dim3((unsigned)grid), dim3(VC_THREADS), 0, st, items + done,
-                               (unsigned)now, sendbuf, recvbuf, stage);
+            hipLaunchKernelGGL(vc_copy_items_kernel<VC_THREADS>, grid, dim3(VC_THREADS), 0, st, items + done, (unsigned)now, sendbuf, recvbuf,
+                               stage);
     }
     return hipGetLastError();
 }

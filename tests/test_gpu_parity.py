@@ -715,6 +715,27 @@ def test_default_mode_picks_the_listless_kernel_for_small_calls(api):
     comm.free()
 
 
+@pytest.mark.parametrize("hi,lanes", [(200, 16), (3000, 64), (12000, 256)])
+def test_three_shapes_of_the_copy_kernel(api, hi, lanes):
+    """The copy kernels give a work item a quarter of a wavefront, a wavefront or a workgroup, by the average piece of
+    the list; the listless kernel always a workgroup."""
+    counts = W.counts_uniform_random(96, hi, seed=hi)
+    counts[3, 7] = 40000                                   # one long block among them, cut into pieces
+    prob = W.make_problem(counts, 1, 1, 1)
+    dp = api.DeviceProblem(prob)
+    ds = dp.new_send_arena()
+    dp.fill_payload(0, 12, ds)
+    for name, fn, packed in (("twophase r=3", lambda d: api.twophase_rbruck_alltoallv(3, dp, ds, d), False),
+                             ("s1 n=8 r=2", lambda d: api.TTPL_BT_alltoallv_s1(8, 2, 5, dp, ds, d), False),
+                             ("scattered", lambda d: api.MPICH_intra_scattered(7, dp, ds, d), False)):
+        dr = dp.new_recv_arena(0xEE)
+        assert fn(dr) == 0, (name, dp.comm.error())
+        assert dp.verify(ds, dr) == 0, name
+        st = dp.comm.last_stats()
+        assert st.lanes_per_item == (256 if st.execution == 2 else lanes), (name, st.lanes_per_item)
+    dp.comm.free()
+
+
 def test_phase_times(api):
     """With timing on, the statistics split the launches as the reference's phase timers do (src/rbruckv.h:13-18):
     inside the nodes and between them."""
