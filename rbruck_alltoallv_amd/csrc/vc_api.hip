@@ -237,18 +237,18 @@ static int plan_sizes(vc_comm *c, const VcSched &S, std::vector<VcLaunchInfo> &L
     HIP_TRY(c->org_run_base.reserve(sizeof(int64_t) * (size_t)P * std::max(S.G, 1)));
     HIP_TRY(c->item_row_tot.reserve(sizeof(int64_t) * (size_t)P * nl));
     HIP_TRY(c->item_row_base.reserve(sizeof(int64_t) * (size_t)P * nl));
-    HIP_TRY(c->row_bytes.reserve(sizeof(int64_t) * (size_t)P * (nl + 2)));
+    HIP_TRY(c->row_bytes.reserve(sizeof(int64_t) * (size_t)P * (std::max(nl, S.w + S.w2) + 2)));
     HIP_TRY(c->header.reserve(sizeof(int64_t) * VC_HEADER_WORDS(VC_MAX_LAUNCHES)));
     HIP_TRY(c->launches.reserve(sizeof(VcLaunchInfo) * VC_MAX_LAUNCHES));
     if (forward) {
         if (vc_hop_slots(S) > VC_MAX_HOP_SLOTS) return fail_arg("too many digits for forwarded execution");
-        HIP_TRY(c->chain_row_tot.reserve(sizeof(int64_t) * 2 * (size_t)P));
+        HIP_TRY(c->chain_row_tot.reserve(sizeof(int64_t) * (2 + (size_t)(P + VC_THREADS - 1) / VC_THREADS) * (size_t)P));
         HIP_TRY(c->chain_row_base.reserve(sizeof(int64_t) * (size_t)P));
     }
     if (c->timing) { int rc = ensure_events(c, (size_t)nl + 4); if (rc) return rc; }
 
     if (c->timing) HIP_TRY(hipEventRecord(c->events[0], st));
-    if (nl > VC_LAUNCH_PACK) {                             // a short launch table travels as a kernel argument instead
+    if (!forward && nl > VC_LAUNCH_PACK) {                 // a short launch table travels as a kernel argument instead
         memcpy(c->h_launches, L.data(), sizeof(VcLaunchInfo) * nl);
         HIP_TRY(hipMemcpyAsync(c->launches.p, c->h_launches, sizeof(VcLaunchInfo) * nl, hipMemcpyHostToDevice, st));
     }
@@ -278,13 +278,22 @@ static int lanes_for(int64_t bytes, int64_t items) {
 
 // Step 3b, after the stream has been synchronised: what the planning kernels found.
 static int plan_read(vc_comm *c, const VcSched &S, const std::vector<VcLaunchInfo> &L, PlanInfo &out, bool forward) {
-    const int nl = (int)L.size();
+    const int nl = forward ? 1 : (int)L.size();           // forwarded execution: one launch, one set of totals
     const int64_t *h = c->h_header;
     if (h[VC_HEADER_BAD] != 0)    // such tables would send the copy kernels outside the arenas
         return fail_arg("negative entries in sendcounts / sdispls / recvcounts / rdispls", VC_ERR_TABLES);
     out.nl = nl; out.n_digits = S.w + S.w2; out.recv_lo = S.recv_lo;
     out.stage_bytes = h[0]; out.payload_bytes = h[1];
     out.first.assign(nl, 0); out.count.assign(nl, 0); out.bytes.assign(nl, 0); out.inter.assign(nl, 0); out.lanes.assign(nl, VC_THREADS);
+    if (forward) {
+        out.bytes[0] = h[VC_HEADER_FIXED];
+        out.chain = true;
+        out.chain_stride = VC_CHAIN_HEAD + vc_hop_slots(S);
+        out.chain_items = h[2];
+        out.chain_lanes = lanes_for(out.payload_bytes, out.chain_items);      // every chain item carries one piece of the payload
+        out.max_pieces = h[VC_HEADER_MAX_PIECES];
+        return VC_OK;
+    }
     int64_t nitems = 0;
     for (int k = 0; k < nl; k++) {
         out.inter[k] = L[k].kind == 1 || L[k].kind == 3 || L[k].kind == 4 || (L[k].kind == 2 && L[k].x == 2);
@@ -295,13 +304,6 @@ static int plan_read(vc_comm *c, const VcSched &S, const std::vector<VcLaunchInf
         nitems += out.count[k];
     }
     out.items_total = nitems;
-    if (forward) {
-        out.chain = true;
-        out.chain_stride = VC_CHAIN_HEAD + vc_hop_slots(S);
-        out.chain_items = h[2];
-        out.chain_lanes = lanes_for(out.payload_bytes, out.chain_items);      // every chain item carries one piece of the payload
-        out.max_pieces = h[VC_HEADER_MAX_PIECES];
-    }
     return VC_OK;
 }
 
@@ -311,7 +313,7 @@ static int plan_emit(vc_comm *c, const VcSched &S, std::vector<VcLaunchInfo> &L,
     if (pi.chain) {
         HIP_TRY(items.reserve(sizeof(int64_t) * (size_t)pi.chain_stride * (size_t)std::max<int64_t>(pi.chain_items, 1)));
         HIP_TRY(vc_launch_chain_plan(S, T, c->slot_off.as<int64_t>(), c->row_base.as<int64_t>(), c->chain_row_base.as<int64_t>(),
-                                     items.as<int64_t>(), pi.chain_items, st));
+                                     c->chain_row_tot.as<int64_t>() + 2 * (size_t)S.P, items.as<int64_t>(), pi.chain_items, st));
     } else {
         HIP_TRY(items.reserve(sizeof(VcDesc) * (size_t)std::max<int64_t>(pi.items_total, 1)));
         HIP_TRY(vc_launch_plan_emit(S, L.data(), c->launches.as<VcLaunchInfo>(), pi.nl, T, c->slot_off.as<int64_t>(), c->row_base.as<int64_t>(),

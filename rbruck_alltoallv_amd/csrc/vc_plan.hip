@@ -18,9 +18,13 @@
 #include "vc_plan_math.h"
 
 // ---- pass 1: row-wise prefix sums ----
-// grid (P, w + w2 + nl [+ 1]).  Rows y < w + w2: staging sizes of region y, slot_off[(y*P + to)*P + id] = offset of the
-// slot inside the row.  Later rows: work-item count, moved bytes (and, for the first launch, payload and the number of
-// negative table entries) of launch y - w - w2.  One more row with chain_row_tot: the chain items of forwarded execution.
+// Launch-per-digit execution: grid (P, regions + nl).  Rows y < regions = w + w2: staging sizes of region y,
+// slot_off[(y*P + to)*P + id] = offset of the slot inside the row.  Later rows: work-item count and moved bytes of launch
+// y - regions; the first of them also sums the payload and counts negative table entries.
+// Forwarded execution (chain_row_tot != null, nl = 0): grid (P, regions + 1).  The region rows also sum the bytes of the
+// blocks themselves (every staged block is one hop), and the last row counts the chain items of the blocks that end on
+// the rank, the most pieces of any of them, the payload and the negative table entries.
+// row_bytes rows: [launch or region][P], then [payload][P], then [negative entries][P].
 __global__ __launch_bounds__(VC_THREADS) void vc_plan_rows(VcSched S, VcLaunchPack pack, const VcLaunchInfo *__restrict__ launches, int nl, VcTables T,
                                                            int64_t *__restrict__ slot_off, int64_t *__restrict__ row_tot,
                                                            int64_t *__restrict__ item_row_tot, int64_t *__restrict__ row_bytes,
@@ -28,45 +32,54 @@ __global__ __launch_bounds__(VC_THREADS) void vc_plan_rows(VcSched S, VcLaunchPa
     __shared__ int64_t lds[VC_WAVES_PER_BLOCK];
     const int to = blockIdx.x, P = S.P;
     const int nreg = S.w + S.w2;                          // the organized region is laid out by vc_plan_org_rows
-    if ((int)blockIdx.y == nreg + nl) {                   // forwarded execution: chain items whose last hop ends on this rank
-        int64_t items = 0, most = 0;
-        for (int s = threadIdx.x; s < P; s += VC_THREADS) {
-            const int64_t cnt = vc_chain_count(S, T, s, to);
-            items += cnt;
-            most = cnt > most ? cnt : most;
-        }
-        items = vc_block_sum(items, lds);
-        most = vc_block_max(most, lds);
-        if (threadIdx.x == 0) { chain_row_tot[to] = items; chain_row_tot[P + to] = most; }
-        return;
-    }
+    const bool forward = chain_row_tot != nullptr;
+    const int nsum = forward ? nreg : nl;                 // rows of row_bytes before the payload row
     if ((int)blockIdx.y < nreg) {
         const int y = blockIdx.y;
-        int64_t carry = 0;
+        int64_t carry = 0, data = 0;
         for (int base = 0; base < P; base += VC_THREADS) {
             const int id = base + threadIdx.x;
-            int64_t total;
-            const int64_t v = (id < P) ? vc_region_slot_size(S, T, y, to, id) : 0;
+            int64_t total, len = 0;
+            const int64_t v = (id < P) ? vc_region_slot_size(S, T, y, to, id, &len) : 0;
             const int64_t ex = vc_block_exclusive_scan(v, lds, total);
             if (id < P) slot_off[((int64_t)y * P + to) * P + id] = carry + ex;
             carry += total;
+            data += len;
         }
-        if (threadIdx.x == 0) row_tot[(int64_t)y * P + to] = carry;
+        if (forward) data = vc_block_sum(data, lds);
+        if (threadIdx.x == 0) {
+            row_tot[(int64_t)y * P + to] = carry;
+            if (forward) row_bytes[(int64_t)y * P + to] = data;
+        }
         return;
     }
+    int64_t items = 0, bytes = 0, payload = 0, most = 0;
+    int64_t bad = 0;                                      // entries of this rank's rows no rank could have passed
     const int L = blockIdx.y - nreg;
-    const VcLaunchInfo info = launches ? launches[L] : pack.info[L];     // a short launch table travels as a kernel argument
-    int64_t items = 0, bytes = 0, payload = 0;
-    const int nent = vc_entries_per_rank(S, info);
-    for (int id = threadIdx.x; id < nent; id += VC_THREADS) {
-        VcEntry e;
-        if (vc_entry_block(S, info, to, id, e)) {
-            const int64_t len = vc_entry_len(S, T, e);
-            items += vc_chunk_count(len, vc_entry_phase(S, T, e), vc_entry_cut(S, T, e));
-            bytes += len;
+    if (forward) {
+        // sources in chunks of VC_THREADS: the items before each chunk let vc_chain_emit give every chunk a workgroup
+        const int nchunk = (P + VC_THREADS - 1) / VC_THREADS;
+        int64_t before = 0;
+        for (int chunk = 0; chunk < nchunk; chunk++) {
+            const int s = chunk * VC_THREADS + threadIdx.x;
+            const int64_t cnt = s < P ? vc_chain_count(S, T, s, to) : 0;
+            most = cnt > most ? cnt : most;
+            if (threadIdx.x == 0) chain_row_tot[2 * (int64_t)P + (int64_t)to * nchunk + chunk] = before;
+            before += vc_block_sum(cnt, lds);
+        }
+        items = threadIdx.x == 0 ? before : 0;            // vc_block_sum below adds the lanes up
+    } else {
+        const VcLaunchInfo info = launches ? launches[L] : pack.info[L];     // a short launch table travels as a kernel argument
+        const int nent = vc_entries_per_rank(S, info);
+        for (int id = threadIdx.x; id < nent; id += VC_THREADS) {
+            VcEntry e;
+            if (vc_entry_block(S, info, to, id, e)) {
+                const int64_t len = vc_entry_len(S, T, e);
+                items += vc_chunk_count(len, vc_entry_phase(S, T, e), vc_entry_cut(S, T, e));
+                bytes += len;
+            }
         }
     }
-    int64_t bad = 0;                                      // entries of this rank's rows no rank could have passed
     if (L == 0)
         for (int id = threadIdx.x; id < P; id += VC_THREADS) {
             const int64_t i = (int64_t)to * P + id;
@@ -74,12 +87,12 @@ __global__ __launch_bounds__(VC_THREADS) void vc_plan_rows(VcSched S, VcLaunchPa
             bad += (T.sc[i] < 0) | (T.sd[i] < 0) | (T.rc[i] < 0) | (!S.packed_recv && T.rd[i] < 0);
         }
     items = vc_block_sum(items, lds);
-    bytes = vc_block_sum(bytes, lds);
+    if (forward) most = vc_block_max(most, lds); else bytes = vc_block_sum(bytes, lds);
     if (L == 0) { payload = vc_block_sum(payload, lds); bad = vc_block_sum(bad, lds); }
     if (threadIdx.x == 0) {
-        item_row_tot[(int64_t)L * P + to] = items;
-        row_bytes[(int64_t)L * P + to] = bytes;
-        if (L == 0) { row_bytes[(int64_t)nl * P + to] = payload; row_bytes[(int64_t)(nl + 1) * P + to] = bad; }
+        if (forward) { chain_row_tot[to] = items; chain_row_tot[P + to] = most; }
+        else { item_row_tot[(int64_t)L * P + to] = items; row_bytes[(int64_t)L * P + to] = bytes; }
+        if (L == 0) { row_bytes[(int64_t)nsum * P + to] = payload; row_bytes[(int64_t)(nsum + 1) * P + to] = bad; }
     }
 }
 
@@ -105,17 +118,21 @@ __global__ __launch_bounds__(VC_THREADS) void vc_plan_org_rows(VcSched S, VcTabl
 }
 
 // ---- pass 2: prefix sums over the rows ----
-// grid (nl + 1 [+ 1]).  Workgroup L < nl: item bases of launch L's rows (relative to the launch's first item), its item
-// count and moved bytes.  Workgroup nl: staging row bases, staging bytes, payload bytes.  Workgroup nl + 1: chain item bases.
-__global__ __launch_bounds__(VC_THREADS) void vc_plan_bases(int P, int w, int nl, const int64_t *__restrict__ row_tot,
+// Launch-per-digit execution: grid (nl + 1).  Workgroup L < nl: item bases of launch L's rows (relative to the launch's
+// first item), its item count and moved bytes.  Workgroup nl: staging row bases, staging bytes, payload bytes, negative
+// table entries.  Forwarded execution (chain_row_tot != null, nl = 0): grid (2).  Workgroup 0 as workgroup nl above, and
+// the moved bytes = payload + bytes of the staged blocks as those of launch 0; workgroup 1: chain item bases.
+__global__ __launch_bounds__(VC_THREADS) void vc_plan_bases(int P, int w, int nreg, int nl, const int64_t *__restrict__ row_tot,
                                                             int64_t *__restrict__ row_base, const int64_t *__restrict__ item_row_tot,
                                                             int64_t *__restrict__ item_row_base, const int64_t *__restrict__ row_bytes,
                                                             const int64_t *__restrict__ chain_row_tot, int64_t *__restrict__ chain_row_base,
                                                             int64_t *__restrict__ header, int64_t *__restrict__ header_host) {
     __shared__ int64_t lds[VC_WAVES_PER_BLOCK];
     const int L = blockIdx.x;
+    const bool forward = chain_row_tot != nullptr;
+    const int nsum = forward ? nreg : nl;                 // rows of row_bytes before the payload row
     int64_t carry = 0, bytes = 0;
-    if (L == nl + 1) {                                    // forwarded execution: first chain item of every final receiver
+    if (forward && L == 1) {                              // first chain item of every final receiver
         int64_t most = 0;
         for (int b0 = 0; b0 < P; b0 += VC_THREADS) {
             const int i = b0 + threadIdx.x;
@@ -141,13 +158,20 @@ __global__ __launch_bounds__(VC_THREADS) void vc_plan_bases(int P, int w, int nl
             if (i < nrows) row_base[i] = carry + ex;
             carry += total;
         }
-        int64_t bad = 0;
-        for (int i = threadIdx.x; i < P; i += VC_THREADS) { bytes += row_bytes[(int64_t)nl * P + i]; bad += row_bytes[(int64_t)(nl + 1) * P + i]; }
+        int64_t bad = 0, staged = 0;
+        for (int i = threadIdx.x; i < P; i += VC_THREADS) { bytes += row_bytes[(int64_t)nsum * P + i]; bad += row_bytes[(int64_t)(nsum + 1) * P + i]; }
+        if (forward)
+            for (int64_t i = threadIdx.x; i < (int64_t)nreg * P; i += VC_THREADS) staged += row_bytes[i];
         bytes = vc_block_sum(bytes, lds);
         bad = vc_block_sum(bad, lds);
+        if (forward) staged = vc_block_sum(staged, lds);
         if (threadIdx.x == 0) {
             header[0] = carry; header[1] = bytes; header[VC_HEADER_BAD] = bad;
             if (header_host) { header_host[0] = carry; header_host[1] = bytes; header_host[VC_HEADER_BAD] = bad; }
+            if (forward) {                                // every staged block is one hop, every block's last hop ends in recvbuf
+                header[VC_HEADER_FIXED] = bytes + staged;
+                if (header_host) header_host[VC_HEADER_FIXED] = bytes + staged;
+            }
         }
         return;
     }
@@ -253,13 +277,15 @@ hipError_t vc_launch_plan_sizes(const VcSched &S, const VcLaunchInfo *launches_h
                                 int64_t *row_tot, int64_t *row_base, int64_t *org_run_base, int64_t *item_row_tot,
                                 int64_t *item_row_base, int64_t *row_bytes, int64_t *chain_row_tot, int64_t *chain_row_base,
                                 int64_t *header, int64_t *header_host, hipStream_t st) {
-    const int chain = chain_row_tot ? 1 : 0;
-    hipLaunchKernelGGL(vc_plan_rows, dim3(S.P, S.w + S.w2 + nlaunch + chain), dim3(VC_THREADS), 0, st, S,
-                       vc_pack_launches(launches_host, nlaunch), nlaunch <= VC_LAUNCH_PACK ? nullptr : launches_dev, nlaunch, T, slot_off,
+    const bool forward = chain_row_tot != nullptr;
+    const int nl = forward ? 0 : nlaunch;                 // forwarded execution has no use for the per-launch rows
+    const int nreg = S.w + S.w2;
+    hipLaunchKernelGGL(vc_plan_rows, dim3(S.P, nreg + (forward ? 1 : nl)), dim3(VC_THREADS), 0, st, S,
+                       vc_pack_launches(launches_host, nl), nl <= VC_LAUNCH_PACK ? nullptr : launches_dev, nl, T, slot_off,
                        row_tot, item_row_tot, row_bytes, chain_row_tot);
     if (S.coalesce)
         hipLaunchKernelGGL(vc_plan_org_rows, dim3(S.P), dim3(VC_THREADS), 0, st, S, T, slot_off, row_tot, org_run_base);
-    hipLaunchKernelGGL(vc_plan_bases, dim3(nlaunch + 1 + chain), dim3(VC_THREADS), 0, st, S.P, vc_regions(S), nlaunch, row_tot, row_base,
+    hipLaunchKernelGGL(vc_plan_bases, dim3(forward ? 2 : nl + 1), dim3(VC_THREADS), 0, st, S.P, vc_regions(S), nreg, nl, row_tot, row_base,
                        item_row_tot, item_row_base, row_bytes, chain_row_tot, chain_row_base, header, header_host);
     return hipGetLastError();
 }
@@ -275,12 +301,15 @@ hipError_t vc_launch_plan_emit(const VcSched &S, const VcLaunchInfo *launches_ho
 }
 
 // ---- forwarded execution ----
-// grid (P, Z): the chain items of the blocks that end on rank t, in source order; workgroup (t, z) writes those of the
-// z-th slice of the sources (few ranks with huge blocks would otherwise leave most of the chip idle); big blocks are
-// written by the whole workgroup as in vc_plan_emit.
+// grid (P, chunks x Z): the chain items of the blocks that end on rank t, in source order.  The sources come in chunks of
+// VC_THREADS (vc_plan_rows has counted the items before each chunk); Z workgroups share a chunk when there are few ranks
+// with huge blocks, which would otherwise leave most of the chip idle: workgroup (t, chunk, z) writes the items of the
+// z-th slice of the chunk's sources.  Big blocks are written by the whole workgroup as in vc_plan_emit.
 __global__ __launch_bounds__(VC_THREADS) void vc_chain_emit(VcSched S, VcTables T, const int64_t *__restrict__ slot_off,
                                                             const int64_t *__restrict__ row_base,
-                                                            const int64_t *__restrict__ chain_row_base, int64_t *__restrict__ items) {
+                                                            const int64_t *__restrict__ chain_row_base,
+                                                            const int64_t *__restrict__ chain_chunk_pre, int slices,
+                                                            int64_t *__restrict__ items) {
     __shared__ int64_t lds[VC_WAVES_PER_BLOCK];
     __shared__ int64_t big_at[VC_THREADS], big_pre[VC_THREADS];
     // a block of many pieces keeps its route here while the whole workgroup writes its items (routes of more hops than
@@ -291,51 +320,53 @@ __global__ __launch_bounds__(VC_THREADS) void vc_chain_emit(VcSched S, VcTables 
     const int t = blockIdx.x, P = S.P;
     const int stride = VC_CHAIN_HEAD + vc_hop_slots(S);
     const bool cached = vc_hop_slots(S) <= VC_ROUTE_CACHE;
-    const int per = (P + (int)gridDim.y - 1) / (int)gridDim.y;
-    const int s_lo = (int)blockIdx.y * per < P ? (int)blockIdx.y * per : P, s_hi = s_lo + per < P ? s_lo + per : P;
-    int64_t before = 0;                                   // items of this receiver's earlier sources
-    for (int s = threadIdx.x; s < s_lo; s += VC_THREADS) before += vc_chain_count(S, T, s, t);
-    int64_t carry = chain_row_base[t] + vc_block_sum(before, lds);
-    for (int base = s_lo; base < s_hi; base += VC_THREADS) {
-        const int s = base + threadIdx.x;
-        const int64_t cnt = s < s_hi ? vc_chain_count(S, T, s, t) : 0;
-        int64_t total;
-        const int64_t at = carry + vc_block_exclusive_scan(cnt, lds, total);
-        const bool big = cnt > 4;
-        if (!big)
-            for (int64_t c = 0; c < cnt; c++) vc_chain_item(S, T, slot_off, row_base, s, t, c, items + (at + c) * stride);
-        else {
-            big_at[threadIdx.x] = at;
-            if (cached) big_nhop[threadIdx.x] = vc_chain_route(S, T, slot_off, row_base, s, t, big_dst[threadIdx.x]);
-        }
-        if (__syncthreads_or(big)) {
-            int64_t btotal;
-            big_pre[threadIdx.x] = vc_block_exclusive_scan(big ? cnt : 0, lds, btotal);
-            __syncthreads();
-            for (int64_t q = threadIdx.x; q < btotal; q += VC_THREADS) {
-                int lo = 0, hi = VC_THREADS - 1;              // last lane whose pieces start at or before q
-                while (lo < hi) {
-                    const int mid = (lo + hi + 1) >> 1;
-                    if (big_pre[mid] <= q) lo = mid; else hi = mid - 1;
-                }
-                const int64_t c = q - big_pre[lo];
-                const int sb = base + lo;
-                if (cached)
-                    vc_chain_piece(VC_SPACE_SEND | vc_send_offset(S, T, sb, t), (int64_t)T.sc[(int64_t)sb * P + t] * S.esz, vc_phase(S, T, sb, t),
-                                   vc_chain_cut(S, T, sb, t), c, big_dst[lo], big_nhop[lo], items + (big_at[lo] + c) * stride);
-                else
-                    vc_chain_item(S, T, slot_off, row_base, sb, t, c, items + (big_at[lo] + c) * stride);
+    const int nchunk = (P + VC_THREADS - 1) / VC_THREADS;
+    const int chunk = (int)blockIdx.y / slices, z = (int)blockIdx.y % slices;
+    const int c_lo = chunk * VC_THREADS, c_hi = c_lo + VC_THREADS < P ? c_lo + VC_THREADS : P;
+    const int per = (c_hi - c_lo + slices - 1) / slices;
+    const int s_lo = c_lo + z * per < c_hi ? c_lo + z * per : c_hi, s_hi = s_lo + per < c_hi ? s_lo + per : c_hi;
+    int64_t before = 0;                                   // items of the chunk's earlier sources
+    if (c_lo + (int)threadIdx.x < s_lo) before = vc_chain_count(S, T, c_lo + threadIdx.x, t);
+    const int64_t carry = chain_row_base[t] + chain_chunk_pre[(int64_t)t * nchunk + chunk] + vc_block_sum(before, lds);
+    const int s = s_lo + threadIdx.x;                     // one source per lane: a slice has at most VC_THREADS of them
+    const int64_t cnt = s < s_hi ? vc_chain_count(S, T, s, t) : 0;
+    int64_t total;
+    const int64_t at = carry + vc_block_exclusive_scan(cnt, lds, total);
+    const bool big = cnt > 4;
+    if (!big)
+        for (int64_t c = 0; c < cnt; c++) vc_chain_item(S, T, slot_off, row_base, s, t, c, items + (at + c) * stride);
+    else {
+        big_at[threadIdx.x] = at;
+        if (cached) big_nhop[threadIdx.x] = vc_chain_route(S, T, slot_off, row_base, s, t, big_dst[threadIdx.x]);
+    }
+    if (__syncthreads_or(big)) {
+        int64_t btotal;
+        big_pre[threadIdx.x] = vc_block_exclusive_scan(big ? cnt : 0, lds, btotal);
+        __syncthreads();
+        for (int64_t q = threadIdx.x; q < btotal; q += VC_THREADS) {
+            int lo = 0, hi = VC_THREADS - 1;              // last lane whose pieces start at or before q
+            while (lo < hi) {
+                const int mid = (lo + hi + 1) >> 1;
+                if (big_pre[mid] <= q) lo = mid; else hi = mid - 1;
             }
-            __syncthreads();
+            const int64_t c = q - big_pre[lo];
+            const int sb = s_lo + lo;
+            if (cached)
+                vc_chain_piece(VC_SPACE_SEND | vc_send_offset(S, T, sb, t), (int64_t)T.sc[(int64_t)sb * P + t] * S.esz, vc_phase(S, T, sb, t),
+                               vc_chain_cut(S, T, sb, t), c, big_dst[lo], big_nhop[lo], items + (big_at[lo] + c) * stride);
+            else
+                vc_chain_item(S, T, slot_off, row_base, sb, t, c, items + (big_at[lo] + c) * stride);
         }
-        carry += total;
     }
 }
 
 hipError_t vc_launch_chain_plan(const VcSched &S, VcTables T, const int64_t *slot_off, const int64_t *row_base,
-                                const int64_t *chain_row_base, int64_t *items, int64_t nitems, hipStream_t st) {
-    const int slices = vc_emit_slices(nitems, S.P);
-    hipLaunchKernelGGL(vc_chain_emit, dim3(S.P, slices), dim3(VC_THREADS), 0, st, S, T, slot_off, row_base, chain_row_base, items);
+                                const int64_t *chain_row_base, const int64_t *chain_chunk_pre, int64_t *items, int64_t nitems,
+                                hipStream_t st) {
+    const int nchunk = (S.P + VC_THREADS - 1) / VC_THREADS;
+    const int slices = nchunk > 1 ? 1 : vc_emit_slices(nitems, S.P);
+    hipLaunchKernelGGL(vc_chain_emit, dim3(S.P, nchunk * slices), dim3(VC_THREADS), 0, st, S, T, slot_off, row_base, chain_row_base,
+                       chain_chunk_pre, slices, items);
     return hipGetLastError();
 }
 

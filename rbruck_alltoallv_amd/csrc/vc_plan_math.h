@@ -118,25 +118,30 @@ VC_HD int vc_phase(const VcSched &S, const VcTables &T, int s, int t) {
 
 // Bytes the staging slot `id` of rank `to` needs for the block that arrives in digit x
 // (0 if nothing arrives there, or if it goes to recvbuf).  Always a multiple of VC_LINE.
-VC_HD int64_t vc_stage_slot_size(const VcSched &S, const VcTables &T, int x, int dist, int to, int id) {
+VC_HD int64_t vc_stage_slot_size(const VcSched &S, const VcTables &T, int x, int dist, int to, int id, int64_t *data_len = nullptr) {
     VcBlock b;
+    if (data_len) *data_len = 0;
     if (!vc_intra_block(S, x, dist, to, id, b) || !b.to_stage || b.to_org) return 0;
     const int64_t len = (int64_t)T.sc[(int64_t)b.s * S.P + b.t] * S.esz;
+    if (data_len) *data_len = len;
     return len ? ((len + vc_phase(S, T, b.s, b.t) + VC_LINE - 1) & ~(int64_t)(VC_LINE - 1)) : 0;
 }
 
-// The same for staging region y of a call: intra-node digits first, then inter-node digits.
-VC_HD int64_t vc_region_slot_size(const VcSched &S, const VcTables &T, int y, int to, int id) {
+// The same for staging region y of a call: intra-node digits first, then inter-node digits.  data_len (optional)
+// receives the bytes of the block itself.
+VC_HD int64_t vc_region_slot_size(const VcSched &S, const VcTables &T, int y, int to, int id, int64_t *data_len = nullptr) {
     int dist = 1;
     if (y < S.w) {
         for (int k = 0; k < y; k++) dist *= S.r;
-        return vc_stage_slot_size(S, T, y, dist, to, id);
+        return vc_stage_slot_size(S, T, y, dist, to, id, data_len);
     }
     for (int k = S.w; k < y; k++) dist *= S.r;
     VcEntry e;
     int z;
+    if (data_len) *data_len = 0;
     if (!vc_inter_block(S, y - S.w, dist, to, id, e, z) || e.xdst < 0) return 0;
     const int64_t len = (int64_t)T.sc[(int64_t)e.s * S.P + e.t] * S.esz;
+    if (data_len) *data_len = len;
     return len ? ((len + vc_phase(S, T, e.s, e.t) + VC_LINE - 1) & ~(int64_t)(VC_LINE - 1)) : 0;
 }
 
