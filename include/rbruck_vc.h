@@ -64,11 +64,13 @@ int vc_comm_set_bases(vc_comm_t comm, const int64_t *sbase_bytes, const int64_t 
  *    once (from sendbuf) and written once per hop (into the staging slot of every intermediate holder, then into
  *    recvbuf).  The batching tunables (b, bblock) then have no effect, and TTPL_BT_alltoallv sends its inter-node data
  *    per block instead of coalesced.  The copy kernel normally works through a list of block pieces that a planning
- *    kernel writes first (after the host has learnt its size).  On communicators of at most 128 ranks, when the last
- *    call consisted of few, short blocks, the next one goes without the list: one workgroup per pair of ranks derives
- *    its block's route itself, the kernel is enqueued right behind the size computation, and the call needs one host
- *    synchronisation instead of two (24 - 35 us instead of 37 - 47 us per call of 16 - 64 ranks on MI355X).
- * 2: forwarded, always through the list.   3: forwarded, always without it (any size; slower beyond ~128 ranks).
+ *    kernel writes first (after the host has learnt its size).  When the last call on the communicator consisted of
+ *    short blocks, the next one goes without the list: every pair of ranks gets a workgroup (at most 128 ranks) or a
+ *    quarter of a wavefront (average piece below 1 KiB, any number of ranks) that derives its block's route itself; the
+ *    kernel is enqueued right behind the size computation and the call needs one host synchronisation instead of two
+ *    (26 - 35 us instead of 42 - 47 us per call at 64 ranks on MI355X, 10 - 25 % less at 256 and 1024 ranks).
+ * 2: forwarded, always through the list.   3 / 4: forwarded, always without it, a workgroup / a quarter of a wavefront
+ *    per pair of ranks (any sizes; not the fastest choice everywhere).
  * 0: one kernel launch per digit phase (or per batch of its rounds, as b / bblock say); every hop reads the block
  *    where the previous hop left it.  This is the mode whose launches vc_comm_last_stats and vc_comm_last_traffic
  *    describe one by one.
@@ -238,9 +240,9 @@ typedef struct {
     float launch_ms[VC_MAX_LAUNCHES];  /* per data-moving launch, HIP events on the comm's stream */
     int32_t execution;           /* how the call ran: 0 launch per digit, 1 forwarded through a work-item list, 2 forwarded
                                     without one (see vc_comm_set_forwarding) */
-    int32_t lanes_per_item;      /* 256: the copy kernel gave every work item a workgroup; 64: a wavefront (lists of short
-                                    pieces); 16: a quarter of one (pieces of a few hundred bytes).  Launch-per-digit
-                                    execution: of the launch that moved the most bytes. */
+    int32_t lanes_per_item;      /* 256: the copy kernel gave every work item (without a list: every pair of ranks) a
+                                    workgroup; 64: a wavefront (lists of short pieces); 16: a quarter of one (pieces of a
+                                    few hundred bytes).  Launch-per-digit execution: of the launch that moved the most bytes. */
 } vc_stats_t;
 
 /* Per-launch HIP-event timing of the following calls (0 = off, default). */

@@ -50,7 +50,7 @@ class VirtualComm:
     def set_forwarding(self, enable: bool | int) -> None:
         """vc_comm_set_forwarding: 0 / False one launch per digit phase; 1 / True forwarded (one launch per call, every
         block piece carried through all its hops in registers; the library picks list or listless); 2 forwarded through
-        a work-item list; 3 forwarded without one."""
+        a work-item list; 3 / 4 forwarded without one, a workgroup / a quarter of a wavefront per pair of ranks."""
         self._check(self.lib.vc_comm_set_forwarding(self.handle, int(enable)))
 
     def last_stats(self) -> _lib.VcStats:

@@ -30,11 +30,16 @@ static int fail_hip(hipError_t e, const char *what, int line) {
     return VC_ERR_HIP;
 }
 
-// The default mode goes without a work-item list only where that was measured to win: at most this many pairs of ranks
-// (128 ranks) and block pieces, no block of more than VC_LISTLESS_MAX_PIECES pieces (one workgroup moves them in turn).
-// 16 - 64 ranks: 24 - 35 us per call against 37 - 47 us; 128 ranks: even; 256 ranks and more: the list wins.
+// Where the default mode goes without a work-item list (measured, blocking calls on MI355X):
+//  - blocks of a few hundred bytes, any number of ranks: a quarter of a wavefront per pair of ranks.  Average piece below
+//    1 KiB: 26 - 30 us per call at 64 ranks (through the list 42), 42 - 73 at 256 (51 - 88), 300 - 900 at 1024 (330 - 990).
+//  - at most 128 ranks and 16384 pieces, longer blocks: a workgroup per pair (35 - 52 us against 47 - 80 at 64 ranks;
+//    even at 128 ranks; at 256 ranks the list wins by 1.3 - 1.8x).
+//  - never after a call with a block of more than VC_LISTLESS_MAX_PIECES pieces (one workgroup moves them in turn).
 #define VC_LISTLESS_MAX_ITEMS 16384
 #define VC_LISTLESS_MAX_PIECES 8
+#define VC_LISTLESS_QUARTER_BELOW 1024        // average piece, any communicator
+#define VC_LISTLESS_SMALL_QUARTER_BELOW 2048  // average piece, communicators of at most 128 ranks
 
 #define HIP_TRY(expr)                                                   \
     do {                                                                \
@@ -72,9 +77,10 @@ struct vc_comm {
     const int64_t *sbase = nullptr, *rbase = nullptr;
     bool timing = false;
     int forward = 1;                      // vc_comm_set_forwarding: 0 launch per digit, 1 forwarded (list or listless as the last
-                                          // call suggests), 2 forwarded through a work-item list, 3 forwarded, listless if possible
+                                          // call suggests), 2 forwarded through a work-item list, 3 / 4 forwarded, listless with a
+                                          // workgroup / a quarter of a wavefront per pair of ranks
     bool hint_valid = false;              // what the last forwarded call on this communicator looked like
-    int64_t hint_items = 0, hint_max_pieces = 0;
+    int64_t hint_items = 0, hint_max_pieces = 0, hint_payload = 0;
     DevBuf chain_row_tot, chain_row_base;
     DevBuf slot_off, row_tot, row_base, org_run_base, item_row_tot, item_row_base, row_bytes, desc, header, launches, stage, rd_packed,
         uni_counts, uni_displs, scratch;
@@ -146,7 +152,7 @@ extern "C" int vc_comm_set_timing(vc_comm_t c, int enable) {
 
 extern "C" int vc_comm_set_forwarding(vc_comm_t c, int enable) {
     if (!c) return fail_arg("null communicator");
-    if (enable < 0 || enable > 3) return fail_arg("vc_comm_set_forwarding: 0, 1, 2 or 3");
+    if (enable < 0 || enable > 4) return fail_arg("vc_comm_set_forwarding: 0 .. 4");
     c->forward = enable;
     return VC_OK;
 }
@@ -365,9 +371,10 @@ static int finish_stats(vc_comm *c, const PlanInfo &pi, const void *items_any, b
         s.launch_ms[0] = 0.f;
         if (c->timing) HIP_TRY(hipEventElapsedTime(&s.launch_ms[0], c->events[2], c->events[3]));
         s.intra_ms = s.launch_ms[0];
-        s.lanes_per_item = pi.listless ? VC_THREADS : pi.chain_lanes;
+        s.lanes_per_item = pi.chain_lanes;
         c->hint_valid = true;
         c->hint_items = pi.chain_items;
+        c->hint_payload = pi.payload_bytes;
         c->hint_max_pieces = pi.max_pieces;
     } else {
         int64_t most = -1;
@@ -412,14 +419,18 @@ static int run_items(vc_comm *c, const PlanInfo &pi, const void *items_any, cons
     return finish_stats(c, pi, items_any, planned_now);
 }
 
-// Whether a forwarded call should try to go without the work-item list: worth it when writing the list (and waiting for
-// its size before that) costs more than the slower per-block kernel loses, i.e. for calls of few, short blocks.  The
-// last forwarded call on the communicator is the guide (mode 1), or the caller says so (mode 3).
-static bool want_listless(const vc_comm *c, const VcSched &S) {
-    if (c->forward == 3) return true;
-    if (c->forward != 1 || !c->hint_valid) return false;
-    return (int64_t)S.P * S.P <= VC_LISTLESS_MAX_ITEMS && c->hint_items <= VC_LISTLESS_MAX_ITEMS &&
-           c->hint_max_pieces <= VC_LISTLESS_MAX_PIECES;
+// Whether a forwarded call should try to go without the work-item list, and with how many lanes per pair of ranks
+// (0: through the list): worth it when writing the list (and waiting for its size before that) costs more than the
+// per-pair kernel loses by working out routes itself, i.e. for calls of short blocks.  The last forwarded call on the
+// communicator is the guide (mode 1), or the caller says so (modes 3 and 4).
+static int listless_lanes(const vc_comm *c, const VcSched &S) {
+    if (c->forward == 3) return VC_THREADS;
+    if (c->forward == 4) return 16;
+    if (c->forward != 1 || !c->hint_valid || c->hint_max_pieces > VC_LISTLESS_MAX_PIECES) return 0;
+    const int64_t average = c->hint_payload / std::max<int64_t>(c->hint_items, 1);
+    if ((int64_t)S.P * S.P <= VC_LISTLESS_MAX_ITEMS && c->hint_items <= VC_LISTLESS_MAX_ITEMS)
+        return average < VC_LISTLESS_SMALL_QUARTER_BELOW ? 16 : VC_THREADS;
+    return average < VC_LISTLESS_QUARTER_BELOW ? 16 : 0;
 }
 
 static int run_schedule(vc_comm *c, VcSched S, std::vector<VcLaunchInfo> &L, const char *sendbuf, char *recvbuf, VcTables T, bool forward) {
@@ -427,7 +438,8 @@ static int run_schedule(vc_comm *c, VcSched S, std::vector<VcLaunchInfo> &L, con
     hipStream_t st = c->stream;
     int rc = plan_sizes(c, S, L, T, forward);
     if (rc) return rc;
-    if (forward && want_listless(c, S)) {
+    const int pair_lanes = forward ? listless_lanes(c, S) : 0;
+    if (pair_lanes) {
         // the copy kernel goes out right behind the planning kernels and checks their verdict on the device; when the
         // staging arena turns out too small it has touched nothing, and goes out once more behind a larger arena
         for (int attempt = 0; attempt < 2; attempt++) {
@@ -437,12 +449,12 @@ static int run_schedule(vc_comm *c, VcSched S, std::vector<VcLaunchInfo> &L, con
                 HIP_TRY(hipEventRecord(c->events[2], st));
             }
             HIP_TRY(vc_launch_copy_blocks(S, T, c->slot_off.as<int64_t>(), c->row_base.as<int64_t>(), c->header.as<int64_t>(), stage_cap,
-                                          sendbuf, recvbuf, c->stage.as<char>(), st));
+                                          pair_lanes, sendbuf, recvbuf, c->stage.as<char>(), st));
             if (c->timing) HIP_TRY(hipEventRecord(c->events[3], st));
             HIP_TRY(hipStreamSynchronize(st));
             rc = plan_read(c, S, L, pi, true);
             if (rc) return rc;
-            if (pi.stage_bytes <= stage_cap) { pi.listless = true; break; }
+            if (pi.stage_bytes <= stage_cap) { pi.listless = true; pi.chain_lanes = pair_lanes; break; }
             HIP_TRY(c->stage.reserve((size_t)pi.stage_bytes + 64));
         }
         if (!pi.listless) return fail_arg("the plan changed between two launches of one call", VC_ERR_HIP);

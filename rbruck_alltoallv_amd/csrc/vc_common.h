@@ -148,6 +148,7 @@ hipError_t vc_launch_copy_chains(const int64_t *items, int stride, int64_t nitem
 // Forwarded execution without a work-item list: one workgroup per (source, destination) pair works out the route of its
 // block from the plan tables and carries it through.  Reads the device `header` the planning kernels before it on the
 // stream have written and does nothing when the plan needs more than stage_cap bytes of staging or found bad tables.
+// lanes: VC_THREADS (a workgroup per pair) or 16 (a quarter of a wavefront per pair, for blocks of a few hundred bytes).
 hipError_t vc_launch_copy_blocks(const VcSched &S, VcTables T, const int64_t *slot_off, const int64_t *row_base, const int64_t *header,
-                                 int64_t stage_cap, const char *sendbuf, char *recvbuf, char *stage, hipStream_t st);
+                                 int64_t stage_cap, int lanes, const char *sendbuf, char *recvbuf, char *stage, hipStream_t st);
 hipError_t vc_launch_calibration_copy(const char *src, char *dst, int64_t nbytes, hipStream_t st);

@@ -231,14 +231,62 @@ __global__ __launch_bounds__(VC_THREADS) void vc_copy_blocks_kernel(VcSched S, V
     }
 }
 
+// The same for pairs whose blocks are a few hundred bytes: a quarter of a wavefront per pair, four pairs in a row per
+// wavefront.  Lane q of a group evaluates hop slots q and q + 16; the four routes of the wavefront go through LDS.
+__global__ __launch_bounds__(VC_WAVE) void vc_copy_blocks_quarter_kernel(VcSched S, VcTables T, const int64_t *__restrict__ slot_off,
+                                                                         const int64_t *__restrict__ row_base,
+                                                                         const int64_t *__restrict__ header, int64_t stage_cap,
+                                                                         int64_t first_pair, const char *__restrict__ sendbuf,
+                                                                         char *__restrict__ recvbuf, char *__restrict__ stage) {
+    if (header[0] > stage_cap || header[VC_HEADER_BAD] != 0) return;
+    __shared__ int64_t route[VC_ITEMS_PER_WAVE][VC_MAX_HOP_SLOTS];
+    const int64_t per = gridDim.x / VC_XCDS;
+    const int64_t wave = (int64_t)(blockIdx.x % VC_XCDS) * per + blockIdx.x / VC_XCDS;
+    const int g = threadIdx.x / VC_QUARTER, q = threadIdx.x % VC_QUARTER;
+    const int64_t idx = first_pair + wave * VC_ITEMS_PER_WAVE + g;
+    int t = 0, s = 0;
+    int64_t len = 0;
+    if (idx < (int64_t)S.P * S.P) {
+        t = (int)(idx / S.P);
+        s = (int)(idx % S.P);
+        len = (int64_t)T.sc[(int64_t)s * S.P + t] * S.esz;
+    }
+    const bool active = len > 0;                          // no lane leaves before the barrier below
+    const int nslots = vc_hop_slots(S);
+    int64_t d0 = 0, d1 = 0;
+    const bool m0 = active && q < nslots && vc_block_hop(S, T, slot_off, row_base, s, t, q, d0);
+    const bool m1 = active && q + VC_QUARTER < nslots && vc_block_hop(S, T, slot_off, row_base, s, t, q + VC_QUARTER, d1);
+    const unsigned g0 = (unsigned)(__ballot(m0) >> (g * VC_QUARTER)) & 0xFFFFu;      // the group's hops among slots 0..15
+    const unsigned g1 = (unsigned)(__ballot(m1) >> (g * VC_QUARTER)) & 0xFFFFu;      // ... among slots 16..31
+    if (m0) route[g][__popc(g0 & ((1u << q) - 1))] = d0;
+    if (m1) route[g][__popc(g0) + __popc(g1 & ((1u << q) - 1))] = d1;
+    __syncthreads();
+    const int nhop = __popc(g0) + __popc(g1);
+    if (!active || nhop <= 0) return;
+    const char *src = sendbuf + vc_send_offset(S, T, s, t);
+    const int phase = vc_phase(S, T, s, t), cut = vc_chain_cut(S, T, s, t);
+    const int64_t pieces = vc_chunk_count(len, phase, cut);
+    for (int64_t c = 0; c < pieces; c++) {
+        int64_t lo, hi;
+        vc_piece_range(len, phase, cut, c, lo, hi);
+        vc_forward_piece_quarter(src + lo, hi - lo, nhop, [&](int k) { return vc_resolve(route[g][k] + lo, sendbuf, recvbuf, stage); });
+    }
+}
+
 hipError_t vc_launch_copy_blocks(const VcSched &S, VcTables T, const int64_t *slot_off, const int64_t *row_base, const int64_t *header,
-                                 int64_t stage_cap, const char *sendbuf, char *recvbuf, char *stage, hipStream_t st) {
+                                 int64_t stage_cap, int lanes, const char *sendbuf, char *recvbuf, char *stage, hipStream_t st) {
     const int64_t npairs = (int64_t)S.P * S.P;
-    for (int64_t done = 0; done < npairs; done += VC_MAX_GRID) {
-        const int64_t now = npairs - done < VC_MAX_GRID ? npairs - done : VC_MAX_GRID;
-        const int64_t grid = (now + VC_XCDS - 1) / VC_XCDS * VC_XCDS;
-        hipLaunchKernelGGL(vc_copy_blocks_kernel, dim3((unsigned)grid), dim3(VC_THREADS), 0, st, S, T, slot_off, row_base, header, stage_cap,
-                           done, sendbuf, recvbuf, stage);
+    const int64_t step = lanes == VC_QUARTER ? VC_MAX_GRID * VC_ITEMS_PER_WAVE : VC_MAX_GRID;
+    for (int64_t done = 0; done < npairs; done += step) {
+        const int64_t now = npairs - done < step ? npairs - done : step;
+        const int64_t units = lanes == VC_QUARTER ? (now + VC_ITEMS_PER_WAVE - 1) / VC_ITEMS_PER_WAVE : now;
+        const dim3 grid((unsigned)((units + VC_XCDS - 1) / VC_XCDS * VC_XCDS));
+        if (lanes == VC_QUARTER)
+            hipLaunchKernelGGL(vc_copy_blocks_quarter_kernel, grid, dim3(VC_WAVE), 0, st, S, T, slot_off, row_base, header, stage_cap, done,
+                               sendbuf, recvbuf, stage);
+        else
+            hipLaunchKernelGGL(vc_copy_blocks_kernel, grid, dim3(VC_THREADS), 0, st, S, T, slot_off, row_base, header, stage_cap, done,
+                               sendbuf, recvbuf, stage);
     }
     return hipGetLastError();
 }
