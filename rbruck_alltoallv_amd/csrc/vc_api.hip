@@ -439,30 +439,42 @@ static int run_schedule(vc_comm *c, VcSched S, std::vector<VcLaunchInfo> &L, con
     int rc = plan_sizes(c, S, L, T, forward);
     if (rc) return rc;
     const int pair_lanes = forward ? listless_lanes(c, S) : 0;
+    bool synced = false;
     if (pair_lanes) {
-        // the copy kernel goes out right behind the planning kernels and checks their verdict on the device; when the
-        // staging arena turns out too small it has touched nothing, and goes out once more behind a larger arena
-        for (int attempt = 0; attempt < 2; attempt++) {
-            const int64_t stage_cap = c->stage.cap >= 64 ? (int64_t)c->stage.cap - 64 : 0;
+        // the copy kernel goes out right behind the planning kernels and checks their verdict on the device: when the
+        // staging arena turns out too small it has touched nothing and goes out once more behind a larger arena; when the
+        // call is not of the kind the last one made the host expect, the call continues through the list
+        VcListlessGuard guard = {0, 0, 0, 0};
+        if (c->forward == 1) {
+            const bool quarter = pair_lanes != VC_THREADS;
+            guard.max_pieces = VC_LISTLESS_MAX_PIECES;
+            guard.max_items = quarter ? 0 : VC_LISTLESS_MAX_ITEMS;
+            guard.max_average = quarter ? 2 * VC_LISTLESS_SMALL_QUARTER_BELOW : 0;
+        }
+        for (int attempt = 0; attempt < 2 && !pi.listless; attempt++) {
+            guard.stage_cap = c->stage.cap >= 64 ? (int64_t)c->stage.cap - 64 : 0;
             if (c->timing) {
                 if (attempt == 0) HIP_TRY(hipEventRecord(c->events[1], st));
                 HIP_TRY(hipEventRecord(c->events[2], st));
             }
-            HIP_TRY(vc_launch_copy_blocks(S, T, c->slot_off.as<int64_t>(), c->row_base.as<int64_t>(), c->header.as<int64_t>(), stage_cap,
+            HIP_TRY(vc_launch_copy_blocks(S, T, c->slot_off.as<int64_t>(), c->row_base.as<int64_t>(), c->header.as<int64_t>(), guard,
                                           pair_lanes, sendbuf, recvbuf, c->stage.as<char>(), st));
             if (c->timing) HIP_TRY(hipEventRecord(c->events[3], st));
             HIP_TRY(hipStreamSynchronize(st));
+            synced = true;
             rc = plan_read(c, S, L, pi, true);
             if (rc) return rc;
-            if (pi.stage_bytes <= stage_cap) { pi.listless = true; pi.chain_lanes = pair_lanes; break; }
+            if (vc_listless_ok(c->h_header, guard)) { pi.listless = true; pi.chain_lanes = pair_lanes; break; }
+            if (pi.stage_bytes <= guard.stage_cap) break;          // not a call for this kernel
             HIP_TRY(c->stage.reserve((size_t)pi.stage_bytes + 64));
         }
-        if (!pi.listless) return fail_arg("the plan changed between two launches of one call", VC_ERR_HIP);
-        return finish_stats(c, pi, nullptr, true);
+        if (pi.listless) return finish_stats(c, pi, nullptr, true);
     }
-    HIP_TRY(hipStreamSynchronize(st));             // the staging arena and the item list are sized from the plan
-    rc = plan_read(c, S, L, pi, forward);
-    if (rc) return rc;
+    if (!synced) {
+        HIP_TRY(hipStreamSynchronize(st));         // the staging arena and the item list are sized from the plan
+        rc = plan_read(c, S, L, pi, forward);
+        if (rc) return rc;
+    }
     rc = plan_emit(c, S, L, T, c->desc, pi);
     if (rc) return rc;
     return run_items(c, pi, c->desc.p, sendbuf, recvbuf, true);

@@ -145,10 +145,26 @@ hipError_t vc_launch_copy_items(const VcDesc *items, int64_t nitems, int lanes, 
                                 hipStream_t st);
 hipError_t vc_launch_copy_chains(const int64_t *items, int stride, int64_t nitems, int lanes, const char *sendbuf, char *recvbuf,
                                  char *stage, hipStream_t st);
-// Forwarded execution without a work-item list: one workgroup per (source, destination) pair works out the route of its
-// block from the plan tables and carries it through.  Reads the device `header` the planning kernels before it on the
-// stream have written and does nothing when the plan needs more than stage_cap bytes of staging or found bad tables.
+// What the plan of a call must look like for the listless kernels to run it; 0 = no limit.  The kernels evaluate it on
+// the device header, the host on its copy after the synchronisation: both then agree on whether anything was moved.
+struct VcListlessGuard {
+    int64_t stage_cap;      // bytes of staging arena there are
+    int64_t max_pieces;     // most pieces of one block
+    int64_t max_items;      // block pieces in all
+    int64_t max_average;    // average piece, bytes
+};
+
+VC_HD bool vc_listless_ok(const int64_t *header, const VcListlessGuard &g) {
+    if (header[0] > g.stage_cap || header[VC_HEADER_BAD] != 0) return false;
+    if (g.max_pieces && header[VC_HEADER_MAX_PIECES] > g.max_pieces) return false;
+    if (g.max_items && header[2] > g.max_items) return false;
+    return !(g.max_average && header[1] > g.max_average * header[2]);
+}
+
+// Forwarded execution without a work-item list: one workgroup (or a quarter of a wavefront) per (source, destination)
+// pair works out the route of its block from the plan tables and carries it through.  Reads the device `header` the
+// planning kernels before it on the stream have written and does nothing unless vc_listless_ok(header, guard).
 // lanes: VC_THREADS (a workgroup per pair) or 16 (a quarter of a wavefront per pair, for blocks of a few hundred bytes).
 hipError_t vc_launch_copy_blocks(const VcSched &S, VcTables T, const int64_t *slot_off, const int64_t *row_base, const int64_t *header,
-                                 int64_t stage_cap, int lanes, const char *sendbuf, char *recvbuf, char *stage, hipStream_t st);
+                                 VcListlessGuard guard, int lanes, const char *sendbuf, char *recvbuf, char *stage, hipStream_t st);
 hipError_t vc_launch_calibration_copy(const char *src, char *dst, int64_t nbytes, hipStream_t st);

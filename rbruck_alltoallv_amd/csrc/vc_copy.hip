@@ -196,13 +196,14 @@ __global__ __launch_bounds__(VC_WAVE) void vc_copy_items_quarter_kernel(const Vc
 // of the pairs per XCD).  The workgroup works out the route of its block in closed form from the plan tables (lane k
 // evaluates hop slot k), then carries the block through it piece by piece.  The kernel is enqueued right behind the
 // planning kernels, before the host has seen their result, so it checks that result itself: nothing is touched when the
-// plan needs more staging than there is or the tables hold negative entries (the host then takes the other path).
+// plan needs more staging than there is, the tables hold negative entries, or the call is not of the kind the host
+// expected when it chose this kernel (the host, which evaluates the same condition afterwards, then takes another path).
 __global__ __launch_bounds__(VC_THREADS) void vc_copy_blocks_kernel(VcSched S, VcTables T, const int64_t *__restrict__ slot_off,
                                                                     const int64_t *__restrict__ row_base,
-                                                                    const int64_t *__restrict__ header, int64_t stage_cap,
+                                                                    const int64_t *__restrict__ header, VcListlessGuard guard,
                                                                     int64_t first_pair, const char *__restrict__ sendbuf,
                                                                     char *__restrict__ recvbuf, char *__restrict__ stage) {
-    if (header[0] > stage_cap || header[VC_HEADER_BAD] != 0) return;
+    if (!vc_listless_ok(header, guard)) return;
     __shared__ int64_t route[VC_MAX_HOP_SLOTS];
     __shared__ int route_len;
     const int64_t per = gridDim.x / VC_XCDS;
@@ -235,10 +236,10 @@ __global__ __launch_bounds__(VC_THREADS) void vc_copy_blocks_kernel(VcSched S, V
 // wavefront.  Lane q of a group evaluates hop slots q and q + 16; the four routes of the wavefront go through LDS.
 __global__ __launch_bounds__(VC_WAVE) void vc_copy_blocks_quarter_kernel(VcSched S, VcTables T, const int64_t *__restrict__ slot_off,
                                                                          const int64_t *__restrict__ row_base,
-                                                                         const int64_t *__restrict__ header, int64_t stage_cap,
+                                                                         const int64_t *__restrict__ header, VcListlessGuard guard,
                                                                          int64_t first_pair, const char *__restrict__ sendbuf,
                                                                          char *__restrict__ recvbuf, char *__restrict__ stage) {
-    if (header[0] > stage_cap || header[VC_HEADER_BAD] != 0) return;
+    if (!vc_listless_ok(header, guard)) return;
     __shared__ int64_t route[VC_ITEMS_PER_WAVE][VC_MAX_HOP_SLOTS];
     const int64_t per = gridDim.x / VC_XCDS;
     const int64_t wave = (int64_t)(blockIdx.x % VC_XCDS) * per + blockIdx.x / VC_XCDS;
@@ -274,7 +275,7 @@ __global__ __launch_bounds__(VC_WAVE) void vc_copy_blocks_quarter_kernel(VcSched
 }
 
 hipError_t vc_launch_copy_blocks(const VcSched &S, VcTables T, const int64_t *slot_off, const int64_t *row_base, const int64_t *header,
-                                 int64_t stage_cap, int lanes, const char *sendbuf, char *recvbuf, char *stage, hipStream_t st) {
+                                 VcListlessGuard guard, int lanes, const char *sendbuf, char *recvbuf, char *stage, hipStream_t st) {
     const int64_t npairs = (int64_t)S.P * S.P;
     const int64_t step = lanes == VC_QUARTER ? VC_MAX_GRID * VC_ITEMS_PER_WAVE : VC_MAX_GRID;
     for (int64_t done = 0; done < npairs; done += step) {
@@ -282,10 +283,10 @@ hipError_t vc_launch_copy_blocks(const VcSched &S, VcTables T, const int64_t *sl
         const int64_t units = lanes == VC_QUARTER ? (now + VC_ITEMS_PER_WAVE - 1) / VC_ITEMS_PER_WAVE : now;
         const dim3 grid((unsigned)((units + VC_XCDS - 1) / VC_XCDS * VC_XCDS));
         if (lanes == VC_QUARTER)
-            hipLaunchKernelGGL(vc_copy_blocks_quarter_kernel, grid, dim3(VC_WAVE), 0, st, S, T, slot_off, row_base, header, stage_cap, done,
+            hipLaunchKernelGGL(vc_copy_blocks_quarter_kernel, grid, dim3(VC_WAVE), 0, st, S, T, slot_off, row_base, header, guard, done,
                                sendbuf, recvbuf, stage);
         else
-            hipLaunchKernelGGL(vc_copy_blocks_kernel, grid, dim3(VC_THREADS), 0, st, S, T, slot_off, row_base, header, stage_cap, done,
+            hipLaunchKernelGGL(vc_copy_blocks_kernel, grid, dim3(VC_THREADS), 0, st, S, T, slot_off, row_base, header, guard, done,
                                sendbuf, recvbuf, stage);
     }
     return hipGetLastError();
