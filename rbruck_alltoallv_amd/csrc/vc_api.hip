@@ -279,7 +279,7 @@ static int plan_sizes(vc_comm *c, const VcSched &S, std::vector<VcLaunchInfo> &L
 static int lanes_for(int64_t bytes, int64_t items) {
     if (items <= 0) return VC_THREADS;
     const int64_t average = bytes / items;
-    return average < 448 ? 16 : (average < 3072 ? VC_WAVE : VC_THREADS);
+    return average < 448 ? VC_QUARTER : (average < 3072 ? VC_WAVE : VC_THREADS);
 }
 
 // Step 3b, after the stream has been synchronised: what the planning kernels found.
@@ -425,12 +425,12 @@ static int run_items(vc_comm *c, const PlanInfo &pi, const void *items_any, cons
 // communicator is the guide (mode 1), or the caller says so (modes 3 and 4).
 static int listless_lanes(const vc_comm *c, const VcSched &S) {
     if (c->forward == 3) return VC_THREADS;
-    if (c->forward == 4) return 16;
+    if (c->forward == 4) return VC_QUARTER;
     if (c->forward != 1 || !c->hint_valid || c->hint_max_pieces > VC_LISTLESS_MAX_PIECES) return 0;
     const int64_t average = c->hint_payload / std::max<int64_t>(c->hint_items, 1);
     if ((int64_t)S.P * S.P <= VC_LISTLESS_MAX_ITEMS && c->hint_items <= VC_LISTLESS_MAX_ITEMS)
-        return average < VC_LISTLESS_SMALL_QUARTER_BELOW ? 16 : VC_THREADS;
-    return average < VC_LISTLESS_QUARTER_BELOW ? 16 : 0;
+        return average < VC_LISTLESS_SMALL_QUARTER_BELOW ? VC_QUARTER : VC_THREADS;
+    return average < VC_LISTLESS_QUARTER_BELOW ? VC_QUARTER : 0;
 }
 
 static int run_schedule(vc_comm *c, VcSched S, std::vector<VcLaunchInfo> &L, const char *sendbuf, char *recvbuf, VcTables T, bool forward) {

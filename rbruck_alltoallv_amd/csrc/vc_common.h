@@ -12,6 +12,8 @@
 #include <stdint.h>
 
 #define VC_THREADS 256
+// lanes of a work item in the copy kernels for short pieces: a wavefront (VC_WAVE, vc_scan.h) or a quarter of one
+#define VC_QUARTER 16
 // window of one workgroup of the copy kernel: 256 lanes x 2 vectors x 16 bytes, starting at a cache-line boundary
 #define VC_CHUNK 8192
 #define VC_LINE 128
@@ -139,7 +141,7 @@ hipError_t vc_launch_plan_emit(const VcSched &S, const VcLaunchInfo *launches_ho
 hipError_t vc_launch_traffic(const VcDesc *desc, int64_t ndesc, int64_t *matrix, int P, hipStream_t st);
 
 // vc_copy.hip
-// lanes: VC_THREADS (a workgroup per item), VC_WAVE (a wavefront per item, for lists of short pieces) or 16 (a quarter of
+// lanes: VC_THREADS (a workgroup per item), VC_WAVE (a wavefront per item, for lists of short pieces) or VC_QUARTER (a quarter of
 // a wavefront, for lists of pieces of a few hundred bytes)
 hipError_t vc_launch_copy_items(const VcDesc *items, int64_t nitems, int lanes, const char *sendbuf, char *recvbuf, char *stage,
                                 hipStream_t st);
@@ -164,7 +166,7 @@ VC_HD bool vc_listless_ok(const int64_t *header, const VcListlessGuard &g) {
 // Forwarded execution without a work-item list: one workgroup (or a quarter of a wavefront) per (source, destination)
 // pair works out the route of its block from the plan tables and carries it through.  Reads the device `header` the
 // planning kernels before it on the stream have written and does nothing unless vc_listless_ok(header, guard).
-// lanes: VC_THREADS (a workgroup per pair) or 16 (a quarter of a wavefront per pair, for blocks of a few hundred bytes).
+// lanes: VC_THREADS (a workgroup per pair) or VC_QUARTER (a quarter of a wavefront per pair, for blocks of a few hundred bytes).
 hipError_t vc_launch_copy_blocks(const VcSched &S, VcTables T, const int64_t *slot_off, const int64_t *row_base, const int64_t *header,
                                  VcListlessGuard guard, int lanes, const char *sendbuf, char *recvbuf, char *stage, hipStream_t st);
 hipError_t vc_launch_calibration_copy(const char *src, char *dst, int64_t nbytes, hipStream_t st);

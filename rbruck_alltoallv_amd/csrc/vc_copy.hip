@@ -159,7 +159,6 @@ __device__ __forceinline__ void vc_forward_piece_quarter(const char *src, int64_
     }
 }
 
-#define VC_QUARTER 16                                     // lanes per item of the kernels below
 #define VC_ITEMS_PER_WAVE (VC_WAVE / VC_QUARTER)
 
 // gridDim.x wavefronts, a multiple of VC_XCDS; XCD k works through the k-th eighth of them, each taking four items in a row
