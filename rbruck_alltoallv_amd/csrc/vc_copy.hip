@@ -4,12 +4,12 @@
 // (src/twophase_tunable_rbruckv.cpp:90-100,119,126-139) collapse into one read of
 // the block where the sender holds it and one write where the receiver wants it.
 //
-// Shape of the kernel, chosen by measurement on MI355X: one 256-lane workgroup per
-// work item (a piece of one block that fits a window of VC_CHUNK = 8 KiB), every lane moving
-// up to two 16-byte vectors whose loads are both issued before the stores,
-// non-temporal on both sides (the data is touched once per hop).  Many small
-// workgroups beat persistent or wider ones for a plain copy on this chip, and the
-// same holds for the scattered variable-size blocks of an alltoallv.
+// Shape of the kernels, chosen by measurement on MI355X: one work item = a piece of one block that fits a window of
+// VC_CHUNK = 8 KiB; every lane moves 16-byte vectors whose loads are all issued before the stores, non-temporal on both
+// sides (the data is touched once per hop).  For pieces of several KiB a 256-lane workgroup per item is fastest (many
+// small workgroups beat persistent or wider ones for a plain copy on this chip, and the same holds for the scattered
+// variable-size blocks of an alltoallv); lists of short pieces are bound by the number of items in flight and get a
+// wavefront, or a quarter of one, per item.  The host chooses per launch (lanes_for in vc_api.hip).
 //
 // Workgroups are handed to the 8 XCDs of the chip in turn (workgroup b runs on XCD
 // b mod 8) and every XCD has its own L2.  Work items that follow each other in the
@@ -42,20 +42,21 @@ __device__ __forceinline__ char *vc_resolve(int64_t loc, const char *sendbuf, ch
     return base + off;
 }
 
-// One workgroup (or one wavefront) of LANES lanes per work item.  Lane t owns the t-th, (t + LANES)-th, ... 16-byte vector
-// of the window that starts at the 128-byte boundary at or below dst, so every wave stores whole cache lines whatever
-// the byte phase of the block (measured: +4 % over counting vectors from the first 16-byte boundary of dst).  Vectors
-// that lie fully inside the block are moved by (possibly unaligned) 16-byte loads and aligned stores; the < 16 bytes
-// before the first and after the last of them are moved byte-wise (lanes 0..15 the head, lanes 16..31 the tail: one byte
-// load and one byte store each).  The planner guarantees len + (dst & 127) <= VC_CHUNK.
 #define VC_XCDS 8
 // Workgroups of one launch: a dispatch counts its grid in work-items in 32 bits, so gridDim.x * VC_THREADS must stay
 // below 2^32 (a larger grid is not refused: it runs truncated); longer lists go out in several launches.  A multiple of
 // VC_XCDS.
 #define VC_MAX_GRID ((int64_t)((1ull << 32) / VC_THREADS) - VC_XCDS)
-// Forwarded execution: one workgroup carries a piece through all the hops of its block.  The piece is read once, from
-// sendbuf; every hop stores the same registers (all destinations of a block share the offset inside their cache line,
-// so one mapping of lanes to window vectors serves them all).  dst_of(k) is where hop k puts the piece.
+
+// One workgroup (or one wavefront) of LANES lanes moves one piece.  Lane t owns the t-th, (t + LANES)-th, ... 16-byte vector
+// of the window that starts at the 128-byte boundary at or below dst, so every wave stores whole cache lines whatever
+// the byte phase of the block (measured: +4 % over counting vectors from the first 16-byte boundary of dst).  Vectors
+// that lie fully inside the block are moved by (possibly unaligned) 16-byte loads and aligned stores; the < 16 bytes
+// before the first and after the last of them are moved byte-wise (lanes 0..15 the head, lanes 16..31 the tail: one byte
+// load and one byte store each).  The planner guarantees len + (dst & 127) <= VC_CHUNK.
+// With nhop > 1 this is forwarded execution: the piece is read once, from sendbuf, and every hop stores the same
+// registers (all destinations of a block share the offset inside their cache line, so one mapping of lanes to window
+// vectors serves them all).  dst_of(k) is where hop k puts the piece.
 template <int LANES, class DstOf>
 __device__ __forceinline__ void vc_forward_piece(const char *src, int64_t len, int nhop, DstOf dst_of) {
     constexpr int VECS = VC_CHUNK / 16 / LANES;           // window vectors per lane: 2 for a workgroup of 256, 8 for one wavefront
