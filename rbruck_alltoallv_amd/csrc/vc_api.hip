@@ -32,13 +32,16 @@ static int fail_hip(hipError_t e, const char *what, int line) {
 
 // Where the default mode goes without a work-item list (measured, blocking calls on MI355X):
 //  - blocks of a few hundred bytes, any number of ranks: a quarter of a wavefront per pair of ranks.  Average piece below
-//    1 KiB: 26 - 30 us per call at 64 ranks (through the list 42), 42 - 73 at 256 (51 - 88), 300 - 900 at 1024 (330 - 990).
-//  - at most 128 ranks and 16384 pieces, longer blocks: a workgroup per pair (35 - 52 us against 47 - 80 at 64 ranks;
-//    even at 128 ranks; at 256 ranks the list wins by 1.3 - 1.8x).
-//  - never after a call with a block of more than VC_LISTLESS_MAX_PIECES pieces (one workgroup moves them in turn).
-#define VC_LISTLESS_MAX_ITEMS 16384
-#define VC_LISTLESS_MAX_PIECES 8
-#define VC_LISTLESS_QUARTER_BELOW 1024        // average piece, any communicator
+//    768 B: 26 - 30 us per call at 64 ranks (through the list 42), 42 - 73 at 256 (51 - 88), 300 - 900 at 1024 (330 - 990).
+//  - at most 128 ranks and 32768 pieces, longer blocks: a workgroup per pair (26 - 42 us against 40 - 57 at 16 and 64 ranks
+//    with blocks up to 8 KB, 31 - 77 against 48 - 92 up to 32 KB; a few per cent at 128 ranks; at 256 ranks the list wins).
+//  - never after a call with a block of more than 8 (quarter) / 16 (workgroup) pieces: one group of lanes moves the
+//    pieces of a block in turn.
+#define VC_LISTLESS_MAX_PAIRS 16384           // "small communicator": at most 128 ranks
+#define VC_LISTLESS_MAX_ITEMS 32768           // pieces of a call for a workgroup per pair
+#define VC_LISTLESS_MAX_PIECES 8              // pieces of one block, quarter of a wavefront per pair
+#define VC_LISTLESS_WG_MAX_PIECES 16          // pieces of one block, workgroup per pair
+#define VC_LISTLESS_QUARTER_BELOW 768         // average piece, any communicator (at 1 KiB the two ways are even)
 #define VC_LISTLESS_SMALL_QUARTER_BELOW 2048  // average piece, communicators of at most 128 ranks
 
 #define HIP_TRY(expr)                                                   \
@@ -426,11 +429,13 @@ static int run_items(vc_comm *c, const PlanInfo &pi, const void *items_any, cons
 static int listless_lanes(const vc_comm *c, const VcSched &S) {
     if (c->forward == 3) return VC_THREADS;
     if (c->forward == 4) return VC_QUARTER;
-    if (c->forward != 1 || !c->hint_valid || c->hint_max_pieces > VC_LISTLESS_MAX_PIECES) return 0;
+    if (c->forward != 1 || !c->hint_valid) return 0;
     const int64_t average = c->hint_payload / std::max<int64_t>(c->hint_items, 1);
-    if ((int64_t)S.P * S.P <= VC_LISTLESS_MAX_ITEMS && c->hint_items <= VC_LISTLESS_MAX_ITEMS)
-        return average < VC_LISTLESS_SMALL_QUARTER_BELOW ? VC_QUARTER : VC_THREADS;
-    return average < VC_LISTLESS_QUARTER_BELOW ? VC_QUARTER : 0;
+    const bool small_comm = (int64_t)S.P * S.P <= VC_LISTLESS_MAX_PAIRS;
+    if (c->hint_max_pieces <= VC_LISTLESS_MAX_PIECES && average < (small_comm ? VC_LISTLESS_SMALL_QUARTER_BELOW : VC_LISTLESS_QUARTER_BELOW))
+        return VC_QUARTER;
+    if (small_comm && c->hint_max_pieces <= VC_LISTLESS_WG_MAX_PIECES && c->hint_items <= VC_LISTLESS_MAX_ITEMS) return VC_THREADS;
+    return 0;
 }
 
 static int run_schedule(vc_comm *c, VcSched S, std::vector<VcLaunchInfo> &L, const char *sendbuf, char *recvbuf, VcTables T, bool forward) {
@@ -447,7 +452,7 @@ static int run_schedule(vc_comm *c, VcSched S, std::vector<VcLaunchInfo> &L, con
         VcListlessGuard guard = {0, 0, 0, 0};
         if (c->forward == 1) {
             const bool quarter = pair_lanes != VC_THREADS;
-            guard.max_pieces = VC_LISTLESS_MAX_PIECES;
+            guard.max_pieces = quarter ? VC_LISTLESS_MAX_PIECES : VC_LISTLESS_WG_MAX_PIECES;
             guard.max_items = quarter ? 0 : VC_LISTLESS_MAX_ITEMS;
             guard.max_average = quarter ? 2 * VC_LISTLESS_SMALL_QUARTER_BELOW : 0;
         }
