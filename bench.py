@@ -152,8 +152,17 @@ def cpu_baseline(name: str, seed: int, budget_s: float) -> dict:
 # vc_stats_t.execution of the timed calls (the library's default mode picks between the two forwarded kernels)
 EXECUTION_NAMES = {0: "launch per digit phase",
                    1: "forwarded (one launch, blocks carried through all hops in registers)",
-                   2: "forwarded, without a work-item list (one workgroup per pair of ranks; one host synchronisation per call)"}
-EXECUTION_KERNELS = {0: "vc_copy_items_kernel", 1: "vc_copy_chains_kernel", 2: "vc_copy_blocks_kernel"}
+                   2: "forwarded, without a work-item list (every pair of ranks derives its block's route in the copy kernel; "
+                      "one host synchronisation per call)"}
+EXECUTION_KERNELS = {0: "vc_copy_items", 1: "vc_copy_chains", 2: "vc_copy_blocks"}
+
+
+def kernel_name(st) -> str:
+    """Name of the copy kernel the timed calls launched, from vc_stats_t.execution and .lanes_per_item."""
+    base, lanes = EXECUTION_KERNELS[int(st.execution)], int(st.lanes_per_item)
+    if lanes == 16:
+        return base + "_quarter_kernel"
+    return base + "_kernel" + ("" if st.execution == 2 else f"<{lanes}>")
 
 
 def main() -> None:
@@ -332,7 +341,7 @@ def main() -> None:
         "one_pass_comparator": {"func": "spreadout_alltoallv", "ms_per_call": round(comp_s * 1e3, 4),
                                 "GBps_effective": round(S / comp_s / 1e9, 1),
                                 "hbm_frac": round(2 * S / comp_s / 1e9 / HBM_PEAK_GBPS, 4), "mismatched_bytes": int(comp_bad)},
-        "roofline": {"bound": "hbm", "kernel": EXECUTION_KERNELS[int(st.execution)] + ("" if st.execution == 2 else f"<{int(st.lanes_per_item)}>"), "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
+        "roofline": {"bound": "hbm", "kernel": kernel_name(st), "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
                      "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
                      "traffic": MEASURED_TRAFFIC_PER_LAUNCH.get((args.workload, func, int(bool(args.forward)))),
                      "avg_launch_ms": round(kern_ms / max(nkern, 1), 4),
