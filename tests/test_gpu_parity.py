@@ -694,6 +694,46 @@ def test_seeded_random_sweep(api):
         dp.comm.free()
 
 
+@pytest.mark.parametrize("P", [24, 100])
+def test_seeded_sweep_on_one_communicator(api, P):
+    """One long-lived communicator, every call with other sizes, another function and another execution mode: buffers
+    grow, the hints of the default mode go stale, the listless kernels refuse calls and the list takes over."""
+    import random
+    rnd = random.Random(P)
+    comm = api.VirtualComm(P)
+    divs = [d for d in range(1, P + 1) if P % d == 0]
+    for it in range(60):
+        hi = rnd.choice([0, 3, 40, 300, 2000, 9000, 30000])
+        esz = rnd.choice([1, 2, 4, 8])
+        counts = W.counts_uniform_random(P, hi, seed=it * 7 + P)
+        if rnd.random() < 0.3:
+            counts[counts % 3 == 0] = 0
+        if rnd.random() < 0.15:
+            counts[rnd.randrange(P), rnd.randrange(P)] = rnd.choice([60000, 250000])
+        layout = rnd.choice([0, 1])
+        prob = W.make_problem(counts, esz, layout, layout)
+        dp = api.DeviceProblem(prob, comm=comm)
+        mode = rnd.choice([0, 1, 1, 1, 1, 2, 3, 4])
+        comm.set_forwarding(mode)
+        ds = dp.new_send_arena()
+        dp.fill_payload(0, it, ds)
+        dr = dp.new_recv_arena(0xEE)
+        n, r, b = rnd.choice(divs), rnd.choice([2, 3, 4, 8, 16, P]), rnd.choice([0, 1, 5])
+        calls = [("twophase", lambda: api.twophase_rbruck_alltoallv(r, dp, ds, dr), False),
+                 ("om", lambda: api.twophase_rbruck_alltoallv_om(r, dp, ds, dr), False),
+                 ("s1", lambda: api.TTPL_BT_alltoallv_s1(n, r, b, dp, ds, dr), False),
+                 ("rbruck", lambda: api.TTPL_rbruck_alltoallv(n, r, dp, ds, dr), False),
+                 ("tuna", lambda: api.tuna_algorithm(r, b, dp, ds, dr), False),
+                 ("spreadout", lambda: api.spreadout_alltoallv(dp, ds, dr), False)]
+        if layout == 0:
+            calls.append(("ttpl", lambda: api.TTPL_BT_alltoallv(n, r, b, dp, ds, dr), True))
+        name, fn, packed = rnd.choice(calls)
+        what = f"call {it} {name}: mode={mode} n={n} r={r} b={b} esz={esz} hi={hi} layout={layout}"
+        assert fn() == 0, (what, comm.error())
+        assert dp.verify(ds, dr, packed_recv=packed) == 0, what
+    comm.free()
+
+
 def test_default_mode_picks_the_listless_kernel_for_small_calls(api):
     """Mode 1 (the library's default): forwarded, and after a call of few short blocks the next one goes without the
     work-item list; a call with long blocks is refused by the listless kernel's own check of the plan and goes through
