@@ -141,22 +141,22 @@ __device__ __forceinline__ void vc_forward_piece_quarter(const char *src, int64_
     char head_byte = 0, tail_byte = 0;
     if (has_head) head_byte = src[t];
     if (has_tail) tail_byte = src[done + t];
-    for (int k = 0; k < nhop; k++) {
-        if (k) dst = dst_of(k);
-        if (has_head) dst[t] = head_byte;
-        if (has_tail) dst[done + t] = tail_byte;
-    }
     const char *sw = src - w;
-    for (int64_t j = t; j < end_full; j += 32) {
-        const bool has0 = j >= first_full, has1 = j + 16 >= first_full && j + 16 < end_full;
+    bool first_pass = true;                               // the pass that also stores the head and tail bytes: there is
+    for (int64_t j = t; first_pass || j < end_full; j += 32) {     // always one, also for a block without a full vector
+        const bool has0 = j >= first_full && j < end_full, has1 = j + 16 >= first_full && j + 16 < end_full;
         vc_u32x4 v0, v1;
         if (has0) v0 = vc_load16(sw + (j << 4));
         if (has1) v1 = vc_load16(sw + ((j + 16) << 4));
         for (int k = 0; k < nhop; k++) {
-            char *dw = dst_of(k) - w;
+            if (k || !first_pass) dst = dst_of(k);
+            char *dw = dst - w;
+            if (first_pass && has_head) dst[t] = head_byte;
+            if (first_pass && has_tail) dst[done + t] = tail_byte;
             if (has0) vc_store16(dw + (j << 4), v0);
             if (has1) vc_store16(dw + ((j + 16) << 4), v1);
         }
+        first_pass = false;
     }
 }
 
