@@ -276,8 +276,8 @@ static int plan_sizes(vc_comm *c, const VcSched &S, std::vector<VcLaunchInfo> &L
 // Lanes per work item, from the average piece of the list.  Short pieces leave most of a workgroup idle, and what bounds
 // the launch is then the number of items in flight: a wavefront per item keeps four times as many as a workgroup, a
 // quarter of a wavefront sixteen times.  Measured on 1 Mi items (P = 1024, times of the copy kernel, workgroup /
-// wavefront / quarter): pieces uniform in 0..16 B 832 / 269 / 86 us, 0..256 B 883 / 350 / 213, 0..1 KiB 922 / 456 / 445,
-// 0..2 KiB 1105 / 695 / 783, 0..4 KiB 1450 / 1318 / 1479; around 4 KiB and above the workgroup is 5 - 8 % faster than the
+// wavefront / quarter): pieces uniform in 0..16 B 830 / 269 / 67 us, 0..256 B 882 / 351 / 189, 0..1 KiB 926 / 455 / 431,
+// 0..2 KiB 1105 / 693 / 770, 0..4 KiB 1449 / 1311 / 1462; around 4 KiB and above the workgroup is 5 - 8 % faster than the
 // wavefront.
 static int lanes_for(int64_t bytes, int64_t items) {
     if (items <= 0) return VC_THREADS;
