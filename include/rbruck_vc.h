@@ -46,8 +46,10 @@ typedef struct vc_comm *vc_comm_t;
 
 /* ---- communicator (replaces MPI_Comm; MPI_Comm_size/MPI_Comm_rank have no per-rank analogue) ---- */
 
-/* Creates a virtual communicator of `nranks` ranks on the current HIP device. */
+/* Creates a virtual communicator of `nranks` ranks on the current HIP device.  A communicator serves one call at a time
+ * (it owns the staging arena and the planning buffers the calls reuse); use one per host thread or stream. */
 int vc_comm_create(int nranks, vc_comm_t *comm_out);
+/* Waits for the communicator's stream, then releases its device and pinned memory.  Free its plans first. */
 int vc_comm_free(vc_comm_t comm);
 int vc_comm_size(vc_comm_t comm);
 
@@ -209,6 +211,7 @@ int vc_plan_execute(vc_plan_t plan, char *sendbuf, char *recvbuf);
  * when the plan was created; a later, larger call on the same communicator may move it, after which graphs captured
  * before are stale.  The caller orders later work after it (same stream, or an event). */
 int vc_plan_execute_async(vc_plan_t plan, char *sendbuf, char *recvbuf);
+/* Waits for the communicator's stream and releases the plan's work items; before vc_comm_free of its communicator. */
 int vc_plan_free(vc_plan_t plan);
 
 /* ---- radix choice.  The reference leaves r to the caller (its drivers sweep a list of bases,
