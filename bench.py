@@ -80,6 +80,38 @@ def call(api, func, tun, dp, send, recv):
     raise SystemExit(func)
 
 
+def short_block_context(api, torch) -> dict:
+    """Context beside the metric: blocking calls at the other end of the metric's range of rank counts and at the block sizes
+    the Bruck family exists for (short ones), microseconds per call by wall clock.  `default` is the library's default
+    mode after its first call on the communicator, `through_list` forces the work-item list (vc_comm_set_forwarding 2)."""
+    out = {}
+    for key, P, hi, what, fn in (
+            ("P64_blocks_0_4096B_twophase_r2", 64, 4096, "benchmark configuration 2", lambda dp, s, d: api.twophase_rbruck_alltoallv(2, dp, s, d)),
+            ("P1024_blocks_0_512B_ttpl_n32_r32", 1024, 512, "configuration 4's shape with short blocks", lambda dp, s, d: api.TTPL_BT_alltoallv_s1(32, 32, 0, dp, s, d))):
+        prob = W.make_problem(W.counts_uniform_random(P, hi, seed=0), 1, 0, 0)
+        dp = api.DeviceProblem(prob)
+        send, recv = dp.new_send_arena(), dp.new_recv_arena()
+        dp.fill_payload(0, 0, send)
+        entry = {"workload": what, "payload_bytes": int(prob.payload_bytes)}
+        for label, mode in (("default", 1), ("through_list", 2)):
+            dp.comm.set_forwarding(mode)
+            for _ in range(3):
+                assert fn(dp, send, recv) == 0, dp.comm.error()
+            reps = 200 if P <= 64 else 30
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(reps):
+                fn(dp, send, recv)
+            entry[label + "_us_per_call"] = round((time.perf_counter() - t0) / reps * 1e6, 1)
+            if mode == 1:
+                st = dp.comm.last_stats()
+                entry["default_kernel"] = kernel_name(st)
+        entry["mismatched_bytes"] = int(dp.verify(send, recv))
+        out[key] = entry
+        dp.comm.free()
+    return out
+
+
 def cpu_baseline(name: str, seed: int, budget_s: float) -> dict:
     """The same algorithm on this box's host cores, on a bounded sample of the workload.
 
@@ -318,6 +350,7 @@ def main() -> None:
     torch.cuda.synchronize()
     comp_s = (time.perf_counter() - c0) / comp_steps
     comp_bad = dp.verify(send, recv, packed_recv=False)
+    short_blocks = short_block_context(api, torch) if args.workload == "C4" and args.func is None else None
     ms_per_step = elapsed / args.steps * 1e3
     value = S / (elapsed / args.steps) / 1e9
     achieved = kern_bytes / (kern_ms * 1e-3) / 1e9 if kern_ms > 0 else 0.0
@@ -338,6 +371,7 @@ def main() -> None:
         "execution": EXECUTION_NAMES[int(st.execution)],
         "persistent_plan": plan_info,
         "other_execution_mode": other,
+        "short_block_calls": short_blocks,
         "one_pass_comparator": {"func": "spreadout_alltoallv", "ms_per_call": round(comp_s * 1e3, 4),
                                 "GBps_effective": round(S / comp_s / 1e9, 1),
                                 "hbm_frac": round(2 * S / comp_s / 1e9 / HBM_PEAK_GBPS, 4), "mismatched_bytes": int(comp_bad)},
