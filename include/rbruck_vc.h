@@ -68,7 +68,7 @@ int vc_comm_set_bases(vc_comm_t comm, const int64_t *sbase_bytes, const int64_t 
  *    per block instead of coalesced.  The copy kernel normally works through a list of block pieces that a planning
  *    kernel writes first (after the host has learnt its size).  When the last call on the communicator consisted of
  *    short blocks, the next one goes without the list: every pair of ranks gets a workgroup (at most 128 ranks) or a
- *    quarter of a wavefront (average piece below 768 B, any number of ranks) that derives its block's route itself; the
+ *    quarter of a wavefront (short blocks: average piece below 768 B on any number of ranks, below 1.75 - 3 KiB on 33 - 128) that derives its block's route itself; the
  *    kernel is enqueued right behind the size computation and the call needs one host synchronisation instead of two
  *    (26 - 35 us instead of 42 - 47 us per call at 64 ranks on MI355X, 10 - 25 % less at 256 and 1024 ranks).
  * 2: forwarded, always through the list.   3 / 4: forwarded, always without it, a workgroup / a quarter of a wavefront

@@ -42,7 +42,10 @@ static int fail_hip(hipError_t e, const char *what, int line) {
 #define VC_LISTLESS_MAX_PIECES 8              // pieces of one block, quarter of a wavefront per pair
 #define VC_LISTLESS_WG_MAX_PIECES 16          // pieces of one block, workgroup per pair
 #define VC_LISTLESS_QUARTER_BELOW 768         // average piece, any communicator (at 1 KiB the two ways are even)
-#define VC_LISTLESS_SMALL_QUARTER_BELOW 2048  // average piece, communicators of at most 128 ranks
+// ... on communicators of at most 128 ranks, where the alternative is a workgroup per pair: never up to 32 ranks (1024
+// pairs leave room for as many workgroups: 26 us either way, the workgroup up to 1.3x faster on KiB blocks), below
+// 1.75 KiB up to 90 ranks (64 ranks: 27 - 33 us against 34 - 38), below 3 KiB above (128 ranks: 30 - 70 us against 64 - 84)
+static int64_t small_quarter_below(int64_t pairs) { return pairs <= 1024 ? 0 : (pairs < 8192 ? 1792 : 3072); }
 
 #define HIP_TRY(expr)                                                   \
     do {                                                                \
@@ -432,7 +435,7 @@ static int listless_lanes(const vc_comm *c, const VcSched &S) {
     if (c->forward != 1 || !c->hint_valid) return 0;
     const int64_t average = c->hint_payload / std::max<int64_t>(c->hint_items, 1);
     const bool small_comm = (int64_t)S.P * S.P <= VC_LISTLESS_MAX_PAIRS;
-    if (c->hint_max_pieces <= VC_LISTLESS_MAX_PIECES && average < (small_comm ? VC_LISTLESS_SMALL_QUARTER_BELOW : VC_LISTLESS_QUARTER_BELOW))
+    if (c->hint_max_pieces <= VC_LISTLESS_MAX_PIECES && average < (small_comm ? small_quarter_below((int64_t)S.P * S.P) : VC_LISTLESS_QUARTER_BELOW))
         return VC_QUARTER;
     if (small_comm && c->hint_max_pieces <= VC_LISTLESS_WG_MAX_PIECES && c->hint_items <= VC_LISTLESS_MAX_ITEMS) return VC_THREADS;
     return 0;
@@ -454,7 +457,7 @@ static int run_schedule(vc_comm *c, VcSched S, std::vector<VcLaunchInfo> &L, con
             const bool quarter = pair_lanes != VC_THREADS;
             guard.max_pieces = quarter ? VC_LISTLESS_MAX_PIECES : VC_LISTLESS_WG_MAX_PIECES;
             guard.max_items = quarter ? 0 : VC_LISTLESS_MAX_ITEMS;
-            guard.max_average = quarter ? 2 * VC_LISTLESS_SMALL_QUARTER_BELOW : 0;
+            guard.max_average = quarter ? 4096 : 0;
         }
         for (int attempt = 0; attempt < 2 && !pi.listless; attempt++) {
             guard.stage_cap = c->stage.cap >= 64 ? (int64_t)c->stage.cap - 64 : 0;
