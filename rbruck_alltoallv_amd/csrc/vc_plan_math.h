@@ -280,9 +280,9 @@ VC_HD VcDesc vc_entry_desc(const VcSched &S, const VcTables &T, const int64_t *s
     return d;
 }
 
-// Blocks are copied in pieces of at most VC_CHUNK bytes, one workgroup each.  Pieces are cut where the DESTINATION
-// address is a multiple of 16, so that only the first piece of a block has a byte-wise head and only the last one a
-// tail; every piece in between is whole aligned vectors.
+// Blocks are copied in pieces of at most VC_CHUNK bytes, one work item (a workgroup, a wavefront or a quarter of one)
+// each.  Pieces are cut where the DESTINATION address is a multiple of the cache line, so that only the first piece of
+// a block has a byte-wise head and only the last one a tail; every piece in between is whole aligned vectors.
 
 // Cache-line phase of the destination address of an entry's copy.  Staging slots and organized runs are laid out at
 // the phase of the block's final address, so this holds whichever arena the copy writes to.
@@ -299,7 +299,7 @@ VC_HD int vc_entry_cut(const VcSched &S, const VcTables &T, const VcEntry &e) {
 
 // A copy that fits one work item (VC_CHUNK bytes from the cache-line boundary below its destination) stays whole; a
 // longer one is cut into pieces of at most VC_PIECE bytes, the size at which a plain copy runs fastest on this chip
-// (one vector per lane).  Only the first piece has a byte-wise head and only the last one a tail.
+// (one vector per lane of a 256-lane workgroup).  Only the first piece has a byte-wise head and only the last one a tail.
 // The copy kernel's window starts at the cache-line boundary at or below the destination: `phase` bytes before it.
 VC_HD bool vc_fits_one_item(int64_t len, int phase) { return len + phase <= VC_CHUNK; }
 
