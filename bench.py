@@ -34,7 +34,9 @@ HBM_PEAK_GBPS = 8000.0
 # execution, profiles/vc_copy_items_kernel_C4_pmc_fetch_write.txt for one launch per digit); counters cannot be read
 # from inside this process, so workloads that were not profiled report null.  Forwarded execution reads every block
 # once and writes it once per hop, so its traffic is below the algorithmic bytes (one read + one write per hop).
-MEASURED_TRAFFIC_PER_LAUNCH = {("C4", "TTPL_BT_alltoallv", 1): 12781523483, ("C4", "TTPL_BT_alltoallv", 0): 8408821395}
+MEASURED_TRAFFIC_PER_LAUNCH = {("C4", "TTPL_BT_alltoallv", 1): 12781523483, ("C4", "TTPL_BT_alltoallv", 0): 8408821395,
+                               ("C5", "tuna_algorithm", 1): 43081601593, ("C3", "twophase_rbruck_alltoallv", 1): 740439781,
+                               ("ML1024", "twophase_rbruck_alltoallv", 1): 35370126039}
 METRIC = "effective alltoallv GB/s + % HBM peak, P=64..1024 virtual ranks, 1 GPU"
 
 
