@@ -379,7 +379,7 @@ def main() -> None:
                                 "hbm_frac": round(2 * S / comp_s / 1e9 / HBM_PEAK_GBPS, 4), "mismatched_bytes": int(comp_bad)},
         "roofline": {"bound": "hbm", "kernel": kernel_name(st), "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
                      "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
-                     "traffic": MEASURED_TRAFFIC_PER_LAUNCH.get((args.workload, func, int(bool(args.forward)))),
+                     "traffic": None if args.radix or args.seed else MEASURED_TRAFFIC_PER_LAUNCH.get((args.workload, func, int(bool(args.forward)))),
                      "avg_launch_ms": round(kern_ms / max(nkern, 1), 4),
                      "algorithmic_bytes_per_launch": int(kern_bytes / max(nkern, 1)),
                      "per_launch": None if per_launch_ms is None else [
