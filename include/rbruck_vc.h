@@ -198,7 +198,9 @@ typedef struct vc_plan *vc_plan_t;
 
 /* `function` is the name of one of the alltoallv-shaped entry points above ("twophase_rbruck_alltoallv", "tuna_algorithm",
  * "TTPL_BT_alltoallv", "spreadout_alltoallv", ...); n, r and batch (b / bblock) are that function's tunables, ignored where
- * it has none.  The tables are read now and not needed afterwards; the communicator's bases are read now too.
+ * it has none; for "uniform_spreadout_twolayer" and "uniform_inverse_isplit_r_bruck" batch is the block length in elements
+ * and the four tables are implied (pass NULL).  The tables are read now and not needed afterwards; the communicator's
+ * bases are read now too.
  * recvbuf_low_bits = (address of the recvbuf that will be passed) & 4095: the low 7 bits must match at execution, the
  * rest only decides where long copies are cut.  Same return codes as the function itself. */
 int vc_plan_create(const char *function, int n, int r, int batch, int *sendcounts, int *sdispls, int elem_size,

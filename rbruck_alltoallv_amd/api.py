@@ -212,11 +212,12 @@ class Plan:
     """vc_plan_t: a planned (persistent) collective for one set of tables."""
 
     def __init__(self, function: str, p: DeviceProblem, recv: torch.Tensor, n: int = 0, r: int = 2, batch: int = 0):
+        """For the uniform_* functions `batch` is the block length in elements and the tables are implied."""
         self.problem = p
         h = C.c_void_p()
-        rc = p.comm.lib.vc_plan_create(function.encode(), n, r, batch, p.sendcounts.data_ptr(), p.sdispls.data_ptr(), p.esz,
-                                       p.recvcounts.data_ptr(), p.rdispls.data_ptr(), recv.data_ptr() & 4095, p.comm.handle,
-                                       C.byref(h))
+        tables = [None] * 4 if function.startswith("uniform_") else [t.data_ptr() for t in (p.sendcounts, p.sdispls, p.recvcounts, p.rdispls)]
+        rc = p.comm.lib.vc_plan_create(function.encode(), n, r, batch, tables[0], tables[1], p.esz, tables[2], tables[3],
+                                       recv.data_ptr() & 4095, p.comm.handle, C.byref(h))
         self.rc = rc
         self.handle = h if rc == 0 else None
 

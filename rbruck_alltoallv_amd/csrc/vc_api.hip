@@ -665,7 +665,8 @@ static bool func_by_name(const char *name, VcFunc &f) {
         {"TTPL_BT_alltoallv", VC_F_TTPL}, {"TTPL_BT_alltoallv_s1", VC_F_TTPL_S1}, {"TTPL_rbruck_alltoallv", VC_F_TTPL_RBRUCK},
         {"twolayer_communicator_linear", VC_F_TWOLAYER_LINEAR}, {"spreadout_alltoallv", VC_F_SPREADOUT},
         {"MPICH_intra_scattered", VC_F_MPICH_SCATTERED}, {"ompi_alltoallv_intra_basic_linear", VC_F_OMPI_LINEAR},
-        {"ompi_alltoallv_intra_pairwise", VC_F_OMPI_PAIRWISE}, {"exclisive_or_alltoallv", VC_F_XOR}};
+        {"ompi_alltoallv_intra_pairwise", VC_F_OMPI_PAIRWISE}, {"exclisive_or_alltoallv", VC_F_XOR},
+        {"uniform_spreadout_twolayer", VC_F_UNIFORM_SPREADOUT}, {"uniform_inverse_isplit_r_bruck", VC_F_UNIFORM_ISPLIT}};
     for (const auto &e : table)
         if (strcmp(name, e.name) == 0) { f = e.f; return true; }
     return false;
@@ -678,12 +679,22 @@ extern "C" int vc_plan_create(const char *function, int n, int r, int batch, int
     if (!c->sbase || !c->rbase) return fail_arg("vc_comm_set_bases has not been called");
     VcFunc f;
     if (!func_by_name(function, f)) return fail_arg("vc_plan_create: unknown function name");
-    if (!sendcounts || !sdispls || !recvcounts || (f != VC_F_TTPL && !rdispls)) return fail_arg("null table");
+    const bool uniform = f == VC_F_UNIFORM_SPREADOUT || f == VC_F_UNIFORM_ISPLIT;      // `batch` is the block length, tables implied
+    if (!uniform && (!sendcounts || !sdispls || !recvcounts || (f != VC_F_TTPL && !rdispls))) return fail_arg("null table");
+    if (uniform && (batch < 0 || (int64_t)batch * c->P > 0x7FFFFFFF)) return fail_arg("block length * P must fit the reference's int displacements");
     VcSched S;
     std::vector<VcLaunchInfo> L;
     const bool forward = c->forward != 0;
-    int rc = vc_make_schedule(f, c->P, n, r, batch, elem_size, 0, S, L, 0, forward);
+    int rc = vc_make_schedule(f, c->P, n, r, uniform ? 0 : batch, elem_size, uniform ? batch : 0, S, L, 0, forward);
     if (rc) return schedule_error(rc);
+    if (uniform) {
+        const size_t PP = (size_t)c->P * c->P;
+        HIP_TRY(c->uni_counts.reserve(sizeof(int) * PP));
+        HIP_TRY(c->uni_displs.reserve(sizeof(int) * PP));
+        HIP_TRY(vc_launch_uniform_tables(c->uni_counts.as<int>(), c->uni_displs.as<int>(), batch, c->P, c->stream));
+        sendcounts = recvcounts = c->uni_counts.as<int>();
+        sdispls = rdispls = c->uni_displs.as<int>();
+    }
     S.recv_lo = recvbuf_low_bits & 4095;
     vc_plan *p = new vc_plan();
     p->comm = c;

@@ -433,6 +433,29 @@ def test_benchmark_shapes_at_reduced_size(api):
         ("uniform isplit n=32 r=3", lambda d: api.uniform_inverse_isplit_r_bruck(32, 3, 2, dp, 300, ds, d), False)])
 
 
+def test_persistent_plans_of_the_uniform_functions(api):
+    """vc_plan_create for the equal-block functions: the block length travels as `batch`, the tables are implied."""
+    up = W.make_uniform_problem(96, 700, 2)
+    dp = api.DeviceProblem(up)
+    ds = dp.new_send_arena()
+    dp.fill_payload(0, 8, ds)
+    for function, n, r, direct in (("uniform_spreadout_twolayer", 8, 3, lambda d: api.uniform_spreadout_twolayer(8, 3, dp, 700, ds, d)),
+                                   ("uniform_inverse_isplit_r_bruck", 12, 2, lambda d: api.uniform_inverse_isplit_r_bruck(12, 2, 2, dp, 700, ds, d))):
+        want = dp.new_recv_arena(0xEE)
+        assert direct(want) == 0, dp.comm.error()
+        assert dp.verify(ds, want) == 0
+        got = dp.new_recv_arena(0xEE)
+        plan = api.Plan(function, dp, got, n=n, r=r, batch=700)
+        assert plan.rc == 0, dp.comm.error()
+        for _ in range(2):
+            got.fill_(0xEE)
+            assert plan.execute(ds, got) == 0, dp.comm.error()
+            assert bool((got == want).all()), function
+        plan.free()
+    assert api.Plan("uniform_spreadout_twolayer", dp, want, n=7, r=2, batch=700).rc == -2       # 7 does not divide 96
+    dp.comm.free()
+
+
 def _transposed(prob):
     """The alltoallv that undoes `prob`: every rank sends back what it received, from where it landed."""
     import dataclasses
