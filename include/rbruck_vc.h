@@ -43,6 +43,7 @@ typedef struct vc_comm *vc_comm_t;
 #define VC_ERR_TABLES (-7)     /* a negative count or displacement in the tables (found on the device before anything is copied) */
 #define VC_ERR_OVERFLOW (-8)   /* vc_displs_from_counts: a rank's counts sum past INT_MAX elements, where the reference's int
                                   displacements wrap (examples/rbruckv_example.cpp:69-72) */
+#define VC_ERR_SCRATCH (-9)    /* twophase_rbruck_alltoallv_noalloc: the call needs more than VC_NOALLOC_SCRATCH_BYTES */
 
 /* ---- communicator (replaces MPI_Comm; MPI_Comm_size/MPI_Comm_rank have no per-rank analogue) ---- */
 
@@ -188,6 +189,19 @@ int twolayer_communicator_linear_s2(int n, int bblock1, int bblock2, char *sendb
 /* benchmarks/common.cpp:10-37 (declared in src/rbruckv.h:88-89; returns void there). */
 int spreadout_alltoallv(char *sendbuf, int *sendcounts, int *sdispls, int sendtype_size, char *recvbuf,
                         int *recvcounts, int *rdispls, int recvtype_size, vc_comm_t comm);
+
+/* No counterpart in the reference.  twophase_rbruck_alltoallv for callers that cannot allocate device memory: code whose
+ * surroundings are under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  Same arguments, same
+ * result (byte for byte) as twophase_rbruck_alltoallv in its forwarded execution, but the plan tables and the staging
+ * arena are slices of one static device array of VC_NOALLOC_SCRATCH_BYTES that each GPU holds for the life of the
+ * process: the call performs no hipMalloc / hipFree and creates no events or streams.  A call whose plan tables
+ * (about 8 * P * P * (digits + 1) bytes) plus staging (the bytes of all blocks that make more than one hop, once per
+ * intermediate hop, each rounded up to 128) exceed the array returns VC_ERR_SCRATCH and leaves recvbuf untouched.  All
+ * calls on one GPU share that GPU's array: calls that overlap on one GPU (two host threads, two streams) race.
+ * Blocking; vc_comm_set_timing has no effect on it. */
+#define VC_NOALLOC_SCRATCH_BYTES (64u << 20)
+int twophase_rbruck_alltoallv_noalloc(int r, char *sendbuf, int *sendcounts, int *sdispls, int sendtype_size, char *recvbuf,
+                                      int *recvcounts, int *rdispls, int recvtype_size, vc_comm_t comm);
 
 /* ---- persistent plans: the analogue of MPI-4 persistent collectives (MPI_Alltoallv_init / MPI_Start).
  * The reference re-exchanges its metadata in every call (src/twophase_tunable_rbruckv.cpp:110); when the same tables are

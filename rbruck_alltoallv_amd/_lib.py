@@ -10,7 +10,8 @@ LIB_PATH = os.path.join(PKG_DIR, "librbruck_vc.so")
 VC_MAX_LAUNCHES = 1024
 
 VC_OK, VC_ERR_RADIX, VC_ERR_GROUP, VC_ERR_TOO_FEW_RANKS, VC_ERR_HIP, VC_ERR_ARG, VC_ERR_NO_DEVICE = 0, -1, -2, -3, -4, -5, -6
-VC_ERR_TABLES, VC_ERR_OVERFLOW = -7, -8
+VC_ERR_TABLES, VC_ERR_OVERFLOW, VC_ERR_SCRATCH = -7, -8, -9
+VC_NOALLOC_SCRATCH_BYTES = 64 << 20
 
 
 class VcStats(C.Structure):
@@ -38,6 +39,7 @@ SYMBOLS = {
     "vc_allreduce_max_count": (_I, [_P, _P, _P]),
     "twophase_rbruck_alltoallv": (_I, [_I] + _V_TAIL),
     "twophase_rbruck_alltoallv_om": (_I, [_I] + _V_TAIL),
+    "twophase_rbruck_alltoallv_noalloc": (_I, [_I] + _V_TAIL),
     "tuna_algorithm": (_I, [_I, _I] + _V_TAIL),
     "tuna2_algorithm": (_I, [_I, _I] + _V_TAIL),
     "TTPL_BT_alltoallv": (_I, [_I, _I, _I] + _V_TAIL),

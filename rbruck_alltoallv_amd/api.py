@@ -141,6 +141,11 @@ def twophase_rbruck_alltoallv(r: int, p: DeviceProblem, send: torch.Tensor, recv
     return p.comm.lib.twophase_rbruck_alltoallv(r, *_tail(p, send, recv))
 
 
+def twophase_rbruck_alltoallv_noalloc(r: int, p: DeviceProblem, send: torch.Tensor, recv: torch.Tensor) -> int:
+    """twophase_rbruck_alltoallv out of the library's static device scratch array: allocates nothing."""
+    return p.comm.lib.twophase_rbruck_alltoallv_noalloc(r, *_tail(p, send, recv))
+
+
 def twophase_rbruck_alltoallv_om(r: int, p: DeviceProblem, send: torch.Tensor, recv: torch.Tensor) -> int:
     """src/twophase_tunable_rbruckv-om.cpp:10-157"""
     return p.comm.lib.twophase_rbruck_alltoallv_om(r, *_tail(p, send, recv))

@@ -23,6 +23,14 @@
 
 static thread_local std::string g_last_error;
 
+// Device memory of the entry point that allocates nothing (twophase_rbruck_alltoallv_noalloc): its plan tables and its
+// staging arena are slices of this array.  Every GPU the library runs on holds its own copy, at its own address, until
+// the process ends; `scratch` itself is only the host-side name of the symbol and never a device address: host code
+// uses the pointer hipGetSymbolAddress returned for the device, resolved once per device in vc_comm_create.
+static __device__ __align__(256) unsigned char scratch[VC_NOALLOC_SCRATCH_BYTES];
+#define VC_MAX_DEVICES 64
+static unsigned char *g_scratch_ptr[VC_MAX_DEVICES];       // per device: where its copy of `scratch` lives (null: not resolved)
+
 static int fail_hip(hipError_t e, const char *what, int line) {
     char buf[256];
     snprintf(buf, sizeof buf, "%s failed at vc_api.hip:%d: %s", what, line, hipGetErrorString(e));
@@ -76,6 +84,15 @@ struct DevBuf {
     template <class T> T *as() const { return static_cast<T *>(p); }
 };
 
+// Device buffers a call plans into: the communicator's grow-only allocations, or slices of memory the caller of the
+// planning functions carved elsewhere.
+struct PlanBufs {
+    int64_t *slot_off = nullptr, *row_tot = nullptr, *row_base = nullptr, *org_run_base = nullptr, *item_row_tot = nullptr,
+            *item_row_base = nullptr, *row_bytes = nullptr, *chain_row_tot = nullptr, *chain_row_base = nullptr, *header = nullptr;
+    VcLaunchInfo *launches = nullptr;
+    int *rd_packed = nullptr;
+};
+
 struct vc_comm {
     int P = 0;
     int device = 0;
@@ -90,6 +107,8 @@ struct vc_comm {
     DevBuf chain_row_tot, chain_row_base;
     DevBuf slot_off, row_tot, row_base, org_run_base, item_row_tot, item_row_base, row_bytes, desc, header, launches, stage, rd_packed,
         uni_counts, uni_displs, scratch;
+    PlanBufs B;                           // where the current call's plan lives
+    const void *last_stage = nullptr;     // staging arena of the last call
     int64_t *h_header = nullptr;          // pinned, coherent: the planner writes its header straight into it
     int64_t *h_header_dev = nullptr;      // the same memory as the device sees it
     VcLaunchInfo *h_launches = nullptr;   // pinned
@@ -111,6 +130,11 @@ extern "C" int vc_comm_create(int nranks, vc_comm_t *comm_out) {
     c->P = nranks;
     memset(&c->stats, 0, sizeof c->stats);
     hipError_t e = hipGetDevice(&c->device);
+    if (e == hipSuccess && c->device >= 0 && c->device < VC_MAX_DEVICES && !g_scratch_ptr[c->device]) {
+        void *ptr = nullptr;                              // this device's copy of the static scratch array
+        e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        if (e == hipSuccess) g_scratch_ptr[c->device] = static_cast<unsigned char *>(ptr);
+    }
     if (e == hipSuccess) e = hipHostMalloc((void **)&c->h_header, sizeof(int64_t) * VC_HEADER_WORDS(VC_MAX_LAUNCHES), hipHostMallocCoherent);
     if (e == hipSuccess) e = hipHostGetDevicePointer((void **)&c->h_header_dev, c->h_header, 0);
     if (e == hipSuccess) e = hipHostMalloc((void **)&c->h_launches, sizeof(VcLaunchInfo) * VC_MAX_LAUNCHES, hipHostMallocDefault);
@@ -233,47 +257,85 @@ struct PlanInfo {
     bool listless = false;                          // forwarded execution that went without the item list
 };
 
-// Step 3a: enqueues the planning kernels that size everything (staging prefix sums, item counts, table check); their
-// result lands in the pinned header.
-static int plan_sizes(vc_comm *c, const VcSched &S, std::vector<VcLaunchInfo> &L, VcTables &T, bool forward) {
+static int plan_sizes(vc_comm *c, const VcSched &S, std::vector<VcLaunchInfo> &L, VcTables &T, bool forward);
+
+// Sizes (bytes) of the plan buffers of a call, in the order of PlanBufs' members.
+struct PlanBufSizes { size_t slot_off, row_tot, row_base, org_run_base, item_row_tot, item_row_base, row_bytes, chain_row_tot, chain_row_base, header, launches, rd_packed; };
+
+static PlanBufSizes plan_buf_sizes(const VcSched &S, int nl, bool forward) {
+    const size_t P = (size_t)S.P, PP = P * P;
+    const size_t wmax = (size_t)std::max(vc_regions(S), 1) + 1;      // staging regions
+    PlanBufSizes z;
+    z.slot_off = sizeof(int64_t) * PP * wmax;
+    z.row_tot = z.row_base = sizeof(int64_t) * P * wmax;
+    z.org_run_base = sizeof(int64_t) * P * (size_t)std::max(S.G, 1);
+    z.item_row_tot = z.item_row_base = sizeof(int64_t) * P * (size_t)std::max(nl, 1);
+    z.row_bytes = sizeof(int64_t) * P * (size_t)(std::max(nl, S.w + S.w2) + 2);
+    z.chain_row_tot = forward ? sizeof(int64_t) * (2 + (P + VC_THREADS - 1) / VC_THREADS) * P : 0;
+    z.chain_row_base = forward ? sizeof(int64_t) * P : 0;
+    z.header = sizeof(int64_t) * VC_HEADER_WORDS(VC_MAX_LAUNCHES);
+    z.launches = sizeof(VcLaunchInfo) * VC_MAX_LAUNCHES;
+    z.rd_packed = S.packed_recv ? sizeof(int) * PP : 0;
+    return z;
+}
+
+// The communicator's own buffers, grown to what the call needs.
+static int reserve_plan_bufs(vc_comm *c, const VcSched &S, int nl, bool forward) {
+    const PlanBufSizes z = plan_buf_sizes(S, nl, forward);
+    HIP_TRY(c->slot_off.reserve(z.slot_off));
+    HIP_TRY(c->row_tot.reserve(z.row_tot));
+    HIP_TRY(c->row_base.reserve(z.row_base));
+    HIP_TRY(c->org_run_base.reserve(z.org_run_base));
+    HIP_TRY(c->item_row_tot.reserve(z.item_row_tot));
+    HIP_TRY(c->item_row_base.reserve(z.item_row_base));
+    HIP_TRY(c->row_bytes.reserve(z.row_bytes));
+    HIP_TRY(c->header.reserve(z.header));
+    HIP_TRY(c->launches.reserve(z.launches));
+    if (forward) {
+        HIP_TRY(c->chain_row_tot.reserve(z.chain_row_tot));
+        HIP_TRY(c->chain_row_base.reserve(z.chain_row_base));
+    }
+    if (S.packed_recv) HIP_TRY(c->rd_packed.reserve(z.rd_packed));
+    PlanBufs &B = c->B;
+    B.slot_off = c->slot_off.as<int64_t>(); B.row_tot = c->row_tot.as<int64_t>(); B.row_base = c->row_base.as<int64_t>();
+    B.org_run_base = c->org_run_base.as<int64_t>(); B.item_row_tot = c->item_row_tot.as<int64_t>();
+    B.item_row_base = c->item_row_base.as<int64_t>(); B.row_bytes = c->row_bytes.as<int64_t>();
+    B.chain_row_tot = forward ? c->chain_row_tot.as<int64_t>() : nullptr;
+    B.chain_row_base = forward ? c->chain_row_base.as<int64_t>() : nullptr;
+    B.header = c->header.as<int64_t>(); B.launches = c->launches.as<VcLaunchInfo>(); B.rd_packed = c->rd_packed.as<int>();
+    return VC_OK;
+}
+
+// Step 3a: enqueues the planning kernels that size everything (staging prefix sums, item counts, table check) into the
+// buffers c->B names; their result lands in the pinned header.
+static int enqueue_plan_sizes(vc_comm *c, const VcSched &S, std::vector<VcLaunchInfo> &L, VcTables &T, bool forward, bool timing) {
     const int P = S.P;
     const int nl = (int)L.size();
-    if (nl > VC_MAX_LAUNCHES) return fail_arg("more than VC_MAX_LAUNCHES launches: raise b / bblock");
     hipStream_t st = c->stream;
-    const size_t PP = (size_t)P * P;
-    const size_t wmax = (size_t)std::max(vc_regions(S), 1) + 1;      // staging regions
-
-    HIP_TRY(c->slot_off.reserve(sizeof(int64_t) * PP * wmax));
-    HIP_TRY(c->row_tot.reserve(sizeof(int64_t) * (size_t)P * wmax));
-    HIP_TRY(c->row_base.reserve(sizeof(int64_t) * (size_t)P * wmax));
-    HIP_TRY(c->org_run_base.reserve(sizeof(int64_t) * (size_t)P * std::max(S.G, 1)));
-    HIP_TRY(c->item_row_tot.reserve(sizeof(int64_t) * (size_t)P * nl));
-    HIP_TRY(c->item_row_base.reserve(sizeof(int64_t) * (size_t)P * nl));
-    HIP_TRY(c->row_bytes.reserve(sizeof(int64_t) * (size_t)P * (std::max(nl, S.w + S.w2) + 2)));
-    HIP_TRY(c->header.reserve(sizeof(int64_t) * VC_HEADER_WORDS(VC_MAX_LAUNCHES)));
-    HIP_TRY(c->launches.reserve(sizeof(VcLaunchInfo) * VC_MAX_LAUNCHES));
-    if (forward) {
-        if (vc_hop_slots(S) > VC_MAX_HOP_SLOTS) return fail_arg("too many digits for forwarded execution");
-        HIP_TRY(c->chain_row_tot.reserve(sizeof(int64_t) * (2 + (size_t)(P + VC_THREADS - 1) / VC_THREADS) * (size_t)P));
-        HIP_TRY(c->chain_row_base.reserve(sizeof(int64_t) * (size_t)P));
-    }
-    if (c->timing) { int rc = ensure_events(c, (size_t)nl + 4); if (rc) return rc; }
-
-    if (c->timing) HIP_TRY(hipEventRecord(c->events[0], st));
+    const PlanBufs &B = c->B;
+    if (timing) HIP_TRY(hipEventRecord(c->events[0], st));
     if (!forward && nl > VC_LAUNCH_PACK) {                 // a short launch table travels as a kernel argument instead
         memcpy(c->h_launches, L.data(), sizeof(VcLaunchInfo) * nl);
-        HIP_TRY(hipMemcpyAsync(c->launches.p, c->h_launches, sizeof(VcLaunchInfo) * nl, hipMemcpyHostToDevice, st));
+        HIP_TRY(hipMemcpyAsync(B.launches, c->h_launches, sizeof(VcLaunchInfo) * nl, hipMemcpyHostToDevice, st));
     }
     if (S.packed_recv) {
-        HIP_TRY(c->rd_packed.reserve(sizeof(int) * PP));
-        HIP_TRY(vc_launch_row_scan(T.rc, c->rd_packed.as<int>(), nullptr, nullptr, P, st));
-        T.rd_packed = c->rd_packed.as<int>();
+        HIP_TRY(vc_launch_row_scan(T.rc, B.rd_packed, nullptr, nullptr, P, st));
+        T.rd_packed = B.rd_packed;
     }
-    HIP_TRY(vc_launch_plan_sizes(S, L.data(), c->launches.as<VcLaunchInfo>(), nl, T, c->slot_off.as<int64_t>(), c->row_tot.as<int64_t>(),
-                                 c->row_base.as<int64_t>(), c->org_run_base.as<int64_t>(), c->item_row_tot.as<int64_t>(),
-                                 c->item_row_base.as<int64_t>(), c->row_bytes.as<int64_t>(), forward ? c->chain_row_tot.as<int64_t>() : nullptr,
-                                 forward ? c->chain_row_base.as<int64_t>() : nullptr, c->header.as<int64_t>(), c->h_header_dev, st));
+    HIP_TRY(vc_launch_plan_sizes(S, L.data(), B.launches, nl, T, B.slot_off, B.row_tot, B.row_base, B.org_run_base, B.item_row_tot,
+                                 B.item_row_base, B.row_bytes, forward ? B.chain_row_tot : nullptr,
+                                 forward ? B.chain_row_base : nullptr, B.header, c->h_header_dev, st));
     return VC_OK;
+}
+
+static int plan_sizes(vc_comm *c, const VcSched &S, std::vector<VcLaunchInfo> &L, VcTables &T, bool forward) {
+    const int nl = (int)L.size();
+    if (nl > VC_MAX_LAUNCHES) return fail_arg("more than VC_MAX_LAUNCHES launches: raise b / bblock");
+    if (forward && vc_hop_slots(S) > VC_MAX_HOP_SLOTS) return fail_arg("too many digits for forwarded execution");
+    int rc = reserve_plan_bufs(c, S, nl, forward);
+    if (rc) return rc;
+    if (c->timing) { rc = ensure_events(c, (size_t)nl + 4); if (rc) return rc; }
+    return enqueue_plan_sizes(c, S, L, T, forward, c->timing);
 }
 
 // Lanes per work item, from the average piece of the list.  Short pieces leave most of a workgroup idle, and what bounds
@@ -324,12 +386,12 @@ static int plan_emit(vc_comm *c, const VcSched &S, std::vector<VcLaunchInfo> &L,
     hipStream_t st = c->stream;
     if (pi.chain) {
         HIP_TRY(items.reserve(sizeof(int64_t) * (size_t)pi.chain_stride * (size_t)std::max<int64_t>(pi.chain_items, 1)));
-        HIP_TRY(vc_launch_chain_plan(S, T, c->slot_off.as<int64_t>(), c->row_base.as<int64_t>(), c->chain_row_base.as<int64_t>(),
-                                     c->chain_row_tot.as<int64_t>() + 2 * (size_t)S.P, items.as<int64_t>(), pi.chain_items, st));
+        HIP_TRY(vc_launch_chain_plan(S, T, c->B.slot_off, c->B.row_base, c->B.chain_row_base, c->B.chain_row_tot + 2 * (size_t)S.P,
+                                     items.as<int64_t>(), pi.chain_items, st));
     } else {
         HIP_TRY(items.reserve(sizeof(VcDesc) * (size_t)std::max<int64_t>(pi.items_total, 1)));
-        HIP_TRY(vc_launch_plan_emit(S, L.data(), c->launches.as<VcLaunchInfo>(), pi.nl, T, c->slot_off.as<int64_t>(), c->row_base.as<int64_t>(),
-                                    c->item_row_base.as<int64_t>(), c->header.as<int64_t>(), items.as<VcDesc>(), pi.items_total, st));
+        HIP_TRY(vc_launch_plan_emit(S, L.data(), c->B.launches, pi.nl, T, c->B.slot_off, c->B.row_base, c->B.item_row_base, c->B.header,
+                                    items.as<VcDesc>(), pi.items_total, st));
     }
     if (c->timing) HIP_TRY(hipEventRecord(c->events[1], st));
     return VC_OK;
@@ -401,6 +463,7 @@ static int finish_stats(vc_comm *c, const PlanInfo &pi, const void *items_any, b
     }
     c->last_nlaunch = pi.chain ? 0 : nl;              // per-launch traffic can only be inspected after launch-per-digit execution
     c->last_items = static_cast<const VcDesc *>(items_any);
+    c->last_stage = c->stage.p;
     return VC_OK;
 }
 
@@ -465,8 +528,8 @@ static int run_schedule(vc_comm *c, VcSched S, std::vector<VcLaunchInfo> &L, con
                 if (attempt == 0) HIP_TRY(hipEventRecord(c->events[1], st));
                 HIP_TRY(hipEventRecord(c->events[2], st));
             }
-            HIP_TRY(vc_launch_copy_blocks(S, T, c->slot_off.as<int64_t>(), c->row_base.as<int64_t>(), c->header.as<int64_t>(), guard,
-                                          pair_lanes, sendbuf, recvbuf, c->stage.as<char>(), st));
+            HIP_TRY(vc_launch_copy_blocks(S, T, c->B.slot_off, c->B.row_base, c->B.header, guard, pair_lanes, sendbuf, recvbuf,
+                                          c->stage.as<char>(), st));
             if (c->timing) HIP_TRY(hipEventRecord(c->events[3], st));
             HIP_TRY(hipStreamSynchronize(st));
             synced = true;
@@ -570,6 +633,82 @@ extern "C" int TTPL_rbruck_alltoallv(int n, int r, char *sendbuf, int *sendcount
                                      int *recvcounts, int *rdispls, int recvtype_size, vc_comm_t c) {
     (void)recvtype_size;
     return run_v(VC_F_TTPL_RBRUCK, n, r, 0, c, sendbuf, sendcounts, sdispls, sendtype_size, recvbuf, recvcounts, rdispls);
+}
+
+// ---- the entry point that allocates nothing ----
+// twophase_rbruck_alltoallv for callers that cannot allocate (code under HIP graph capture of its surroundings, tight
+// serving loops, harnesses that forbid hipMalloc): the same schedule, planning kernels and copy kernel as the forwarded,
+// listless execution of twophase_rbruck_alltoallv, with the plan tables and the staging arena carved out of the static
+// device array `scratch` instead of the communicator's grow-only buffers.  No hipMalloc, hipFree, event or stream
+// creation happens here; the pinned header the planner reports through was allocated by vc_comm_create.  Every call on
+// a GPU uses that GPU's one array, so calls that overlap on one GPU race.  Nothing in the array needs to start at
+// zero: the planning kernels overwrite every word they or the copy kernel later read.
+static size_t carve(size_t &at, size_t bytes) {
+    const size_t here = at;
+    at += (bytes + 255) & ~(size_t)255;
+    return here;
+}
+
+extern "C" int twophase_rbruck_alltoallv_noalloc(int r, char *sendbuf, int *sendcounts, int *sdispls, int sendtype_size, char *recvbuf,
+                                                 int *recvcounts, int *rdispls, int recvtype_size, vc_comm_t c) {
+    (void)recvtype_size;
+    int rc = check_common(c, sendbuf, recvbuf, sendtype_size);
+    if (rc) return rc;
+    if (!sendcounts || !sdispls || !recvcounts || !rdispls) return fail_arg("null table");
+    unsigned char *base = c->device < VC_MAX_DEVICES ? g_scratch_ptr[c->device] : nullptr;
+    if (!base) return fail_arg("the static scratch array was not resolved on this device", VC_ERR_HIP);
+    VcSched S;
+    std::vector<VcLaunchInfo> L;
+    rc = vc_make_schedule(VC_F_TWOPHASE, c->P, 0, r, 0, sendtype_size, 0, S, L, 0, true);
+    if (rc) return schedule_error(rc);
+    if (vc_hop_slots(S) > VC_MAX_HOP_SLOTS) return fail_arg("too many digits for forwarded execution");
+    S.recv_lo = (int)((uintptr_t)recvbuf & 4095);
+    // slices of the scratch array: plan tables first, the rest is the staging arena
+    const PlanBufSizes z = plan_buf_sizes(S, 1, true);
+    size_t at = 0;
+    PlanBufs &B = c->B;
+    B = PlanBufs();
+    B.header = reinterpret_cast<int64_t *>(base + carve(at, z.header));
+    B.slot_off = reinterpret_cast<int64_t *>(base + carve(at, z.slot_off));
+    B.row_tot = reinterpret_cast<int64_t *>(base + carve(at, z.row_tot));
+    B.row_base = reinterpret_cast<int64_t *>(base + carve(at, z.row_base));
+    B.row_bytes = reinterpret_cast<int64_t *>(base + carve(at, z.row_bytes));
+    B.chain_row_tot = reinterpret_cast<int64_t *>(base + carve(at, z.chain_row_tot));
+    B.chain_row_base = reinterpret_cast<int64_t *>(base + carve(at, z.chain_row_base));
+    if (at + 64 > (size_t)VC_NOALLOC_SCRATCH_BYTES) {
+        char msg[200];
+        snprintf(msg, sizeof msg, "twophase_rbruck_alltoallv_noalloc: the plan tables of %d ranks with radix %d need %zu bytes, the static "
+                 "scratch array has %zu", c->P, S.r, at, (size_t)VC_NOALLOC_SCRATCH_BYTES);
+        return fail_arg(msg, VC_ERR_SCRATCH);
+    }
+    char *stage = reinterpret_cast<char *>(base + at);
+    VcListlessGuard guard = {(int64_t)((size_t)VC_NOALLOC_SCRATCH_BYTES - at - 64), 0, 0, 0};
+    VcTables T = make_tables(c, sendcounts, sdispls, recvcounts, rdispls);
+    rc = enqueue_plan_sizes(c, S, L, T, true, false);
+    if (rc) return rc;
+    // a quarter of a wavefront per pair of ranks after a call of short blocks on this communicator, else a workgroup
+    const bool quarter = c->hint_valid && c->hint_max_pieces <= VC_LISTLESS_MAX_PIECES &&
+                         c->hint_payload / std::max<int64_t>(c->hint_items, 1) < VC_LISTLESS_QUARTER_BELOW;
+    const int lanes = quarter ? VC_QUARTER : VC_THREADS;
+    HIP_TRY(vc_launch_copy_blocks(S, T, B.slot_off, B.row_base, B.header, guard, lanes, sendbuf, recvbuf, stage, c->stream));
+    HIP_TRY(hipStreamSynchronize(c->stream));
+    PlanInfo pi;
+    rc = plan_read(c, S, L, pi, true);
+    if (rc) return rc;
+    if (!vc_listless_ok(c->h_header, guard)) {            // the copy kernel saw the same header and has touched nothing
+        char msg[200];
+        snprintf(msg, sizeof msg, "twophase_rbruck_alltoallv_noalloc: the call needs %lld bytes of staging, the static scratch array "
+                 "has %lld left after the plan tables", (long long)pi.stage_bytes, (long long)guard.stage_cap);
+        return fail_arg(msg, VC_ERR_SCRATCH);
+    }
+    pi.listless = true;
+    pi.chain_lanes = lanes;
+    const bool timing = c->timing;
+    c->timing = false;                                    // no events were recorded
+    rc = finish_stats(c, pi, nullptr, true);
+    c->timing = timing;
+    c->last_stage = stage;
+    return rc;
 }
 
 // The linear comparators (src/MPICH_scattered.cpp, src/OpenMPI_basic_linear.cpp, src/OpenMPI_pairwise.cpp,
@@ -795,7 +934,7 @@ extern "C" int vc_comm_last_traffic(vc_comm_t c, int launch, int64_t *matrix_out
 
 extern "C" int vc_comm_staging(vc_comm_t c, void **ptr_out, int64_t *bytes_out) {
     if (!c || !ptr_out || !bytes_out) return fail_arg("vc_comm_staging: null argument");
-    *ptr_out = c->stage.p;
+    *ptr_out = const_cast<void *>(c->last_stage);
     *bytes_out = c->stats.staging_bytes;
     return VC_OK;
 }
