@@ -40,9 +40,12 @@ typedef struct vc_comm *vc_comm_t;
 #define VC_ERR_HIP (-4)        /* a HIP runtime call failed; vc_last_error_string() says which */
 #define VC_ERR_ARG (-5)        /* null handle / pointer, element size < 1, bases not set */
 #define VC_ERR_NO_DEVICE (-6)  /* no HIP device */
-#define VC_ERR_TABLES (-7)     /* a negative count or displacement in the tables (found on the device before anything is copied) */
-#define VC_ERR_OVERFLOW (-8)   /* vc_displs_from_counts: a rank's counts sum past INT_MAX elements, where the reference's int
-                                  displacements wrap (examples/rbruckv_example.cpp:69-72) */
+#define VC_ERR_TABLES (-7)     /* a negative count or displacement in the tables, or recvcounts[t][s] != sendcounts[s][t] (the reference
+                                  fails with an MPI truncation error); found on the device before anything is copied */
+#define VC_ERR_OVERFLOW (-8)   /* a rank's counts sum past INT_MAX elements, where the reference's int displacements wrap
+                                  (examples/rbruckv_example.cpp:69-72): vc_displs_from_counts, and the packed receive layout of
+                                  TTPL_BT_alltoallv (src/twophase_twolayer_rbruck.cpp:406-418) */
+#define VC_ERR_BUSY (-10)      /* the communicator is serving another call (a second host thread): one call at a time */
 #define VC_ERR_SCRATCH (-9)    /* twophase_rbruck_alltoallv_noalloc: the call needs more than VC_NOALLOC_SCRATCH_BYTES */
 
 /* ---- communicator (replaces MPI_Comm; MPI_Comm_size/MPI_Comm_rank have no per-rank analogue) ---- */
@@ -224,8 +227,9 @@ int vc_plan_create(const char *function, int n, int r, int batch, int *sendcount
 int vc_plan_execute(vc_plan_t plan, char *sendbuf, char *recvbuf);
 /* Only enqueues the copy kernels on the communicator's stream and returns: no synchronisation, no allocation, no
  * host-side bookkeeping — usable while the stream is being captured into a HIP graph.  The staging arena was sized
- * when the plan was created; a later, larger call on the same communicator may move it, after which graphs captured
- * before are stale.  The caller orders later work after it (same stream, or an event). */
+ * when the plan was created and stays where it is for as long as any plan of the communicator exists (a later, larger
+ * call gets a second arena; the outgrown one is released with the last plan), so a graph captured from this call stays
+ * valid until its plan is freed.  The caller orders later work after it (same stream, or an event). */
 int vc_plan_execute_async(vc_plan_t plan, char *sendbuf, char *recvbuf);
 /* Waits for the communicator's stream and releases the plan's work items; before vc_comm_free of its communicator. */
 int vc_plan_free(vc_plan_t plan);

@@ -10,7 +10,7 @@ LIB_PATH = os.path.join(PKG_DIR, "librbruck_vc.so")
 VC_MAX_LAUNCHES = 1024
 
 VC_OK, VC_ERR_RADIX, VC_ERR_GROUP, VC_ERR_TOO_FEW_RANKS, VC_ERR_HIP, VC_ERR_ARG, VC_ERR_NO_DEVICE = 0, -1, -2, -3, -4, -5, -6
-VC_ERR_TABLES, VC_ERR_OVERFLOW, VC_ERR_SCRATCH = -7, -8, -9
+VC_ERR_TABLES, VC_ERR_OVERFLOW, VC_ERR_SCRATCH, VC_ERR_BUSY = -7, -8, -9, -10
 VC_NOALLOC_SCRATCH_BYTES = 64 << 20
 
 

@@ -10,6 +10,7 @@
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
+#include <atomic>
 #include <cstdio>
 #include <cstring>
 #include <string>
@@ -107,6 +108,10 @@ struct vc_comm {
     DevBuf chain_row_tot, chain_row_base;
     DevBuf slot_off, row_tot, row_base, org_run_base, item_row_tot, item_row_base, row_bytes, desc, header, launches, stage, rd_packed,
         uni_counts, uni_displs, scratch;
+    int live_plans = 0;                   // plans created on this communicator and not yet freed
+    std::vector<void *> retired_stage;    // staging arenas that were outgrown while plans existed: a HIP graph captured from
+                                          // vc_plan_execute_async holds the arena's address, so they stay until the plans go
+    std::atomic_flag busy = ATOMIC_FLAG_INIT;   // a call is in progress (a communicator serves one call at a time)
     PlanBufs B;                           // where the current call's plan lives
     const void *last_stage = nullptr;     // staging arena of the last call
     int64_t *h_header = nullptr;          // pinned, coherent: the planner writes its header straight into it
@@ -118,6 +123,35 @@ struct vc_comm {
     int64_t launch_first[VC_MAX_LAUNCHES], launch_items[VC_MAX_LAUNCHES];   // work items of the last call
     const VcDesc *last_items = nullptr;
 };
+
+// Grows the staging arena.  While plans exist the outgrown arena is kept (not freed): graphs captured from their
+// launches write to its address.
+static hipError_t reserve_stage(vc_comm *c, size_t bytes) {
+    if (bytes <= c->stage.cap) return hipSuccess;
+    if (c->live_plans > 0 && c->stage.p) {
+        c->retired_stage.push_back(c->stage.p);
+        c->stage.p = nullptr;
+        c->stage.cap = 0;
+    }
+    return c->stage.reserve(bytes);
+}
+
+static void free_retired_stage(vc_comm *c) {
+    for (void *p : c->retired_stage) (void)hipFree(p);
+    c->retired_stage.clear();
+}
+
+// One call at a time per communicator: a second host thread gets VC_ERR_BUSY instead of a race on the plan buffers.
+struct BusyGuard {
+    vc_comm *c;
+    bool mine;
+    explicit BusyGuard(vc_comm *comm) : c(comm), mine(comm && !comm->busy.test_and_set(std::memory_order_acquire)) {}
+    ~BusyGuard() { if (mine) c->busy.clear(std::memory_order_release); }
+    bool ok() const { return !c || mine; }
+};
+#define VC_ONE_CALL(c)                                                                                              \
+    BusyGuard busy_guard_(c);                                                                                       \
+    if (!busy_guard_.ok()) return fail_arg("the communicator is serving another call (one call at a time)", VC_ERR_BUSY)
 
 // ------------------------------------------------------------------ communicator
 
@@ -152,6 +186,7 @@ extern "C" int vc_comm_free(vc_comm_t c) {
     for (DevBuf *b : {&c->slot_off, &c->row_tot, &c->row_base, &c->org_run_base, &c->item_row_tot, &c->item_row_base, &c->row_bytes, &c->desc, &c->header, &c->launches, &c->stage, &c->rd_packed,
                       &c->uni_counts, &c->uni_displs, &c->scratch, &c->chain_row_tot, &c->chain_row_base})
         b->release();
+    free_retired_stage(c);
     for (hipEvent_t e : c->events) (void)hipEventDestroy(e);
     if (c->h_header) (void)hipHostFree(c->h_header);
     if (c->h_launches) (void)hipHostFree(c->h_launches);
@@ -354,8 +389,12 @@ static int lanes_for(int64_t bytes, int64_t items) {
 static int plan_read(vc_comm *c, const VcSched &S, const std::vector<VcLaunchInfo> &L, PlanInfo &out, bool forward) {
     const int nl = forward ? 1 : (int)L.size();           // forwarded execution: one launch, one set of totals
     const int64_t *h = c->h_header;
+    if (h[VC_HEADER_BAD] >= VC_BAD_OVERFLOW)
+        return fail_arg("a rank receives more than INT_MAX elements: the packed receive displacements of TTPL_BT_alltoallv do not fit an int",
+                        VC_ERR_OVERFLOW);
     if (h[VC_HEADER_BAD] != 0)    // such tables would send the copy kernels outside the arenas
-        return fail_arg("negative entries in sendcounts / sdispls / recvcounts / rdispls", VC_ERR_TABLES);
+        return fail_arg("sendcounts / sdispls / recvcounts / rdispls hold negative entries, or recvcounts[t][s] != sendcounts[s][t]",
+                        VC_ERR_TABLES);
     out.nl = nl; out.n_digits = S.w + S.w2; out.recv_lo = S.recv_lo;
     out.stage_bytes = h[0]; out.payload_bytes = h[1];
     out.first.assign(nl, 0); out.count.assign(nl, 0); out.bytes.assign(nl, 0); out.inter.assign(nl, 0); out.lanes.assign(nl, VC_THREADS);
@@ -471,7 +510,7 @@ static int run_items(vc_comm *c, const PlanInfo &pi, const void *items_any, cons
     hipStream_t st = c->stream;
     const int nl = pi.chain ? 1 : pi.nl;              // kernel launches of this execution
     const VcDesc *items = static_cast<const VcDesc *>(items_any);
-    HIP_TRY(c->stage.reserve((size_t)pi.stage_bytes + 64));
+    HIP_TRY(reserve_stage(c, (size_t)pi.stage_bytes + 64));
     if (c->timing) { int rc = ensure_events(c, (size_t)nl + 4); if (rc) return rc; }
     if (pi.chain) {
         if (c->timing) HIP_TRY(hipEventRecord(c->events[2], st));
@@ -537,7 +576,7 @@ static int run_schedule(vc_comm *c, VcSched S, std::vector<VcLaunchInfo> &L, con
             if (rc) return rc;
             if (vc_listless_ok(c->h_header, guard)) { pi.listless = true; pi.chain_lanes = pair_lanes; break; }
             if (pi.stage_bytes <= guard.stage_cap) break;          // not a call for this kernel
-            HIP_TRY(c->stage.reserve((size_t)pi.stage_bytes + 64));
+            HIP_TRY(reserve_stage(c, (size_t)pi.stage_bytes + 64));
         }
         if (pi.listless) return finish_stats(c, pi, nullptr, true);
     }
@@ -583,6 +622,7 @@ static int run_v(VcFunc f, int n, int r, int batch, vc_comm *c, char *sendbuf, i
                  char *recvbuf, int *recvcounts, int *rdispls, int batch2 = 0) {
     int rc = check_common(c, sendbuf, recvbuf, esz);
     if (rc) return rc;
+    VC_ONE_CALL(c);
     if (!sendcounts || !sdispls || !recvcounts || (f != VC_F_TTPL && !rdispls)) return fail_arg("null table");
     VcSched S;
     std::vector<VcLaunchInfo> L;
@@ -654,6 +694,7 @@ extern "C" int twophase_rbruck_alltoallv_noalloc(int r, char *sendbuf, int *send
     (void)recvtype_size;
     int rc = check_common(c, sendbuf, recvbuf, sendtype_size);
     if (rc) return rc;
+    VC_ONE_CALL(c);
     if (!sendcounts || !sdispls || !recvcounts || !rdispls) return fail_arg("null table");
     unsigned char *base = c->device < VC_MAX_DEVICES ? g_scratch_ptr[c->device] : nullptr;
     if (!base) return fail_arg("the static scratch array was not resolved on this device", VC_ERR_HIP);
@@ -762,6 +803,7 @@ extern "C" int twolayer_communicator_linear_s2(int n, int bblock1, int bblock2, 
 static int run_uniform(VcFunc f, int n, int r, vc_comm *c, char *sendbuf, int sendcount, int esz, char *recvbuf) {
     int rc = check_common(c, sendbuf, recvbuf, esz);
     if (rc) return rc;
+    VC_ONE_CALL(c);
     if (sendcount < 0) return fail_arg("negative block length");
     if ((int64_t)sendcount * c->P > 0x7FFFFFFF) return fail_arg("sendcount * P must fit the reference's int displacements");
     VcSched S;
@@ -816,6 +858,7 @@ extern "C" int vc_plan_create(const char *function, int n, int r, int batch, int
     if (!c || !function || !plan_out) return fail_arg("vc_plan_create: null argument");
     if (elem_size < 1) return fail_arg("element size must be >= 1");
     if (!c->sbase || !c->rbase) return fail_arg("vc_comm_set_bases has not been called");
+    VC_ONE_CALL(c);
     VcFunc f;
     if (!func_by_name(function, f)) return fail_arg("vc_plan_create: unknown function name");
     const bool uniform = f == VC_F_UNIFORM_SPREADOUT || f == VC_F_UNIFORM_ISPLIT;      // `batch` is the block length, tables implied
@@ -839,9 +882,10 @@ extern "C" int vc_plan_create(const char *function, int n, int r, int batch, int
     p->comm = c;
     rc = build_plan(c, S, L, make_tables(c, sendcounts, sdispls, recvcounts, rdispls), p->items, p->info, forward);
     if (rc == VC_OK && hipStreamSynchronize(c->stream) != hipSuccess) rc = fail_arg("vc_plan_create: stream error", VC_ERR_HIP);
-    if (rc == VC_OK && c->stage.reserve((size_t)p->info.stage_bytes + 64) != hipSuccess)       // so that executing never allocates
+    if (rc == VC_OK && reserve_stage(c, (size_t)p->info.stage_bytes + 64) != hipSuccess)       // so that executing never allocates
         rc = fail_arg("vc_plan_create: cannot allocate the staging arena", VC_ERR_HIP);
     if (rc) { p->items.release(); delete p; return rc; }
+    c->live_plans++;
     *plan_out = p;
     return VC_OK;
 }
@@ -850,6 +894,7 @@ extern "C" int vc_plan_execute(vc_plan_t p, char *sendbuf, char *recvbuf) {
     if (!p || !sendbuf || !recvbuf) return fail_arg("vc_plan_execute: null argument");
     if ((int)((uintptr_t)recvbuf & (VC_LINE - 1)) != (p->info.recv_lo & (VC_LINE - 1)))
         return fail_arg("vc_plan_execute: recvbuf must have the low address bits the plan was made for");
+    VC_ONE_CALL(p->comm);
     return run_items(p->comm, p->info, p->items.p, sendbuf, recvbuf, false);
 }
 
@@ -865,6 +910,7 @@ extern "C" int vc_plan_free(vc_plan_t p) {
     (void)hipStreamSynchronize(p->comm->stream);
     if (p->comm->last_items == p->items.as<VcDesc>()) { p->comm->last_items = nullptr; p->comm->last_nlaunch = 0; }
     p->items.release();
+    if (--p->comm->live_plans == 0) free_retired_stage(p->comm);
     delete p;
     return VC_OK;
 }

@@ -110,12 +110,15 @@ hipError_t vc_launch_uniform_tables(int *counts, int *displs, int count, int P, 
 // vc_plan.hip
 // header layout (int64), nl = number of launches:
 //   [0] staging bytes   [1] payload bytes   [2] chain items (forwarded execution)
-//   [3] negative entries found in the count / displacement tables
+//   [3] entries of the count / displacement tables no set of ranks could have passed: negative ones, recvcounts[t][s] that
+//       differ from sendcounts[s][t]; plus VC_BAD_OVERFLOW per rank whose packed receive layout overflows an int
 //   [4] the most pieces any block is cut into (forwarded execution)
 //   [5 + L] bytes moved by launch L   [5 + nl + L] work items of launch L
 //   (forwarded execution: [5] all moved bytes, no per-launch words)
 #define VC_HEADER_FIXED 5
 #define VC_HEADER_BAD 3
+// added to header[VC_HEADER_BAD] once per rank whose packed receive displacements would pass INT_MAX elements
+#define VC_BAD_OVERFLOW (1ll << 40)
 #define VC_HEADER_MAX_PIECES 4
 #define VC_HEADER_WORDS(nl) (VC_HEADER_FIXED + 2 * (nl))
 // Passes 1 and 2: staging prefix sums and the number of work items of every launch (sizes only).  The launch table

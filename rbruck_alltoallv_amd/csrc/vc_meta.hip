@@ -1,6 +1,8 @@
 // vc_meta.hip — the caller-side metadata steps of the reference drivers as kernels
 // (count-matrix exchange, displacement prefix sums, global maximum), plus the
 // payload fill and the exact receiver-side check used by the harness.
+#include <climits>
+
 #include "vc_common.h"
 #include "vc_scan.h"
 
@@ -88,17 +90,17 @@ hipError_t vc_launch_bases(const int64_t *extent, int esz, int64_t align, int64_
 // MPI_Allreduce(MAX) of the block length (src/twophase_tunable_rbruckv.cpp:40-44).
 // ---------------------------------------------------------------------------
 __global__ __launch_bounds__(VC_THREADS) void vc_max_kernel(const int *__restrict__ counts, int *__restrict__ out, int64_t n) {
-    int m = 0;
+    int m = INT_MIN;
     for (int64_t i = (int64_t)blockIdx.x * VC_THREADS + threadIdx.x; i < n; i += (int64_t)gridDim.x * VC_THREADS) m = max(m, counts[i]);
 #pragma unroll
     for (int o = VC_WAVE / 2; o > 0; o >>= 1) m = max(m, __shfl_xor(m, o, VC_WAVE));
     if ((threadIdx.x & (VC_WAVE - 1)) == 0) atomicMax(out, m);
 }
 
-__global__ void vc_zero_int_kernel(int *p) { *p = 0; }
+__global__ void vc_lowest_int_kernel(int *p) { *p = INT_MIN; }
 
 hipError_t vc_launch_max(const int *counts, int *out, int64_t nelem, hipStream_t st) {
-    hipLaunchKernelGGL(vc_zero_int_kernel, dim3(1), dim3(1), 0, st, out);
+    hipLaunchKernelGGL(vc_lowest_int_kernel, dim3(1), dim3(1), 0, st, out);
     int64_t blocks = (nelem + VC_THREADS - 1) / VC_THREADS;
     if (blocks > 1024) blocks = 1024;
     if (blocks < 1) blocks = 1;

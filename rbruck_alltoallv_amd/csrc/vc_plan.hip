@@ -63,6 +63,8 @@ __global__ __launch_bounds__(VC_THREADS) void vc_plan_rows(VcSched S, VcLaunchPa
         for (int chunk = 0; chunk < nchunk; chunk++) {
             const int s = chunk * VC_THREADS + threadIdx.x;
             const int64_t cnt = s < P ? vc_chain_count(S, T, s, to) : 0;
+            // the receiver must expect exactly what the source sends (the reference fails with an MPI truncation error)
+            bad += s < P && T.rc[(int64_t)to * P + s] != T.sc[(int64_t)s * P + to];
             most = cnt > most ? cnt : most;
             if (threadIdx.x == 0) chain_row_tot[2 * (int64_t)P + (int64_t)to * nchunk + chunk] = before;
             before += vc_block_sum(cnt, lds);
@@ -85,10 +87,16 @@ __global__ __launch_bounds__(VC_THREADS) void vc_plan_rows(VcSched S, VcLaunchPa
             const int64_t i = (int64_t)to * P + id;
             payload += (int64_t)T.rc[i] * S.esz;
             bad += (T.sc[i] < 0) | (T.sd[i] < 0) | (T.rc[i] < 0) | (!S.packed_recv && T.rd[i] < 0);
+            if (!forward) bad += T.rc[i] != T.sc[(int64_t)id * P + to];      // forwarded execution has compared them above
         }
     items = vc_block_sum(items, lds);
     if (forward) most = vc_block_max(most, lds); else bytes = vc_block_sum(bytes, lds);
-    if (L == 0) { payload = vc_block_sum(payload, lds); bad = vc_block_sum(bad, lds); }
+    if (L == 0) {
+        payload = vc_block_sum(payload, lds);
+        bad = vc_block_sum(bad, lds);
+        // the packed receive layout is an int prefix sum of the rank's receive counts, like the reference's displacements
+        if (S.packed_recv && payload > (int64_t)0x7FFFFFFF * S.esz) bad += VC_BAD_OVERFLOW;
+    }
     if (threadIdx.x == 0) {
         if (forward) { chain_row_tot[to] = items; chain_row_tot[P + to] = most; }
         else { item_row_tot[(int64_t)L * P + to] = items; row_bytes[(int64_t)L * P + to] = bytes; }
@@ -380,8 +388,12 @@ __global__ __launch_bounds__(VC_THREADS) void vc_traffic_kernel(const VcDesc *__
 }
 
 hipError_t vc_launch_traffic(const VcDesc *desc, int64_t ndesc, int64_t *matrix, int P, hipStream_t st) {
-    int64_t nb = (ndesc + VC_THREADS - 1) / VC_THREADS;
-    if (nb < 1) nb = 1;
-    hipLaunchKernelGGL(vc_traffic_kernel, dim3((unsigned)nb), dim3(VC_THREADS), 0, st, desc, ndesc, matrix, P);
+    // a dispatch counts its grid in work-items in 32 bits: at most 2^24 - 1 workgroups of VC_THREADS per launch
+    const int64_t step = (((int64_t)1 << 24) - 1) * VC_THREADS;
+    for (int64_t done = 0; done < ndesc; done += step) {
+        const int64_t now = ndesc - done < step ? ndesc - done : step;
+        hipLaunchKernelGGL(vc_traffic_kernel, dim3((unsigned)((now + VC_THREADS - 1) / VC_THREADS)), dim3(VC_THREADS), 0, st, desc + done,
+                           now, matrix, P);
+    }
     return hipGetLastError();
 }

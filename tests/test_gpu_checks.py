@@ -1,0 +1,260 @@
+"""Checks of the checkers and of the library's default execution mode, through the C ABI on a real MI355X.
+
+* vc_verify_alltoallv (the on-device definition check the full-size tests and the benchmark lean on) must count exactly
+  the bytes that are wrong, not merely return 0 on a correct arena;
+* the library's default mode (vc_comm_set_forwarding 1: the last call on the communicator decides between the work-item
+  list and the listless kernels, which may refuse a call on the device and have it redone) against the oracle's bytes;
+* table validation beyond negative entries; the staging arena under live plans."""
+import collections
+
+import numpy as np
+import pytest
+
+from oracle import oracle_py as O
+from rbruck_alltoallv_amd import _lib
+from rbruck_alltoallv_amd import workloads as W
+from tests.helpers import digest_problem, load_golden, problem_for_case, run_on
+
+pytestmark = pytest.mark.gpu
+
+CASES = load_golden()
+
+
+@pytest.fixture(scope="module")
+def api():
+    import torch
+    assert torch.cuda.is_available(), "these tests need the GPU"
+    from rbruck_alltoallv_amd import api as A
+    A.DEFAULT_FORWARDING = None
+    return A
+
+
+def _host_mismatch(prob, send, recv, rdispls=None, packed=False):
+    """Bytes of recv that differ from the definition, counted block by block on the host (numpy)."""
+    rd = prob.rdispls if rdispls is None else rdispls
+    bad = 0
+    for t in range(prob.P):
+        at_packed = 0
+        for s in range(prob.P):
+            nb = int(prob.sendcounts[s, t]) * prob.esz
+            a = int(prob.sbase[s]) + int(prob.sdispls[s, t]) * prob.esz
+            b = int(prob.rbase[t]) + (at_packed if packed else int(rd[t, s]) * prob.esz)
+            bad += int(np.count_nonzero(send[a:a + nb] != recv[b:b + nb]))
+            at_packed += int(prob.recvcounts[t, s]) * prob.esz
+    return bad
+
+
+@pytest.mark.parametrize("packed", [False, True])
+def test_verify_counts_exactly_the_wrong_bytes(api, packed):
+    import torch
+    P, esz = 24, 2
+    counts = W.counts_uniform_random(P, 900, seed=31)
+    counts[counts % 7 == 0] = 0
+    prob = W.make_problem(counts, esz, 0, 0)
+    send = W.fill_send_arena(prob, 0, 17)
+    dp = api.DeviceProblem(prob)
+    ds = torch.from_numpy(send).to("cuda:0")
+    dr = dp.new_recv_arena(0xEE)
+    fn = (lambda: api.TTPL_BT_alltoallv(6, 3, 0, dp, ds, dr)) if packed else (lambda: api.twophase_rbruck_alltoallv(3, dp, ds, dr))
+    assert fn() == 0, dp.comm.error()
+    assert dp.verify(ds, dr, packed_recv=packed) == 0
+    good = dr.clone()
+
+    # one flipped byte inside a block
+    t, s = 5, 9
+    assert counts[s, t] > 0
+    at = int(prob.rbase[t]) + int(prob.rdispls[t, s]) * esz + 3
+    dr[at] ^= 0x40
+    assert dp.verify(ds, dr, packed_recv=packed) == 1
+    dr.copy_(good)
+
+    # a byte between the ranks' buffers or in a gap is nobody's: not counted (the arena comparison of the parity tests covers those)
+    # two blocks of one receiver swapped (the first min(len) bytes of each)
+    s1, s2 = 2, 11
+    n1, n2 = int(counts[s1, t]) * esz, int(counts[s2, t]) * esz
+    assert n1 > 0 and n2 > 0
+    a1 = int(prob.rbase[t]) + int(prob.rdispls[t, s1]) * esz
+    a2 = int(prob.rbase[t]) + int(prob.rdispls[t, s2]) * esz
+    m = min(n1, n2)
+    tmp = dr[a1:a1 + m].clone()
+    dr[a1:a1 + m] = dr[a2:a2 + m]
+    dr[a2:a2 + m] = tmp
+    want = _host_mismatch(prob, send, dr.cpu().numpy(), packed=packed)
+    assert want > m                                           # random payload: nearly all 2 m bytes differ
+    assert dp.verify(ds, dr, packed_recv=packed) == want
+    dr.copy_(good)
+
+    # a whole rank's buffer wiped
+    t2 = 13
+    lo, hi = int(prob.rbase[t2]), int(prob.rbase[t2]) + int(counts[:, t2].sum()) * esz
+    dr[lo:hi] = 0
+    want = _host_mismatch(prob, send, dr.cpu().numpy(), packed=packed)
+    assert dp.verify(ds, dr, packed_recv=packed) == want > 0
+    dr.copy_(good)
+
+    if not packed:
+        # one receive displacement shifted by one element: the check reads the block one element further on
+        rd = prob.rdispls.copy()
+        rd[t, s] += 1
+        drd = torch.from_numpy(rd).to("cuda:0")
+        keep = dp.rdispls
+        dp.rdispls = drd
+        want = _host_mismatch(prob, send, good.cpu().numpy(), rdispls=rd)
+        assert want > 0
+        assert dp.verify(ds, good) == want
+        dp.rdispls = keep
+    # a receive count that disagrees with the send count is one mismatch of its own
+    rc = prob.recvcounts.copy()
+    rc[t, s] += 1
+    keep = dp.recvcounts
+    dp.recvcounts = torch.from_numpy(rc).to("cuda:0")
+    got = dp.verify(ds, good, packed_recv=packed)
+    dp.recvcounts = keep
+    if packed:                                                # the packed layout follows the receive counts: later blocks shift too
+        assert got >= 1
+    else:
+        assert got == 1
+    dp.comm.free()
+
+
+def test_default_mode_on_the_golden_cases(api):
+    """vc_comm_set_forwarding 1, the library's default: one long-lived communicator per rank count, the golden cases in
+    file order, two calls each.  The first call of a case runs on whatever the previous case left as a hint (the listless
+    kernels refuse what they were not made for and the call is redone through the list, or redone behind a larger
+    staging arena); the second on the hint of the first.  Every call must leave the oracle's bytes."""
+    import torch
+    comms = {}
+    ran = collections.Counter()
+    for case in CASES:
+        print("case", case["id"], flush=True)
+        prob = problem_for_case(case)
+        send = W.fill_send_arena(prob, case["payload"], case["seed"])
+        want = np.full(prob.recv_bytes, 0xEE, dtype=np.uint8)
+        assert run_on(O, case, prob, send.copy(), want) == 0
+        if prob.P not in comms:
+            comms[prob.P] = api.VirtualComm(prob.P)
+            comms[prob.P].set_forwarding(1)
+        dp = api.DeviceProblem(prob, comm=comms[prob.P])
+        dsend = torch.from_numpy(send).to("cuda:0")
+        for call in range(2):
+            drecv = dp.new_recv_arena(0xEE)
+            rc = run_on(api, case, dp, dsend, drecv)
+            assert rc == 0, (case["id"], call, dp.comm.error())
+            got = drecv.cpu().numpy()
+            assert np.array_equal(got, want), (case["id"], call)
+            st = dp.comm.last_stats()
+            assert st.n_launches == 1 and st.payload_bytes == prob.payload_bytes
+            ran[(int(st.execution), int(st.lanes_per_item))] += 1
+        assert [f"{int(h):016x}" for h in O.digest_recv(digest_problem(case, prob), got)] == case["digests"]
+    for c in comms.values():
+        c.free()
+    print("executions (mode, lanes):", dict(ran), flush=True)
+    assert any(k[0] == 1 for k in ran) and any(k[0] == 2 for k in ran)      # both ways were taken
+
+
+def test_refused_listless_call_is_redone(api):
+    """The two ways a listless attempt ends without having moved anything, both compared with the oracle's bytes: the
+    staging arena was too small (the call is enqueued again behind a larger one) and the call was not of the kind the
+    hint promised (it continues through the work-item list)."""
+    import torch
+    P = 48
+    comm = api.VirtualComm(P)
+    comm.set_forwarding(1)
+    tiny = W.make_problem(W.counts_uniform_random(P, 8, seed=1), 1, 0, 0)
+    short = W.make_problem(W.counts_uniform_random(P, 700, seed=2), 1, 1, 1)        # same kind, 100 times the staging
+    long_counts = W.counts_uniform_random(P, 700, seed=3)
+    long_counts[7, 30] = 500000                                                       # one block of 123 pieces
+    long = W.make_problem(long_counts, 1, 0, 0)
+    seen = []
+    for prob in (tiny, tiny, short, long, short):
+        send = W.fill_send_arena(prob, 0, 5)
+        want = np.full(prob.recv_bytes, 0xEE, dtype=np.uint8)
+        assert O.twophase_rbruck_alltoallv(3, prob, send, want) == 0
+        dp = api.DeviceProblem(prob, comm=comm)
+        ds = torch.from_numpy(send).to("cuda:0")
+        dr = dp.new_recv_arena(0xEE)
+        assert api.twophase_rbruck_alltoallv(3, dp, ds, dr) == 0, comm.error()
+        assert np.array_equal(dr.cpu().numpy(), want)
+        st = comm.last_stats()
+        seen.append((int(st.execution), int(st.staging_bytes)))
+    assert [e for e, _ in seen] == [1, 2, 2, 1, 1], seen      # list, listless, listless behind a grown arena, refused -> list, list
+    assert seen[2][1] > 2 * seen[1][1]                       # the third call needed a larger arena than there was
+    comm.free()
+
+
+def test_tables_that_disagree_are_refused(api):
+    """recvcounts must be the transpose of sendcounts (the reference fails with an MPI truncation error); a packed receive
+    layout past INT_MAX elements is an overflow, as in vc_displs_from_counts."""
+    import torch
+    counts = W.counts_uniform_random(12, 40, seed=5)
+    prob = W.make_problem(counts, 4, 0, 0)
+    dp = api.DeviceProblem(prob)
+    s, d = dp.new_send_arena(), dp.new_recv_arena()
+    dp.fill_payload(0, 1, s)
+    keep = int(dp.recvcounts[7, 3].item())
+    for mode in (0, 1, 2, 3, 4):
+        dp.comm.set_forwarding(mode)
+        for delta in (1, -1):
+            dp.recvcounts[7, 3] = keep + delta
+            for call in (lambda: api.twophase_rbruck_alltoallv(3, dp, s, d), lambda: api.TTPL_BT_alltoallv(4, 2, 0, dp, s, d),
+                         lambda: api.spreadout_alltoallv(dp, s, d)):
+                assert call() == _lib.VC_ERR_TABLES and "recvcounts" in dp.comm.error(), mode
+            assert bool((d == 0xEE).all())
+        dp.recvcounts[7, 3] = keep
+        assert api.twophase_rbruck_alltoallv(3, dp, s, d) == 0 and dp.verify(s, d) == 0
+        d.fill_(0xEE)
+    dp.comm.free()
+    # 2 ranks that each receive 2^31 one-byte elements: found by the planner, nothing is touched
+    comm = api.VirtualComm(2)
+    z = torch.zeros(2, dtype=torch.int64, device="cuda:0")
+    comm.set_bases(z, z)
+    big = torch.full((2, 2), 2 ** 30, dtype=torch.int32, device="cuda:0")
+    displs = torch.tensor([[0, 2 ** 30], [0, 2 ** 30]], dtype=torch.int32, device="cuda:0")
+    buf = torch.full((256,), 0xEE, dtype=torch.uint8, device="cuda:0")
+    for mode in (0, 2, 3):
+        comm.set_forwarding(mode)
+        rc = comm.lib.TTPL_BT_alltoallv(1, 2, 0, buf.data_ptr(), big.data_ptr(), displs.data_ptr(), 1, buf.data_ptr(), big.data_ptr(),
+                                        None, 1, comm.handle)
+        assert rc == _lib.VC_ERR_OVERFLOW, (mode, rc, comm.error())
+        assert bool((buf == 0xEE).all())
+    comm.free()
+
+
+def test_staging_arena_stays_put_while_a_plan_lives(api):
+    """A HIP graph captured from vc_plan_execute_async holds the staging arena's address.  A later call on the same
+    communicator that needs a larger arena must not free the one the graph writes to: the replay after it is still exact."""
+    import torch
+    P = 32
+    small = W.make_problem(W.counts_uniform_random(P, 900, seed=8), 1, 0, 0)
+    large = W.make_problem(W.counts_uniform_random(P, 60000, seed=9), 1, 0, 0)
+    comm = api.VirtualComm(P)
+    comm.set_forwarding(2)
+    dp = api.DeviceProblem(small, comm=comm)
+    send = W.fill_send_arena(small, 0, 3)
+    want = W.expected_recv_arena(small, send, fill=0)
+    ds = torch.from_numpy(send).to("cuda:0")
+    dr = dp.new_recv_arena(0)
+    plan = api.Plan("twophase_rbruck_alltoallv", dp, dr, r=2)
+    assert plan.rc == 0, comm.error()
+    assert plan.execute(ds, dr) == 0 and np.array_equal(dr.cpu().numpy(), want)
+    before = comm.staging()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        comm.use_current_stream()
+        assert plan.execute_async(ds, dr) == 0, comm.error()
+    comm.use_current_stream()
+    # a larger call on the same communicator: its bases are another problem's
+    dpl = api.DeviceProblem(large, comm=comm)
+    dsl, drl = dpl.new_send_arena(), dpl.new_recv_arena()
+    dpl.fill_payload(0, 4, dsl)
+    assert api.twophase_rbruck_alltoallv(2, dpl, dsl, drl) == 0 and dpl.verify(dsl, drl) == 0
+    after = comm.staging()
+    assert after[1] > before[1] and after[0] != before[0]    # a second arena; the first one is still allocated
+    for rep in range(3):
+        dr.zero_()
+        torch.cuda.synchronize()
+        g.replay()
+        torch.cuda.synchronize()
+        assert np.array_equal(dr.cpu().numpy(), want), rep
+    plan.free()
+    comm.free()
