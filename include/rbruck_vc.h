@@ -234,14 +234,28 @@ int vc_plan_execute_async(vc_plan_t plan, char *sendbuf, char *recvbuf);
 /* Waits for the communicator's stream and releases the plan's work items; before vc_comm_free of its communicator. */
 int vc_plan_free(vc_plan_t plan);
 
-/* ---- radix choice.  The reference leaves r to the caller (its drivers sweep a list of bases,
- * examples/rbruckv_example.cpp:33-35).  Given candidate radices this evaluates, on the device, the bytes each would
- * move (sum over blocks of hops x bytes; hops = non-zero base-r digits of the offset inside the node, + 1 if the node
- * differs) and returns the candidate with the smallest modelled time: 2 * moved / (sustained copy rate) + launches x
- * launch latency for one launch per digit, moved / rate (one write per hop, one launch) for forwarded execution.  n = ranks per node for the two-layer functions, 0 or P for the one-layer ones.  `candidates` and the
- * outputs are HOST arrays; moved_bytes_out (may be NULL) receives the moved bytes per candidate. ---- */
+/* ---- tunables.  The reference leaves r and b to the caller; its drivers sweep a list of bases and batch sizes and time
+ * every combination (examples/rbruckv_example.cpp:33-35, 98-103; src/tuna.cpp:21, 69).  vc_suggest_tunables replaces the
+ * sweep by a model priced in figures measured once per communicator (vc_comm_calibration): the rate of a plain copy on
+ * this GPU, the cost of one more kernel launch, and of a launch the host waits for.  For every candidate radix it evaluates on the device the bytes and
+ * work items the call would move (sum over blocks of hops x bytes; hops = non-zero base-r digits of the offset inside the
+ * node, + 1 if the node differs) and models the call in the communicator's execution mode (vc_comm_set_forwarding):
+ *   one launch per digit:  (planning) + launches x launch cost + (2 x moved bytes + 64 x moved items) / rate
+ *   forwarded:             (planning) + launch cost + (payload + moved bytes + 2 x items x (24 + 8 x hop slots)) / rate
+ * with rate = 0.85 x the plain copy's.  n = ranks per node for the two-layer functions, 0 or P for the one-layer ones.
+ * candidates / ncand: HOST array of radices; ncand = 0 searches every radix from 2 to min(n, 63) and n itself.
+ * r_out: the candidate with the smallest modelled time; b_out (may be NULL): rounds of a digit per launch for
+ * tuna_algorithm: always all of them (r - 1), because on one GPU the rounds of a digit are independent copies and
+ * splitting them over launches only adds launch costs; seconds_out / moved_bytes_out (HOST, ncand entries, may be NULL;
+ * pass NULL with ncand = 0): modelled time and hop-weighted bytes per candidate. ---- */
+int vc_suggest_tunables(const int *sendcounts, int elem_size, int n, const int *candidates, int ncand, int *r_out, int *b_out,
+                        double *seconds_out, int64_t *moved_bytes_out, vc_comm_t comm);
+/* The radix alone, from a non-empty candidate list (vc_suggest_tunables without b and the modelled times). */
 int vc_suggest_radix(const int *sendcounts, int elem_size, int n, const int *candidates, int ncand, int *best_out,
                      int64_t *moved_bytes_out, vc_comm_t comm);
+/* Measures (once per communicator, then remembered) what the model is priced in: bytes per second of a plain 256 MiB copy
+ * (read + written bytes) and seconds per kernel launch in a row of empty launches.  Allocates 512 MiB for the moment. */
+int vc_comm_calibration(vc_comm_t comm, double *copy_bytes_per_s_out, double *launch_seconds_out);
 
 /* ---- measurement and inspection (the reference's global phase timers, src/rbruckv.h:13-18) ---- */
 

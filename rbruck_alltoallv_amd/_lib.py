@@ -59,6 +59,8 @@ SYMBOLS = {
     "vc_plan_execute_async": (_I, [_P, _P, _P]),
     "vc_plan_free": (_I, [_P]),
     "vc_suggest_radix": (_I, [_P, _I, _I, _P, _I, C.POINTER(_I), _P, _P]),
+    "vc_suggest_tunables": (_I, [_P, _I, _I, _P, _I, C.POINTER(_I), C.POINTER(_I), _P, _P, _P]),
+    "vc_comm_calibration": (_I, [_P, C.POINTER(C.c_double), C.POINTER(C.c_double)]),
     "vc_comm_set_timing": (_I, [_P, _I]),
     "vc_comm_last_stats": (_I, [_P, C.POINTER(VcStats)]),
     "vc_comm_last_traffic": (_I, [_P, _I, _P]),

@@ -248,6 +248,24 @@ def suggest_radix(p: DeviceProblem, candidates: list[int], n: int = 0) -> tuple[
     return best.value, list(moved)
 
 
+def suggest_tunables(p: DeviceProblem, candidates: list[int] | None = None, n: int = 0) -> tuple[int, int, list[float]]:
+    """vc_suggest_tunables: (radix, rounds per launch, modelled seconds per candidate); no candidates = search 2..min(n, 63), n."""
+    ncand = len(candidates) if candidates else 0
+    cand = (C.c_int * max(ncand, 1))(*(candidates or [0]))
+    secs = (C.c_double * max(ncand, 1))()
+    r, b = C.c_int(0), C.c_int(0)
+    p.comm._check(p.comm.lib.vc_suggest_tunables(p.sendcounts.data_ptr(), p.esz, n, cand if ncand else None, ncand, C.byref(r),
+                                                 C.byref(b), secs if ncand else None, None, p.comm.handle))
+    return r.value, b.value, list(secs)[:ncand]
+
+
+def calibration(comm: VirtualComm) -> tuple[float, float]:
+    """vc_comm_calibration: (bytes per second of a plain copy, seconds per kernel launch)."""
+    rate, launch = C.c_double(0), C.c_double(0)
+    comm._check(comm.lib.vc_comm_calibration(comm.handle, C.byref(rate), C.byref(launch)))
+    return rate.value, launch.value
+
+
 def twolayer_communicator_linear(n: int, p: DeviceProblem, send: torch.Tensor, recv: torch.Tensor) -> int:
     """src/twolayer_communicator_linear.cpp:13-88"""
     return p.comm.lib.twolayer_communicator_linear(n, *_tail(p, send, recv))

@@ -11,6 +11,7 @@
 
 #include <algorithm>
 #include <atomic>
+#include <chrono>
 #include <cstdio>
 #include <cstring>
 #include <string>
@@ -108,6 +109,8 @@ struct vc_comm {
     DevBuf chain_row_tot, chain_row_base;
     DevBuf slot_off, row_tot, row_base, org_run_base, item_row_tot, item_row_base, row_bytes, desc, header, launches, stage, rd_packed,
         uni_counts, uni_displs, scratch;
+    double cal_copy_bytes_per_s = 0, cal_launch_s = 0, cal_sync_s = 0;   // calibrate(): the plain copy's rate, the cost of a
+                                          // launch, of a launch the host waits for
     int live_plans = 0;                   // plans created on this communicator and not yet freed
     std::vector<void *> retired_stage;    // staging arenas that were outgrown while plans existed: a HIP graph captured from
                                           // vc_plan_execute_async holds the arena's address, so they stay until the plans go
@@ -926,40 +929,126 @@ static int launches_for(int span, int r, bool inter) {
     return n + (inter ? 1 : 0);
 }
 
-extern "C" int vc_suggest_radix(const int *sendcounts, int elem_size, int n, const int *candidates, int ncand, int *best_out,
-                                int64_t *moved_bytes_out, vc_comm_t c) {
-    if (!c || !sendcounts || !candidates || !best_out || elem_size < 1 || ncand < 1 || ncand > 64)
-        return fail_arg("vc_suggest_radix: bad argument (1..64 candidates)");
+// What this GPU sustains, measured once per communicator: a plain copy of 256 MiB (best of 3) and the cost of one more
+// kernel launch on the stream (a row of 64 empty kernels).  The model below is priced in these two figures.
+static int calibrate(vc_comm *c) {
+    if (c->cal_copy_bytes_per_s > 0) return VC_OK;
+    int rc = ensure_events(c, 2);
+    if (rc) return rc;
+    const size_t nb = (size_t)256 << 20;
+    char *buf = nullptr;
+    HIP_TRY(hipMalloc((void **)&buf, 2 * nb));
+    float best = 0.f, ms = 0.f;
+    hipError_t e = hipSuccess;
+    for (int rep = 0; rep < 4 && e == hipSuccess; rep++) {         // the first one warms up
+        e = hipEventRecord(c->events[0], c->stream);
+        if (e == hipSuccess) e = vc_launch_calibration_copy(buf, buf + nb, (int64_t)nb, c->stream);
+        if (e == hipSuccess) e = hipEventRecord(c->events[1], c->stream);
+        if (e == hipSuccess) e = hipEventSynchronize(c->events[1]);
+        if (e == hipSuccess) e = hipEventElapsedTime(&ms, c->events[0], c->events[1]);
+        if (rep > 0 && (best == 0.f || ms < best)) best = ms;
+    }
+    const int row = 64;
+    if (e == hipSuccess) e = hipEventRecord(c->events[0], c->stream);
+    for (int k = 0; k < row && e == hipSuccess; k++) e = vc_launch_empty(c->stream);
+    if (e == hipSuccess) e = hipEventRecord(c->events[1], c->stream);
+    if (e == hipSuccess) e = hipEventSynchronize(c->events[1]);
+    if (e == hipSuccess) e = hipEventElapsedTime(&ms, c->events[0], c->events[1]);
+    (void)hipFree(buf);
+    // a launch the host waits for, by the host's clock: what each of a blocking call's synchronisations costs
+    const auto t0 = std::chrono::steady_clock::now();
+    const int waits = 16;
+    for (int k = 0; k < waits && e == hipSuccess; k++) {
+        e = vc_launch_empty(c->stream);
+        if (e == hipSuccess) e = hipStreamSynchronize(c->stream);
+    }
+    const double waited = std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count();
+    if (e != hipSuccess) return fail_hip(e, "calibrate", __LINE__);
+    c->cal_copy_bytes_per_s = 2.0 * (double)nb / (best * 1e-3);
+    c->cal_launch_s = (double)ms * 1e-3 / row;
+    c->cal_sync_s = waited / waits;
+    return VC_OK;
+}
+
+extern "C" int vc_comm_calibration(vc_comm_t c, double *copy_bytes_per_s_out, double *launch_seconds_out) {
+    if (!c) return fail_arg("null communicator");
+    VC_ONE_CALL(c);
+    int rc = calibrate(c);
+    if (rc) return rc;
+    if (copy_bytes_per_s_out) *copy_bytes_per_s_out = c->cal_copy_bytes_per_s;
+    if (launch_seconds_out) *launch_seconds_out = c->cal_launch_s;
+    return VC_OK;
+}
+
+#define VC_MAX_CANDIDATES 64
+// the block movers sustain this share of the plain copy's rate on scattered, unaligned blocks (0.80 - 0.97 measured)
+#define VC_BLOCK_COPY_EFFICIENCY 0.85
+
+extern "C" int vc_suggest_tunables(const int *sendcounts, int elem_size, int n, const int *candidates, int ncand, int *r_out, int *b_out,
+                                   double *seconds_out, int64_t *moved_bytes_out, vc_comm_t c) {
+    if (!c || !sendcounts || !r_out || elem_size < 1 || ncand < 0 || ncand > VC_MAX_CANDIDATES || (ncand > 0 && !candidates))
+        return fail_arg("vc_suggest_tunables: bad argument (0..64 candidates)");
+    VC_ONE_CALL(c);
     const int P = c->P;
     if (n <= 0) n = P;
     if (P % n != 0) return fail_arg("n must divide the number of ranks", VC_ERR_GROUP);
-    int cand[64];
-    for (int k = 0; k < ncand; k++) {
-        if (candidates[k] < 2) return fail_arg("radix must be >= 2", VC_ERR_RADIX);
-        cand[k] = std::min(candidates[k], std::max(n, 2));
+    const int span = std::max(n, 2);
+    int given[VC_MAX_CANDIDATES], cand[VC_MAX_CANDIDATES];
+    if (ncand == 0) {                                     // every radix from 2 to min(span, 64), and the span itself (one hop)
+        for (int r = 2; r <= std::min(span, VC_MAX_CANDIDATES - 1); r++) given[ncand++] = r;
+        if (span > VC_MAX_CANDIDATES - 1) given[ncand++] = span;
+    } else {
+        for (int k = 0; k < ncand; k++) given[k] = candidates[k];
     }
-    HIP_TRY(c->scratch.reserve(sizeof(unsigned long long) * 64 + sizeof(int) * 64));
+    for (int k = 0; k < ncand; k++) {
+        if (given[k] < 2) return fail_arg("radix must be >= 2", VC_ERR_RADIX);
+        cand[k] = std::min(given[k], span);
+    }
+    int rc = calibrate(c);
+    if (rc) return rc;
+    const int words = 2 * (ncand + 1);
+    HIP_TRY(c->scratch.reserve(sizeof(unsigned long long) * 2 * (VC_MAX_CANDIDATES + 1) + sizeof(int) * VC_MAX_CANDIDATES));
     unsigned long long *moved_dev = c->scratch.as<unsigned long long>();
-    int *cand_dev = reinterpret_cast<int *>(moved_dev + 64);
-    HIP_TRY(hipMemsetAsync(moved_dev, 0, sizeof(unsigned long long) * 64, c->stream));
+    int *cand_dev = reinterpret_cast<int *>(moved_dev + 2 * (VC_MAX_CANDIDATES + 1));
+    HIP_TRY(hipMemsetAsync(moved_dev, 0, sizeof(unsigned long long) * words, c->stream));
     HIP_TRY(hipMemcpyAsync(cand_dev, cand, sizeof(int) * ncand, hipMemcpyHostToDevice, c->stream));
     HIP_TRY(vc_launch_hop_bytes(sendcounts, elem_size, P, n, cand_dev, ncand, moved_dev, c->stream));
-    unsigned long long moved[64];
-    HIP_TRY(hipMemcpyAsync(moved, moved_dev, sizeof(unsigned long long) * ncand, hipMemcpyDeviceToHost, c->stream));
+    unsigned long long got[2 * (VC_MAX_CANDIDATES + 1)];
+    HIP_TRY(hipMemcpyAsync(got, moved_dev, sizeof(unsigned long long) * words, hipMemcpyDeviceToHost, c->stream));
     HIP_TRY(hipStreamSynchronize(c->stream));
-    // time model, at the rate the copy kernels sustain on scattered blocks.  One launch per digit: every moved byte is
-    // read and written once and every launch costs a fixed latency.  Forwarded execution: one launch; every byte is
-    // written once per hop, and read only once (moved[k] counts one payload for every hop, so the payload itself is the
-    // same for all candidates and drops out of the comparison).
-    const double bytes_per_s = 5.2e12, launch_s = 7e-6;
+    // Time model.  A blocking call waits for the stream twice (after sizing the plan, at the end) and launches three planning
+    // kernels besides its copy kernels.  Every launch costs one launch latency; bytes move at the rate
+    // of the plain copy times what the block movers keep of it.  One launch per digit: every hop reads and writes its
+    // bytes and its 32-byte work items are written and read once.  Forwarded execution: one launch; the payload is read
+    // once, every hop writes its bytes, and every piece has one item of 24 + 8 x (hop slots) bytes.  The planning kernels
+    // read the count tables once per staging region.
+    const double rate = c->cal_copy_bytes_per_s * VC_BLOCK_COPY_EFFICIENCY, launch = c->cal_launch_s;
+    const double payload = (double)got[ncand], pieces = (double)got[2 * ncand + 1];
     double best = 0;
+    int best_k = 0;
     for (int k = 0; k < ncand; k++) {
-        const double t = c->forward != 0 ? (double)moved[k] / bytes_per_s
-                                    : 2.0 * (double)moved[k] / bytes_per_s + launch_s * launches_for(n, cand[k], n < P);
-        if (moved_bytes_out) moved_bytes_out[k] = (int64_t)moved[k];
-        if (k == 0 || t < best) { best = t; *best_out = candidates[k]; }
+        const double moved = (double)got[k], hop_pieces = (double)got[ncand + 1 + k];
+        int w, d;
+        vc_radix_params(n, cand[k], w, d);
+        const double plan = 2 * c->cal_sync_s + 3 * launch + (double)P * P * (w + 2) * 16.0 / rate;
+        const double t = c->forward != 0
+            ? plan + launch + (payload + moved + 2.0 * pieces * (24 + 8 * (w + 1))) / rate
+            : plan + launch * launches_for(n, cand[k], n < P) + (2.0 * moved + 2.0 * 32 * hop_pieces) / rate;
+        if (moved_bytes_out) moved_bytes_out[k] = (int64_t)got[k];
+        if (seconds_out) seconds_out[k] = t;
+        if (k == 0 || t < best) { best = t; best_k = k; }
     }
+    *r_out = given[best_k];
+    // rounds of a digit per launch (b of tuna_algorithm): on one GPU the rounds of a digit are independent copies, so
+    // splitting them over launches only adds launch latencies; all of them (r - 1) share a launch
+    if (b_out) *b_out = std::max(cand[best_k] - 1, 1);
     return VC_OK;
+}
+
+extern "C" int vc_suggest_radix(const int *sendcounts, int elem_size, int n, const int *candidates, int ncand, int *best_out,
+                                int64_t *moved_bytes_out, vc_comm_t c) {
+    if (!candidates || ncand < 1) return fail_arg("vc_suggest_radix: bad argument (1..64 candidates)");
+    return vc_suggest_tunables(sendcounts, elem_size, n, candidates, ncand, best_out, nullptr, nullptr, moved_bytes_out, c);
 }
 
 // ------------------------------------------------------------------ inspection

@@ -103,9 +103,12 @@ hipError_t vc_launch_fill_payload(int mode, uint64_t seed, char *sendbuf, const 
                                   int esz, int P, hipStream_t st);
 hipError_t vc_launch_verify(const char *sendbuf, const char *recvbuf, VcTables t, int esz, int P, int packed,
                             unsigned long long *mismatch, hipStream_t st);
+// moved_dev: 2 (ncand + 1) words the caller has zeroed: hop-weighted bytes per candidate, the payload, hop-weighted work
+// items per candidate, the work items of the payload
 hipError_t vc_launch_hop_bytes(const int *sc, int esz, int P, int n, const int *cand_dev, int ncand, unsigned long long *moved_dev,
                                hipStream_t st);
 hipError_t vc_launch_uniform_tables(int *counts, int *displs, int count, int P, hipStream_t st);
+hipError_t vc_launch_empty(hipStream_t st);
 
 // vc_plan.hip
 // header layout (int64), nl = number of launches:

@@ -206,27 +206,44 @@ hipError_t vc_launch_verify(const char *sendbuf, const char *recvbuf, VcTables t
 }
 
 // ---------------------------------------------------------------------------
-// Traffic model for choosing the radix: moved[c] = sum over all blocks of hops_r(s, t) * bytes(s, t) for radix
-// r = cand[c], where hops = non-zero base-r digits of the (local) offset, plus one if the node differs, and 1 for a
-// rank's block to itself.  grid (P, ncand).
+// Traffic model for choosing the radix.  For radix r = cand[c]: moved[c] = sum over all blocks of hops_r(s, t) *
+// bytes(s, t) and moved[ncand + 1 + c] = sum of hops_r(s, t) * pieces(s, t), where hops = non-zero base-r digits of the
+// (local) offset, plus one if the node differs, and 1 for a rank's block to itself; pieces = the 4 KiB work items a
+// block is cut into.  moved[ncand] and moved[2 ncand + 1] receive the payload and the pieces of all blocks (one hop
+// each).  grid (P, ncand + 1); the last row of workgroups adds up the radix-independent totals.
 // ---------------------------------------------------------------------------
-__global__ __launch_bounds__(VC_THREADS) void vc_hop_bytes_kernel(const int *__restrict__ sc, int esz, int P, int n,
+__global__ __launch_bounds__(VC_THREADS) void vc_hop_bytes_kernel(const int *__restrict__ sc, int esz, int P, int n, int ncand,
                                                                   const int *__restrict__ cand, unsigned long long *__restrict__ moved) {
     __shared__ int64_t lds[VC_WAVES_PER_BLOCK];
-    const int s = blockIdx.x, r = cand[blockIdx.y];
-    int64_t acc = 0;
+    const int s = blockIdx.x, c = blockIdx.y;
+    const int r = c < ncand ? cand[c] : 0;                // r = 0: every block counts once
+    int64_t acc = 0, items = 0;
     for (int t = threadIdx.x; t < P; t += VC_THREADS) {
-        int hops = (s / n != t / n) ? 1 : 0;
-        for (int j = (s % n - t % n + n) % n; j; j /= r) hops += (j % r) != 0;
-        if (s == t) hops = 1;
-        acc += (int64_t)hops * sc[(int64_t)s * P + t] * esz;
+        int hops = 1;
+        if (r && s != t) {
+            hops = (s / n != t / n) ? 1 : 0;
+            for (int j = (s % n - t % n + n) % n; j; j /= r) hops += (j % r) != 0;
+        }
+        const int64_t len = (int64_t)sc[(int64_t)s * P + t] * esz;
+        acc += hops * len;
+        items += hops * (len <= VC_CHUNK ? (len > 0) : (len + VC_PIECE - 1) / VC_PIECE);
     }
     acc = vc_block_sum(acc, lds);
-    if (threadIdx.x == 0 && acc) atomicAdd(&moved[blockIdx.y], (unsigned long long)acc);
+    items = vc_block_sum(items, lds);
+    if (threadIdx.x == 0 && acc) atomicAdd(&moved[c], (unsigned long long)acc);
+    if (threadIdx.x == 0 && items) atomicAdd(&moved[ncand + 1 + c], (unsigned long long)items);
 }
 
 hipError_t vc_launch_hop_bytes(const int *sc, int esz, int P, int n, const int *cand_dev, int ncand, unsigned long long *moved_dev,
                                hipStream_t st) {
-    hipLaunchKernelGGL(vc_hop_bytes_kernel, dim3(P, ncand), dim3(VC_THREADS), 0, st, sc, esz, P, n, cand_dev, moved_dev);
+    hipLaunchKernelGGL(vc_hop_bytes_kernel, dim3(P, ncand + 1), dim3(VC_THREADS), 0, st, sc, esz, P, n, ncand, cand_dev, moved_dev);
+    return hipGetLastError();
+}
+
+// A kernel that does nothing: what one launch costs is measured with a row of these.
+__global__ void vc_empty_kernel() {}
+
+hipError_t vc_launch_empty(hipStream_t st) {
+    hipLaunchKernelGGL(vc_empty_kernel, dim3(1), dim3(VC_WAVE), 0, st);
     return hipGetLastError();
 }

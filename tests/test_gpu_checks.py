@@ -258,3 +258,52 @@ def test_staging_arena_stays_put_while_a_plan_lives(api):
         assert np.array_equal(dr.cpu().numpy(), want), rep
     plan.free()
     comm.free()
+
+
+@pytest.mark.parametrize("mode", [2, 0], ids=["forwarded", "launch-per-digit"])
+@pytest.mark.parametrize("name", ["C3", "C5", "ML256"])
+def test_suggested_radix_is_within_ten_percent_of_the_best_measured(api, name, mode):
+    """vc_suggest_tunables replaces the sweep over bases of the reference's drivers (examples/rbruckv_example.cpp:33-35,
+    98-103): the radix it picks from the model must run within 10 % of the fastest candidate when all are timed, on the
+    shapes of configurations 3 and 5 and on one of the reference's input matrices (reduced sizes)."""
+    import os
+    import time
+    import torch
+    from tests.helpers import INPUTS_DIR
+    if name == "C3":
+        counts, esz = W.counts_zipf(256, 16384, 1.2, 5, 0), 4
+        fn = lambda r, dp, s, d: api.twophase_rbruck_alltoallv(r, dp, s, d)
+    elif name == "C5":
+        counts, esz = W.counts_fft_rows(512, 32, 8192), 8
+        fn = lambda r, dp, s, d: api.tuna_algorithm(r, 0, dp, s, d)
+    else:
+        counts, esz = W.counts_from_npz(os.path.join(INPUTS_DIR, "global_comm_pattern_256proc.npz"), 32), 1
+        fn = lambda r, dp, s, d: api.twophase_rbruck_alltoallv(r, dp, s, d)
+    prob = W.make_problem(counts, esz, 0, 0)
+    dp = api.DeviceProblem(prob)
+    dp.comm.set_forwarding(mode)
+    ds, dr = dp.new_send_arena(), dp.new_recv_arena()
+    dp.fill_payload(0, 3, ds)
+    cands = [2, 4, 8, 16, 32, prob.P]
+    best, b, modelled = api.suggest_tunables(dp, cands)
+    assert best in cands and b == min(best, prob.P) - 1
+    measured = {}
+    for r in cands:
+        for _ in range(2):
+            assert fn(r, dp, ds, dr) == 0, dp.comm.error()
+        times = []
+        for _ in range(7):
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            fn(r, dp, ds, dr)
+            times.append(time.perf_counter() - t0)
+        measured[r] = sorted(times)[len(times) // 2]
+        assert dp.verify(ds, dr) == 0
+    print(name, "mode", mode, "suggested", best, {r: (round(measured[r] * 1e3, 3), round(m * 1e3, 3)) for r, m in zip(cands, modelled)}, flush=True)
+    assert measured[best] <= 1.10 * min(measured.values()), (best, measured)
+    # without a candidate list: the whole range 2 .. min(P, 63) and P
+    free_choice, _, _ = api.suggest_tunables(dp)
+    assert 2 <= free_choice <= prob.P
+    rate, launch = api.calibration(dp.comm)
+    assert 1e12 < rate < 8e12 and 2e-7 < launch < 1e-4, (rate, launch)
+    dp.comm.free()
