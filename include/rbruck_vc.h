@@ -193,6 +193,36 @@ int twolayer_communicator_linear_s2(int n, int bblock1, int bblock2, char *sendb
 int spreadout_alltoallv(char *sendbuf, int *sendcounts, int *sdispls, int sendtype_size, char *recvbuf,
                         int *recvcounts, int *rdispls, int recvtype_size, vc_comm_t comm);
 
+/* ---- _async twins of the seven collectives above (same reference functions: src/rbruckv.h:24-26, 28-33, 39-45, 84-93).
+ * The reference's calls are blocking; on a GPU a caller wants to enqueue a collective behind its producer kernels, time it
+ * with its own events, or overlap two communicators on two streams.  Same arguments plus the stream (a hipStream_t; it
+ * becomes the communicator's stream): the planning kernels and the copy kernel are enqueued and the call returns without
+ * having waited for the device.  The execution is the forwarded one without a work-item list (the copy kernel derives
+ * every block's route itself and checks the planner's verdict on the device before it touches anything), so the batching
+ * tunables have no effect; a workgroup serves each pair of ranks, or a quarter of a wavefront after a call of short blocks.
+ * Calls of very long blocks are served faster by a persistent plan (vc_plan_execute_async).
+ * Until vc_comm_wait the communicator is busy (other calls on it return VC_ERR_BUSY) and the tables, bases and buffers
+ * must stay valid.  The return code covers what the host can check (0, -1, -2, -3, -5); vc_comm_wait reports the rest. */
+int twophase_rbruck_alltoallv_async(int r, char *sendbuf, int *sendcounts, int *sdispls, int sendtype_size, char *recvbuf,
+                                    int *recvcounts, int *rdispls, int recvtype_size, vc_comm_t comm, void *hip_stream);
+int twophase_rbruck_alltoallv_om_async(int r, char *sendbuf, int *sendcounts, int *sdispls, int sendtype_size, char *recvbuf,
+                                       int *recvcounts, int *rdispls, int recvtype_size, vc_comm_t comm, void *hip_stream);
+int tuna_algorithm_async(int r, int b, char *sendbuf, int *sendcounts, int *sdispls, int sendtype_size, char *recvbuf,
+                         int *recvcounts, int *rdispls, int recvtype_size, vc_comm_t comm, void *hip_stream);
+int TTPL_BT_alltoallv_async(int n, int r, int bblock, char *sendbuf, int *sendcounts, int *sdispls, int sendtype_size,
+                            char *recvbuf, int *recvcounts, int *rdispls, int recvtype_size, vc_comm_t comm, void *hip_stream);
+int TTPL_BT_alltoallv_s1_async(int n, int r, int bblock, char *sendbuf, int *sendcounts, int *sdispls, int sendtype_size,
+                               char *recvbuf, int *recvcounts, int *rdispls, int recvtype_size, vc_comm_t comm, void *hip_stream);
+int uniform_spreadout_twolayer_async(int n, int r, char *sendbuf, int sendcount, int sendtype_size, char *recvbuf,
+                                     int recvcount, int recvtype_size, vc_comm_t comm, void *hip_stream);
+int uniform_inverse_isplit_r_bruck_async(int n, int r1, int r2, char *sendbuf, int sendcount, int sendtype_size,
+                                         char *recvbuf, int recvcount, int recvtype_size, vc_comm_t comm, void *hip_stream);
+/* Waits for the communicator's stream and completes the call an _async entry point enqueued: returns VC_ERR_TABLES /
+ * VC_ERR_OVERFLOW when the planner refused the tables (recvbuf is then untouched), VC_ERR_HIP for a runtime failure; when the
+ * staging arena was too small for the call (the copy kernel has then moved nothing) it grows the arena and runs the copy
+ * kernel again before returning.  0 with nothing pending.  vc_comm_last_stats describes the call afterwards. */
+int vc_comm_wait(vc_comm_t comm);
+
 /* No counterpart in the reference.  twophase_rbruck_alltoallv for callers that cannot allocate device memory: code whose
  * surroundings are under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  Same arguments, same
  * result (byte for byte) as twophase_rbruck_alltoallv in its forwarded execution, but the plan tables and the staging

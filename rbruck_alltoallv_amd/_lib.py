@@ -45,6 +45,14 @@ SYMBOLS = {
     "TTPL_BT_alltoallv": (_I, [_I, _I, _I] + _V_TAIL),
     "TTPL_BT_alltoallv_s1": (_I, [_I, _I, _I] + _V_TAIL),
     "TTPL_rbruck_alltoallv": (_I, [_I, _I] + _V_TAIL),
+    "twophase_rbruck_alltoallv_async": (_I, [_I] + _V_TAIL + [_P]),
+    "twophase_rbruck_alltoallv_om_async": (_I, [_I] + _V_TAIL + [_P]),
+    "tuna_algorithm_async": (_I, [_I, _I] + _V_TAIL + [_P]),
+    "TTPL_BT_alltoallv_async": (_I, [_I, _I, _I] + _V_TAIL + [_P]),
+    "TTPL_BT_alltoallv_s1_async": (_I, [_I, _I, _I] + _V_TAIL + [_P]),
+    "uniform_spreadout_twolayer_async": (_I, [_I, _I, _P, _I, _I, _P, _I, _I, _P, _P]),
+    "uniform_inverse_isplit_r_bruck_async": (_I, [_I, _I, _I, _P, _I, _I, _P, _I, _I, _P, _P]),
+    "vc_comm_wait": (_I, [_P]),
     "uniform_spreadout_twolayer": (_I, [_I, _I, _P, _I, _I, _P, _I, _I, _P]),
     "uniform_inverse_isplit_r_bruck": (_I, [_I, _I, _I, _P, _I, _I, _P, _I, _I, _P]),
     "MPICH_intra_scattered": (_I, [_I] + _V_TAIL),

@@ -69,6 +69,10 @@ class VirtualComm:
         self._check(self.lib.vc_comm_staging(self.handle, C.byref(ptr), C.byref(size)))
         return ptr.value or 0, size.value
 
+    def wait(self) -> int:
+        """vc_comm_wait: completes the call an _async entry point enqueued; returns its code."""
+        return self.lib.vc_comm_wait(self.handle)
+
     def error(self) -> str:
         return self.lib.vc_last_error_string().decode()
 
@@ -211,6 +215,19 @@ def exclisive_or_alltoallv(p: DeviceProblem, send: torch.Tensor, recv: torch.Ten
 def spreadout_alltoallv(p: DeviceProblem, send: torch.Tensor, recv: torch.Tensor) -> int:
     """benchmarks/common.cpp:10-37"""
     return p.comm.lib.spreadout_alltoallv(*_tail(p, send, recv))
+
+
+def call_async(name: str, tunables: tuple, p: DeviceProblem, send: torch.Tensor, recv: torch.Tensor, stream: torch.cuda.Stream) -> int:
+    """The _async twin of the alltoallv-shaped entry point `name` (e.g. "tuna_algorithm" with tunables (r, b)): enqueues on
+    `stream` and returns; VirtualComm.wait() completes the call."""
+    return getattr(p.comm.lib, name + "_async")(*tunables, *_tail(p, send, recv), C.c_void_p(stream.cuda_stream))
+
+
+def uniform_async(name: str, tunables: tuple, p: DeviceProblem, count: int, send: torch.Tensor, recv: torch.Tensor,
+                  stream: torch.cuda.Stream) -> int:
+    """The _async twin of uniform_spreadout_twolayer (tunables (n, r)) or uniform_inverse_isplit_r_bruck ((n, r1, r2))."""
+    return getattr(p.comm.lib, name + "_async")(*tunables, send.data_ptr(), count, p.esz, recv.data_ptr(), count, p.esz, p.comm.handle,
+                                                C.c_void_p(stream.cuda_stream))
 
 
 class Plan:

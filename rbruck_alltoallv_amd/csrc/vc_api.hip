@@ -115,6 +115,15 @@ struct vc_comm {
     std::vector<void *> retired_stage;    // staging arenas that were outgrown while plans existed: a HIP graph captured from
                                           // vc_plan_execute_async holds the arena's address, so they stay until the plans go
     std::atomic_flag busy = ATOMIC_FLAG_INIT;   // a call is in progress (a communicator serves one call at a time)
+    struct {                              // a call enqueued by an _async entry point that vc_comm_wait has not collected yet
+        bool active = false;
+        VcSched S;
+        VcTables T;
+        const char *sendbuf = nullptr;
+        char *recvbuf = nullptr;
+        int lanes = 0;
+        int n_launch_infos = 0;
+    } pending;
     PlanBufs B;                           // where the current call's plan lives
     const void *last_stage = nullptr;     // staging arena of the last call
     int64_t *h_header = nullptr;          // pinned, coherent: the planner writes its header straight into it
@@ -151,6 +160,7 @@ struct BusyGuard {
     explicit BusyGuard(vc_comm *comm) : c(comm), mine(comm && !comm->busy.test_and_set(std::memory_order_acquire)) {}
     ~BusyGuard() { if (mine) c->busy.clear(std::memory_order_release); }
     bool ok() const { return !c || mine; }
+    void keep() { mine = false; }         // the call stays in progress after the entry point returns (vc_comm_wait ends it)
 };
 #define VC_ONE_CALL(c)                                                                                              \
     BusyGuard busy_guard_(c);                                                                                       \
@@ -186,6 +196,7 @@ extern "C" int vc_comm_create(int nranks, vc_comm_t *comm_out) {
 extern "C" int vc_comm_free(vc_comm_t c) {
     if (!c) return VC_OK;
     (void)hipStreamSynchronize(c->stream);
+    c->pending.active = false;
     for (DevBuf *b : {&c->slot_off, &c->row_tot, &c->row_base, &c->org_run_base, &c->item_row_tot, &c->item_row_base, &c->row_bytes, &c->desc, &c->header, &c->launches, &c->stage, &c->rd_packed,
                       &c->uni_counts, &c->uni_displs, &c->scratch, &c->chain_row_tot, &c->chain_row_base})
         b->release();
@@ -593,6 +604,53 @@ static int run_schedule(vc_comm *c, VcSched S, std::vector<VcLaunchInfo> &L, con
     return run_items(c, pi, c->desc.p, sendbuf, recvbuf, true);
 }
 
+// The _async entry points: planning kernels and the listless copy kernel are enqueued and the call returns.  The copy
+// kernel checks the planner's verdict on the device (tables, staging arena) and touches nothing when it is bad;
+// vc_comm_wait reads the same verdict and reports it, or grows the arena and runs the copy again.
+static int enqueue_async(vc_comm *c, const VcSched &S, std::vector<VcLaunchInfo> &L, const char *sendbuf, char *recvbuf, VcTables T) {
+    int rc = plan_sizes(c, S, L, T, true);
+    if (rc) return rc;
+    hipStream_t st = c->stream;
+    // a quarter of a wavefront per pair of ranks after a call of short blocks on this communicator, else a workgroup
+    const bool quarter = c->hint_valid && c->hint_max_pieces <= VC_LISTLESS_MAX_PIECES &&
+                         c->hint_payload / std::max<int64_t>(c->hint_items, 1) < VC_LISTLESS_QUARTER_BELOW;
+    const int lanes = quarter ? VC_QUARTER : VC_THREADS;
+    const VcListlessGuard guard = {c->stage.cap >= 64 ? (int64_t)c->stage.cap - 64 : 0, 0, 0, 0};
+    if (c->timing) { HIP_TRY(hipEventRecord(c->events[1], st)); HIP_TRY(hipEventRecord(c->events[2], st)); }
+    HIP_TRY(vc_launch_copy_blocks(S, T, c->B.slot_off, c->B.row_base, c->B.header, guard, lanes, sendbuf, recvbuf, c->stage.as<char>(), st));
+    if (c->timing) HIP_TRY(hipEventRecord(c->events[3], st));
+    c->pending.active = true;
+    c->pending.S = S; c->pending.T = T; c->pending.sendbuf = sendbuf; c->pending.recvbuf = recvbuf; c->pending.lanes = lanes;
+    c->pending.n_launch_infos = (int)L.size();
+    return VC_OK;
+}
+
+extern "C" int vc_comm_wait(vc_comm_t c) {
+    if (!c) return fail_arg("null communicator");
+    HIP_TRY(hipStreamSynchronize(c->stream));
+    if (!c->pending.active) return VC_OK;
+    c->pending.active = false;
+    struct Release { vc_comm *c; ~Release() { c->busy.clear(std::memory_order_release); } } release{c};
+    const VcSched &S = c->pending.S;
+    std::vector<VcLaunchInfo> L((size_t)c->pending.n_launch_infos);     // plan_read only needs their number here
+    PlanInfo pi;
+    int rc = plan_read(c, S, L, pi, true);
+    if (rc) return rc;
+    VcListlessGuard guard = {c->stage.cap >= 64 ? (int64_t)c->stage.cap - 64 : 0, 0, 0, 0};
+    if (!vc_listless_ok(c->h_header, guard)) {            // the arena was too small: nothing has been moved yet
+        HIP_TRY(reserve_stage(c, (size_t)pi.stage_bytes + 64));
+        guard.stage_cap = (int64_t)c->stage.cap - 64;
+        if (c->timing) HIP_TRY(hipEventRecord(c->events[2], c->stream));
+        HIP_TRY(vc_launch_copy_blocks(S, c->pending.T, c->B.slot_off, c->B.row_base, c->B.header, guard, c->pending.lanes,
+                                      c->pending.sendbuf, c->pending.recvbuf, c->stage.as<char>(), c->stream));
+        if (c->timing) HIP_TRY(hipEventRecord(c->events[3], c->stream));
+        HIP_TRY(hipStreamSynchronize(c->stream));
+    }
+    pi.listless = true;
+    pi.chain_lanes = c->pending.lanes;
+    return finish_stats(c, pi, nullptr, true);
+}
+
 static int check_common(vc_comm *c, const void *sendbuf, const void *recvbuf, int esz) {
     if (!c) return fail_arg("null communicator");
     if (!sendbuf || !recvbuf) return fail_arg("null buffer");
@@ -621,19 +679,24 @@ static int schedule_error(int code) {
 }
 
 // The alltoallv-shaped functions.
+// `async_stream` (null: the blocking call): the stream the call is enqueued on; vc_comm_wait collects it.
 static int run_v(VcFunc f, int n, int r, int batch, vc_comm *c, char *sendbuf, int *sendcounts, int *sdispls, int esz,
-                 char *recvbuf, int *recvcounts, int *rdispls, int batch2 = 0) {
+                 char *recvbuf, int *recvcounts, int *rdispls, int batch2 = 0, void **async_stream = nullptr) {
     int rc = check_common(c, sendbuf, recvbuf, esz);
     if (rc) return rc;
     VC_ONE_CALL(c);
     if (!sendcounts || !sdispls || !recvcounts || (f != VC_F_TTPL && !rdispls)) return fail_arg("null table");
     VcSched S;
     std::vector<VcLaunchInfo> L;
-    const bool forward = c->forward != 0;
+    const bool forward = c->forward != 0 || async_stream;
     rc = vc_make_schedule(f, c->P, n, r, batch, esz, 0, S, L, batch2, forward);
     if (rc) return schedule_error(rc);
     S.recv_lo = (int)((uintptr_t)recvbuf & 4095);
-    return run_schedule(c, S, L, sendbuf, recvbuf, make_tables(c, sendcounts, sdispls, recvcounts, rdispls), forward);
+    if (!async_stream) return run_schedule(c, S, L, sendbuf, recvbuf, make_tables(c, sendcounts, sdispls, recvcounts, rdispls), forward);
+    c->stream = static_cast<hipStream_t>(*async_stream);
+    rc = enqueue_async(c, S, L, sendbuf, recvbuf, make_tables(c, sendcounts, sdispls, recvcounts, rdispls));
+    if (rc == VC_OK) busy_guard_.keep();
+    return rc;
 }
 
 extern "C" int twophase_rbruck_alltoallv(int r, char *sendbuf, int *sendcounts, int *sdispls, int sendtype_size, char *recvbuf,
@@ -803,7 +866,7 @@ extern "C" int twolayer_communicator_linear_s2(int n, int bblock1, int bblock2, 
 }
 
 // The alltoall-shaped (equal blocks) functions: the count tables are implied.
-static int run_uniform(VcFunc f, int n, int r, vc_comm *c, char *sendbuf, int sendcount, int esz, char *recvbuf) {
+static int run_uniform(VcFunc f, int n, int r, vc_comm *c, char *sendbuf, int sendcount, int esz, char *recvbuf, void **async_stream = nullptr) {
     int rc = check_common(c, sendbuf, recvbuf, esz);
     if (rc) return rc;
     VC_ONE_CALL(c);
@@ -811,16 +874,20 @@ static int run_uniform(VcFunc f, int n, int r, vc_comm *c, char *sendbuf, int se
     if ((int64_t)sendcount * c->P > 0x7FFFFFFF) return fail_arg("sendcount * P must fit the reference's int displacements");
     VcSched S;
     std::vector<VcLaunchInfo> L;
-    const bool forward = c->forward != 0;
+    const bool forward = c->forward != 0 || async_stream;
     rc = vc_make_schedule(f, c->P, n, r, 0, esz, sendcount, S, L, 0, forward);
     if (rc) return schedule_error(rc);
     S.recv_lo = (int)((uintptr_t)recvbuf & 4095);
+    if (async_stream) c->stream = static_cast<hipStream_t>(*async_stream);
     const size_t PP = (size_t)c->P * c->P;
     HIP_TRY(c->uni_counts.reserve(sizeof(int) * PP));
     HIP_TRY(c->uni_displs.reserve(sizeof(int) * PP));
     HIP_TRY(vc_launch_uniform_tables(c->uni_counts.as<int>(), c->uni_displs.as<int>(), sendcount, c->P, c->stream));
     const int *cnt = c->uni_counts.as<int>(), *dsp = c->uni_displs.as<int>();
-    return run_schedule(c, S, L, sendbuf, recvbuf, make_tables(c, cnt, dsp, cnt, dsp), forward);
+    if (!async_stream) return run_schedule(c, S, L, sendbuf, recvbuf, make_tables(c, cnt, dsp, cnt, dsp), forward);
+    rc = enqueue_async(c, S, L, sendbuf, recvbuf, make_tables(c, cnt, dsp, cnt, dsp));
+    if (rc == VC_OK) busy_guard_.keep();
+    return rc;
 }
 
 extern "C" int uniform_spreadout_twolayer(int n, int r, char *sendbuf, int sendcount, int sendtype_size, char *recvbuf,
@@ -833,6 +900,50 @@ extern "C" int uniform_inverse_isplit_r_bruck(int n, int r1, int r2, char *sendb
                                               char *recvbuf, int recvcount, int recvtype_size, vc_comm_t c) {
     (void)recvcount; (void)recvtype_size; (void)r2;          // r2 is overwritten with the group count (:158)
     return run_uniform(VC_F_UNIFORM_ISPLIT, n, r1, c, sendbuf, sendcount, sendtype_size, recvbuf);
+}
+
+// ---- the _async twins of the seven collectives: enqueue on `hip_stream` (which becomes the communicator's stream) and
+// return; vc_comm_wait completes the call and reports what the planner found.
+extern "C" int twophase_rbruck_alltoallv_async(int r, char *sendbuf, int *sendcounts, int *sdispls, int sendtype_size, char *recvbuf,
+                                               int *recvcounts, int *rdispls, int recvtype_size, vc_comm_t c, void *hip_stream) {
+    (void)recvtype_size;
+    return run_v(VC_F_TWOPHASE, 0, r, 0, c, sendbuf, sendcounts, sdispls, sendtype_size, recvbuf, recvcounts, rdispls, 0, &hip_stream);
+}
+
+extern "C" int twophase_rbruck_alltoallv_om_async(int r, char *sendbuf, int *sendcounts, int *sdispls, int sendtype_size, char *recvbuf,
+                                                  int *recvcounts, int *rdispls, int recvtype_size, vc_comm_t c, void *hip_stream) {
+    (void)recvtype_size;
+    return run_v(VC_F_OM, 0, r, 0, c, sendbuf, sendcounts, sdispls, sendtype_size, recvbuf, recvcounts, rdispls, 0, &hip_stream);
+}
+
+extern "C" int tuna_algorithm_async(int r, int b, char *sendbuf, int *sendcounts, int *sdispls, int sendtype_size, char *recvbuf,
+                                    int *recvcounts, int *rdispls, int recvtype_size, vc_comm_t c, void *hip_stream) {
+    (void)recvtype_size;
+    return run_v(VC_F_TUNA, 0, r, b, c, sendbuf, sendcounts, sdispls, sendtype_size, recvbuf, recvcounts, rdispls, 0, &hip_stream);
+}
+
+extern "C" int TTPL_BT_alltoallv_async(int n, int r, int bblock, char *sendbuf, int *sendcounts, int *sdispls, int sendtype_size,
+                                       char *recvbuf, int *recvcounts, int *rdispls, int recvtype_size, vc_comm_t c, void *hip_stream) {
+    (void)recvtype_size;
+    return run_v(VC_F_TTPL, n, r, bblock, c, sendbuf, sendcounts, sdispls, sendtype_size, recvbuf, recvcounts, rdispls, 0, &hip_stream);
+}
+
+extern "C" int TTPL_BT_alltoallv_s1_async(int n, int r, int bblock, char *sendbuf, int *sendcounts, int *sdispls, int sendtype_size,
+                                          char *recvbuf, int *recvcounts, int *rdispls, int recvtype_size, vc_comm_t c, void *hip_stream) {
+    (void)recvtype_size;
+    return run_v(VC_F_TTPL_S1, n, r, bblock, c, sendbuf, sendcounts, sdispls, sendtype_size, recvbuf, recvcounts, rdispls, 0, &hip_stream);
+}
+
+extern "C" int uniform_spreadout_twolayer_async(int n, int r, char *sendbuf, int sendcount, int sendtype_size, char *recvbuf,
+                                                int recvcount, int recvtype_size, vc_comm_t c, void *hip_stream) {
+    (void)recvcount; (void)recvtype_size;
+    return run_uniform(VC_F_UNIFORM_SPREADOUT, n, r, c, sendbuf, sendcount, sendtype_size, recvbuf, &hip_stream);
+}
+
+extern "C" int uniform_inverse_isplit_r_bruck_async(int n, int r1, int r2, char *sendbuf, int sendcount, int sendtype_size,
+                                                    char *recvbuf, int recvcount, int recvtype_size, vc_comm_t c, void *hip_stream) {
+    (void)recvcount; (void)recvtype_size; (void)r2;
+    return run_uniform(VC_F_UNIFORM_ISPLIT, n, r1, c, sendbuf, sendcount, sendtype_size, recvbuf, &hip_stream);
 }
 
 // ------------------------------------------------------------- persistent plans

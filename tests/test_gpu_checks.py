@@ -307,3 +307,79 @@ def test_suggested_radix_is_within_ten_percent_of_the_best_measured(api, name, m
     rate, launch = api.calibration(dp.comm)
     assert 1e12 < rate < 8e12 and 2e-7 < launch < 1e-4, (rate, launch)
     dp.comm.free()
+
+
+def test_async_twins_overlap_two_communicators(api):
+    """The _async entry points only enqueue: two communicators on two streams run their collectives side by side, each is
+    completed by vc_comm_wait, and both leave the oracle's bytes.  All seven twins, errors reported at the wait, the arena
+    grown at the wait, and the communicator busy in between."""
+    import torch
+    s1, s2 = torch.cuda.Stream(), torch.cuda.Stream()
+    pa = W.make_problem(W.counts_uniform_random(48, 2500, seed=41), 2, 1, 1)
+    pb = W.make_problem(W.counts_normal(64, 700.0, 300.0, 0, 3000, 5), 1, 0, 0)
+    senda, sendb = W.fill_send_arena(pa, 0, 6), W.fill_send_arena(pb, 0, 7)
+    dpa, dpb = api.DeviceProblem(pa), api.DeviceProblem(pb)
+    dsa, dsb = torch.from_numpy(senda).to("cuda:0"), torch.from_numpy(sendb).to("cuda:0")
+    twins = [("twophase_rbruck_alltoallv", (3,), lambda p, s, r: O.twophase_rbruck_alltoallv(3, p, s, r), False),
+             ("twophase_rbruck_alltoallv_om", (4,), lambda p, s, r: O.twophase_rbruck_alltoallv_om(4, p, s, r), False),
+             ("tuna_algorithm", (2, 1), lambda p, s, r: O.tuna_algorithm(2, 1, p, s, r), False),
+             ("TTPL_BT_alltoallv_s1", (8, 2, 3), lambda p, s, r: O.TTPL_BT_alltoallv_s1(8, 2, 3, p, s, r), False),
+             ("TTPL_BT_alltoallv", (8, 8, 0), lambda p, s, r: O.TTPL_BT_alltoallv(8, 8, 0, p, s, r), True)]
+    torch.cuda.synchronize()
+    for k, (name, tun, ofn, packed) in enumerate(twins):
+        print("  async", name, flush=True)
+        other = twins[(k + 1) % 4]                            # another function on the second communicator, at the same time
+        if packed:                                            # the packed layout needs packed receive displacements: pb has them
+            wa = None
+        else:
+            wa = np.full(pa.recv_bytes, 0xEE, dtype=np.uint8)
+            assert ofn(pa, senda, wa) == 0
+        wb = np.full(pb.recv_bytes, 0xEE, dtype=np.uint8)
+        assert (ofn if packed else other[2])(pb, sendb, wb) == 0
+        dra, drb = dpa.new_recv_arena(0xEE), dpb.new_recv_arena(0xEE)
+        torch.cuda.synchronize()
+        if not packed:
+            assert api.call_async(name, tun, dpa, dsa, dra, s1) == 0, dpa.comm.error()
+        bname, btun = (name, tun) if packed else (other[0], other[1])
+        assert api.call_async(bname, btun, dpb, dsb, drb, s2) == 0, dpb.comm.error()
+        # busy until collected
+        assert api.twophase_rbruck_alltoallv(2, dpb, dsb, drb) == _lib.VC_ERR_BUSY
+        assert dpb.comm.wait() == 0, dpb.comm.error()
+        assert np.array_equal(drb.cpu().numpy(), wb), (bname, "second communicator")
+        assert dpb.comm.last_stats().execution == 2 and dpb.comm.last_stats().payload_bytes == pb.payload_bytes
+        if not packed:
+            assert dpa.comm.wait() == 0, dpa.comm.error()
+            assert np.array_equal(dra.cpu().numpy(), wa), (name, "first communicator")
+        assert dpa.comm.wait() == 0                           # nothing pending: just a synchronisation
+    # a table error is found on the device and reported by the wait; recvbuf stays untouched
+    keep = int(dpa.sdispls[5, 6].item())
+    dpa.sdispls[5, 6] = -3
+    dra = dpa.new_recv_arena(0xEE)
+    assert api.call_async("tuna_algorithm", (3, 0), dpa, dsa, dra, s1) == 0
+    assert dpa.comm.wait() == _lib.VC_ERR_TABLES
+    assert bool((dra == 0xEE).all())
+    dpa.sdispls[5, 6] = keep
+    assert api.call_async("twophase_rbruck_alltoallv", (1,), dpa, dsa, dra, s1) == -1 and dpa.comm.wait() == 0
+    dpa.comm.free()
+    dpb.comm.free()
+    # a fresh communicator has no staging arena: the copy kernel refuses on the device and the wait redoes it
+    pc = W.make_problem(W.counts_uniform_random(40, 5000, seed=43), 1, 0, 0)
+    sendc = W.fill_send_arena(pc, 0, 8)
+    dpc = api.DeviceProblem(pc)
+    dsc, drc = torch.from_numpy(sendc).to("cuda:0"), dpc.new_recv_arena(0xEE)
+    assert api.call_async("twophase_rbruck_alltoallv", (2,), dpc, dsc, drc, s1) == 0
+    assert dpc.comm.wait() == 0, dpc.comm.error()
+    assert dpc.comm.last_stats().staging_bytes > 0
+    assert np.array_equal(drc.cpu().numpy(), W.expected_recv_arena(pc, sendc))
+    dpc.comm.free()
+    # the equal-block twins
+    up = W.make_uniform_problem(48, 333, 2)
+    dpu = api.DeviceProblem(up)
+    dsu = dpu.new_send_arena()
+    dpu.fill_payload(0, 9, dsu)
+    for name, tun in (("uniform_spreadout_twolayer", (8, 3)), ("uniform_inverse_isplit_r_bruck", (6, 2, 2))):
+        dru = dpu.new_recv_arena(0xEE)
+        assert api.uniform_async(name, tun, dpu, 333, dsu, dru, s2) == 0, dpu.comm.error()
+        assert dpu.comm.wait() == 0, dpu.comm.error()
+        assert dpu.verify(dsu, dru) == 0, name
+    dpu.comm.free()
