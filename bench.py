@@ -217,8 +217,10 @@ def cpu_baseline(name: str, seed: int, budget_s: float) -> dict:
 EXECUTION_NAMES = {0: "launch per digit phase",
                    1: "forwarded (one launch, blocks carried through all hops in registers)",
                    2: "forwarded, without a work-item list (every pair of ranks derives its block's route in the copy kernel; "
-                      "one host synchronisation per call)"}
-EXECUTION_KERNELS = {0: "vc_copy_items", 1: "vc_copy_chains", 2: "vc_copy_blocks"}
+                      "one host synchronisation per call)",
+                   3: "forwarded, without a work-item list, staging slots at a fixed stride (one pass over the count tables "
+                      "instead of the planner's prefix sums; one host synchronisation per call)"}
+EXECUTION_KERNELS = {0: "vc_copy_items", 1: "vc_copy_chains", 2: "vc_copy_blocks", 3: "vc_copy_blocks"}
 
 
 def kernel_name(st) -> str:
@@ -226,7 +228,7 @@ def kernel_name(st) -> str:
     base, lanes = EXECUTION_KERNELS[int(st.execution)], int(st.lanes_per_item)
     if lanes == 16:
         return base + "_quarter_kernel"
-    return base + "_kernel" + ("" if st.execution == 2 else f"<{lanes}>")
+    return base + "_kernel" + f"<{lanes}>"
 
 
 def copy_ceiling(comm, torch, mib: int = 2048, reps: int = 5) -> dict:

@@ -73,8 +73,12 @@ int vc_comm_set_bases(vc_comm_t comm, const int64_t *sbase_bytes, const int64_t 
  *    kernel writes first (after the host has learnt its size).  When the last call on the communicator consisted of
  *    short blocks, the next one goes without the list: every pair of ranks gets a workgroup (at most 128 ranks) or a
  *    quarter of a wavefront (short blocks: average piece below 768 B on any number of ranks, below 1.75 - 3 KiB on 33 - 128) that derives its block's route itself; the
- *    kernel is enqueued right behind the size computation and the call needs one host synchronisation instead of two
- *    (26 - 35 us instead of 42 - 47 us per call at 64 ranks on MI355X, 10 - 25 % less at 256 and 1024 ranks).
+ *    kernel is enqueued right behind the size computation and the call needs one host synchronisation instead of two.
+ *    Such a call also gets the reference's own staging layout, every slot as long as the longest block
+ *    (src/twophase_tunable_rbruckv.cpp:59; the stride comes from the last call's longest block, and the copy kernel checks
+ *    on the device that this call's blocks fit): slot addresses are then closed forms, and one pass over the count tables
+ *    replaces the planner's prefix sums and slot tables.  Only on at most 128 ranks and while regions x P x P x stride
+ *    stays below 256 MiB.
  * 2: forwarded, always through the list.   3 / 4: forwarded, always without it, a workgroup / a quarter of a wavefront
  *    per pair of ranks (any sizes; not the fastest choice everywhere).
  * 0: one kernel launch per digit phase (or per batch of its rounds, as b / bblock say); every hop reads the block
@@ -306,9 +310,9 @@ typedef struct {
     int64_t launch_bytes[VC_MAX_LAUNCHES];   /* bytes the hops of a launch copy (forwarded execution: [0] = moved_bytes) */
     float launch_ms[VC_MAX_LAUNCHES];  /* per data-moving launch, HIP events on the comm's stream */
     int32_t execution;           /* how the call ran: 0 launch per digit, 1 forwarded through a work-item list, 2 forwarded
-                                    without one (see vc_comm_set_forwarding) */
+                                    without one, 3 forwarded without one on fixed-stride staging (see vc_comm_set_forwarding) */
     int32_t lanes_per_item;      /* 256: the copy kernel gave every work item (without a list: every pair of ranks) a
-                                    workgroup; 64: a wavefront (lists of short pieces); 16: a quarter of one (pieces of a
+                                    workgroup; 64: a wavefront (short pieces); 16: a quarter of one (pieces of a
                                     few hundred bytes).  Launch-per-digit execution: of the launch that moved the most bytes. */
 } vc_stats_t;
 

@@ -55,6 +55,10 @@ struct VcSched {
     int last_hop;     // which blocks make a hop that is no digit round and ends in recvbuf, besides every rank's block to
                       // itself: 0 none (one-layer Bruck; Bruck over the nodes), 1 those that change node (inter-node
                       // messages), 2 all (direct one-hop functions)
+    int stride;       // > 0: staging slots at a fixed stride of this many bytes (a multiple of VC_LINE that holds the longest block
+                      //    at any cache-line phase), the reference's own layout (src/twophase_tunable_rbruckv.cpp:59): slot `id`
+                      //    of rank `holder` in region x starts at ((x P + holder) P + id) stride, a closed form, and the planner's
+                      //    prefix sums and slot tables are not needed.  0: compact slots at prefix-sum offsets.
     int coalesce;     // 1: blocks that are about to leave their node wait in "organized" runs — the n blocks one rank
                       //    holds for one destination rank back to back in source order — so that an inter-node message
                       //    is a contiguous copy (TTPL_BT_alltoallv, src/twophase_twolayer_rbruck.cpp:388-398, 430-453).
@@ -117,8 +121,10 @@ hipError_t vc_launch_empty(hipStream_t st);
 //       differ from sendcounts[s][t]; plus VC_BAD_OVERFLOW per rank whose packed receive layout overflows an int
 //   [4] the most pieces any block is cut into (forwarded execution)
 //   [5 + L] bytes moved by launch L   [5 + nl + L] work items of launch L
-//   (forwarded execution: [5] all moved bytes, no per-launch words)
+//   (forwarded execution: [5] all moved bytes, [6] the longest block, no per-launch words)
 #define VC_HEADER_FIXED 5
+// forwarded execution: the longest block of the call, bytes
+#define VC_HEADER_MAX_LEN (VC_HEADER_FIXED + 1)
 #define VC_HEADER_BAD 3
 // added to header[VC_HEADER_BAD] once per rank whose packed receive displacements would pass INT_MAX elements
 #define VC_BAD_OVERFLOW (1ll << 40)
@@ -133,6 +139,10 @@ hipError_t vc_launch_plan_sizes(const VcSched &S, const VcLaunchInfo *launches_h
                                 int64_t *row_tot, int64_t *row_base, int64_t *org_run_base, int64_t *item_row_tot,
                                 int64_t *item_row_base, int64_t *row_bytes, int64_t *chain_row_tot, int64_t *chain_row_base,
                                 int64_t *header, int64_t *header_host, hipStream_t st);
+// Fixed-stride staging (S.stride > 0), forwarded execution: one pass over the tables instead of the prefix sums —
+// validation, payload, block pieces, longest block, hop-weighted bytes — added up into `header` (device; the caller has
+// zeroed words 0 .. VC_HEADER_MAX_LEN).  header[0] is set to the bytes the fixed-stride arena takes.
+hipError_t vc_launch_scan_tables(const VcSched &S, VcTables T, int64_t *header, hipStream_t st);
 // Forwarded execution: the chain items (every block's route in closed form, staging addresses from the plan tables).
 // chain_chunk_pre: [P][chunks of VC_THREADS sources] items of a receiver before each chunk (vc_launch_plan_sizes leaves it
 // behind chain_row_tot's first 2 P words).
@@ -160,10 +170,12 @@ struct VcListlessGuard {
     int64_t max_pieces;     // most pieces of one block
     int64_t max_items;      // block pieces in all
     int64_t max_average;    // average piece, bytes
+    int64_t max_len;        // longest block, bytes (fixed-stride staging: what a slot holds at any phase)
 };
 
 VC_HD bool vc_listless_ok(const int64_t *header, const VcListlessGuard &g) {
     if (header[0] > g.stage_cap || header[VC_HEADER_BAD] != 0) return false;
+    if (g.max_len && header[VC_HEADER_MAX_LEN] > g.max_len) return false;
     if (g.max_pieces && header[VC_HEADER_MAX_PIECES] > g.max_pieces) return false;
     if (g.max_items && header[2] > g.max_items) return false;
     return !(g.max_average && header[1] > g.max_average * header[2]);
@@ -172,7 +184,12 @@ VC_HD bool vc_listless_ok(const int64_t *header, const VcListlessGuard &g) {
 // Forwarded execution without a work-item list: one workgroup (or a quarter of a wavefront) per (source, destination)
 // pair works out the route of its block from the plan tables and carries it through.  Reads the device `header` the
 // planning kernels before it on the stream have written and does nothing unless vc_listless_ok(header, guard).
-// lanes: VC_THREADS (a workgroup per pair) or VC_QUARTER (a quarter of a wavefront per pair, for blocks of a few hundred bytes).
+// lanes: VC_THREADS (a workgroup per pair), VC_WAVE (a wavefront per pair, blocks of a KiB or two) or VC_QUARTER (a quarter of a
+// wavefront per pair, for blocks of a few hundred bytes).
+// header_host (pinned, may be null): the first workgroup copies the fixed words of `header` there, for planners that add
+// the header up with atomics and cannot write it to the host themselves.  header_zero (may be null): ... and clears the
+// fixed words there: the header the next call's planner will add up into.
 hipError_t vc_launch_copy_blocks(const VcSched &S, VcTables T, const int64_t *slot_off, const int64_t *row_base, const int64_t *header,
-                                 VcListlessGuard guard, int lanes, const char *sendbuf, char *recvbuf, char *stage, hipStream_t st);
+                                 VcListlessGuard guard, int lanes, const char *sendbuf, char *recvbuf, char *stage, hipStream_t st,
+                                 int64_t *header_host = nullptr, int64_t *header_zero = nullptr);
 hipError_t vc_launch_calibration_copy(const char *src, char *dst, int64_t nbytes, hipStream_t st);

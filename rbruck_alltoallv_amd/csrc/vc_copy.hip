@@ -198,23 +198,35 @@ __global__ __launch_bounds__(VC_WAVE) void vc_copy_items_quarter_kernel(const Vc
 // planning kernels, before the host has seen their result, so it checks that result itself: nothing is touched when the
 // plan needs more staging than there is, the tables hold negative entries, or the call is not of the kind the host
 // expected when it chose this kernel (the host, which evaluates the same condition afterwards, then takes another path).
-__global__ __launch_bounds__(VC_THREADS) void vc_copy_blocks_kernel(VcSched S, VcTables T, const int64_t *__restrict__ slot_off,
-                                                                    const int64_t *__restrict__ row_base,
-                                                                    const int64_t *__restrict__ header, VcListlessGuard guard,
-                                                                    int64_t first_pair, const char *__restrict__ sendbuf,
-                                                                    char *__restrict__ recvbuf, char *__restrict__ stage) {
-    if (!vc_listless_ok(header, guard)) return;
+// LANES = VC_THREADS: a workgroup of four wavefronts per pair; LANES = VC_WAVE: one wavefront per pair, for blocks of a
+// KiB or two (a quarter of the wavefronts to start, all of them with work).
+template <int LANES>
+__global__ __launch_bounds__(LANES) void vc_copy_blocks_kernel(VcSched S, VcTables T, const int64_t *__restrict__ slot_off,
+                                                               const int64_t *__restrict__ row_base,
+                                                               const int64_t *__restrict__ header, VcListlessGuard guard,
+                                                               int64_t first_pair, const char *__restrict__ sendbuf,
+                                                               char *__restrict__ recvbuf, char *__restrict__ stage,
+                                                               int64_t *__restrict__ header_host, int64_t *__restrict__ header_zero) {
     __shared__ int64_t route[VC_MAX_HOP_SLOTS];
     __shared__ int route_len;
     const int64_t per = gridDim.x / VC_XCDS;
     const int64_t idx = first_pair + (int64_t)(blockIdx.x % VC_XCDS) * per + blockIdx.x / VC_XCDS;
-    if (idx >= (int64_t)S.P * S.P) return;
-    const int t = (int)(idx / S.P), s = (int)(idx % S.P);
+    const bool inside = idx < (int64_t)S.P * S.P;
+    const int t = inside ? (int)(idx / S.P) : 0, s = inside ? (int)(idx % S.P) : 0;
+    // Everything the block's addresses depend on is loaded before the planner's verdict is looked at: the loads are
+    // independent of each other and of the verdict (tables are always readable), so they travel together instead of one
+    // memory round trip after the other; nothing is stored before the verdict is known.
     const int64_t len = (int64_t)T.sc[(int64_t)s * S.P + t] * S.esz;
-    if (len <= 0) return;
+    const int64_t send_off = vc_send_offset(S, T, s, t);
+    const int64_t recv_off = vc_recv_offset(S, T, s, t);
+    int64_t dst = 0;
+    const bool moves = threadIdx.x < VC_WAVE && (int)threadIdx.x < vc_hop_slots(S) && vc_block_hop(S, T, slot_off, row_base, s, t, threadIdx.x, dst);
+    if (blockIdx.x == 0 && first_pair == 0 && threadIdx.x <= VC_HEADER_MAX_LEN) {
+        if (header_host) header_host[threadIdx.x] = header[threadIdx.x];
+        if (header_zero) header_zero[threadIdx.x] = 0;    // the header the next call will add up into
+    }
+    if (!vc_listless_ok(header, guard) || !inside || len <= 0) return;
     if (threadIdx.x < VC_WAVE) {                          // hop slots <= VC_MAX_HOP_SLOTS < lanes of the first wavefront
-        int64_t dst = 0;
-        const bool moves = (int)threadIdx.x < vc_hop_slots(S) && vc_block_hop(S, T, slot_off, row_base, s, t, threadIdx.x, dst);
         const unsigned long long mask = __ballot(moves);
         if (moves) route[__popcll(mask & ((1ull << threadIdx.x) - 1))] = dst;
         if (threadIdx.x == 0) route_len = __popcll(mask);
@@ -222,13 +234,13 @@ __global__ __launch_bounds__(VC_THREADS) void vc_copy_blocks_kernel(VcSched S, V
     __syncthreads();
     const int nhop = route_len;
     if (nhop <= 0) return;
-    const char *src = sendbuf + vc_send_offset(S, T, s, t);
-    const int phase = vc_phase(S, T, s, t), cut = vc_chain_cut(S, T, s, t);
+    const char *src = sendbuf + send_off;
+    const int phase = (int)((recv_off + S.recv_lo) & (VC_LINE - 1)), cut = (int)((recv_off + S.recv_lo) & (VC_PIECE - 1));
     const int64_t pieces = vc_chunk_count(len, phase, cut);
     for (int64_t c = 0; c < pieces; c++) {                // the same cuts as the chain items of this block
         int64_t lo, hi;
         vc_piece_range(len, phase, cut, c, lo, hi);
-        vc_forward_piece<VC_THREADS>(src + lo, hi - lo, nhop, [&](int k) { return vc_resolve(route[k] + lo, sendbuf, recvbuf, stage); });
+        vc_forward_piece<LANES>(src + lo, hi - lo, nhop, [&](int k) { return vc_resolve(route[k] + lo, sendbuf, recvbuf, stage); });
     }
 }
 
@@ -238,25 +250,29 @@ __global__ __launch_bounds__(VC_WAVE) void vc_copy_blocks_quarter_kernel(VcSched
                                                                          const int64_t *__restrict__ row_base,
                                                                          const int64_t *__restrict__ header, VcListlessGuard guard,
                                                                          int64_t first_pair, const char *__restrict__ sendbuf,
-                                                                         char *__restrict__ recvbuf, char *__restrict__ stage) {
-    if (!vc_listless_ok(header, guard)) return;
+                                                                         char *__restrict__ recvbuf, char *__restrict__ stage,
+                                                                         int64_t *__restrict__ header_host, int64_t *__restrict__ header_zero) {
     __shared__ int64_t route[VC_ITEMS_PER_WAVE][VC_MAX_HOP_SLOTS];
     const int64_t per = gridDim.x / VC_XCDS;
     const int64_t wave = (int64_t)(blockIdx.x % VC_XCDS) * per + blockIdx.x / VC_XCDS;
     const int g = threadIdx.x / VC_QUARTER, q = threadIdx.x % VC_QUARTER;
     const int64_t idx = first_pair + wave * VC_ITEMS_PER_WAVE + g;
-    int t = 0, s = 0;
-    int64_t len = 0;
-    if (idx < (int64_t)S.P * S.P) {
-        t = (int)(idx / S.P);
-        s = (int)(idx % S.P);
-        len = (int64_t)T.sc[(int64_t)s * S.P + t] * S.esz;
-    }
+    const bool inside = idx < (int64_t)S.P * S.P;
+    const int t = inside ? (int)(idx / S.P) : 0, s = inside ? (int)(idx % S.P) : 0;
+    // all loads the addresses depend on go out before the planner's verdict is looked at (see vc_copy_blocks_kernel)
+    const int64_t len = inside ? (int64_t)T.sc[(int64_t)s * S.P + t] * S.esz : 0;
+    const int64_t send_off = vc_send_offset(S, T, s, t);
+    const int64_t recv_off = vc_recv_offset(S, T, s, t);
     const bool active = len > 0;                          // no lane leaves before the barrier below
     const int nslots = vc_hop_slots(S);
     int64_t d0 = 0, d1 = 0;
     const bool m0 = active && q < nslots && vc_block_hop(S, T, slot_off, row_base, s, t, q, d0);
     const bool m1 = active && q + VC_QUARTER < nslots && vc_block_hop(S, T, slot_off, row_base, s, t, q + VC_QUARTER, d1);
+    if (blockIdx.x == 0 && first_pair == 0 && threadIdx.x <= VC_HEADER_MAX_LEN) {
+        if (header_host) header_host[threadIdx.x] = header[threadIdx.x];
+        if (header_zero) header_zero[threadIdx.x] = 0;
+    }
+    if (!vc_listless_ok(header, guard)) return;           // the same for every lane of the grid
     const unsigned g0 = (unsigned)(__ballot(m0) >> (g * VC_QUARTER)) & 0xFFFFu;      // the group's hops among slots 0..15
     const unsigned g1 = (unsigned)(__ballot(m1) >> (g * VC_QUARTER)) & 0xFFFFu;      // ... among slots 16..31
     if (m0) route[g][__popc(g0 & ((1u << q) - 1))] = d0;
@@ -264,8 +280,8 @@ __global__ __launch_bounds__(VC_WAVE) void vc_copy_blocks_quarter_kernel(VcSched
     __syncthreads();
     const int nhop = __popc(g0) + __popc(g1);
     if (!active || nhop <= 0) return;
-    const char *src = sendbuf + vc_send_offset(S, T, s, t);
-    const int phase = vc_phase(S, T, s, t), cut = vc_chain_cut(S, T, s, t);
+    const char *src = sendbuf + send_off;
+    const int phase = (int)((recv_off + S.recv_lo) & (VC_LINE - 1)), cut = (int)((recv_off + S.recv_lo) & (VC_PIECE - 1));
     const int64_t pieces = vc_chunk_count(len, phase, cut);
     for (int64_t c = 0; c < pieces; c++) {
         int64_t lo, hi;
@@ -275,7 +291,8 @@ __global__ __launch_bounds__(VC_WAVE) void vc_copy_blocks_quarter_kernel(VcSched
 }
 
 hipError_t vc_launch_copy_blocks(const VcSched &S, VcTables T, const int64_t *slot_off, const int64_t *row_base, const int64_t *header,
-                                 VcListlessGuard guard, int lanes, const char *sendbuf, char *recvbuf, char *stage, hipStream_t st) {
+                                 VcListlessGuard guard, int lanes, const char *sendbuf, char *recvbuf, char *stage, hipStream_t st,
+                                 int64_t *header_host, int64_t *header_zero) {
     const int64_t npairs = (int64_t)S.P * S.P;
     const int64_t step = lanes == VC_QUARTER ? VC_MAX_GRID * VC_ITEMS_PER_WAVE : VC_MAX_GRID;
     for (int64_t done = 0; done < npairs; done += step) {
@@ -284,10 +301,13 @@ hipError_t vc_launch_copy_blocks(const VcSched &S, VcTables T, const int64_t *sl
         const dim3 grid((unsigned)((units + VC_XCDS - 1) / VC_XCDS * VC_XCDS));
         if (lanes == VC_QUARTER)
             hipLaunchKernelGGL(vc_copy_blocks_quarter_kernel, grid, dim3(VC_WAVE), 0, st, S, T, slot_off, row_base, header, guard, done,
-                               sendbuf, recvbuf, stage);
+                               sendbuf, recvbuf, stage, header_host, header_zero);
+        else if (lanes == VC_WAVE)
+            hipLaunchKernelGGL(vc_copy_blocks_kernel<VC_WAVE>, grid, dim3(VC_WAVE), 0, st, S, T, slot_off, row_base, header, guard, done,
+                               sendbuf, recvbuf, stage, header_host, header_zero);
         else
-            hipLaunchKernelGGL(vc_copy_blocks_kernel, grid, dim3(VC_THREADS), 0, st, S, T, slot_off, row_base, header, guard, done,
-                               sendbuf, recvbuf, stage);
+            hipLaunchKernelGGL(vc_copy_blocks_kernel<VC_THREADS>, grid, dim3(VC_THREADS), 0, st, S, T, slot_off, row_base, header, guard,
+                               done, sendbuf, recvbuf, stage, header_host, header_zero);
     }
     return hipGetLastError();
 }

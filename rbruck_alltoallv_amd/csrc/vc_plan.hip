@@ -24,7 +24,7 @@
 // Forwarded execution (chain_row_tot != null, nl = 0): grid (P, regions + 1).  The region rows also sum the bytes of the
 // blocks themselves (every staged block is one hop), and the last row counts the chain items of the blocks that end on
 // the rank, the most pieces of any of them, the payload and the negative table entries.
-// row_bytes rows: [launch or region][P], then [payload][P], then [negative entries][P].
+// row_bytes rows: [launch or region][P], then [payload][P], then [negative entries][P], then (forwarded) [longest block][P].
 __global__ __launch_bounds__(VC_THREADS) void vc_plan_rows(VcSched S, VcLaunchPack pack, const VcLaunchInfo *__restrict__ launches, int nl, VcTables T,
                                                            int64_t *__restrict__ slot_off, int64_t *__restrict__ row_tot,
                                                            int64_t *__restrict__ item_row_tot, int64_t *__restrict__ row_bytes,
@@ -53,7 +53,7 @@ __global__ __launch_bounds__(VC_THREADS) void vc_plan_rows(VcSched S, VcLaunchPa
         }
         return;
     }
-    int64_t items = 0, bytes = 0, payload = 0, most = 0;
+    int64_t items = 0, bytes = 0, payload = 0, most = 0, longest = 0;
     int64_t bad = 0;                                      // entries of this rank's rows no rank could have passed
     const int L = blockIdx.y - nreg;
     if (forward) {
@@ -66,6 +66,8 @@ __global__ __launch_bounds__(VC_THREADS) void vc_plan_rows(VcSched S, VcLaunchPa
             // the receiver must expect exactly what the source sends (the reference fails with an MPI truncation error)
             bad += s < P && T.rc[(int64_t)to * P + s] != T.sc[(int64_t)s * P + to];
             most = cnt > most ? cnt : most;
+            const int64_t len = s < P ? (int64_t)T.sc[(int64_t)s * P + to] * S.esz : 0;
+            longest = len > longest ? len : longest;
             if (threadIdx.x == 0) chain_row_tot[2 * (int64_t)P + (int64_t)to * nchunk + chunk] = before;
             before += vc_block_sum(cnt, lds);
         }
@@ -90,7 +92,7 @@ __global__ __launch_bounds__(VC_THREADS) void vc_plan_rows(VcSched S, VcLaunchPa
             if (!forward) bad += T.rc[i] != T.sc[(int64_t)id * P + to];      // forwarded execution has compared them above
         }
     items = vc_block_sum(items, lds);
-    if (forward) most = vc_block_max(most, lds); else bytes = vc_block_sum(bytes, lds);
+    if (forward) { most = vc_block_max(most, lds); longest = vc_block_max(longest, lds); } else bytes = vc_block_sum(bytes, lds);
     if (L == 0) {
         payload = vc_block_sum(payload, lds);
         bad = vc_block_sum(bad, lds);
@@ -98,7 +100,7 @@ __global__ __launch_bounds__(VC_THREADS) void vc_plan_rows(VcSched S, VcLaunchPa
         if (S.packed_recv && payload > (int64_t)0x7FFFFFFF * S.esz) bad += VC_BAD_OVERFLOW;
     }
     if (threadIdx.x == 0) {
-        if (forward) { chain_row_tot[to] = items; chain_row_tot[P + to] = most; }
+        if (forward) { chain_row_tot[to] = items; chain_row_tot[P + to] = most; row_bytes[(int64_t)(nsum + 2) * P + to] = longest; }
         else { item_row_tot[(int64_t)L * P + to] = items; row_bytes[(int64_t)L * P + to] = bytes; }
         if (L == 0) { row_bytes[(int64_t)nsum * P + to] = payload; row_bytes[(int64_t)(nsum + 1) * P + to] = bad; }
     }
@@ -141,18 +143,24 @@ __global__ __launch_bounds__(VC_THREADS) void vc_plan_bases(int P, int w, int nr
     const int nsum = forward ? nreg : nl;                 // rows of row_bytes before the payload row
     int64_t carry = 0, bytes = 0;
     if (forward && L == 1) {                              // first chain item of every final receiver
-        int64_t most = 0;
+        int64_t most = 0, longest = 0;
         for (int b0 = 0; b0 < P; b0 += VC_THREADS) {
             const int i = b0 + threadIdx.x;
             int64_t total;
             const int64_t ex = vc_block_exclusive_scan((i < P) ? chain_row_tot[i] : 0, lds, total);
-            if (i < P) { chain_row_base[i] = carry + ex; most = chain_row_tot[P + i] > most ? chain_row_tot[P + i] : most; }
+            if (i < P) {
+                chain_row_base[i] = carry + ex;
+                most = chain_row_tot[P + i] > most ? chain_row_tot[P + i] : most;
+                const int64_t len = row_bytes[(int64_t)(nsum + 2) * P + i];
+                longest = len > longest ? len : longest;
+            }
             carry += total;
         }
         most = vc_block_max(most, lds);
+        longest = vc_block_max(longest, lds);
         if (threadIdx.x == 0) {
-            header[2] = carry; header[VC_HEADER_MAX_PIECES] = most;
-            if (header_host) { header_host[2] = carry; header_host[VC_HEADER_MAX_PIECES] = most; }
+            header[2] = carry; header[VC_HEADER_MAX_PIECES] = most; header[VC_HEADER_MAX_LEN] = longest;
+            if (header_host) { header_host[2] = carry; header_host[VC_HEADER_MAX_PIECES] = most; header_host[VC_HEADER_MAX_LEN] = longest; }
         }
         return;
     }
@@ -375,6 +383,54 @@ hipError_t vc_launch_chain_plan(const VcSched &S, VcTables T, const int64_t *slo
     const int slices = nchunk > 1 ? 1 : vc_emit_slices(nitems, S.P);
     hipLaunchKernelGGL(vc_chain_emit, dim3(S.P, nchunk * slices), dim3(VC_THREADS), 0, st, S, T, slot_off, row_base, chain_row_base,
                        chain_chunk_pre, slices, items);
+    return hipGetLastError();
+}
+
+// ---- fixed-stride staging: one pass over the tables instead of the prefix sums ----
+// One pair of ranks per lane (pairs in the order of the chain items: by receiver, then source).  Every workgroup adds
+// its part into the header (zeroed before): [1] payload, [2] block pieces, [3] table entries no rank could have passed,
+// [4] the most pieces of a block (max), [5] hop-weighted bytes, [6] the longest block (max).
+// [0] is the size of the fixed-stride arena.
+__global__ __launch_bounds__(VC_THREADS) void vc_scan_tables_kernel(VcSched S, VcTables T, int64_t *__restrict__ header) {
+    __shared__ int64_t lds[VC_WAVES_PER_BLOCK];
+    const int P = S.P;
+    const int64_t idx = (int64_t)blockIdx.x * VC_THREADS + threadIdx.x;
+    int64_t payload = 0, items = 0, bad = 0, most = 0, moved = 0, longest = 0;
+    if (idx < (int64_t)P * P) {
+        const int to = (int)(idx / P), s = (int)(idx % P);
+        const int64_t i = (int64_t)to * P + s, k = (int64_t)s * P + to;
+        const int sc = T.sc[k], rc = T.rc[i];
+        bad = (sc < 0) | (rc != sc) | (T.sd[i] < 0) | (!S.packed_recv && T.rd[i] < 0);
+        // (a packed receive layout past INT_MAX elements shows as a negative packed displacement of a later source)
+        if (S.packed_recv && (T.rd_packed[i] < 0 || (s == P - 1 && (int64_t)T.rd_packed[i] + rc > 0x7FFFFFFF))) bad += VC_BAD_OVERFLOW;
+        const int64_t len = (int64_t)sc * S.esz;
+        const int64_t cnt = sc > 0 ? vc_chain_count(S, T, s, to) : 0;
+        payload = len;
+        items = most = cnt;
+        moved = len * vc_block_hops(S, s, to);
+        longest = len;
+    }
+    payload = vc_block_sum(payload, lds);
+    items = vc_block_sum(items, lds);
+    bad = vc_block_sum(bad, lds);
+    moved = vc_block_sum(moved, lds);
+    most = vc_block_max(most, lds);
+    longest = vc_block_max(longest, lds);
+    if (threadIdx.x == 0) {
+        unsigned long long *h = reinterpret_cast<unsigned long long *>(header);
+        if (blockIdx.x == 0) header[0] = vc_strided_stage_bytes(S);
+        if (payload) atomicAdd(&h[1], (unsigned long long)payload);
+        if (items) atomicAdd(&h[2], (unsigned long long)items);
+        if (bad) atomicAdd(&h[VC_HEADER_BAD], (unsigned long long)bad);
+        if (moved) atomicAdd(&h[VC_HEADER_FIXED], (unsigned long long)moved);
+        if (most) atomicMax(&h[VC_HEADER_MAX_PIECES], (unsigned long long)most);
+        if (longest) atomicMax(&h[VC_HEADER_MAX_LEN], (unsigned long long)longest);
+    }
+}
+
+hipError_t vc_launch_scan_tables(const VcSched &S, VcTables T, int64_t *header, hipStream_t st) {
+    const int64_t pairs = (int64_t)S.P * S.P;
+    hipLaunchKernelGGL(vc_scan_tables_kernel, dim3((unsigned)((pairs + VC_THREADS - 1) / VC_THREADS)), dim3(VC_THREADS), 0, st, S, T, header);
     return hipGetLastError();
 }
 

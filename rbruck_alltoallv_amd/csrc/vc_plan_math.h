@@ -150,7 +150,22 @@ VC_HD int64_t vc_region_slot_size(const VcSched &S, const VcTables &T, int y, in
 VC_HD int64_t vc_stage_addr(const VcSched &S, const VcTables &T, const int64_t *slot_off, const int64_t *row_base,
                             int x, int holder, int id, int s, int t) {
     const int64_t row = (int64_t)x * S.P + holder;
+    if (S.stride) return (row * S.P + id) * S.stride + vc_phase(S, T, s, t);
     return row_base[row] + slot_off[row * S.P + id] + vc_phase(S, T, s, t);
+}
+
+// Bytes of staging arena a fixed-stride layout takes.
+VC_HD int64_t vc_strided_stage_bytes(const VcSched &S) { return (int64_t)(S.w + S.w2) * S.P * S.P * S.stride; }
+
+// Hops of block (s, t): the digit rounds it moves in, plus the hop that is no digit round (vc_block_hop's last slot).
+VC_HD int vc_block_hops(const VcSched &S, int s, int t) {
+    if (s == t) return 1;
+    const int n = S.n, G = S.G, r = S.r;
+    const int gs = s / n, gt = t / n;
+    int hops = (S.last_hop == 2 || (S.last_hop == 1 && gs != gt)) ? 1 : 0;
+    if (S.w) for (int j = (s % n - t % n + n) % n; j; j /= r) hops += (j % r) != 0;
+    if (S.w2) for (int j = (gs - gt + G) % G; j; j /= r) hops += (j % r) != 0;
+    return hops;
 }
 
 VC_HD int64_t vc_send_offset(const VcSched &S, const VcTables &T, int s, int t) {

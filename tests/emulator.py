@@ -43,7 +43,7 @@ class Result:
         self.traffic = traffic[: self.nlaunch] if rc == 0 else None
 
 
-def emulate(func, prob, send, recv, n=0, r=2, batch=0, uniform_count=0, recv_lo=0, batch2=0, forward=None) -> Result:
+def emulate(func, prob, send, recv, n=0, r=2, batch=0, uniform_count=0, recv_lo=0, batch2=0, forward=None, stride=0) -> Result:
     global _lib
     if _lib is None:
         _lib = C.CDLL(build())
@@ -54,7 +54,7 @@ def emulate(func, prob, send, recv, n=0, r=2, batch=0, uniform_count=0, recv_lo=
                            C.c_int(uniform_count), _p(send), C.c_int64(send.size), _p(recv), C.c_int64(recv.size),
                            _p(prob.sbase), _p(prob.rbase), _p(prob.sendcounts), _p(prob.sdispls), _p(prob.recvcounts),
                            _p(prob.rdispls), C.c_int(recv_lo), _p(stats), _p(traffic), C.c_int(MAX_LAUNCHES), C.c_int(batch2),
-                           C.c_int(int(FORWARD if forward is None else forward)))
+                           C.c_int(int(FORWARD if forward is None else forward)), C.c_int(stride))
     return Result(rc, stats, traffic)
 
 
@@ -62,11 +62,20 @@ def emulate(func, prob, send, recv, n=0, r=2, batch=0, uniform_count=0, recv_lo=
 last = None
 # module-wide switch: emulate forwarded execution (and check it against the launch-per-digit execution)
 FORWARD = False
+# module-wide switch: fixed-stride staging, every slot as long as the call's longest block at any cache-line phase
+STRIDED = False
 
 
-def _run(*a, **k):
+def stride_for(prob, uniform_count=0) -> int:
+    longest = (uniform_count if uniform_count else int(prob.sendcounts.max(initial=0))) * prob.esz
+    return (longest + 255) // 128 * 128
+
+
+def _run(func, prob, *a, **k):
     global last
-    last = emulate(*a, **k)
+    if STRIDED:
+        k["stride"] = stride_for(prob, k.get("uniform_count", 0))
+    last = emulate(func, prob, *a, **k)
     if last.rc == 0 and last.errors:
         return 1000 + last.errors
     return last.rc

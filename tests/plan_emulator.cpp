@@ -41,13 +41,15 @@ static int count_overlaps(std::vector<Range> &dst, std::vector<Range> &src) {
 extern "C" int plan_emulate(int func, int P, int n, int r, int batch, int esz, int uniform_count, const char *send,
                             int64_t send_bytes, char *recv, int64_t recv_bytes, const int64_t *sbase, const int64_t *rbase,
                             const int *sc, const int *sd, const int *rc, const int *rd, int recv_lo, int64_t *stats_out,
-                            int64_t *traffic_out, int max_launches, int batch2, int forward) {
+                            int64_t *traffic_out, int max_launches, int batch2, int forward, int stride) {
     VcSched S;
     std::vector<VcLaunchInfo> L;
     int code = vc_make_schedule((VcFunc)func, P, n, r, batch, esz, uniform_count, S, L, batch2, forward != 0);
     if (code) return code;
     S.recv_lo = recv_lo;
     const int64_t PP = (int64_t)P * P;
+    if (stride > 0 && S.coalesce) return -100;            // fixed-stride staging has no organized region
+    S.stride = stride > 0 ? stride : 0;
 
     std::vector<int> ucnt, udsp, rdp;
     VcTables T;
@@ -68,8 +70,8 @@ extern "C" int plan_emulate(int func, int P, int n, int r, int batch, int esz, i
     // passes 1 and 2 of the planner
     const int w = std::max(vc_regions(S), 1) + 1;         // staging regions
     std::vector<int64_t> slot_off(PP * w, 0), row_base((int64_t)P * w, 0);
-    int64_t stage_bytes = 0;
-    for (int x = 0; x < S.w + S.w2; x++) {
+    int64_t stage_bytes = S.stride ? vc_strided_stage_bytes(S) : 0;
+    for (int x = 0; x < S.w + S.w2 && !S.stride; x++) {
         for (int to = 0; to < P; to++) {
             row_base[(int64_t)x * P + to] = stage_bytes;
             int64_t acc = 0;

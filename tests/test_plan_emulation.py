@@ -488,3 +488,45 @@ def test_distributions_of_the_reference_drivers(name, counts):
             assert np.array_equal(recv, want)
             ref = np.full(prob.recv_bytes, 0xEE, dtype=np.uint8)
             assert ofn(ref) == 0 and np.array_equal(ref, want)
+
+
+# ---- fixed-stride staging (the layout calls of short blocks get in the library's default mode) ----
+
+@pytest.fixture
+def strided():
+    E.FORWARD = True
+    E.STRIDED = True
+    yield
+    E.FORWARD = False
+    E.STRIDED = False
+
+
+@pytest.mark.parametrize("case", [c for c in CASES if c["P"] <= 128], ids=[c["id"] for c in CASES if c["P"] <= 128])
+def test_strided_plan_reproduces_reference_digests(case, strided):
+    """Slots at the closed-form addresses ((region P + holder) P + slot) x stride: every copy stays inside the arena, no
+    two slots overlap, forwarded and launch-per-digit execution agree, and the result has the reference's digests."""
+    prob = problem_for_case(case)
+    send = W.fill_send_arena(prob, case["payload"], case["seed"])
+    recv = np.full(prob.recv_bytes, 0xEE, dtype=np.uint8)
+    assert run_on(E, case, prob, send, recv) == 0
+    assert E.last.errors == 0
+    assert [f"{int(h):016x}" for h in O.digest_recv(digest_problem(case, prob), recv)] == case["digests"]
+    assert np.array_equal(recv, W.expected_recv_arena(prob, send))
+
+
+@pytest.mark.parametrize("P", [1, 2, 3, 5, 8, 12, 17, 27, 32, 50])
+def test_strided_plans_all_radices(P, strided):
+    for layout in (0, 1):
+        prob = _prob(P, layout, 3, seed=P + 90)
+        send = W.fill_send_arena(prob, 0, 3)
+        want = W.expected_recv_arena(prob, send)
+        for r in sorted({2, 3, 5, P, P + 3} - {1}):
+            calls = [lambda d: E.twophase_rbruck_alltoallv(r, prob, send, d), lambda d: E.twophase_rbruck_alltoallv_om(r, prob, send, d)]
+            if P >= 3:
+                calls += [lambda d: E.tuna_algorithm(r, 2, prob, send, d)]
+            for n in [d for d in (1, 2, 3, 4, 8) if P % d == 0]:
+                calls += [lambda d, n=n: E.TTPL_BT_alltoallv_s1(n, r, 0, prob, send, d), lambda d, n=n: E.TTPL_rbruck_alltoallv(n, r, prob, send, d)]
+            for fn in calls:
+                recv = np.full(prob.recv_bytes, 0xEE, dtype=np.uint8)
+                assert fn(recv) == 0 and E.last.errors == 0, (P, r)
+                assert np.array_equal(recv, want)
