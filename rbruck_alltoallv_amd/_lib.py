@@ -32,6 +32,7 @@ SYMBOLS = {
     "vc_comm_set_stream": (_I, [_P, _P]),
     "vc_comm_set_forwarding": (_I, [_P, _I]),
     "vc_comm_set_bases": (_I, [_P, _P, _P]),
+    "vc_comm_set_staging_bound": (_I, [_P, _I]),
     "vc_last_error_string": (C.c_char_p, []),
     "vc_alltoall_counts": (_I, [_P, _P, _P]),
     "vc_displs_from_counts": (_I, [_P, _P, _P, _P]),

@@ -53,6 +53,11 @@ class VirtualComm:
         a work-item list; 3 / 4 forwarded without one, a workgroup / a quarter of a wavefront per pair of ranks."""
         self._check(self.lib.vc_comm_set_forwarding(self.handle, int(enable)))
 
+    def set_staging_bound(self, on: bool) -> None:
+        """vc_comm_set_staging_bound: reuse staging memory in launch-per-digit execution and run forwarded calls that would
+        need more than twice their payload (and 1 GiB) that way (default), or give every digit phase its own region."""
+        self._check(self.lib.vc_comm_set_staging_bound(self.handle, int(on)))
+
     def last_stats(self) -> _lib.VcStats:
         s = _lib.VcStats()
         self._check(self.lib.vc_comm_last_stats(self.handle, C.byref(s)))

@@ -114,6 +114,7 @@ struct vc_comm {
         uni_counts, uni_displs, scratch;
     double cal_copy_bytes_per_s = 0, cal_launch_s = 0, cal_sync_s = 0;   // calibrate(): the plain copy's rate, the cost of a
                                           // launch, of a launch the host waits for
+    int bound_staging = 1;                // vc_comm_set_staging_bound
     int live_plans = 0;                   // plans created on this communicator and not yet freed
     std::vector<void *> retired_stage;    // staging arenas that were outgrown while plans existed: a HIP graph captured from
                                           // vc_plan_execute_async holds the arena's address, so they stay until the plans go
@@ -239,6 +240,12 @@ extern "C" int vc_comm_set_forwarding(vc_comm_t c, int enable) {
     return VC_OK;
 }
 
+extern "C" int vc_comm_set_staging_bound(vc_comm_t c, int enable) {
+    if (!c) return fail_arg("null communicator");
+    c->bound_staging = enable != 0;
+    return VC_OK;
+}
+
 extern "C" int vc_comm_last_stats(vc_comm_t c, vc_stats_t *out) {
     if (!c || !out) return fail_arg("vc_comm_last_stats: null argument");
     *out = c->stats;
@@ -293,6 +300,33 @@ static int ensure_events(vc_comm *c, size_t n) {
     return VC_OK;
 }
 
+static int schedule_error(int code);
+
+// What a call asked for: enough to derive its schedule again in the other execution mode.
+struct CallParams {
+    VcFunc f;
+    int n, r, batch, esz, uniform, batch2;
+};
+
+// The schedule of a call in one of the two execution modes.  Launch-per-digit execution reuses staging memory when the
+// communicator bounds its staging (the default) and there is something to reuse: with fewer than three staging regions
+// no sub-region is written after another one has been read for the last time.
+static int make_schedule(const vc_comm *c, const CallParams &q, bool forward, VcSched &S, std::vector<VcLaunchInfo> &L) {
+    const int rc = vc_make_schedule(q.f, c->P, q.n, q.r, q.batch, q.esz, q.uniform, S, L, q.batch2, forward);
+    if (rc) return rc;
+    const int nreg = S.w + S.w2;
+    if (!forward && c->bound_staging && nreg >= 3 && nreg + 1 <= VC_RECYCLE_MAX_SLOTS) S.recycle = 1;
+    return VC_OK;
+}
+
+// Forwarded execution keeps every hop's copy of every block (nothing reads them, so nothing says when one could be
+// overwritten): its staging is the sum over the blocks of (hops - 1) x bytes, 3.5 x the payload for a radix-2 Bruck
+// over 512 ranks.  A communicator that bounds its staging runs such a call one launch per digit instead, where staging
+// memory is reused: beyond twice the payload, and only when it matters (more than 1 GiB).
+static bool staging_out_of_bound(const vc_comm *c, int64_t stage_bytes, int64_t payload_bytes) {
+    return c->bound_staging && stage_bytes > ((int64_t)1 << 30) && stage_bytes > 2 * payload_bytes;
+}
+
 // What the planner leaves behind for the copy launches.
 struct PlanInfo {
     int nl = 0, n_digits = 0;
@@ -321,7 +355,7 @@ static PlanBufSizes plan_buf_sizes(const VcSched &S, int nl, bool forward) {
     const size_t wmax = (size_t)std::max(vc_regions(S), 1) + 1;      // staging regions
     PlanBufSizes z;
     z.slot_off = sizeof(int64_t) * PP * wmax;
-    z.row_tot = z.row_base = sizeof(int64_t) * P * wmax;
+    z.row_tot = z.row_base = sizeof(int64_t) * P * std::max(wmax, (size_t)vc_row_families(S) + 1);
     z.org_run_base = sizeof(int64_t) * P * (size_t)std::max(S.G, 1);
     z.item_row_tot = z.item_row_base = sizeof(int64_t) * P * (size_t)std::max(nl, 1);
     z.row_bytes = sizeof(int64_t) * P * (size_t)(std::max(nl, S.w + S.w2) + 3);
@@ -456,12 +490,18 @@ static int plan_emit(vc_comm *c, const VcSched &S, std::vector<VcLaunchInfo> &L,
     return VC_OK;
 }
 
-static int build_plan(vc_comm *c, VcSched S, std::vector<VcLaunchInfo> &L, VcTables T, DevBuf &items, PlanInfo &out, bool forward) {
-    int rc = plan_sizes(c, S, L, T, forward);
+static int build_plan(vc_comm *c, const CallParams &q, int recv_lo, VcTables T, DevBuf &items, PlanInfo &out, bool forward) {
+    VcSched S;
+    std::vector<VcLaunchInfo> L;
+    int rc = make_schedule(c, q, forward, S, L);
+    if (rc) return schedule_error(rc);
+    S.recv_lo = recv_lo;
+    rc = plan_sizes(c, S, L, T, forward);
     if (rc) return rc;
     HIP_TRY(hipStreamSynchronize(c->stream));     // the staging arena and the item list are sized from the plan
     rc = plan_read(c, S, L, out, forward);
     if (rc) return rc;
+    if (forward && staging_out_of_bound(c, out.stage_bytes, out.payload_bytes)) return build_plan(c, q, recv_lo, T, items, out, false);
     return plan_emit(c, S, L, T, items, out);
 }
 
@@ -626,7 +666,12 @@ static int try_strided(vc_comm *c, VcSched S, std::vector<VcLaunchInfo> &L, cons
     return rc ? rc : 1;
 }
 
-static int run_schedule(vc_comm *c, VcSched S, std::vector<VcLaunchInfo> &L, const char *sendbuf, char *recvbuf, VcTables T, bool forward) {
+static int run_schedule(vc_comm *c, const CallParams &q, const char *sendbuf, char *recvbuf, VcTables T, bool forward) {
+    VcSched S;
+    std::vector<VcLaunchInfo> L;
+    const int rc_sched = make_schedule(c, q, forward, S, L);
+    if (rc_sched) return schedule_error(rc_sched);
+    S.recv_lo = (int)((uintptr_t)recvbuf & 4095);
     PlanInfo pi;
     hipStream_t st = c->stream;
     const int pair_lanes = forward ? listless_lanes(c, S) : 0;
@@ -661,6 +706,7 @@ static int run_schedule(vc_comm *c, VcSched S, std::vector<VcLaunchInfo> &L, con
             if (rc) return rc;
             if (vc_listless_ok(c->h_header, guard)) { pi.listless = true; pi.chain_lanes = pair_lanes; break; }
             if (pi.stage_bytes <= guard.stage_cap) break;          // not a call for this kernel
+            if (staging_out_of_bound(c, pi.stage_bytes, pi.payload_bytes)) break;
             HIP_TRY(reserve_stage(c, (size_t)pi.stage_bytes + 64));
         }
         if (pi.listless) return finish_stats(c, pi, nullptr, true);
@@ -670,6 +716,7 @@ static int run_schedule(vc_comm *c, VcSched S, std::vector<VcLaunchInfo> &L, con
         rc = plan_read(c, S, L, pi, forward);
         if (rc) return rc;
     }
+    if (forward && staging_out_of_bound(c, pi.stage_bytes, pi.payload_bytes)) return run_schedule(c, q, sendbuf, recvbuf, T, false);
     rc = plan_emit(c, S, L, T, c->desc, pi);
     if (rc) return rc;
     return run_items(c, pi, c->desc.p, sendbuf, recvbuf, true);
@@ -757,13 +804,14 @@ static int run_v(VcFunc f, int n, int r, int batch, vc_comm *c, char *sendbuf, i
     if (rc) return rc;
     VC_ONE_CALL(c);
     if (!sendcounts || !sdispls || !recvcounts || (f != VC_F_TTPL && !rdispls)) return fail_arg("null table");
+    const CallParams q = {f, n, r, batch, esz, 0, batch2};
+    const bool forward = c->forward != 0 || async_stream;
+    if (!async_stream) return run_schedule(c, q, sendbuf, recvbuf, make_tables(c, sendcounts, sdispls, recvcounts, rdispls), forward);
     VcSched S;
     std::vector<VcLaunchInfo> L;
-    const bool forward = c->forward != 0 || async_stream;
-    rc = vc_make_schedule(f, c->P, n, r, batch, esz, 0, S, L, batch2, forward);
+    rc = make_schedule(c, q, true, S, L);
     if (rc) return schedule_error(rc);
     S.recv_lo = (int)((uintptr_t)recvbuf & 4095);
-    if (!async_stream) return run_schedule(c, S, L, sendbuf, recvbuf, make_tables(c, sendcounts, sdispls, recvcounts, rdispls), forward);
     c->stream = static_cast<hipStream_t>(*async_stream);
     rc = enqueue_async(c, S, L, sendbuf, recvbuf, make_tables(c, sendcounts, sdispls, recvcounts, rdispls));
     if (rc == VC_OK) busy_guard_.keep();
@@ -943,10 +991,11 @@ static int run_uniform(VcFunc f, int n, int r, vc_comm *c, char *sendbuf, int se
     VC_ONE_CALL(c);
     if (sendcount < 0) return fail_arg("negative block length");
     if ((int64_t)sendcount * c->P > 0x7FFFFFFF) return fail_arg("sendcount * P must fit the reference's int displacements");
+    const CallParams q = {f, n, r, 0, esz, sendcount, 0};
     VcSched S;
     std::vector<VcLaunchInfo> L;
     const bool forward = c->forward != 0 || async_stream;
-    rc = vc_make_schedule(f, c->P, n, r, 0, esz, sendcount, S, L, 0, forward);
+    rc = make_schedule(c, q, forward, S, L);              // (validates the tunables before anything is enqueued)
     if (rc) return schedule_error(rc);
     S.recv_lo = (int)((uintptr_t)recvbuf & 4095);
     if (async_stream) c->stream = static_cast<hipStream_t>(*async_stream);
@@ -955,7 +1004,7 @@ static int run_uniform(VcFunc f, int n, int r, vc_comm *c, char *sendbuf, int se
     HIP_TRY(c->uni_displs.reserve(sizeof(int) * PP));
     HIP_TRY(vc_launch_uniform_tables(c->uni_counts.as<int>(), c->uni_displs.as<int>(), sendcount, c->P, c->stream));
     const int *cnt = c->uni_counts.as<int>(), *dsp = c->uni_displs.as<int>();
-    if (!async_stream) return run_schedule(c, S, L, sendbuf, recvbuf, make_tables(c, cnt, dsp, cnt, dsp), forward);
+    if (!async_stream) return run_schedule(c, q, sendbuf, recvbuf, make_tables(c, cnt, dsp, cnt, dsp), forward);
     rc = enqueue_async(c, S, L, sendbuf, recvbuf, make_tables(c, cnt, dsp, cnt, dsp));
     if (rc == VC_OK) busy_guard_.keep();
     return rc;
@@ -1049,11 +1098,15 @@ extern "C" int vc_plan_create(const char *function, int n, int r, int batch, int
     const bool uniform = f == VC_F_UNIFORM_SPREADOUT || f == VC_F_UNIFORM_ISPLIT;      // `batch` is the block length, tables implied
     if (!uniform && (!sendcounts || !sdispls || !recvcounts || (f != VC_F_TTPL && !rdispls))) return fail_arg("null table");
     if (uniform && (batch < 0 || (int64_t)batch * c->P > 0x7FFFFFFF)) return fail_arg("block length * P must fit the reference's int displacements");
-    VcSched S;
-    std::vector<VcLaunchInfo> L;
+    const CallParams q = {f, n, r, uniform ? 0 : batch, elem_size, uniform ? batch : 0, 0};
     const bool forward = c->forward != 0;
-    int rc = vc_make_schedule(f, c->P, n, r, uniform ? 0 : batch, elem_size, uniform ? batch : 0, S, L, 0, forward);
-    if (rc) return schedule_error(rc);
+    int rc = VC_OK;
+    {
+        VcSched S;
+        std::vector<VcLaunchInfo> L;
+        rc = make_schedule(c, q, forward, S, L);          // validates the tunables before anything is allocated
+        if (rc) return schedule_error(rc);
+    }
     if (uniform) {
         const size_t PP = (size_t)c->P * c->P;
         HIP_TRY(c->uni_counts.reserve(sizeof(int) * PP));
@@ -1062,10 +1115,9 @@ extern "C" int vc_plan_create(const char *function, int n, int r, int batch, int
         sendcounts = recvcounts = c->uni_counts.as<int>();
         sdispls = rdispls = c->uni_displs.as<int>();
     }
-    S.recv_lo = recvbuf_low_bits & 4095;
     vc_plan *p = new vc_plan();
     p->comm = c;
-    rc = build_plan(c, S, L, make_tables(c, sendcounts, sdispls, recvcounts, rdispls), p->items, p->info, forward);
+    rc = build_plan(c, q, recvbuf_low_bits & 4095, make_tables(c, sendcounts, sdispls, recvcounts, rdispls), p->items, p->info, forward);
     if (rc == VC_OK && hipStreamSynchronize(c->stream) != hipSuccess) rc = fail_arg("vc_plan_create: stream error", VC_ERR_HIP);
     if (rc == VC_OK && reserve_stage(c, (size_t)p->info.stage_bytes + 64) != hipSuccess)       // so that executing never allocates
         rc = fail_arg("vc_plan_create: cannot allocate the staging arena", VC_ERR_HIP);

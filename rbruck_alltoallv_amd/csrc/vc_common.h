@@ -59,6 +59,10 @@ struct VcSched {
                       //    at any cache-line phase), the reference's own layout (src/twophase_tunable_rbruckv.cpp:59): slot `id`
                       //    of rank `holder` in region x starts at ((x P + holder) P + id) stride, a closed form, and the planner's
                       //    prefix sums and slot tables are not needed.  0: compact slots at prefix-sum offsets.
+    int recycle;      // 1 (launch-per-digit execution only): staging memory is reused.  A staged block arrives in one hop slot and
+                      //    leaves in a later one; blocks with the same (arrival, departure) pair of hop slots form a sub-region,
+                      //    and a sub-region may take the memory of another one whose blocks have all left before it is written
+                      //    (the reference reuses its extra_buffer slots the same way, src/twophase_tunable_rbruckv-om.cpp:52-75).
     int coalesce;     // 1: blocks that are about to leave their node wait in "organized" runs — the n blocks one rank
                       //    holds for one destination rank back to back in source order — so that an inter-node message
                       //    is a contiguous copy (TTPL_BT_alltoallv, src/twophase_twolayer_rbruck.cpp:388-398, 430-453).
@@ -73,6 +77,15 @@ struct VcSched {
 
 // Staging regions of a call: one per intra-node digit, one per inter-node digit, the organized region.
 VC_HD int vc_regions(const VcSched &S) { return S.w + S.w2 + S.coalesce; }
+
+// Reused staging (S.recycle): hop slots a call may have at most, and rows of the row tables per rank: one per (arrival,
+// departure) pair of hop slots plus one for the organized region.
+#define VC_RECYCLE_MAX_SLOTS 12
+#define VC_RECYCLE_MAX_PAIRS (VC_RECYCLE_MAX_SLOTS * VC_RECYCLE_MAX_SLOTS + 1)
+VC_HD int vc_row_families(const VcSched &S) {
+    const int ns = S.w + S.w2 + 1;
+    return S.recycle ? ns * ns + 1 : vc_regions(S);
+}
 
 // One data-moving kernel launch.
 struct VcLaunchInfo {

@@ -34,6 +34,31 @@ __global__ __launch_bounds__(VC_THREADS) void vc_plan_rows(VcSched S, VcLaunchPa
     const int nreg = S.w + S.w2;                          // the organized region is laid out by vc_plan_org_rows
     const bool forward = chain_row_tot != nullptr;
     const int nsum = forward ? nreg : nl;                 // rows of row_bytes before the payload row
+    if ((int)blockIdx.y < nreg && S.recycle) {
+        // reused staging: the slots of the region in one prefix sum per hop slot in which their blocks leave again
+        __shared__ int64_t family_carry[VC_RECYCLE_MAX_SLOTS];
+        const int y = blockIdx.y, ns = nreg + 1, t_arrive = vc_slot_time(S, y);
+        if (threadIdx.x < VC_RECYCLE_MAX_SLOTS) family_carry[threadIdx.x] = 0;
+        __syncthreads();
+        for (int base = 0; base < P; base += VC_THREADS) {
+            const int id = base + threadIdx.x;
+            int st[2] = {0, 0};
+            const int64_t v = (id < P) ? vc_region_slot_size(S, T, y, to, id, nullptr, st) : 0;
+            const int leaves = v ? vc_next_hop(S, st[0], st[1], y) : -1;
+            for (int time = t_arrive + 1; time < ns; time++) {
+                const int kd = vc_slot_time(S, time);
+                int64_t total;
+                const int64_t ex = vc_block_exclusive_scan(leaves == kd ? v : 0, lds, total);
+                if (leaves == kd) slot_off[((int64_t)y * P + to) * P + id] = family_carry[kd] + ex;
+                __syncthreads();
+                if (threadIdx.x == 0) family_carry[kd] += total;
+                __syncthreads();
+            }
+            if (id < P && !v) slot_off[((int64_t)y * P + to) * P + id] = 0;
+        }
+        if ((int)threadIdx.x < ns) row_tot[(int64_t)(y * ns + threadIdx.x) * P + to] = vc_slot_time(S, threadIdx.x) > t_arrive ? family_carry[threadIdx.x] : 0;
+        return;
+    }
     if ((int)blockIdx.y < nreg) {
         const int y = blockIdx.y;
         int64_t carry = 0, data = 0;
@@ -121,7 +146,8 @@ __global__ __launch_bounds__(VC_THREADS) void vc_plan_org_rows(VcSched S, VcTabl
         if (g < G) org_run_base[(int64_t)to * G + g] = carry + ex;
         carry += total;
     }
-    if (threadIdx.x == 0) row_tot[(int64_t)S.w * P + to] = carry;
+    const int ns = S.w + S.w2 + 1;
+    if (threadIdx.x == 0) row_tot[(int64_t)(S.recycle ? ns * ns : S.w) * P + to] = carry;
     __syncthreads();                                      // org_run_base of this rank is complete (same workgroup wrote it)
     for (int id = threadIdx.x; id < P; id += VC_THREADS)
         slot_off[((int64_t)S.w * P + to) * P + id] = org_run_base[(int64_t)to * G + id / S.n] + vc_org_slot_rel(S, T, to, id);
@@ -132,14 +158,14 @@ __global__ __launch_bounds__(VC_THREADS) void vc_plan_org_rows(VcSched S, VcTabl
 // first item), its item count and moved bytes.  Workgroup nl: staging row bases, staging bytes, payload bytes, negative
 // table entries.  Forwarded execution (chain_row_tot != null, nl = 0): grid (2).  Workgroup 0 as workgroup nl above, and
 // the moved bytes = payload + bytes of the staged blocks as those of launch 0; workgroup 1: chain item bases.
-__global__ __launch_bounds__(VC_THREADS) void vc_plan_bases(int P, int w, int nreg, int nl, const int64_t *__restrict__ row_tot,
+__global__ __launch_bounds__(VC_THREADS) void vc_plan_bases(VcSched S, int P, int w, int nreg, int nl, const int64_t *__restrict__ row_tot,
                                                             int64_t *__restrict__ row_base, const int64_t *__restrict__ item_row_tot,
                                                             int64_t *__restrict__ item_row_base, const int64_t *__restrict__ row_bytes,
                                                             const int64_t *__restrict__ chain_row_tot, int64_t *__restrict__ chain_row_base,
                                                             int64_t *__restrict__ header, int64_t *__restrict__ header_host) {
     __shared__ int64_t lds[VC_WAVES_PER_BLOCK];
     const int L = blockIdx.x;
-    const bool forward = chain_row_tot != nullptr;
+    const bool forward = chain_row_tot != nullptr, recycle = S.recycle != 0;
     const int nsum = forward ? nreg : nl;                 // rows of row_bytes before the payload row
     int64_t carry = 0, bytes = 0;
     if (forward && L == 1) {                              // first chain item of every final receiver
@@ -161,6 +187,40 @@ __global__ __launch_bounds__(VC_THREADS) void vc_plan_bases(int P, int w, int nr
         if (threadIdx.x == 0) {
             header[2] = carry; header[VC_HEADER_MAX_PIECES] = most; header[VC_HEADER_MAX_LEN] = longest;
             if (header_host) { header_host[2] = carry; header_host[VC_HEADER_MAX_PIECES] = most; header_host[VC_HEADER_MAX_LEN] = longest; }
+        }
+        return;
+    }
+    if (L == nl && recycle) {
+        // reused staging: row bases inside every sub-region, the sub-regions' sizes, their places in the arena
+        __shared__ int64_t family_size[VC_RECYCLE_MAX_PAIRS], family_base[VC_RECYCLE_MAX_PAIRS], hole_lo[VC_RECYCLE_MAX_PAIRS],
+            hole_hi[VC_RECYCLE_MAX_PAIRS];
+        const int ns = nreg + 1, nfam = ns * ns + 1;
+        for (int f = 0; f < nfam; f++) {
+            const int ka = f / ns, kd = f % ns;
+            const bool used = f == ns * ns ? w > nreg : (ka < nreg && vc_slot_time(S, kd) > vc_slot_time(S, ka));
+            int64_t fam_carry = 0;
+            if (used)
+                for (int b0 = 0; b0 < P; b0 += VC_THREADS) {
+                    const int i = b0 + threadIdx.x;
+                    int64_t total;
+                    const int64_t ex = vc_block_exclusive_scan((i < P) ? row_tot[(int64_t)f * P + i] : 0, lds, total);
+                    if (i < P) row_base[(int64_t)f * P + i] = fam_carry + ex;
+                    fam_carry += total;
+                }
+            if (threadIdx.x == 0) family_size[f] = fam_carry;
+        }
+        __syncthreads();
+        if (threadIdx.x == 0) carry = vc_allocate_staging(S, family_size, family_base, hole_lo, hole_hi);
+        __syncthreads();
+        for (int64_t i = threadIdx.x; i < (int64_t)nfam * P; i += VC_THREADS)
+            if (family_size[i / P] > 0) row_base[i] += family_base[i / P];
+        int64_t bad = 0;
+        for (int i = threadIdx.x; i < P; i += VC_THREADS) { bytes += row_bytes[(int64_t)nsum * P + i]; bad += row_bytes[(int64_t)(nsum + 1) * P + i]; }
+        bytes = vc_block_sum(bytes, lds);
+        bad = vc_block_sum(bad, lds);
+        if (threadIdx.x == 0) {
+            header[0] = carry; header[1] = bytes; header[VC_HEADER_BAD] = bad;
+            if (header_host) { header_host[0] = carry; header_host[1] = bytes; header_host[VC_HEADER_BAD] = bad; }
         }
         return;
     }
@@ -301,7 +361,7 @@ hipError_t vc_launch_plan_sizes(const VcSched &S, const VcLaunchInfo *launches_h
                        row_tot, item_row_tot, row_bytes, chain_row_tot);
     if (S.coalesce)
         hipLaunchKernelGGL(vc_plan_org_rows, dim3(S.P), dim3(VC_THREADS), 0, st, S, T, slot_off, row_tot, org_run_base);
-    hipLaunchKernelGGL(vc_plan_bases, dim3(forward ? 2 : nl + 1), dim3(VC_THREADS), 0, st, S.P, vc_regions(S), nreg, nl, row_tot, row_base,
+    hipLaunchKernelGGL(vc_plan_bases, dim3(forward ? 2 : nl + 1), dim3(VC_THREADS), 0, st, S, S.P, vc_regions(S), nreg, nl, row_tot, row_base,
                        item_row_tot, item_row_base, row_bytes, chain_row_tot, chain_row_base, header, header_host);
     return hipGetLastError();
 }

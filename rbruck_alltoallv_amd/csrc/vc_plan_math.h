@@ -117,11 +117,14 @@ VC_HD int vc_phase(const VcSched &S, const VcTables &T, int s, int t) {
 
 
 // Bytes the staging slot `id` of rank `to` needs for the block that arrives in digit x
-// (0 if nothing arrives there, or if it goes to recvbuf).  Always a multiple of VC_LINE.
-VC_HD int64_t vc_stage_slot_size(const VcSched &S, const VcTables &T, int x, int dist, int to, int id, int64_t *data_len = nullptr) {
+// (0 if nothing arrives there, or if it goes to recvbuf).  Always a multiple of VC_LINE.  st (optional) receives the
+// block's source and destination rank.
+VC_HD int64_t vc_stage_slot_size(const VcSched &S, const VcTables &T, int x, int dist, int to, int id, int64_t *data_len = nullptr,
+                                 int *st = nullptr) {
     VcBlock b;
     if (data_len) *data_len = 0;
     if (!vc_intra_block(S, x, dist, to, id, b) || !b.to_stage || b.to_org) return 0;
+    if (st) { st[0] = b.s; st[1] = b.t; }
     const int64_t len = (int64_t)T.sc[(int64_t)b.s * S.P + b.t] * S.esz;
     if (data_len) *data_len = len;
     return len ? ((len + vc_phase(S, T, b.s, b.t) + VC_LINE - 1) & ~(int64_t)(VC_LINE - 1)) : 0;
@@ -129,17 +132,18 @@ VC_HD int64_t vc_stage_slot_size(const VcSched &S, const VcTables &T, int x, int
 
 // The same for staging region y of a call: intra-node digits first, then inter-node digits.  data_len (optional)
 // receives the bytes of the block itself.
-VC_HD int64_t vc_region_slot_size(const VcSched &S, const VcTables &T, int y, int to, int id, int64_t *data_len = nullptr) {
+VC_HD int64_t vc_region_slot_size(const VcSched &S, const VcTables &T, int y, int to, int id, int64_t *data_len = nullptr, int *st = nullptr) {
     int dist = 1;
     if (y < S.w) {
         for (int k = 0; k < y; k++) dist *= S.r;
-        return vc_stage_slot_size(S, T, y, dist, to, id, data_len);
+        return vc_stage_slot_size(S, T, y, dist, to, id, data_len, st);
     }
     for (int k = S.w; k < y; k++) dist *= S.r;
     VcEntry e;
     int z;
     if (data_len) *data_len = 0;
     if (!vc_inter_block(S, y - S.w, dist, to, id, e, z) || e.xdst < 0) return 0;
+    if (st) { st[0] = e.s; st[1] = e.t; }
     const int64_t len = (int64_t)T.sc[(int64_t)e.s * S.P + e.t] * S.esz;
     if (data_len) *data_len = len;
     return len ? ((len + vc_phase(S, T, e.s, e.t) + VC_LINE - 1) & ~(int64_t)(VC_LINE - 1)) : 0;
@@ -147,10 +151,18 @@ VC_HD int64_t vc_region_slot_size(const VcSched &S, const VcTables &T, int y, in
 
 // Address (inside the staging arena) of the data of block (s, t) while it sits in slot `id`
 // of `holder` in staging region x.
+// With reused staging (S.recycle) the rows of a region are split by the hop slot in which their blocks leave again:
+// row family (arrival slot) * slots + (departure slot), the organized region last.
+VC_HD int vc_next_hop(const VcSched &S, int s, int t, int k);
 VC_HD int64_t vc_stage_addr(const VcSched &S, const VcTables &T, const int64_t *slot_off, const int64_t *row_base,
                             int x, int holder, int id, int s, int t) {
     const int64_t row = (int64_t)x * S.P + holder;
     if (S.stride) return (row * S.P + id) * S.stride + vc_phase(S, T, s, t);
+    if (S.recycle) {
+        const int ns = S.w + S.w2 + 1;
+        const int family = (S.coalesce && x == S.w) ? ns * ns : x * ns + vc_next_hop(S, s, t, x);
+        return row_base[(int64_t)family * S.P + holder] + slot_off[row * S.P + id] + vc_phase(S, T, s, t);
+    }
     return row_base[row] + slot_off[row * S.P + id] + vc_phase(S, T, s, t);
 }
 
@@ -373,6 +385,88 @@ VC_HD int64_t vc_chain_count(const VcSched &S, const VcTables &T, int s, int t) 
 #define VC_CHAIN_LEN 1
 #define VC_CHAIN_NHOP 2
 #define VC_CHAIN_HEAD 3   // followed by the space-tagged destination of the piece at every hop
+
+// Hop slots in the order in which a call works through them: the intra-node digits (most significant first for the
+// functions that run them that way), the inter-node digits, the last slot.  The mapping is its own inverse.
+VC_HD int vc_slot_time(const VcSched &S, int k) { return (k < S.w && S.msd) ? S.w - 1 - k : k; }
+
+// Whether block (s, t) moves in hop slot k (vc_block_hop without the destination).
+VC_HD bool vc_block_moves(const VcSched &S, int s, int t, int k) {
+    const int n = S.n, G = S.G, r = S.r, final_slot = S.w + S.w2;
+    if (s == t) return k == final_slot;
+    const int gs = s / n, gt = t / n;
+    if (k == final_slot) return S.last_hop == 2 || (S.last_hop == 1 && gs != gt);
+    const bool intra = k < S.w;
+    const int x = intra ? k : k - S.w;
+    const int span = intra ? n : G;
+    const int j = intra ? (s % n - t % n + n) % n : (gs - gt + G) % G;
+    int64_t dist = 1;
+    for (int i = 0; i < x; i++) dist *= r;
+    return dist < span && (j / dist) % r != 0;
+}
+
+// The hop slot in which block (s, t) moves next after hop slot k (in the call's order), or -1.
+VC_HD int vc_next_hop(const VcSched &S, int s, int t, int k) {
+    const int ns = S.w + S.w2 + 1;
+    for (int time = vc_slot_time(S, k) + 1; time < ns; time++) {
+        const int k2 = vc_slot_time(S, time);
+        if (vc_block_moves(S, s, t, k2)) return k2;
+    }
+    return -1;
+}
+
+// Where the sub-regions of reused staging go.  size[family] (family = arrival slot * slots + departure slot; the
+// organized region at slots * slots) are the bytes of the sub-regions, multiples of VC_LINE; base[family] receives
+// their offsets in the arena; returns the arena's size.  A sub-region is written in the launches of its arrival slot
+// and read for the last time in those of its departure slot, so its memory is free for sub-regions that arrive in
+// any later slot.  First fit, the longest-lived sub-regions of an arrival slot first.  hole_lo / hole_hi: work space of
+// VC_RECYCLE_MAX_PAIRS entries each.
+VC_HD int64_t vc_allocate_staging(const VcSched &S, const int64_t *size, int64_t *base, int64_t *hole_lo, int64_t *hole_hi) {
+    const int ns = S.w + S.w2 + 1, org = ns * ns;
+    int nh = 0;
+    int64_t top = 0, peak = 0;
+    base[org] = 0;                                        // lives from the first launch to the last
+    top = peak = size[org];
+    for (int ta = 0; ta < ns; ta++) {
+        if (ta >= 1) {                                    // what the launches of the slot before have read for the last time
+            const int kd = vc_slot_time(S, ta - 1);
+            for (int ka = 0; ka < ns - 1; ka++)
+                if (size[ka * ns + kd] > 0 && vc_slot_time(S, ka) < ta - 1) {
+                    hole_lo[nh] = base[ka * ns + kd]; hole_hi[nh] = hole_lo[nh] + size[ka * ns + kd]; nh++;
+                }
+            for (bool again = true; again;) {             // merge neighbours, give the top of the arena back
+                again = false;
+                for (int a = 0; a < nh && !again; a++) {
+                    if (hole_hi[a] == top) { top = hole_lo[a]; hole_lo[a] = hole_lo[nh - 1]; hole_hi[a] = hole_hi[nh - 1]; nh--; again = true; break; }
+                    for (int b = 0; b < nh; b++)
+                        if (b != a && hole_hi[a] == hole_lo[b]) {
+                            hole_hi[a] = hole_hi[b]; hole_lo[b] = hole_lo[nh - 1]; hole_hi[b] = hole_hi[nh - 1]; nh--; again = true; break;
+                        }
+                }
+            }
+        }
+        const int ka = vc_slot_time(S, ta);
+        if (ka >= ns - 1) continue;                       // the last slot has no staging region
+        for (int td = ns - 1; td > ta; td--) {
+            const int f = ka * ns + vc_slot_time(S, td);
+            const int64_t sz = size[f];
+            if (sz <= 0) { base[f] = 0; continue; }
+            int best = -1;
+            for (int a = 0; a < nh; a++)
+                if (hole_hi[a] - hole_lo[a] >= sz && (best < 0 || hole_lo[a] < hole_lo[best])) best = a;
+            if (best >= 0) {
+                base[f] = hole_lo[best];
+                hole_lo[best] += sz;
+                if (hole_lo[best] == hole_hi[best]) { hole_lo[best] = hole_lo[nh - 1]; hole_hi[best] = hole_hi[nh - 1]; nh--; }
+            } else {
+                base[f] = top;
+                top += sz;
+                if (top > peak) peak = top;
+            }
+        }
+    }
+    return peak;
+}
 
 // The route of block (s, t) in closed form: does it move in hop slot k, and where to?  After digit x of a Bruck that
 // runs least significant digit first a block has travelled (offset mod r^(x+1)) ranks down from its source, most

@@ -43,7 +43,7 @@ class Result:
         self.traffic = traffic[: self.nlaunch] if rc == 0 else None
 
 
-def emulate(func, prob, send, recv, n=0, r=2, batch=0, uniform_count=0, recv_lo=0, batch2=0, forward=None, stride=0) -> Result:
+def emulate(func, prob, send, recv, n=0, r=2, batch=0, uniform_count=0, recv_lo=0, batch2=0, forward=None, stride=0, recycle=None) -> Result:
     global _lib
     if _lib is None:
         _lib = C.CDLL(build())
@@ -54,7 +54,8 @@ def emulate(func, prob, send, recv, n=0, r=2, batch=0, uniform_count=0, recv_lo=
                            C.c_int(uniform_count), _p(send), C.c_int64(send.size), _p(recv), C.c_int64(recv.size),
                            _p(prob.sbase), _p(prob.rbase), _p(prob.sendcounts), _p(prob.sdispls), _p(prob.recvcounts),
                            _p(prob.rdispls), C.c_int(recv_lo), _p(stats), _p(traffic), C.c_int(MAX_LAUNCHES), C.c_int(batch2),
-                           C.c_int(int(FORWARD if forward is None else forward)), C.c_int(stride))
+                           C.c_int(int(FORWARD if forward is None else forward)), C.c_int(stride),
+                           C.c_int(int(RECYCLE if recycle is None else recycle)))
     return Result(rc, stats, traffic)
 
 
@@ -62,6 +63,8 @@ def emulate(func, prob, send, recv, n=0, r=2, batch=0, uniform_count=0, recv_lo=
 last = None
 # module-wide switch: emulate forwarded execution (and check it against the launch-per-digit execution)
 FORWARD = False
+# module-wide switch: launch-per-digit execution reuses staging memory where the library would (its default)
+RECYCLE = True
 # module-wide switch: fixed-stride staging, every slot as long as the call's longest block at any cache-line phase
 STRIDED = False
 

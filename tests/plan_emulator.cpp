@@ -41,7 +41,7 @@ static int count_overlaps(std::vector<Range> &dst, std::vector<Range> &src) {
 extern "C" int plan_emulate(int func, int P, int n, int r, int batch, int esz, int uniform_count, const char *send,
                             int64_t send_bytes, char *recv, int64_t recv_bytes, const int64_t *sbase, const int64_t *rbase,
                             const int *sc, const int *sd, const int *rc, const int *rd, int recv_lo, int64_t *stats_out,
-                            int64_t *traffic_out, int max_launches, int batch2, int forward, int stride) {
+                            int64_t *traffic_out, int max_launches, int batch2, int forward, int stride, int recycle) {
     VcSched S;
     std::vector<VcLaunchInfo> L;
     int code = vc_make_schedule((VcFunc)func, P, n, r, batch, esz, uniform_count, S, L, batch2, forward != 0);
@@ -50,6 +50,9 @@ extern "C" int plan_emulate(int func, int P, int n, int r, int batch, int esz, i
     const int64_t PP = (int64_t)P * P;
     if (stride > 0 && S.coalesce) return -100;            // fixed-stride staging has no organized region
     S.stride = stride > 0 ? stride : 0;
+    // reused staging under the library's own rule (make_schedule in csrc/vc_api.hip): launch-per-digit execution with at
+    // least three staging regions
+    if (recycle && !forward && !S.stride && S.w + S.w2 >= 3 && S.w + S.w2 + 1 <= VC_RECYCLE_MAX_SLOTS) S.recycle = 1;
 
     std::vector<int> ucnt, udsp, rdp;
     VcTables T;
@@ -69,9 +72,48 @@ extern "C" int plan_emulate(int func, int P, int n, int r, int batch, int esz, i
 
     // passes 1 and 2 of the planner
     const int w = std::max(vc_regions(S), 1) + 1;         // staging regions
-    std::vector<int64_t> slot_off(PP * w, 0), row_base((int64_t)P * w, 0);
+    std::vector<int64_t> slot_off(PP * w, 0), row_base((int64_t)P * std::max(w, vc_row_families(S) + 1), 0);
     int64_t stage_bytes = S.stride ? vc_strided_stage_bytes(S) : 0;
-    for (int x = 0; x < S.w + S.w2 && !S.stride; x++) {
+    if (S.recycle) {
+        // the planner's passes for reused staging: slots numbered per (arrival, departure) family, rows inside a family,
+        // families placed by the allocator the planning kernel uses
+        const int ns = S.w + S.w2 + 1, nfam = ns * ns + 1;
+        std::vector<int64_t> row_tot((int64_t)nfam * P, 0), fam_size(nfam, 0), fam_base(nfam, 0), hole_lo(VC_RECYCLE_MAX_PAIRS), hole_hi(VC_RECYCLE_MAX_PAIRS);
+        for (int y = 0; y < S.w + S.w2; y++)
+            for (int to = 0; to < P; to++) {
+                std::vector<int64_t> carry(ns, 0);
+                for (int id = 0; id < P; id++) {
+                    int st[2] = {0, 0};
+                    const int64_t v = vc_region_slot_size(S, T, y, to, id, nullptr, st);
+                    if (!v) continue;
+                    const int kd = vc_next_hop(S, st[0], st[1], y);
+                    if (kd < 0 || vc_slot_time(S, kd) <= vc_slot_time(S, y)) return -101;
+                    slot_off[((int64_t)y * P + to) * P + id] = carry[kd];
+                    carry[kd] += v;
+                }
+                for (int kd = 0; kd < ns; kd++) row_tot[(int64_t)(y * ns + kd) * P + to] = carry[kd];
+            }
+        if (S.coalesce)
+            for (int to = 0; to < P; to++) {
+                std::vector<int64_t> run_base(S.G);
+                int64_t acc = 0;
+                for (int g = 0; g < S.G; g++) { run_base[g] = acc; acc += vc_org_run_size(S, T, to, g); }
+                for (int id = 0; id < P; id++)
+                    slot_off[((int64_t)S.w * P + to) * P + id] = run_base[id / S.n] + vc_org_slot_rel(S, T, to, id);
+                row_tot[(int64_t)(ns * ns) * P + to] = acc;
+            }
+        for (int f = 0; f < nfam; f++) {
+            int64_t acc = 0;
+            for (int to = 0; to < P; to++) { row_base[(int64_t)f * P + to] = acc; acc += row_tot[(int64_t)f * P + to]; }
+            fam_size[f] = acc;
+        }
+        stage_bytes = vc_allocate_staging(S, fam_size.data(), fam_base.data(), hole_lo.data(), hole_hi.data());
+        for (int f = 0; f < nfam; f++) {
+            if (fam_size[f] > 0 && fam_base[f] + fam_size[f] > stage_bytes) return -102;
+            for (int to = 0; to < P; to++) row_base[(int64_t)f * P + to] += fam_base[f];
+        }
+    }
+    for (int x = 0; x < S.w + S.w2 && !S.stride && !S.recycle; x++) {
         for (int to = 0; to < P; to++) {
             row_base[(int64_t)x * P + to] = stage_bytes;
             int64_t acc = 0;
@@ -82,7 +124,7 @@ extern "C" int plan_emulate(int func, int P, int n, int r, int batch, int esz, i
             stage_bytes += acc;
         }
     }
-    if (S.coalesce)                                       // pass 1b: organized region
+    if (S.coalesce && !S.recycle)                         // pass 1b: organized region
         for (int to = 0; to < P; to++) {
             row_base[(int64_t)S.w * P + to] = stage_bytes;
             std::vector<int64_t> run_base(S.G);
@@ -135,8 +177,8 @@ extern "C" int plan_emulate(int func, int P, int n, int r, int batch, int esz, i
                 const int64_t dlim = dspace == 1 ? recv_bytes : (dspace == 2 ? stage_bytes : -1);
                 if (so < 0 || so + d.len > slim || dof < 0 || dof + d.len > dlim) { errors++; continue; }
                 if (d.from < 0 || d.from >= P || d.to != to) errors++;
-                if (sspace == 2)
-                    for (int64_t b = 0; b < d.len; b++) errors += !written[so + b];
+                if (sspace == 2)                          // every staged byte is read exactly once: by the block's next hop
+                    for (int64_t b = 0; b < d.len; b++) { errors += !written[so + b]; written[so + b] = 0; }
                 descs.push_back(d);
                 dst_ranges.push_back({dof, dof + d.len, dspace});
                 src_ranges.push_back({so, so + d.len, sspace});
@@ -150,10 +192,14 @@ extern "C" int plan_emulate(int func, int P, int n, int r, int batch, int esz, i
             const char *from = (sspace == 0 ? send : stage.data()) + (d.src & VC_OFFSET_MASK);
             char *to = (dspace == 1 ? recv : stage.data()) + (d.dst & VC_OFFSET_MASK);
             memcpy(to, from, (size_t)d.len);
-            if (dspace == 2) memset(written.data() + (d.dst & VC_OFFSET_MASK), 1, (size_t)d.len);
+            if (dspace == 2) {                            // ... and nothing lands on bytes that are still waiting for theirs
+                char *wr = written.data() + (d.dst & VC_OFFSET_MASK);
+                for (int64_t b = 0; b < d.len; b++) { errors += wr[b] != 0; wr[b] = 1; }
+            }
             moved += d.len;
         }
     }
+    for (int64_t b = 0; b < stage_bytes; b++) errors += written[b] != 0;          // every staged block has moved on
     if (forward) {
         const int nslots = vc_hop_slots(S), stride = VC_CHAIN_HEAD + nslots;
         if (nslots > VC_MAX_HOP_SLOTS) errors++;

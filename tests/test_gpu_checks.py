@@ -387,3 +387,40 @@ def test_async_twins_overlap_two_communicators(api):
         assert dpu.comm.wait() == 0, dpu.comm.error()
         assert dpu.verify(dsu, dru) == 0, name
     dpu.comm.free()
+
+
+def test_staging_bound(api):
+    """A radix-2 Bruck on the pencil pattern of configuration 5 (512 ranks, rows of 32, here 64 KiB blocks: 1 GiB of
+    payload, 4.5 hops per block) would keep 3.5 x the payload in separate staging regions.  A communicator that bounds its
+    staging (the default) runs the call one launch per digit on reused staging, below twice the payload; unbounded it stays
+    forwarded.  Both exact."""
+    counts = W.counts_fft_rows(512, 32, 8192)
+    prob = W.make_problem(counts, 8, 0, 0)
+    S = prob.payload_bytes
+    assert S == 1 << 30
+    dp = api.DeviceProblem(prob)
+    ds = dp.new_send_arena()
+    dp.fill_payload(0, 21, ds)
+    seen = {}
+    for bound in (True, False):
+        dp.comm.set_staging_bound(bound)
+        for mode in (2, 0):
+            dp.comm.set_forwarding(mode)
+            dr = dp.new_recv_arena(0xEE)
+            assert api.tuna_algorithm(2, 0, dp, ds, dr) == 0, dp.comm.error()
+            assert dp.verify(ds, dr) == 0
+            st = dp.comm.last_stats()
+            seen[(bound, mode)] = (int(st.execution), int(st.staging_bytes), int(st.n_launches))
+            assert st.moved_bytes * 2 == W.algorithmic_bytes(counts, 8, W.hops_flat(512, 2))
+    print(seen, flush=True)
+    assert seen[(False, 2)][0] == 1 and seen[(False, 2)][1] > 3.4 * S            # forwarded, every region of its own
+    assert seen[(False, 0)][0] == 0 and seen[(False, 0)][1] == seen[(False, 2)][1]
+    assert seen[(True, 0)][0] == 0 and seen[(True, 0)][1] < 2 * S                  # reused
+    assert seen[(True, 2)] == seen[(True, 0)]                                      # asked for forwarded, run per digit
+    # a radix with few hops stays forwarded under the bound
+    dp.comm.set_staging_bound(True)
+    dp.comm.set_forwarding(2)
+    dr = dp.new_recv_arena(0xEE)
+    assert api.tuna_algorithm(32, 0, dp, ds, dr) == 0 and dp.verify(ds, dr) == 0
+    assert dp.comm.last_stats().execution == 1 and dp.comm.last_stats().staging_bytes < S
+    dp.comm.free()

@@ -874,6 +874,7 @@ def test_both_execution_modes_leave_the_same_staging(api):
                                           ("twophase r=7", lambda dp, s, d: api.twophase_rbruck_alltoallv(7, dp, s, d)),
                                           ("tuna r=3", lambda dp, s, d: api.tuna_algorithm(3, 2, dp, s, d))])):
         dp = api.DeviceProblem(prob)
+        dp.comm.set_staging_bound(False)             # every digit phase its own region: the layout all four modes share
         ds = dp.new_send_arena()
         dp.fill_payload(0, 11, ds)
         lib, h = dp.comm.lib, dp.comm.handle
@@ -899,6 +900,16 @@ def test_both_execution_modes_leave_the_same_staging(api):
             assert sizes[0] == sizes[1] == sizes[2] == sizes[3], name
             assert all(np.array_equal(snaps[0], other) for other in snaps[1:]), name
             assert np.count_nonzero(snaps[0] != 0xAB) > sizes[0] // 4, name        # the slots were written
+            # with the staging bound on (the default), launch-per-digit execution reuses staging memory: never more, and
+            # the same result
+            dp.comm.set_staging_bound(True)
+            dp.comm.set_forwarding(0)
+            dr = dp.new_recv_arena(0xEE)
+            assert fn(dp, ds, dr) == 0 and dp.verify(ds, dr) == 0, name
+            assert dp.comm.last_stats().staging_bytes <= sizes[0], name
+            if name == "twophase r=2":               # (two-layer calls keep most staged blocks until the inter-node phase)
+                assert dp.comm.last_stats().staging_bytes < 0.85 * sizes[0], name
+            dp.comm.set_staging_bound(False)
         dp.comm.free()
 
 
@@ -919,6 +930,7 @@ def test_forwarded_shapes_plans_and_graphs(api):
                                           ("spreadout", lambda dp, s, d: api.spreadout_alltoallv(dp, s, d), False)])):
         dp = api.DeviceProblem(prob)
         dp.comm.set_forwarding(api.DEFAULT_FORWARDING or 2)
+        dp.comm.set_staging_bound(False)             # (the radix-4 two-layer Bruck on 256-byte blocks stages 4 x its payload)
         ds = dp.new_send_arena()
         dp.fill_payload(0, 3, ds)
         for name, fn, packed in calls:

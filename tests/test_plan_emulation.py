@@ -530,3 +530,54 @@ def test_strided_plans_all_radices(P, strided):
                 recv = np.full(prob.recv_bytes, 0xEE, dtype=np.uint8)
                 assert fn(recv) == 0 and E.last.errors == 0, (P, r)
                 assert np.array_equal(recv, want)
+
+
+# ---- reused staging (launch-per-digit execution with at least three staging regions) ----
+
+@pytest.mark.parametrize("P,r,func", [(64, 2, "tuna"), (64, 2, "twophase"), (81, 3, "om"), (100, 2, "twophase"), (50, 3, "tuna"),
+                                      (64, 4, "om"), (128, 2, "tuna")])
+def test_reused_staging_is_smaller_and_stays_below_twice_the_payload(P, r, func):
+    """A sub-region of staging takes the memory of sub-regions whose blocks have all left before it is written.  The
+    emulator checks every launch (nothing lands on bytes that still wait for their next hop, every staged byte is read
+    exactly once, all have left at the end); here: the arena shrinks and stays below twice the payload, on all-pairs
+    traffic and on the pencil pattern of configuration 5 (rows of a grid)."""
+    fn = {"tuna": lambda rec, p, s, d: E.emulate(E.F_TUNA, p, s, d, r=r, recycle=rec),
+          "twophase": lambda rec, p, s, d: E.emulate(E.F_TWOPHASE, p, s, d, r=r, recycle=rec),
+          "om": lambda rec, p, s, d: E.emulate(E.F_OM, p, s, d, r=r, recycle=rec)}[func]
+    for counts in (W.counts_uniform_random(P, 300, seed=P + r), W.counts_fft_rows(P, 8 if P % 8 == 0 else 10 if P % 10 == 0 else 9, 64)):
+        prob = W.make_problem(counts, 2, 0, 0)
+        send = W.fill_send_arena(prob, 0, 2)
+        want = W.expected_recv_arena(prob, send)
+        sizes = []
+        for rec in (False, True):
+            recv = np.full(prob.recv_bytes, 0xEE, dtype=np.uint8)
+            res = fn(rec, prob, send, recv)
+            assert res.rc == 0 and res.errors == 0, (P, r, func, rec, res.errors)
+            assert np.array_equal(recv, want)
+            sizes.append(res.stage_bytes)
+        assert sizes[1] <= sizes[0] and (r > 2 or sizes[1] < 0.8 * sizes[0]), sizes      # (first fit: a hole must hold a whole sub-region)
+        assert sizes[1] <= 2 * prob.payload_bytes + 128 * P * P, (sizes, prob.payload_bytes)
+
+
+@pytest.mark.parametrize("P,n,r", [(64, 8, 2), (64, 16, 2), (81, 27, 3), (128, 32, 2), (64, 8, 3)])
+def test_reused_staging_twolayer(P, n, r):
+    prob = _prob(P, 0, 3, seed=P + n + r, recv_layout=0)
+    send = W.fill_send_arena(prob, 0, 3)
+    want = W.expected_recv_arena(prob, send)
+    for func, kw in ((E.F_TTPL, dict(n=n, r=r, batch=2)), (E.F_TTPL_S1, dict(n=n, r=r, batch=7)), (E.F_TTPL_RBRUCK, dict(n=n, r=r)),
+                     (E.F_TUNA, dict(r=r, batch=1))):
+        sizes = []
+        for rec in (False, True):
+            recv = np.full(prob.recv_bytes, 0xEE, dtype=np.uint8)
+            res = E.emulate(func, prob, send, recv, recycle=rec, **kw)
+            assert res.rc == 0 and res.errors == 0, (func, rec, res.errors)
+            assert np.array_equal(recv, want)
+            sizes.append(res.stage_bytes)
+        assert sizes[1] <= sizes[0], (func, sizes)
+    up = W.make_uniform_problem(P, 5, 4)
+    us = W.fill_send_arena(up, 0, 1)
+    for func, kw in ((E.F_UNIFORM_SPREADOUT, dict(n=n, r=r, uniform_count=5)), (E.F_UNIFORM_ISPLIT, dict(n=n, r=r, uniform_count=5))):
+        ur = np.full(up.recv_bytes, 0xEE, dtype=np.uint8)
+        res = E.emulate(func, up, us, ur, recycle=True, **kw)
+        assert res.rc == 0 and res.errors == 0, func
+        assert np.array_equal(ur, W.expected_recv_arena(up, us))
