@@ -442,6 +442,7 @@ static int lanes_for(int64_t bytes, int64_t items) {
 static int plan_read(vc_comm *c, const VcSched &S, const std::vector<VcLaunchInfo> &L, PlanInfo &out, bool forward) {
     const int nl = forward ? 1 : (int)L.size();           // forwarded execution: one launch, one set of totals
     const int64_t *h = c->h_header;
+    out = PlanInfo();                                     // (a plan that is derived again in the other execution mode reuses `out`)
     if (h[VC_HEADER_BAD] >= VC_BAD_OVERFLOW)
         return fail_arg("a rank receives more than INT_MAX elements: the packed receive displacements of TTPL_BT_alltoallv do not fit an int",
                         VC_ERR_OVERFLOW);
@@ -478,6 +479,7 @@ static int plan_read(vc_comm *c, const VcSched &S, const std::vector<VcLaunchInf
 static int plan_emit(vc_comm *c, const VcSched &S, std::vector<VcLaunchInfo> &L, const VcTables &T, DevBuf &items, const PlanInfo &pi) {
     hipStream_t st = c->stream;
     if (pi.chain) {
+        if (!c->B.chain_row_base || !c->B.chain_row_tot) return fail_arg("internal: chain items asked for a plan that was not sized for them", VC_ERR_HIP);
         HIP_TRY(items.reserve(sizeof(int64_t) * (size_t)pi.chain_stride * (size_t)std::max<int64_t>(pi.chain_items, 1)));
         HIP_TRY(vc_launch_chain_plan(S, T, c->B.slot_off, c->B.row_base, c->B.chain_row_base, c->B.chain_row_tot + 2 * (size_t)S.P,
                                      items.as<int64_t>(), pi.chain_items, st));

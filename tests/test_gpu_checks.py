@@ -413,6 +413,18 @@ def test_staging_bound(api):
             seen[(bound, mode)] = (int(st.execution), int(st.staging_bytes), int(st.n_launches))
             assert st.moved_bytes * 2 == W.algorithmic_bytes(counts, 8, W.hops_flat(512, 2))
     print(seen, flush=True)
+    # a persistent plan made in forwarded mode for a call beyond the bound is a launch-per-digit plan too
+    dp.comm.set_staging_bound(True)
+    dp.comm.set_forwarding(2)
+    dr = dp.new_recv_arena(0xEE)
+    plan = api.Plan("tuna_algorithm", dp, dr, r=2, batch=0)
+    assert plan.rc == 0, dp.comm.error()
+    for _ in range(2):
+        dr.fill_(0xEE)
+        assert plan.execute(ds, dr) == 0, dp.comm.error()
+        assert dp.verify(ds, dr) == 0
+        assert (dp.comm.last_stats().execution, dp.comm.last_stats().staging_bytes) == seen[(True, 0)][:2]
+    plan.free()
     assert seen[(False, 2)][0] == 1 and seen[(False, 2)][1] > 3.4 * S            # forwarded, every region of its own
     assert seen[(False, 0)][0] == 0 and seen[(False, 0)][1] == seen[(False, 2)][1]
     assert seen[(True, 0)][0] == 0 and seen[(True, 0)][1] < 2 * S                  # reused
