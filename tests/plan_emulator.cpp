@@ -280,3 +280,12 @@ extern "C" int plan_emulate(int func, int P, int n, int r, int batch, int esz, i
     stats_out[0] = nl; stats_out[1] = stage_bytes; stats_out[2] = moved; stats_out[3] = errors; stats_out[4] = items;
     return 0;
 }
+
+// The staging allocator of the planning kernel on its own: sizes per (arrival, departure) family in, bases out.
+extern "C" int64_t staging_allocate(int w, int w2, int msd, int coalesce, const int64_t *size, int64_t *base) {
+    VcSched S;
+    memset(&S, 0, sizeof S);
+    S.w = w; S.w2 = w2; S.msd = msd; S.coalesce = coalesce; S.recycle = 1;
+    std::vector<int64_t> lo(VC_RECYCLE_MAX_PAIRS), hi(VC_RECYCLE_MAX_PAIRS);
+    return vc_allocate_staging(S, size, base, lo.data(), hi.data());
+}

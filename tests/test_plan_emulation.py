@@ -581,3 +581,38 @@ def test_reused_staging_twolayer(P, n, r):
         res = E.emulate(func, up, us, ur, recycle=True, **kw)
         assert res.rc == 0 and res.errors == 0, func
         assert np.array_equal(ur, W.expected_recv_arena(up, us))
+
+
+@pytest.mark.parametrize("msd", [0, 1])
+def test_staging_allocator_never_overlaps_live_sub_regions(msd):
+    """vc_allocate_staging on random sizes: two sub-regions whose lifetimes (arrival slot .. departure slot, in the call's
+    order) touch never share memory; the arena is no larger than separate regions and no smaller than the most bytes alive
+    during any digit's launches."""
+    import ctypes as C
+    lib = C.CDLL(E.build())
+    lib.staging_allocate.restype = C.c_int64
+    rng = np.random.default_rng(7 + msd)
+    for trial in range(300):
+        w = int(rng.integers(1, 9))
+        w2 = int(rng.integers(0, 11 - w)) if not msd else 0
+        ns = w + w2 + 1
+        time = lambda k: (w - 1 - k) if (k < w and msd) else k
+        size = np.zeros(ns * ns + 1, dtype=np.int64)
+        fams = [(ka, kd) for ka in range(ns - 1) for kd in range(ns) if time(kd) > time(ka)]
+        for ka, kd in fams:
+            if rng.random() < 0.8:
+                size[ka * ns + kd] = 128 * int(rng.integers(1, 2000))
+        if rng.random() < 0.3:
+            size[ns * ns] = 128 * int(rng.integers(1, 500))
+        base = np.zeros_like(size)
+        peak = lib.staging_allocate(w, w2, msd, int(size[ns * ns] > 0), size.ctypes.data_as(C.c_void_p), base.ctypes.data_as(C.c_void_p))
+        live = [(time(ka), time(kd), int(base[ka * ns + kd]), int(size[ka * ns + kd])) for ka, kd in fams if size[ka * ns + kd]]
+        if size[ns * ns]:
+            live.append((0, ns - 1, int(base[ns * ns]), int(size[ns * ns])))
+        for i, (a0, d0, b0, s0) in enumerate(live):
+            assert 0 <= b0 and b0 + s0 <= peak
+            for a1, d1, b1, s1 in live[i + 1:]:
+                if a0 <= d1 and a1 <= d0:                      # alive during the launches of a common slot
+                    assert b0 + s0 <= b1 or b1 + s1 <= b0, (trial, (a0, d0, b0, s0), (a1, d1, b1, s1))
+        assert peak <= int(size.sum())
+        assert peak >= max(sum(s for a, d, _, s in live if a <= t <= d) for t in range(ns))
