@@ -96,8 +96,8 @@ int vc_comm_set_forwarding(vc_comm_t comm, int enable);
  *    peak then stays below about 1.5 x the payload where separate regions need the sum over the blocks of
  *    (hops - 1) x bytes (configuration 5 with radix 2: 60 GB);
  *  - forwarded execution keeps every hop's copy of every block, because nothing reads them and so nothing says when one
- *    may be overwritten.  A call whose staging would pass both 1 GiB and twice its payload is therefore run one launch
- *    per digit instead (vc_stats_t.execution says so).
+ *    may be overwritten.  A call whose staging would pass both 1 GiB and three times its payload is therefore run one
+ *    launch per digit instead (vc_stats_t.execution says so).
  * Unbounded: every digit phase has its own region and forwarded calls stay forwarded, whatever they need. */
 int vc_comm_set_staging_bound(vc_comm_t comm, int enable);
 

@@ -55,7 +55,7 @@ class VirtualComm:
 
     def set_staging_bound(self, on: bool) -> None:
         """vc_comm_set_staging_bound: reuse staging memory in launch-per-digit execution and run forwarded calls that would
-        need more than twice their payload (and 1 GiB) that way (default), or give every digit phase its own region."""
+        need more than three times their payload (and 1 GiB) that way (default), or give every digit phase its own region."""
         self._check(self.lib.vc_comm_set_staging_bound(self.handle, int(on)))
 
     def last_stats(self) -> _lib.VcStats:
