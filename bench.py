@@ -77,6 +77,12 @@ def workload(name: str, seed: int):
         # equal blocks of U<bytes> bytes at configuration 4's shape: separates the cost of variable, unaligned blocks
         counts = np.full((1024, 1024), int(name[1:]), dtype=np.int32)
         return counts, 1, "TTPL_BT_alltoallv", dict(n=32, r=32, bblock=0), W.hops_twolayer(1024, 32, 32)
+    if name.startswith("C4m"):
+        # configuration 4 with every count rounded to a multiple of C4m<bytes>: sources and destinations then share their
+        # phase modulo that many bytes, which prices the byte phases of the real configuration
+        m = int(name[3:])
+        counts = ((W.config_counts("C4", seed)[0] + m // 2) // m * m).astype(np.int32)
+        return counts, 1, "TTPL_BT_alltoallv", dict(n=32, r=32, bblock=0), W.hops_twolayer(1024, 32, 32)
     counts, esz, tun = W.config_counts(name, seed)
     P = counts.shape[0]
     if name == "C4":
@@ -424,7 +430,8 @@ def main() -> None:
         "metric": METRIC, "value": round(S / call_s / 1e9, 2), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "u8", "data": "synthetic",
-        "config": {"workload": (f"benchmark configuration {args.workload[1:]}" if args.workload[0] == "C" else
+        "config": {"workload": (f"benchmark configuration 4 with counts rounded to multiples of {args.workload[3:]} bytes" if args.workload.startswith("C4m") else
+                                f"benchmark configuration {args.workload[1:]}" if args.workload[0] == "C" else
                                 f"equal blocks of {args.workload[1:]} bytes" if args.workload[0] == "U" else
                                 f"reference input matrix inputs/{prob.P}proc") + f": {func}, P={prob.P} virtual ranks, "
                                + ", ".join(f"{k}={v}" for k, v in tun.items()) + f", {esz}-byte elements",

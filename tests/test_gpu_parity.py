@@ -605,6 +605,37 @@ def test_reference_input_matrices(api):
             (f"ML{P} tuna r=8", lambda d: api.tuna_algorithm(8, 0, dp, ds, d), False)])
 
 
+@pytest.mark.parametrize("P", [64, 1024])
+def test_reference_input_matrices_at_full_size(api, P):
+    """The smallest and the largest of the reference's communication patterns at their real sizes (5.2 and 12.8 GB of
+    payload, examples/MLinputs_example.cpp:96: twophase_rbruck_alltoallv on 1-byte elements), checked as the benchmark
+    configurations are: definition check on the device, byte sum, and the transposed alltoallv by another function."""
+    if api.DEFAULT_FORWARDING not in (0, 2):
+        pytest.skip("blocks of megabytes belong to the work-item list and to launch-per-digit execution")
+    import os
+    import torch
+    from tests.helpers import INPUTS_DIR
+    counts = W.counts_from_npz(os.path.join(INPUTS_DIR, f"global_comm_pattern_{P}proc.npz"))
+    prob = W.make_problem(counts, 1, 0, 0)
+    dp = api.DeviceProblem(prob)
+    ds = dp.new_send_arena()
+    ds.zero_()
+    dp.fill_payload(0, 13, ds)
+    checksum = _byte_sum(ds)
+    dr = dp.new_recv_arena(0)
+    print("  ML", P, "payload", prob.payload_bytes, flush=True)
+    assert api.twophase_rbruck_alltoallv(32, dp, ds, dr) == 0, dp.comm.error()
+    assert dp.verify(ds, dr) == 0
+    assert _byte_sum(dr) == checksum
+    assert dp.comm.last_stats().payload_bytes == prob.payload_bytes
+    dp.comm.free()
+    tp = api.DeviceProblem(_transposed(prob))
+    dback = tp.new_recv_arena(0)
+    assert api.tuna_algorithm(8, 0, tp, dr, dback) == 0, tp.comm.error()
+    assert torch.equal(dback, ds)
+    tp.comm.free()
+
+
 def test_suggest_radix_matches_the_traffic_model(api):
     for P, n in ((64, 0), (100, 0), (256, 0), (128, 32), (64, 8)):
         counts = W.counts_zipf(P, 4096, 1.2, 5, P)
