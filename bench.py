@@ -234,6 +234,8 @@ def kernel_name(st) -> str:
     base, lanes = EXECUTION_KERNELS[int(st.execution)], int(st.lanes_per_item)
     if lanes == 16:
         return base + "_quarter_kernel"
+    if lanes == 1:
+        return base + "_batch_kernel"
     return base + "_kernel" + f"<{lanes}>"
 
 

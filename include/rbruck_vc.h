@@ -79,8 +79,10 @@ int vc_comm_set_bases(vc_comm_t comm, const int64_t *sbase_bytes, const int64_t 
  *    on the device that this call's blocks fit): slot addresses are then closed forms, and one pass over the count tables
  *    replaces the planner's prefix sums and slot tables.  Only on at most 128 ranks and while regions x P x P x stride
  *    stays below 256 MiB.
- * 2: forwarded, always through the list.   3 / 4: forwarded, always without it, a workgroup / a quarter of a wavefront
- *    per pair of ranks (any sizes; not the fastest choice everywhere).
+ *    On more than 128 ranks and blocks below 384 B on average a wavefront takes a batch of 16 - 64 pairs instead: a lane per
+ *    pair works out the route, then the quarters of the wavefront carry the blocks one after the other.
+ * 2: forwarded, always through the list.   3 / 4 / 5: forwarded, always without it, a workgroup / a quarter of a
+ *    wavefront per pair of ranks / a batch of pairs per wavefront (any sizes; not the fastest choice everywhere).
  * 0: one kernel launch per digit phase (or per batch of its rounds, as b / bblock say); every hop reads the block
  *    where the previous hop left it.  This is the mode whose launches vc_comm_last_stats and vc_comm_last_traffic
  *    describe one by one.
@@ -326,7 +328,8 @@ typedef struct {
                                     without one, 3 forwarded without one on fixed-stride staging (see vc_comm_set_forwarding) */
     int32_t lanes_per_item;      /* 256: the copy kernel gave every work item (without a list: every pair of ranks) a
                                     workgroup; 64: a wavefront (short pieces); 16: a quarter of one (pieces of a
-                                    few hundred bytes).  Launch-per-digit execution: of the launch that moved the most bytes. */
+                                    few hundred bytes); 1: a wavefront took a batch of pairs of ranks (many very short
+                                    blocks).  Launch-per-digit execution: of the launch that moved the most bytes. */
 } vc_stats_t;
 
 /* Per-launch HIP-event timing of the following calls (0 = off, default). */

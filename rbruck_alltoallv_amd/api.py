@@ -50,7 +50,8 @@ class VirtualComm:
     def set_forwarding(self, enable: bool | int) -> None:
         """vc_comm_set_forwarding: 0 / False one launch per digit phase; 1 / True forwarded (one launch per call, every
         block piece carried through all its hops in registers; the library picks list or listless); 2 forwarded through
-        a work-item list; 3 / 4 forwarded without one, a workgroup / a quarter of a wavefront per pair of ranks."""
+        a work-item list; 3 / 4 / 5 forwarded without one, a workgroup / a quarter of a wavefront per pair of ranks / a
+        batch of pairs per wavefront."""
         self._check(self.lib.vc_comm_set_forwarding(self.handle, int(enable)))
 
     def set_staging_bound(self, on: bool) -> None:

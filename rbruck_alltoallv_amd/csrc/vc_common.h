@@ -14,6 +14,9 @@
 #define VC_THREADS 256
 // lanes of a work item in the copy kernels for short pieces: a wavefront (VC_WAVE, vc_scan.h) or a quarter of one
 #define VC_QUARTER 16
+// lane code of the listless copy kernel that gives a wavefront a batch of pairs: a lane per pair works out the route, then
+// the quarters of the wavefront carry the blocks one after the other
+#define VC_BATCHED 1
 // window of one workgroup of the copy kernel: 256 lanes x 2 vectors x 16 bytes, starting at a cache-line boundary
 #define VC_CHUNK 8192
 #define VC_LINE 128

@@ -196,7 +196,7 @@ def test_tables_that_disagree_are_refused(api):
     s, d = dp.new_send_arena(), dp.new_recv_arena()
     dp.fill_payload(0, 1, s)
     keep = int(dp.recvcounts[7, 3].item())
-    for mode in (0, 1, 2, 3, 4):
+    for mode in (0, 1, 2, 3, 4, 5):
         dp.comm.set_forwarding(mode)
         for delta in (1, -1):
             dp.recvcounts[7, 3] = keep + delta

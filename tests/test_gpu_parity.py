@@ -15,9 +15,9 @@ pytestmark = pytest.mark.gpu
 CASES = load_golden()
 
 
-# vc_comm_set_forwarding: 2 forwarded through a work-item list, 3 / 4 forwarded without one (a workgroup / a quarter of a
-# wavefront per pair of ranks), 0 one launch per digit phase
-MODES = {"forwarded": 2, "forwarded-listless": 3, "forwarded-listless-quarter": 4, "launch-per-digit": 0}
+# vc_comm_set_forwarding: 2 forwarded through a work-item list, 3 / 4 / 5 forwarded without one (a workgroup / a quarter of a
+# wavefront per pair of ranks / a batch of pairs per wavefront), 0 one launch per digit phase
+MODES = {"forwarded": 2, "forwarded-listless": 3, "forwarded-listless-quarter": 4, "forwarded-listless-batch": 5, "launch-per-digit": 0}
 
 
 @pytest.fixture(scope="module", params=list(MODES))
@@ -520,7 +520,7 @@ def test_benchmark_configurations_at_full_size(api, name):
 def test_blocks_beyond_two_gib(api):
     """Counts and displacements are int32 elements, byte offsets 64-bit: a 2.4 GB block (300 M elements of 8 bytes; the
     reference's int byte arithmetic, src/twophase_tunable_rbruckv.cpp:98, would overflow) next to empty and tiny ones."""
-    if api.DEFAULT_FORWARDING == 4:
+    if api.DEFAULT_FORWARDING in (4, 5):
         pytest.skip("one 2.4 GB block moved by the 16 lanes of its pair: exact, but half a minute")
     import torch
     counts = np.array([[3, 300_000_000, 0], [1, 0, 7], [200_000_000, 5, 2]], dtype=np.int32)
@@ -828,19 +828,21 @@ def test_default_mode_picks_the_listless_kernel_for_small_calls(api):
     # device (longer blocks than the stride holds), and redone through the list
     assert seen == [1, 3, 3, 1, 1, 1, 3]
     comm.free()
-    # blocks of a few hundred bytes go without the list on any number of ranks, a quarter of a wavefront per pair
-    prob = W.make_problem(W.counts_uniform_random(300, 600, seed=2), 1, 0, 0)
-    dp = api.DeviceProblem(prob)
-    dp.comm.set_forwarding(1)
-    ds, dr = dp.new_send_arena(), dp.new_recv_arena()
-    dp.fill_payload(0, 5, ds)
-    seen = []
-    for _ in range(3):
-        assert api.TTPL_BT_alltoallv_s1(10, 3, 0, dp, ds, dr) == 0 and dp.verify(ds, dr) == 0
-        st = dp.comm.last_stats()
-        seen.append((st.execution, st.lanes_per_item))
-    assert seen == [(1, 16), (2, 16), (2, 16)]             # (fixed-stride staging only on at most 128 ranks)
-    dp.comm.free()
+    # blocks of a few hundred bytes go without the list on any number of ranks: a quarter of a wavefront per pair, or (average
+    # block below 384 bytes on more than 128 ranks) a batch of pairs per wavefront, reported as 1 lane per pair
+    for top, lanes in ((900, 16), (600, 1)):
+        prob = W.make_problem(W.counts_uniform_random(300, top, seed=2), 1, 0, 0)
+        dp = api.DeviceProblem(prob)
+        dp.comm.set_forwarding(1)
+        ds, dr = dp.new_send_arena(), dp.new_recv_arena()
+        dp.fill_payload(0, 5, ds)
+        seen = []
+        for _ in range(3):
+            assert api.TTPL_BT_alltoallv_s1(10, 3, 0, dp, ds, dr) == 0 and dp.verify(ds, dr) == 0
+            st = dp.comm.last_stats()
+            seen.append((st.execution, st.lanes_per_item))
+        assert seen[0][0] == 1 and seen[1:] == [(2, lanes), (2, lanes)], (top, seen)      # (fixed-stride staging only on at most 128 ranks)
+        dp.comm.free()
 
 
 @pytest.mark.parametrize("hi,lanes", [(200, 16), (3000, 64), (12000, 256)])
@@ -860,7 +862,7 @@ def test_three_shapes_of_the_copy_kernel(api, hi, lanes):
         assert fn(dr) == 0, (name, dp.comm.error())
         assert dp.verify(ds, dr) == 0, name
         st = dp.comm.last_stats()
-        assert st.lanes_per_item == ({3: 256, 4: 16}[api.DEFAULT_FORWARDING] if st.execution == 2 else lanes), (name, st.lanes_per_item)
+        assert st.lanes_per_item == ({3: 256, 4: 16, 5: 1}[api.DEFAULT_FORWARDING] if st.execution == 2 else lanes), (name, st.lanes_per_item)
     dp.comm.free()
 
 
@@ -912,7 +914,7 @@ def test_both_execution_modes_leave_the_same_staging(api):
         for name, fn in calls:
             print("  ", name, flush=True)
             snaps, sizes = [], []
-            for mode in (0, 2, 3, 4):
+            for mode in (0, 2, 3, 4, 5):
                 dp.comm.set_forwarding(mode)
                 dr = dp.new_recv_arena(0xEE)
                 assert fn(dp, ds, dr) == 0, (name, dp.comm.error())          # sizes the arena
@@ -925,7 +927,7 @@ def test_both_execution_modes_leave_the_same_staging(api):
                 assert dp.comm.staging() == (ptr, size)
                 snap = torch.empty(n, dtype=torch.uint8, device="cuda:0")
                 assert lib.vc_calibration_copy(snap.data_ptr(), ptr, n, h) == 0
-                assert dp.comm.last_stats().execution == {0: 0, 2: 1, 3: 2, 4: 2}[mode]
+                assert dp.comm.last_stats().execution == {0: 0, 2: 1, 3: 2, 4: 2, 5: 2}[mode]
                 snaps.append(snap.cpu().numpy())
                 sizes.append(size)
             assert sizes[0] == sizes[1] == sizes[2] == sizes[3], name
