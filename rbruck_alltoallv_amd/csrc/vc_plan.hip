@@ -62,14 +62,24 @@ __global__ __launch_bounds__(VC_THREADS) void vc_plan_rows(VcSched S, VcLaunchPa
     if ((int)blockIdx.y < nreg) {
         const int y = blockIdx.y;
         int64_t carry = 0, data = 0;
-        for (int base = 0; base < P; base += VC_THREADS) {
-            const int id = base + threadIdx.x;
-            int64_t total, len = 0;
-            const int64_t v = (id < P) ? vc_region_slot_size(S, T, y, to, id, &len) : 0;
-            const int64_t ex = vc_block_exclusive_scan(v, lds, total);
-            if (id < P) slot_off[((int64_t)y * P + to) * P + id] = carry + ex;
-            carry += total;
-            data += len;
+        for (int base0 = 0; base0 < P; base0 += 4 * VC_THREADS) {       // four chunks at a time: their table reads travel together
+            int64_t v[4], len[4];
+#pragma unroll
+            for (int u = 0; u < 4; u++) {
+                const int id = base0 + u * VC_THREADS + threadIdx.x;
+                len[u] = 0;
+                v[u] = (id < P) ? vc_region_slot_size(S, T, y, to, id, &len[u]) : 0;
+            }
+#pragma unroll
+            for (int u = 0; u < 4; u++) {
+                const int id = base0 + u * VC_THREADS + threadIdx.x;
+                if (base0 + u * VC_THREADS >= P) break;
+                int64_t total;
+                const int64_t ex = vc_block_exclusive_scan(v[u], lds, total);
+                if (id < P) slot_off[((int64_t)y * P + to) * P + id] = carry + ex;
+                carry += total;
+                data += len[u];
+            }
         }
         if (forward) data = vc_block_sum(data, lds);
         if (threadIdx.x == 0) {
@@ -82,19 +92,35 @@ __global__ __launch_bounds__(VC_THREADS) void vc_plan_rows(VcSched S, VcLaunchPa
     int64_t bad = 0;                                      // entries of this rank's rows no rank could have passed
     const int L = blockIdx.y - nreg;
     if (forward) {
-        // sources in chunks of VC_THREADS: the items before each chunk let vc_chain_emit give every chunk a workgroup
+        // sources in chunks of VC_THREADS: the items before each chunk let vc_chain_emit give every chunk a workgroup.
+        // Four chunks at a time, so that the table reads of all of them travel together before the first sum needs them;
+        // the checks of this rank's own rows (the loop over ids below, for launch-per-digit execution) ride along.
         const int nchunk = (P + VC_THREADS - 1) / VC_THREADS;
         int64_t before = 0;
-        for (int chunk = 0; chunk < nchunk; chunk++) {
-            const int s = chunk * VC_THREADS + threadIdx.x;
-            const int64_t cnt = s < P ? vc_chain_count(S, T, s, to) : 0;
-            // the receiver must expect exactly what the source sends (the reference fails with an MPI truncation error)
-            bad += s < P && T.rc[(int64_t)to * P + s] != T.sc[(int64_t)s * P + to];
-            most = cnt > most ? cnt : most;
-            const int64_t len = s < P ? (int64_t)T.sc[(int64_t)s * P + to] * S.esz : 0;
-            longest = len > longest ? len : longest;
-            if (threadIdx.x == 0) chain_row_tot[2 * (int64_t)P + (int64_t)to * nchunk + chunk] = before;
-            before += vc_block_sum(cnt, lds);
+        for (int chunk0 = 0; chunk0 < nchunk; chunk0 += 4) {
+            int64_t cnt[4];
+#pragma unroll
+            for (int u = 0; u < 4; u++) {
+                const int s = (chunk0 + u) * VC_THREADS + threadIdx.x;
+                cnt[u] = 0;
+                if (chunk0 + u >= nchunk || s >= P) continue;
+                cnt[u] = vc_chain_count(S, T, s, to);
+                const int64_t i = (int64_t)to * P + s;
+                const int expected = T.rc[i], sent = T.sc[(int64_t)s * P + to];
+                // the receiver must expect exactly what the source sends (the reference fails with an MPI truncation error)
+                bad += expected != sent;
+                bad += (T.sc[i] < 0) | (T.sd[i] < 0) | (expected < 0) | (!S.packed_recv && T.rd[i] < 0);
+                payload += (int64_t)expected * S.esz;
+                most = cnt[u] > most ? cnt[u] : most;
+                const int64_t len = (int64_t)sent * S.esz;
+                longest = len > longest ? len : longest;
+            }
+#pragma unroll
+            for (int u = 0; u < 4; u++) {
+                if (chunk0 + u >= nchunk) break;
+                if (threadIdx.x == 0) chain_row_tot[2 * (int64_t)P + (int64_t)to * nchunk + chunk0 + u] = before;
+                before += vc_block_sum(cnt[u], lds);
+            }
         }
         items = threadIdx.x == 0 ? before : 0;            // vc_block_sum below adds the lanes up
     } else {
@@ -109,12 +135,12 @@ __global__ __launch_bounds__(VC_THREADS) void vc_plan_rows(VcSched S, VcLaunchPa
             }
         }
     }
-    if (L == 0)
+    if (L == 0 && !forward)                               // forwarded execution has done this above
         for (int id = threadIdx.x; id < P; id += VC_THREADS) {
             const int64_t i = (int64_t)to * P + id;
             payload += (int64_t)T.rc[i] * S.esz;
             bad += (T.sc[i] < 0) | (T.sd[i] < 0) | (T.rc[i] < 0) | (!S.packed_recv && T.rd[i] < 0);
-            if (!forward) bad += T.rc[i] != T.sc[(int64_t)id * P + to];      // forwarded execution has compared them above
+            bad += T.rc[i] != T.sc[(int64_t)id * P + to];
         }
     items = vc_block_sum(items, lds);
     if (forward) { most = vc_block_max(most, lds); longest = vc_block_max(longest, lds); } else bytes = vc_block_sum(bytes, lds);
