@@ -224,8 +224,8 @@ EXECUTION_NAMES = {0: "launch per digit phase",
                    1: "forwarded (one launch, blocks carried through all hops in registers)",
                    2: "forwarded, without a work-item list (every pair of ranks derives its block's route in the copy kernel; "
                       "one host synchronisation per call)",
-                   3: "forwarded, without a work-item list, staging slots at a fixed stride (one pass over the count tables "
-                      "instead of the planner's prefix sums; one host synchronisation per call)"}
+                   3: "forwarded, without a work-item list, staging slots at a fixed stride (no planner: the one launch of the call "
+                      "also adds up the tables' totals; one host synchronisation per call)"}
 EXECUTION_KERNELS = {0: "vc_copy_items", 1: "vc_copy_chains", 2: "vc_copy_blocks", 3: "vc_copy_blocks"}
 
 

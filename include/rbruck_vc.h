@@ -41,7 +41,8 @@ typedef struct vc_comm *vc_comm_t;
 #define VC_ERR_ARG (-5)        /* null handle / pointer, element size < 1, bases not set */
 #define VC_ERR_NO_DEVICE (-6)  /* no HIP device */
 #define VC_ERR_TABLES (-7)     /* a negative count or displacement in the tables, or recvcounts[t][s] != sendcounts[s][t] (the reference
-                                  fails with an MPI truncation error); found on the device before anything is copied */
+                                  fails with an MPI truncation error); found on the device before anything is copied
+                                  (single-launch execution of small calls: before the pair's own block is) */
 #define VC_ERR_OVERFLOW (-8)   /* a rank's counts sum past INT_MAX elements, where the reference's int displacements wrap
                                   (examples/rbruckv_example.cpp:69-72): vc_displs_from_counts, and the packed receive layout of
                                   TTPL_BT_alltoallv (src/twophase_twolayer_rbruck.cpp:406-418) */
@@ -75,10 +76,12 @@ int vc_comm_set_bases(vc_comm_t comm, const int64_t *sbase_bytes, const int64_t 
  *    quarter of a wavefront (short blocks: average piece below 768 B on any number of ranks, below 1.75 - 3 KiB on 33 - 128) that derives its block's route itself; the
  *    kernel is enqueued right behind the size computation and the call needs one host synchronisation instead of two.
  *    Such a call also gets the reference's own staging layout, every slot as long as the longest block
- *    (src/twophase_tunable_rbruckv.cpp:59; the stride comes from the last call's longest block, and the copy kernel checks
- *    on the device that this call's blocks fit): slot addresses are then closed forms, and one pass over the count tables
- *    replaces the planner's prefix sums and slot tables.  Only on at most 128 ranks and while regions x P x P x stride
- *    stays below 256 MiB.
+ *    (src/twophase_tunable_rbruckv.cpp:59; the stride comes from the last call's longest block): slot addresses are then
+ *    closed forms and the call is a single kernel launch, without a planner before it.  Every pair of ranks checks its own
+ *    table entries, and that its block fits a slot, before it moves anything, and the kernel's first wavefronts add up
+ *    what the host needs afterwards; a call with a longer block is redone the general way.  Only on at most 128 ranks
+ *    and while regions x P x P x stride stays below 256 MiB.  This is the one execution in which a call that returns
+ *    VC_ERR_TABLES may already have delivered the blocks of the pairs whose entries were in order.
  *    On more than 128 ranks and blocks below 384 B on average a wavefront takes a batch of 16 - 64 pairs instead: a lane per
  *    pair works out the route, then the quarters of the wavefront carry the blocks one after the other.
  * 2: forwarded, always through the list.   3 / 4 / 5: forwarded, always without it, a workgroup / a quarter of a

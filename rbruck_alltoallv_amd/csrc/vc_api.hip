@@ -624,17 +624,20 @@ static int listless_lanes(const vc_comm *c, const VcSched &S) {
 
 // Fixed-stride staging for calls of short blocks (the default mode, after a call that the listless kernels could serve):
 // the reference's own layout, every slot as long as the longest block (src/twophase_tunable_rbruckv.cpp:59), makes slot
-// addresses closed forms, so the call needs neither the planner's prefix sums nor its slot tables: one pass over the count
-// tables (validation, totals, the longest block), the listless copy kernel right behind it, one host synchronisation.  The
-// stride comes from the last call's longest block; the copy kernel checks on the device that this call's blocks fit and
-// touches nothing otherwise (the call then goes the general way).  Costs arena: regions x P x P x stride bytes, so only
+// addresses closed forms, so the call needs neither the planner's prefix sums nor its slot tables, and no planner at all
+// before the copy kernel: the call is ONE launch and one host synchronisation.  The first wavefronts of the copy kernel
+// add up what the host wants to know afterwards (validation, totals, the longest block); every pair of ranks checks its
+// own table entries, and that its block fits a slot, before it moves anything.  The stride comes from the last call's
+// longest block; a call with a longer block is redone the general way, and a call with bad tables returns the same
+// code as elsewhere — but blocks of the pairs whose entries were in order may have been delivered by then (everywhere
+// else nothing moves before the tables have been checked).  Costs arena: regions x P x P x stride bytes, so only
 // up to VC_STRIDED_MAX_BYTES, and only on communicators of at most 128 ranks: measured on MI355X, 64 ranks with blocks of
-// 0 - 4 KiB 41 -> 29 us per call, but 1024 ranks with blocks of 0 - 512 B 380 -> 560 us (805 MB of slots 768 bytes apart
-// instead of 270 MB of compact ones).  Returns 1 when the call has been served, 0 when it must go the general way, < 0 on
-// errors.
+// 0 - 4 KiB 41 -> 29 us per call with a pass over the tables before the copy kernel, 25 us with the pass inside it, but
+// 1024 ranks with blocks of 0 - 512 B 380 -> 560 us (805 MB of slots 768 bytes apart instead of 270 MB of compact ones).
+// Returns 1 when the call has been served, 0 when it must go the general way, < 0 on errors.
 #define VC_STRIDED_MAX_BYTES ((int64_t)256 << 20)
 static int try_strided(vc_comm *c, VcSched S, std::vector<VcLaunchInfo> &L, const char *sendbuf, char *recvbuf, VcTables T, int pair_lanes) {
-    if (c->forward != 1 || !pair_lanes || S.coalesce || vc_hop_slots(S) > VC_MAX_HOP_SLOTS) return 0;
+    if (c->forward != 1 || !pair_lanes || pair_lanes == VC_BATCHED || S.coalesce || vc_hop_slots(S) > VC_MAX_HOP_SLOTS) return 0;
     if ((int64_t)S.P * S.P > VC_LISTLESS_MAX_PAIRS) return 0;
     const int64_t stride = (c->hint_max_len + 2 * VC_LINE - 1) & ~(int64_t)(VC_LINE - 1);     // the block at any cache-line phase
     if (stride > 0x7FFFFF80) return 0;
@@ -661,13 +664,14 @@ static int try_strided(vc_comm *c, VcSched S, std::vector<VcLaunchInfo> &L, cons
         HIP_TRY(vc_launch_row_scan(T.rc, c->rd_packed.as<int>(), nullptr, nullptr, S.P, st));
         T.rd_packed = c->rd_packed.as<int>();
     }
-    HIP_TRY(vc_launch_scan_tables(S, T, header, st));
-    const bool quarter = pair_lanes == VC_QUARTER || pair_lanes == VC_BATCHED;
+    const bool quarter = pair_lanes == VC_QUARTER;
     VcListlessGuard guard = {(int64_t)c->stage.cap - 64, quarter ? VC_LISTLESS_MAX_PIECES : VC_LISTLESS_WG_MAX_PIECES,
                              quarter ? 0 : VC_LISTLESS_MAX_ITEMS, quarter ? 4096 : 0, stride - VC_LINE + 1};
     if (c->timing) { HIP_TRY(hipEventRecord(c->events[1], st)); HIP_TRY(hipEventRecord(c->events[2], st)); }
+    // the one launch of the call: its first wavefronts add the tables' totals up into `header`, every pair checks its own
+    // entries and the length of its block before it moves anything
     HIP_TRY(vc_launch_copy_blocks(S, T, nullptr, nullptr, header, guard, pair_lanes, sendbuf, recvbuf, c->stage.as<char>(), st, c->h_header_dev,
-                                  header_next));
+                                  header_next, header));
     c->strided_clean = true;
     if (c->timing) HIP_TRY(hipEventRecord(c->events[3], st));
     HIP_TRY(hipStreamSynchronize(st));

@@ -145,6 +145,8 @@ hipError_t vc_launch_empty(hipStream_t st);
 // added to header[VC_HEADER_BAD] once per rank whose packed receive displacements would pass INT_MAX elements
 #define VC_BAD_OVERFLOW (1ll << 40)
 #define VC_HEADER_MAX_PIECES 4
+// fixed-stride staging: wavefronts that have added their part of the tables' totals into the header
+#define VC_HEADER_SYNC (VC_HEADER_MAX_LEN + 1)
 #define VC_HEADER_WORDS(nl) (VC_HEADER_FIXED + 2 * (nl))
 // Passes 1 and 2: staging prefix sums and the number of work items of every launch (sizes only).  The launch table
 // travels as a kernel argument when it has at most VC_LAUNCH_PACK entries (launches_dev is then not read).  With chain_row_tot /
@@ -155,10 +157,6 @@ hipError_t vc_launch_plan_sizes(const VcSched &S, const VcLaunchInfo *launches_h
                                 int64_t *row_tot, int64_t *row_base, int64_t *org_run_base, int64_t *item_row_tot,
                                 int64_t *item_row_base, int64_t *row_bytes, int64_t *chain_row_tot, int64_t *chain_row_base,
                                 int64_t *header, int64_t *header_host, hipStream_t st);
-// Fixed-stride staging (S.stride > 0), forwarded execution: one pass over the tables instead of the prefix sums —
-// validation, payload, block pieces, longest block, hop-weighted bytes — added up into `header` (device; the caller has
-// zeroed words 0 .. VC_HEADER_MAX_LEN).  header[0] is set to the bytes the fixed-stride arena takes.
-hipError_t vc_launch_scan_tables(const VcSched &S, VcTables T, int64_t *header, hipStream_t st);
 // Forwarded execution: the chain items (every block's route in closed form, staging addresses from the plan tables).
 // chain_chunk_pre: [P][chunks of VC_THREADS sources] items of a receiver before each chunk (vc_launch_plan_sizes leaves it
 // behind chain_row_tot's first 2 P words).
@@ -205,7 +203,14 @@ VC_HD bool vc_listless_ok(const int64_t *header, const VcListlessGuard &g) {
 // header_host (pinned, may be null): the first workgroup copies the fixed words of `header` there, for planners that add
 // the header up with atomics and cannot write it to the host themselves.  header_zero (may be null): ... and clears the
 // fixed words there: the header the next call's planner will add up into.
+// totals (device, non-null: fixed-stride staging, S.stride > 0, at most VC_MAX_GRID pairs): the kernel needs no planner
+// before it.  Its first wavefronts add up the tables' totals — validation, payload, block pieces, longest block,
+// hop-weighted bytes — into `totals` (words 0 .. VC_HEADER_SYNC zeroed by the caller) and the last of them to finish
+// copies the words to header_host, with [0] = the bytes the fixed-stride arena takes; `header` is not read.  Every pair
+// checks its own table entries and the guard's max_len / max_pieces and leaves its block alone when one of them fails, so
+// no address is formed from a bad entry; the host, which evaluates the same conditions on the totals afterwards, reports
+// the call as refused then.  Blocks of the other pairs may already have been delivered.
 hipError_t vc_launch_copy_blocks(const VcSched &S, VcTables T, const int64_t *slot_off, const int64_t *row_base, const int64_t *header,
                                  VcListlessGuard guard, int lanes, const char *sendbuf, char *recvbuf, char *stage, hipStream_t st,
-                                 int64_t *header_host = nullptr, int64_t *header_zero = nullptr);
+                                 int64_t *header_host = nullptr, int64_t *header_zero = nullptr, int64_t *totals = nullptr);
 hipError_t vc_launch_calibration_copy(const char *src, char *dst, int64_t nbytes, hipStream_t st);

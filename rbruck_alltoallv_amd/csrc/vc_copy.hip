@@ -191,6 +191,90 @@ __global__ __launch_bounds__(VC_WAVE) void vc_copy_items_quarter_kernel(const Vc
     vc_forward_piece_quarter(vc_resolve(d.src, sendbuf, recvbuf, stage), d.len, 1, [&](int) { return dst; });
 }
 
+// ---- fixed-stride staging in one launch (the `totals` of vc_launch_copy_blocks) ----
+__device__ __forceinline__ int64_t vc_wave_sum(int64_t v) {
+#pragma unroll
+    for (int o = VC_WAVE / 2; o > 0; o >>= 1) v += __shfl_xor(v, o, VC_WAVE);
+    return v;
+}
+
+__device__ __forceinline__ int64_t vc_wave_max(int64_t v) {
+#pragma unroll
+    for (int o = VC_WAVE / 2; o > 0; o >>= 1) {
+        const int64_t u = __shfl_xor(v, o, VC_WAVE);
+        v = u > v ? u : v;
+    }
+    return v;
+}
+
+// The wavefronts of the first vc_totals_blocks workgroups of the grid: one pair of ranks per lane (by receiver, then source), the wavefront's
+// sums and maxima added into `totals` with one atomic each: [1] payload, [2] block pieces, [3] table entries no rank could
+// have passed, [4] the most pieces of a block, [5] hop-weighted bytes, [6] the longest block.  The wavefront that finishes
+// last hands the words to the host.
+__device__ __forceinline__ void vc_add_totals(const VcSched &S, const VcTables &T, int64_t *totals, int64_t *header_host) {
+    const int P = S.P;
+    const int64_t pairs = (int64_t)P * P, nwaves = (pairs + VC_WAVE - 1) / VC_WAVE;
+    const int64_t wave = (int64_t)blockIdx.x * (blockDim.x / VC_WAVE) + threadIdx.x / VC_WAVE;
+    if (wave >= nwaves) return;
+    const int lane = threadIdx.x & (VC_WAVE - 1);
+    const int64_t idx = wave * VC_WAVE + lane;
+    int64_t payload = 0, items = 0, bad = 0, most = 0, moved = 0, longest = 0;
+    if (idx < pairs) {
+        const int to = (int)(idx / P), s = (int)(idx % P);
+        const int64_t i = (int64_t)to * P + s, k = (int64_t)s * P + to;
+        const int sc = T.sc[k], rc = T.rc[i];
+        bad = (sc < 0) | (rc != sc) | (T.sd[i] < 0) | (!S.packed_recv && T.rd[i] < 0);
+        // (a packed receive layout past INT_MAX elements shows as a negative packed displacement of a later source)
+        if (S.packed_recv && (T.rd_packed[i] < 0 || (s == P - 1 && (int64_t)T.rd_packed[i] + rc > 0x7FFFFFFF))) bad += VC_BAD_OVERFLOW;
+        const int64_t len = (int64_t)sc * S.esz;
+        payload = longest = len;
+        items = most = sc > 0 ? vc_chain_count(S, T, s, to) : 0;
+        moved = len * vc_block_hops(S, s, to);
+    }
+    payload = vc_wave_sum(payload);
+    items = vc_wave_sum(items);
+    bad = vc_wave_sum(bad);
+    moved = vc_wave_sum(moved);
+    most = vc_wave_max(most);
+    longest = vc_wave_max(longest);
+    unsigned long long *h = reinterpret_cast<unsigned long long *>(totals);
+    int last = 0;
+    if (lane == 0) {
+        if (payload) atomicAdd(&h[1], (unsigned long long)payload);
+        if (items) atomicAdd(&h[2], (unsigned long long)items);
+        if (bad) atomicAdd(&h[VC_HEADER_BAD], (unsigned long long)bad);
+        if (moved) atomicAdd(&h[VC_HEADER_FIXED], (unsigned long long)moved);
+        if (most) atomicMax(&h[VC_HEADER_MAX_PIECES], (unsigned long long)most);
+        if (longest) atomicMax(&h[VC_HEADER_MAX_LEN], (unsigned long long)longest);
+        __threadfence();                                  // the words above before the count below
+        last = atomicAdd(&h[VC_HEADER_SYNC], 1ull) == (unsigned long long)(nwaves - 1);
+    }
+    last = __shfl(last, 0, VC_WAVE);
+    if (last && lane <= VC_HEADER_MAX_LEN)
+        header_host[lane] = lane == 0 ? vc_strided_stage_bytes(S)
+                                      : (int64_t)__hip_atomic_load(&h[lane], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// Workgroups at the head of the grid that only add up the totals (none without `totals`): their round trips run beside the
+// copying instead of in front of it.  A multiple of VC_XCDS, so that the workgroups behind them keep their XCDs.
+__host__ __device__ __forceinline__ unsigned vc_totals_blocks(const VcSched &S, const int64_t *totals, int lanes) {
+    if (!totals) return 0;
+    const int64_t waves = ((int64_t)S.P * S.P + VC_WAVE - 1) / VC_WAVE, per = lanes / VC_WAVE;
+    return (unsigned)(((waves + per - 1) / per + VC_XCDS - 1) / VC_XCDS * VC_XCDS);
+}
+
+// Whether the pair's own table entries allow its block to be moved: none negative, the receiver expecting what the
+// source sends, the block no longer than a slot and cut into no more pieces than the kernel was chosen for.
+__device__ __forceinline__ bool vc_pair_allowed(const VcSched &S, const VcTables &T, const VcListlessGuard &g, int s, int t) {
+    const int64_t i = (int64_t)t * S.P + s, k = (int64_t)s * S.P + t;
+    const int sc = T.sc[k];
+    if (sc < 0 || T.rc[i] != sc || T.sd[k] < 0 || (S.packed_recv ? T.rd_packed[i] < 0 : T.rd[i] < 0)) return false;
+    if (S.packed_recv && (int64_t)T.rd_packed[i] + sc > 0x7FFFFFFF) return false;
+    const int64_t len = (int64_t)sc * S.esz;
+    if (g.max_len && len > g.max_len) return false;
+    return !(g.max_pieces && sc > 0 && vc_chain_count(S, T, s, t) > g.max_pieces);
+}
+
 // Forwarded execution without a work-item list, for calls whose planning would otherwise cost more than their copying:
 // one workgroup per (source, destination) pair, in the order of the chain items (by destination, then source, an eighth
 // of the pairs per XCD).  The workgroup works out the route of its block in closed form from the plan tables (lane k
@@ -206,11 +290,15 @@ __global__ __launch_bounds__(LANES) void vc_copy_blocks_kernel(VcSched S, VcTabl
                                                                const int64_t *__restrict__ header, VcListlessGuard guard,
                                                                int64_t first_pair, const char *__restrict__ sendbuf,
                                                                char *__restrict__ recvbuf, char *__restrict__ stage,
-                                                               int64_t *__restrict__ header_host, int64_t *__restrict__ header_zero) {
+                                                               int64_t *__restrict__ header_host, int64_t *__restrict__ header_zero,
+                                                               int64_t *totals) {
     __shared__ int64_t route[VC_MAX_HOP_SLOTS];
     __shared__ int route_len;
-    const int64_t per = gridDim.x / VC_XCDS;
-    const int64_t idx = first_pair + (int64_t)(blockIdx.x % VC_XCDS) * per + blockIdx.x / VC_XCDS;
+    const unsigned head = vc_totals_blocks(S, totals, LANES);
+    if (blockIdx.x < head) { vc_add_totals(S, T, totals, header_host); return; }
+    const unsigned block = blockIdx.x - head;
+    const int64_t per = (gridDim.x - head) / VC_XCDS;
+    const int64_t idx = first_pair + (int64_t)(block % VC_XCDS) * per + block / VC_XCDS;
     const bool inside = idx < (int64_t)S.P * S.P;
     const int t = inside ? (int)(idx / S.P) : 0, s = inside ? (int)(idx % S.P) : 0;
     // Everything the block's addresses depend on is loaded before the planner's verdict is looked at: the loads are
@@ -221,11 +309,12 @@ __global__ __launch_bounds__(LANES) void vc_copy_blocks_kernel(VcSched S, VcTabl
     const int64_t recv_off = vc_recv_offset(S, T, s, t);
     int64_t dst = 0;
     const bool moves = threadIdx.x < VC_WAVE && (int)threadIdx.x < vc_hop_slots(S) && vc_block_hop(S, T, slot_off, row_base, s, t, threadIdx.x, dst);
-    if (blockIdx.x == 0 && first_pair == 0 && threadIdx.x <= VC_HEADER_MAX_LEN) {
-        if (header_host) header_host[threadIdx.x] = header[threadIdx.x];
+    if (block == 0 && first_pair == 0 && threadIdx.x <= VC_HEADER_SYNC) {
+        if (header_host && !totals && threadIdx.x <= VC_HEADER_MAX_LEN) header_host[threadIdx.x] = header[threadIdx.x];
         if (header_zero) header_zero[threadIdx.x] = 0;    // the header the next call will add up into
     }
-    if (!vc_listless_ok(header, guard) || !inside || len <= 0) return;
+    if (!inside || len <= 0) return;
+    if (totals ? !vc_pair_allowed(S, T, guard, s, t) : !vc_listless_ok(header, guard)) return;
     if (threadIdx.x < VC_WAVE) {                          // hop slots <= VC_MAX_HOP_SLOTS < lanes of the first wavefront
         const unsigned long long mask = __ballot(moves);
         if (moves) route[__popcll(mask & ((1ull << threadIdx.x) - 1))] = dst;
@@ -251,10 +340,14 @@ __global__ __launch_bounds__(VC_WAVE) void vc_copy_blocks_quarter_kernel(VcSched
                                                                          const int64_t *__restrict__ header, VcListlessGuard guard,
                                                                          int64_t first_pair, const char *__restrict__ sendbuf,
                                                                          char *__restrict__ recvbuf, char *__restrict__ stage,
-                                                                         int64_t *__restrict__ header_host, int64_t *__restrict__ header_zero) {
+                                                                         int64_t *__restrict__ header_host, int64_t *__restrict__ header_zero,
+                                                                         int64_t *totals) {
     __shared__ int64_t route[VC_ITEMS_PER_WAVE][VC_MAX_HOP_SLOTS];
-    const int64_t per = gridDim.x / VC_XCDS;
-    const int64_t wave = (int64_t)(blockIdx.x % VC_XCDS) * per + blockIdx.x / VC_XCDS;
+    const unsigned head = vc_totals_blocks(S, totals, VC_WAVE);
+    if (blockIdx.x < head) { vc_add_totals(S, T, totals, header_host); return; }
+    const unsigned block = blockIdx.x - head;
+    const int64_t per = (gridDim.x - head) / VC_XCDS;
+    const int64_t wave = (int64_t)(block % VC_XCDS) * per + block / VC_XCDS;
     const int g = threadIdx.x / VC_QUARTER, q = threadIdx.x % VC_QUARTER;
     const int64_t idx = first_pair + wave * VC_ITEMS_PER_WAVE + g;
     const bool inside = idx < (int64_t)S.P * S.P;
@@ -263,16 +356,17 @@ __global__ __launch_bounds__(VC_WAVE) void vc_copy_blocks_quarter_kernel(VcSched
     const int64_t len = inside ? (int64_t)T.sc[(int64_t)s * S.P + t] * S.esz : 0;
     const int64_t send_off = vc_send_offset(S, T, s, t);
     const int64_t recv_off = vc_recv_offset(S, T, s, t);
-    const bool active = len > 0;                          // no lane leaves before the barrier below
+    // no lane leaves before the barrier below
+    const bool active = len > 0 && (!totals || vc_pair_allowed(S, T, guard, s, t));
     const int nslots = vc_hop_slots(S);
     int64_t d0 = 0, d1 = 0;
     const bool m0 = active && q < nslots && vc_block_hop(S, T, slot_off, row_base, s, t, q, d0);
     const bool m1 = active && q + VC_QUARTER < nslots && vc_block_hop(S, T, slot_off, row_base, s, t, q + VC_QUARTER, d1);
-    if (blockIdx.x == 0 && first_pair == 0 && threadIdx.x <= VC_HEADER_MAX_LEN) {
-        if (header_host) header_host[threadIdx.x] = header[threadIdx.x];
+    if (block == 0 && first_pair == 0 && threadIdx.x <= VC_HEADER_SYNC) {
+        if (header_host && !totals && threadIdx.x <= VC_HEADER_MAX_LEN) header_host[threadIdx.x] = header[threadIdx.x];
         if (header_zero) header_zero[threadIdx.x] = 0;
     }
-    if (!vc_listless_ok(header, guard)) return;           // the same for every lane of the grid
+    if (!totals && !vc_listless_ok(header, guard)) return;      // the same for every lane of the grid
     const unsigned g0 = (unsigned)(__ballot(m0) >> (g * VC_QUARTER)) & 0xFFFFu;      // the group's hops among slots 0..15
     const unsigned g1 = (unsigned)(__ballot(m1) >> (g * VC_QUARTER)) & 0xFFFFu;      // ... among slots 16..31
     if (m0) route[g][__popc(g0 & ((1u << q) - 1))] = d0;
@@ -373,14 +467,16 @@ int vc_batch_pairs(int64_t pairs) { return pairs >= ((int64_t)1 << 19) ? 64 : (p
 
 hipError_t vc_launch_copy_blocks(const VcSched &S, VcTables T, const int64_t *slot_off, const int64_t *row_base, const int64_t *header,
                                  VcListlessGuard guard, int lanes, const char *sendbuf, char *recvbuf, char *stage, hipStream_t st,
-                                 int64_t *header_host, int64_t *header_zero) {
+                                 int64_t *header_host, int64_t *header_zero, int64_t *totals) {
     const int64_t npairs = (int64_t)S.P * S.P;
     const int64_t step = lanes == VC_QUARTER || lanes == VC_BATCHED ? VC_MAX_GRID * VC_ITEMS_PER_WAVE : VC_MAX_GRID;
     for (int64_t done = 0; done < npairs; done += step) {
         const int64_t now = npairs - done < step ? npairs - done : step;
         const int64_t units = lanes == VC_QUARTER ? (now + VC_ITEMS_PER_WAVE - 1) / VC_ITEMS_PER_WAVE : now;
-        const dim3 grid((unsigned)((units + VC_XCDS - 1) / VC_XCDS * VC_XCDS));
+        if (totals && done) return hipErrorInvalidValue;    // the totals belong to a call that one launch takes
+        const dim3 grid((unsigned)((units + VC_XCDS - 1) / VC_XCDS * VC_XCDS) + vc_totals_blocks(S, totals, lanes == VC_THREADS ? VC_THREADS : VC_WAVE));
         if (lanes == VC_BATCHED) {
+            if (totals) return hipErrorInvalidValue;      // the batches are for more pairs than one launch with totals takes
             const int batch = vc_batch_pairs(npairs);
             if (batch == 64)
                 vc_launch_batch<64>(now, S, T, slot_off, row_base, header, guard, done, sendbuf, recvbuf, stage, st, header_host, header_zero);
@@ -390,13 +486,13 @@ hipError_t vc_launch_copy_blocks(const VcSched &S, VcTables T, const int64_t *sl
                 vc_launch_batch<16>(now, S, T, slot_off, row_base, header, guard, done, sendbuf, recvbuf, stage, st, header_host, header_zero);
         } else if (lanes == VC_QUARTER)
             hipLaunchKernelGGL(vc_copy_blocks_quarter_kernel, grid, dim3(VC_WAVE), 0, st, S, T, slot_off, row_base, header, guard, done,
-                               sendbuf, recvbuf, stage, header_host, header_zero);
+                               sendbuf, recvbuf, stage, header_host, header_zero, totals);
         else if (lanes == VC_WAVE)
             hipLaunchKernelGGL(vc_copy_blocks_kernel<VC_WAVE>, grid, dim3(VC_WAVE), 0, st, S, T, slot_off, row_base, header, guard, done,
-                               sendbuf, recvbuf, stage, header_host, header_zero);
+                               sendbuf, recvbuf, stage, header_host, header_zero, totals);
         else
             hipLaunchKernelGGL(vc_copy_blocks_kernel<VC_THREADS>, grid, dim3(VC_THREADS), 0, st, S, T, slot_off, row_base, header, guard,
-                               done, sendbuf, recvbuf, stage, header_host, header_zero);
+                               done, sendbuf, recvbuf, stage, header_host, header_zero, totals);
     }
     return hipGetLastError();
 }

@@ -472,54 +472,6 @@ hipError_t vc_launch_chain_plan(const VcSched &S, VcTables T, const int64_t *slo
     return hipGetLastError();
 }
 
-// ---- fixed-stride staging: one pass over the tables instead of the prefix sums ----
-// One pair of ranks per lane (pairs in the order of the chain items: by receiver, then source).  Every workgroup adds
-// its part into the header (zeroed before): [1] payload, [2] block pieces, [3] table entries no rank could have passed,
-// [4] the most pieces of a block (max), [5] hop-weighted bytes, [6] the longest block (max).
-// [0] is the size of the fixed-stride arena.
-__global__ __launch_bounds__(VC_THREADS) void vc_scan_tables_kernel(VcSched S, VcTables T, int64_t *__restrict__ header) {
-    __shared__ int64_t lds[VC_WAVES_PER_BLOCK];
-    const int P = S.P;
-    const int64_t idx = (int64_t)blockIdx.x * VC_THREADS + threadIdx.x;
-    int64_t payload = 0, items = 0, bad = 0, most = 0, moved = 0, longest = 0;
-    if (idx < (int64_t)P * P) {
-        const int to = (int)(idx / P), s = (int)(idx % P);
-        const int64_t i = (int64_t)to * P + s, k = (int64_t)s * P + to;
-        const int sc = T.sc[k], rc = T.rc[i];
-        bad = (sc < 0) | (rc != sc) | (T.sd[i] < 0) | (!S.packed_recv && T.rd[i] < 0);
-        // (a packed receive layout past INT_MAX elements shows as a negative packed displacement of a later source)
-        if (S.packed_recv && (T.rd_packed[i] < 0 || (s == P - 1 && (int64_t)T.rd_packed[i] + rc > 0x7FFFFFFF))) bad += VC_BAD_OVERFLOW;
-        const int64_t len = (int64_t)sc * S.esz;
-        const int64_t cnt = sc > 0 ? vc_chain_count(S, T, s, to) : 0;
-        payload = len;
-        items = most = cnt;
-        moved = len * vc_block_hops(S, s, to);
-        longest = len;
-    }
-    payload = vc_block_sum(payload, lds);
-    items = vc_block_sum(items, lds);
-    bad = vc_block_sum(bad, lds);
-    moved = vc_block_sum(moved, lds);
-    most = vc_block_max(most, lds);
-    longest = vc_block_max(longest, lds);
-    if (threadIdx.x == 0) {
-        unsigned long long *h = reinterpret_cast<unsigned long long *>(header);
-        if (blockIdx.x == 0) header[0] = vc_strided_stage_bytes(S);
-        if (payload) atomicAdd(&h[1], (unsigned long long)payload);
-        if (items) atomicAdd(&h[2], (unsigned long long)items);
-        if (bad) atomicAdd(&h[VC_HEADER_BAD], (unsigned long long)bad);
-        if (moved) atomicAdd(&h[VC_HEADER_FIXED], (unsigned long long)moved);
-        if (most) atomicMax(&h[VC_HEADER_MAX_PIECES], (unsigned long long)most);
-        if (longest) atomicMax(&h[VC_HEADER_MAX_LEN], (unsigned long long)longest);
-    }
-}
-
-hipError_t vc_launch_scan_tables(const VcSched &S, VcTables T, int64_t *header, hipStream_t st) {
-    const int64_t pairs = (int64_t)S.P * S.P;
-    hipLaunchKernelGGL(vc_scan_tables_kernel, dim3((unsigned)((pairs + VC_THREADS - 1) / VC_THREADS)), dim3(VC_THREADS), 0, st, S, T, header);
-    return hipGetLastError();
-}
-
 // ---- route inspection: bytes sent from every rank to every rank in one launch ----
 __global__ __launch_bounds__(VC_THREADS) void vc_traffic_kernel(const VcDesc *__restrict__ desc, int64_t ndesc, int64_t *__restrict__ matrix, int P) {
     int64_t i = (int64_t)blockIdx.x * VC_THREADS + threadIdx.x;

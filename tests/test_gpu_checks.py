@@ -188,7 +188,8 @@ def test_refused_listless_call_is_redone(api):
 
 def test_tables_that_disagree_are_refused(api):
     """recvcounts must be the transpose of sendcounts (the reference fails with an MPI truncation error); a packed receive
-    layout past INT_MAX elements is an overflow, as in vc_displs_from_counts."""
+    layout past INT_MAX elements is an overflow, as in vc_displs_from_counts.  Nothing moves before the tables have been
+    checked, except in the single-launch execution of small calls, where only the blocks of the offending pairs stay put."""
     import torch
     counts = W.counts_uniform_random(12, 40, seed=5)
     prob = W.make_problem(counts, 4, 0, 0)
@@ -203,7 +204,14 @@ def test_tables_that_disagree_are_refused(api):
             for call in (lambda: api.twophase_rbruck_alltoallv(3, dp, s, d), lambda: api.TTPL_BT_alltoallv(4, 2, 0, dp, s, d),
                          lambda: api.spreadout_alltoallv(dp, s, d)):
                 assert call() == _lib.VC_ERR_TABLES and "recvcounts" in dp.comm.error(), mode
-            assert bool((d == 0xEE).all())
+            if mode != 1:
+                assert bool((d == 0xEE).all())
+            else:
+                # the default mode serves a small call like this one in a single launch, in which every pair of ranks checks
+                # its own table entries: the block of the pair that disagrees stays where it is, the others may have landed
+                lo = int(prob.rbase[7]) + int(dp.rdispls[7, 3].item()) * 4
+                assert bool((d[lo:lo + 4 * min(keep, keep + delta)] == 0xEE).all())
+                d.fill_(0xEE)
         dp.recvcounts[7, 3] = keep
         assert api.twophase_rbruck_alltoallv(3, dp, s, d) == 0 and dp.verify(s, d) == 0
         d.fill_(0xEE)
