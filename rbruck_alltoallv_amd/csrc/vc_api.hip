@@ -632,8 +632,10 @@ static int listless_lanes(const vc_comm *c, const VcSched &S) {
 // code as elsewhere — but blocks of the pairs whose entries were in order may have been delivered by then (everywhere
 // else nothing moves before the tables have been checked).  Costs arena: regions x P x P x stride bytes, so only
 // up to VC_STRIDED_MAX_BYTES, and only on communicators of at most 128 ranks: measured on MI355X, 64 ranks with blocks of
-// 0 - 4 KiB 41 -> 29 us per call with a pass over the tables before the copy kernel, 25 us with the pass inside it, but
-// 1024 ranks with blocks of 0 - 512 B 380 -> 560 us (805 MB of slots 768 bytes apart instead of 270 MB of compact ones).
+// 0 - 4 KiB 41 -> 29 us per call with a pass over the tables before the copy kernel, 24.6 us with the pass inside it, but
+// 1024 ranks with blocks of 0 - 512 B 380 -> 560 us (805 MB of slots 768 bytes apart instead of 270 MB of compact ones), and
+// the atomics of the totals, a handful per 256 pairs, add up with the square of the ranks (even at 192 ranks, 1.3 - 1.4 x
+// slower on 256, 2 x on 512).
 // Returns 1 when the call has been served, 0 when it must go the general way, < 0 on errors.
 #define VC_STRIDED_MAX_BYTES ((int64_t)256 << 20)
 static int try_strided(vc_comm *c, VcSched S, std::vector<VcLaunchInfo> &L, const char *sendbuf, char *recvbuf, VcTables T, int pair_lanes) {

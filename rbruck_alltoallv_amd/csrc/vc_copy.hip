@@ -207,29 +207,36 @@ __device__ __forceinline__ int64_t vc_wave_max(int64_t v) {
     return v;
 }
 
-// The wavefronts of the first vc_totals_blocks workgroups of the grid: one pair of ranks per lane (by receiver, then source), the wavefront's
+// The wavefronts of the first vc_totals_blocks workgroups of the grid: four pairs of ranks per lane (by receiver, then
+// source; the atomics on the same few words are what limits this at many ranks), the wavefront's
 // sums and maxima added into `totals` with one atomic each: [1] payload, [2] block pieces, [3] table entries no rank could
 // have passed, [4] the most pieces of a block, [5] hop-weighted bytes, [6] the longest block.  The wavefront that finishes
 // last hands the words to the host.
+#define VC_TOTALS_PER_LANE 4
 __device__ __forceinline__ void vc_add_totals(const VcSched &S, const VcTables &T, int64_t *totals, int64_t *header_host) {
     const int P = S.P;
-    const int64_t pairs = (int64_t)P * P, nwaves = (pairs + VC_WAVE - 1) / VC_WAVE;
+    const int64_t pairs = (int64_t)P * P, per_wave = VC_WAVE * VC_TOTALS_PER_LANE, nwaves = (pairs + per_wave - 1) / per_wave;
     const int64_t wave = (int64_t)blockIdx.x * (blockDim.x / VC_WAVE) + threadIdx.x / VC_WAVE;
     if (wave >= nwaves) return;
     const int lane = threadIdx.x & (VC_WAVE - 1);
-    const int64_t idx = wave * VC_WAVE + lane;
     int64_t payload = 0, items = 0, bad = 0, most = 0, moved = 0, longest = 0;
-    if (idx < pairs) {
+#pragma unroll
+    for (int u = 0; u < VC_TOTALS_PER_LANE; u++) {
+        const int64_t idx = wave * per_wave + u * VC_WAVE + lane;
+        if (idx >= pairs) continue;
         const int to = (int)(idx / P), s = (int)(idx % P);
         const int64_t i = (int64_t)to * P + s, k = (int64_t)s * P + to;
         const int sc = T.sc[k], rc = T.rc[i];
-        bad = (sc < 0) | (rc != sc) | (T.sd[i] < 0) | (!S.packed_recv && T.rd[i] < 0);
+        bad += (sc < 0) | (rc != sc) | (T.sd[i] < 0) | (!S.packed_recv && T.rd[i] < 0);
         // (a packed receive layout past INT_MAX elements shows as a negative packed displacement of a later source)
         if (S.packed_recv && (T.rd_packed[i] < 0 || (s == P - 1 && (int64_t)T.rd_packed[i] + rc > 0x7FFFFFFF))) bad += VC_BAD_OVERFLOW;
         const int64_t len = (int64_t)sc * S.esz;
-        payload = longest = len;
-        items = most = sc > 0 ? vc_chain_count(S, T, s, to) : 0;
-        moved = len * vc_block_hops(S, s, to);
+        const int64_t cnt = sc > 0 ? vc_chain_count(S, T, s, to) : 0;
+        payload += len;
+        items += cnt;
+        moved += len * vc_block_hops(S, s, to);
+        most = cnt > most ? cnt : most;
+        longest = len > longest ? len : longest;
     }
     payload = vc_wave_sum(payload);
     items = vc_wave_sum(items);
@@ -259,7 +266,8 @@ __device__ __forceinline__ void vc_add_totals(const VcSched &S, const VcTables &
 // copying instead of in front of it.  A multiple of VC_XCDS, so that the workgroups behind them keep their XCDs.
 __host__ __device__ __forceinline__ unsigned vc_totals_blocks(const VcSched &S, const int64_t *totals, int lanes) {
     if (!totals) return 0;
-    const int64_t waves = ((int64_t)S.P * S.P + VC_WAVE - 1) / VC_WAVE, per = lanes / VC_WAVE;
+    const int64_t per_wave = VC_WAVE * VC_TOTALS_PER_LANE;
+    const int64_t waves = ((int64_t)S.P * S.P + per_wave - 1) / per_wave, per = lanes / VC_WAVE;
     return (unsigned)(((waves + per - 1) / per + VC_XCDS - 1) / VC_XCDS * VC_XCDS);
 }
 
