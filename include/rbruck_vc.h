@@ -93,7 +93,8 @@ int vc_comm_set_bases(vc_comm_t comm, const int64_t *sbase_bytes, const int64_t 
  * (plans always hold a list). */
 int vc_comm_set_forwarding(vc_comm_t comm, int enable);
 
-/* Whether the communicator bounds its staging memory (1, the default) or not (0).  The reference keeps one fixed-stride slot
+/* Whether the communicator bounds its staging memory (1, the default; a larger value: bounded, with an allowance of that many
+ * MiB instead of an eighth of the device's memory, see below) or not (0).  The reference keeps one fixed-stride slot
  * per multi-hop offset and reuses it in every round (src/twophase_tunable_rbruckv-om.cpp:52-75).  Here, bounded:
  *  - one launch per digit: a staged block arrives in one digit phase and leaves in a later one; blocks with the same
  *    (arrival, departure) pair form a sub-region of the arena, and a sub-region is placed over the memory of sub-regions
@@ -101,8 +102,8 @@ int vc_comm_set_forwarding(vc_comm_t comm, int enable);
  *    peak then stays below about 1.5 x the payload where separate regions need the sum over the blocks of
  *    (hops - 1) x bytes (configuration 5 with radix 2: 60 GB);
  *  - forwarded execution keeps every hop's copy of every block, because nothing reads them and so nothing says when one
- *    may be overwritten.  A call whose staging would pass both 1 GiB and three times its payload is therefore run one
- *    launch per digit instead (vc_stats_t.execution says so).
+ *    may be overwritten.  A call whose staging would pass both the allowance (an eighth of the device's memory, at least
+ *    1 GiB) and three times its payload is therefore run one launch per digit instead (vc_stats_t.execution says so).
  * Unbounded: every digit phase has its own region and forwarded calls stay forwarded, whatever they need. */
 int vc_comm_set_staging_bound(vc_comm_t comm, int enable);
 

@@ -54,9 +54,10 @@ class VirtualComm:
         batch of pairs per wavefront."""
         self._check(self.lib.vc_comm_set_forwarding(self.handle, int(enable)))
 
-    def set_staging_bound(self, on: bool) -> None:
+    def set_staging_bound(self, on: bool | int) -> None:
         """vc_comm_set_staging_bound: reuse staging memory in launch-per-digit execution and run forwarded calls that would
-        need more than three times their payload (and 1 GiB) that way (default), or give every digit phase its own region."""
+        need more than three times their payload (and an eighth of the device's memory; an int > 1: that many MiB) that
+        way (default), or give every digit phase its own region."""
         self._check(self.lib.vc_comm_set_staging_bound(self.handle, int(on)))
 
     def last_stats(self) -> _lib.VcStats:

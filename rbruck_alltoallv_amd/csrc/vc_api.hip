@@ -116,6 +116,7 @@ struct vc_comm {
     double cal_copy_bytes_per_s = 0, cal_launch_s = 0, cal_sync_s = 0;   // calibrate(): the plain copy's rate, the cost of a
                                           // launch, of a launch the host waits for
     int bound_staging = 1;                // vc_comm_set_staging_bound
+    int64_t staging_allowance = 0;        // bytes of staging a forwarded call may take whatever its payload (set with the bound)
     int live_plans = 0;                   // plans created on this communicator and not yet freed
     std::vector<void *> retired_stage;    // staging arenas that were outgrown while plans existed: a HIP graph captured from
                                           // vc_plan_execute_async holds the arena's address, so they stay until the plans go
@@ -173,6 +174,8 @@ struct BusyGuard {
 
 // ------------------------------------------------------------------ communicator
 
+static int64_t default_staging_allowance();
+
 extern "C" int vc_comm_create(int nranks, vc_comm_t *comm_out) {
     if (!comm_out || nranks < 1) return fail_arg("vc_comm_create: need nranks >= 1 and an output pointer");
     int ndev = 0;
@@ -194,6 +197,7 @@ extern "C" int vc_comm_create(int nranks, vc_comm_t *comm_out) {
         (void)vc_comm_free(c);
         return fail_hip(e, "vc_comm_create", __LINE__);
     }
+    c->staging_allowance = default_staging_allowance();
     *comm_out = c;
     return VC_OK;
 }
@@ -241,9 +245,19 @@ extern "C" int vc_comm_set_forwarding(vc_comm_t c, int enable) {
     return VC_OK;
 }
 
+// An eighth of the device's memory, at least 1 GiB: what a forwarded call may keep in staging before its ratio to the
+// payload is looked at.
+static int64_t default_staging_allowance() {
+    size_t free_bytes = 0, total = 0;
+    if (hipMemGetInfo(&free_bytes, &total) != hipSuccess) { (void)hipGetLastError(); total = 0; }
+    return std::max<int64_t>((int64_t)1 << 30, (int64_t)(total / 8));
+}
+
 extern "C" int vc_comm_set_staging_bound(vc_comm_t c, int enable) {
     if (!c) return fail_arg("null communicator");
+    if (enable < 0) return fail_arg("vc_comm_set_staging_bound: 0, 1 or an allowance in MiB");
     c->bound_staging = enable != 0;
+    c->staging_allowance = enable > 1 ? (int64_t)enable << 20 : default_staging_allowance();
     return VC_OK;
 }
 
@@ -324,10 +338,11 @@ static int make_schedule(const vc_comm *c, const CallParams &q, bool forward, Vc
 // overwritten): its staging is the sum over the blocks of (hops - 1) x bytes, 3.5 x the payload for a radix-2 Bruck
 // over 512 ranks.  A communicator that bounds its staging runs such a call one launch per digit instead, where staging
 // memory is reused (and stays below about twice the payload): beyond three times the payload, and only when it
-// matters (more than 1 GiB).  Measured on MI355X: configuration 5 with radix 2, 60 GB forwarded in 17.4 ms against 30 GB
-// in 25.5 ms; a radix-4 two-layer Bruck at configuration 4 (2.4 x its payload) stays forwarded: 4.8 ms against 6.8.
+// matters (more than an eighth of the device's memory, 36 GB here; vc_comm_set_staging_bound takes another allowance).
+// Measured on MI355X: configuration 5 with radix 2, 60 GB forwarded in 17.4 ms against 30 GB in 25.5 ms; a radix-4
+// two-layer Bruck at configuration 4 (13 GB, 3.1 x its payload) stays forwarded: 4.8 ms against 6.8.
 static bool staging_out_of_bound(const vc_comm *c, int64_t stage_bytes, int64_t payload_bytes) {
-    return c->bound_staging && stage_bytes > ((int64_t)1 << 30) && stage_bytes > 3 * payload_bytes;
+    return c->bound_staging && stage_bytes > c->staging_allowance && stage_bytes > 3 * payload_bytes;
 }
 
 // What the planner leaves behind for the copy launches.

@@ -411,7 +411,7 @@ def test_staging_bound(api):
     dp.fill_payload(0, 21, ds)
     seen = {}
     for bound in (True, False):
-        dp.comm.set_staging_bound(bound)
+        dp.comm.set_staging_bound(1024 if bound else 0)      # an allowance of 1 GiB (the default is an eighth of the device's memory)
         for mode in (2, 0):
             dp.comm.set_forwarding(mode)
             dr = dp.new_recv_arena(0xEE)
@@ -422,7 +422,7 @@ def test_staging_bound(api):
             assert st.moved_bytes * 2 == W.algorithmic_bytes(counts, 8, W.hops_flat(512, 2))
     print(seen, flush=True)
     # a persistent plan made in forwarded mode for a call beyond the bound is a launch-per-digit plan too
-    dp.comm.set_staging_bound(True)
+    dp.comm.set_staging_bound(1024)
     dp.comm.set_forwarding(2)
     dr = dp.new_recv_arena(0xEE)
     plan = api.Plan("tuna_algorithm", dp, dr, r=2, batch=0)
@@ -438,9 +438,13 @@ def test_staging_bound(api):
     assert seen[(True, 0)][0] == 0 and seen[(True, 0)][1] < 2 * S                  # reused
     assert seen[(True, 2)] == seen[(True, 0)]                                      # asked for forwarded, run per digit
     # a radix with few hops stays forwarded under the bound
-    dp.comm.set_staging_bound(True)
+    dp.comm.set_staging_bound(1024)
     dp.comm.set_forwarding(2)
     dr = dp.new_recv_arena(0xEE)
     assert api.tuna_algorithm(32, 0, dp, ds, dr) == 0 and dp.verify(ds, dr) == 0
     assert dp.comm.last_stats().execution == 1 and dp.comm.last_stats().staging_bytes < S
+    # ... and so does the radix-2 call under the default allowance, which 3.5 GiB do not reach
+    dp.comm.set_staging_bound(True)
+    assert api.tuna_algorithm(2, 0, dp, ds, dr) == 0 and dp.verify(ds, dr) == 0
+    assert dp.comm.last_stats().execution == 1 and dp.comm.last_stats().staging_bytes > 3.4 * S
     dp.comm.free()
