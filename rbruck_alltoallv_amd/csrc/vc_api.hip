@@ -1301,7 +1301,9 @@ extern "C" int vc_suggest_tunables(const int *sendcounts, int elem_size, int n, 
         int w, d;
         vc_radix_params(n, cand[k], w, d);
         const double plan = 2 * c->cal_sync_s + 3 * launch + (double)P * P * (w + 2) * 16.0 / rate;
-        const double t = c->forward != 0
+        // (a forwarded call whose staging, the bytes of all hops but the last, is out of bound runs per digit)
+        const bool forwarded = c->forward != 0 && !staging_out_of_bound(c, (int64_t)(moved - payload), (int64_t)payload);
+        const double t = forwarded
             ? plan + launch + (payload + moved + 2.0 * pieces * (24 + 8 * (w + 1))) / rate
             : plan + launch * launches_for(n, cand[k], n < P) + (2.0 * moved + 2.0 * 32 * hop_pieces) / rate;
         if (moved_bytes_out) moved_bytes_out[k] = (int64_t)got[k];
