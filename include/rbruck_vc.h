@@ -79,10 +79,10 @@ int vc_comm_set_bases(vc_comm_t comm, const int64_t *sbase_bytes, const int64_t 
  *    (src/twophase_tunable_rbruckv.cpp:59; the stride comes from the last call's longest block): slot addresses are then
  *    closed forms and the call is a single kernel launch, without a planner before it.  Every pair of ranks checks its own
  *    table entries, and that its block fits a slot, before it moves anything, and the kernel's first wavefronts add up
- *    what the host needs afterwards; a call with a longer block is redone the general way.  Only on at most 128 ranks
+ *    what the host needs afterwards; a call with a longer block is redone the general way.  Only on at most 192 ranks
  *    and while regions x P x P x stride stays below 256 MiB.  This is the one execution in which a call that returns
  *    VC_ERR_TABLES may already have delivered the blocks of the pairs whose entries were in order.
- *    On more than 128 ranks and blocks below 384 B on average a wavefront takes a batch of 16 - 64 pairs instead: a lane per
+ *    On more than 192 ranks and blocks below 384 B on average a wavefront takes a batch of 16 - 64 pairs instead: a lane per
  *    pair works out the route, then the quarters of the wavefront carry the blocks one after the other.
  * 2: forwarded, always through the list.   3 / 4 / 5: forwarded, always without it, a workgroup / a quarter of a
  *    wavefront per pair of ranks / a batch of pairs per wavefront (any sizes; not the fastest choice everywhere).

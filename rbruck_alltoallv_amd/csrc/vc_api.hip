@@ -646,16 +646,19 @@ static int listless_lanes(const vc_comm *c, const VcSched &S) {
 // longest block; a call with a longer block is redone the general way, and a call with bad tables returns the same
 // code as elsewhere — but blocks of the pairs whose entries were in order may have been delivered by then (everywhere
 // else nothing moves before the tables have been checked).  Costs arena: regions x P x P x stride bytes, so only
-// up to VC_STRIDED_MAX_BYTES, and only on communicators of at most 128 ranks: measured on MI355X, 64 ranks with blocks of
-// 0 - 4 KiB 41 -> 29 us per call with a pass over the tables before the copy kernel, 24.6 us with the pass inside it, but
-// 1024 ranks with blocks of 0 - 512 B 380 -> 560 us (805 MB of slots 768 bytes apart instead of 270 MB of compact ones), and
-// the atomics of the totals, a handful per 256 pairs, add up with the square of the ranks (even at 192 ranks, 1.3 - 1.4 x
-// slower on 256, 2 x on 512).
+// up to VC_STRIDED_MAX_BYTES, and only on communicators of at most 192 ranks.  Measured on MI355X, microseconds per
+// blocking call: 64 ranks with blocks of 0 - 4 KiB 41 -> 29 with a pass over the tables before the copy kernel, 24.6 with
+// the pass inside it; 128 ranks, 0 - 512 B: 41 -> 25.6; 160 ranks: 31 - 42 -> 26 - 34; 192 ranks: 31 - 50 -> 30 - 42; but
+// 256 ranks 34 - 68 -> 44 - 68, 384 ranks 44 - 55 -> 85 - 88 (the atomics of the totals, six per 256 pairs on the same
+// words, and the arena grow with the square of the ranks), 1024 ranks with blocks of 0 - 512 B 380 -> 560 (805 MB of
+// slots 768 bytes apart instead of 270 MB of compact ones).
 // Returns 1 when the call has been served, 0 when it must go the general way, < 0 on errors.
 #define VC_STRIDED_MAX_BYTES ((int64_t)256 << 20)
+#define VC_STRIDED_MAX_PAIRS 36864           // 192 ranks
 static int try_strided(vc_comm *c, VcSched S, std::vector<VcLaunchInfo> &L, const char *sendbuf, char *recvbuf, VcTables T, int pair_lanes) {
-    if (c->forward != 1 || !pair_lanes || pair_lanes == VC_BATCHED || S.coalesce || vc_hop_slots(S) > VC_MAX_HOP_SLOTS) return 0;
-    if ((int64_t)S.P * S.P > VC_LISTLESS_MAX_PAIRS) return 0;
+    if (c->forward != 1 || !pair_lanes || S.coalesce || vc_hop_slots(S) > VC_MAX_HOP_SLOTS) return 0;
+    if ((int64_t)S.P * S.P > VC_STRIDED_MAX_PAIRS) return 0;
+    if (pair_lanes == VC_BATCHED) pair_lanes = VC_QUARTER;      // (the batches come without the totals)
     const int64_t stride = (c->hint_max_len + 2 * VC_LINE - 1) & ~(int64_t)(VC_LINE - 1);     // the block at any cache-line phase
     if (stride > 0x7FFFFF80) return 0;
     S.stride = (int)stride;

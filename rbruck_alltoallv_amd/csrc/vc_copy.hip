@@ -247,14 +247,19 @@ __device__ __forceinline__ void vc_add_totals(const VcSched &S, const VcTables &
     unsigned long long *h = reinterpret_cast<unsigned long long *>(totals);
     int last = 0;
     if (lane == 0) {
-        if (payload) atomicAdd(&h[1], (unsigned long long)payload);
-        if (items) atomicAdd(&h[2], (unsigned long long)items);
-        if (bad) atomicAdd(&h[VC_HEADER_BAD], (unsigned long long)bad);
-        if (moved) atomicAdd(&h[VC_HEADER_FIXED], (unsigned long long)moved);
-        if (most) atomicMax(&h[VC_HEADER_MAX_PIECES], (unsigned long long)most);
-        if (longest) atomicMax(&h[VC_HEADER_MAX_LEN], (unsigned long long)longest);
-        __threadfence();                                  // the words above before the count below
-        last = atomicAdd(&h[VC_HEADER_SYNC], 1ull) == (unsigned long long)(nwaves - 1);
+        // The count below must not be seen before the words above.  A release fence would do, but at device scope it writes
+        // this XCD's L2 back, once per wavefront here.  Instead every atomic returns its old value: when the values are
+        // back the atomics have been performed where the count is kept too, and the count's operand is made from them.
+        unsigned long long seen = 0;
+        if (payload) seen += atomicAdd(&h[1], (unsigned long long)payload);
+        if (items) seen += atomicAdd(&h[2], (unsigned long long)items);
+        if (bad) seen += atomicAdd(&h[VC_HEADER_BAD], (unsigned long long)bad);
+        if (moved) seen += atomicAdd(&h[VC_HEADER_FIXED], (unsigned long long)moved);
+        if (most) seen += atomicMax(&h[VC_HEADER_MAX_PIECES], (unsigned long long)most);
+        if (longest) seen += atomicMax(&h[VC_HEADER_MAX_LEN], (unsigned long long)longest);
+        unsigned zero;
+        asm volatile("v_mov_b32 %0, 0" : "=v"(zero) : "v"((unsigned)seen), "v"((unsigned)(seen >> 32)));      // (opaque to the compiler)
+        last = atomicAdd(&h[VC_HEADER_SYNC], 1ull + zero) == (unsigned long long)(nwaves - 1);
     }
     last = __shfl(last, 0, VC_WAVE);
     if (last && lane <= VC_HEADER_MAX_LEN)

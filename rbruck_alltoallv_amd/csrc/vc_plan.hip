@@ -180,6 +180,10 @@ __global__ __launch_bounds__(VC_THREADS) void vc_plan_org_rows(VcSched S, VcTabl
 }
 
 // ---- pass 2: prefix sums over the rows ----
+// (A kernel of its own although a boundary between two kernels of one stream costs as much as the pass itself: folding it
+// into pass 1 — every workgroup counts itself when its rows are written, the last one does the prefix sums — needs a
+// device-wide release fence per workgroup, which on this chip writes the XCD's L2 back; measured, calls on 160 - 512 ranks
+// took twice as long that way.)
 // Launch-per-digit execution: grid (nl + 1).  Workgroup L < nl: item bases of launch L's rows (relative to the launch's
 // first item), its item count and moved bytes.  Workgroup nl: staging row bases, staging bytes, payload bytes, negative
 // table entries.  Forwarded execution (chain_row_tot != null, nl = 0): grid (2).  Workgroup 0 as workgroup nl above, and
