@@ -163,32 +163,38 @@ __device__ __forceinline__ void vc_forward_piece_quarter(const char *src, int64_
 #define VC_ITEMS_PER_WAVE (VC_WAVE / VC_QUARTER)
 
 // gridDim.x wavefronts, a multiple of VC_XCDS; XCD k works through the k-th eighth of them, each taking four items in a row
+// `rounds`: groups of four items in a row a wavefront takes, one after the other (long lists of very short pieces: fewer
+// wavefronts, each paying its start-up once for more items)
 __global__ __launch_bounds__(VC_WAVE) void vc_copy_chains_quarter_kernel(const int64_t *__restrict__ items, int stride, unsigned nitems,
-                                                                         const char *__restrict__ sendbuf, char *__restrict__ recvbuf,
-                                                                         char *__restrict__ stage) {
+                                                                         int rounds, const char *__restrict__ sendbuf,
+                                                                         char *__restrict__ recvbuf, char *__restrict__ stage) {
     const unsigned per = gridDim.x / VC_XCDS;
     const unsigned wave = (blockIdx.x % VC_XCDS) * per + blockIdx.x / VC_XCDS;
-    const int64_t idx = (int64_t)wave * VC_ITEMS_PER_WAVE + threadIdx.x / VC_QUARTER;
-    if (idx >= nitems) return;
-    const int64_t *it = items + idx * stride;
-    const int64_t len = it[VC_CHAIN_LEN];
-    const int nhop = (int)it[VC_CHAIN_NHOP];
-    if (len <= 0 || nhop <= 0) return;
-    vc_forward_piece_quarter(vc_resolve(it[VC_CHAIN_SRC], sendbuf, recvbuf, stage), len, nhop,
-                             [&](int k) { return vc_resolve(it[VC_CHAIN_HEAD + k], sendbuf, recvbuf, stage); });
+    for (int round = 0; round < rounds; round++) {
+        const int64_t idx = ((int64_t)wave * rounds + round) * VC_ITEMS_PER_WAVE + threadIdx.x / VC_QUARTER;
+        if (idx >= nitems) continue;
+        const int64_t *it = items + idx * stride;
+        const int64_t len = it[VC_CHAIN_LEN];
+        const int nhop = (int)it[VC_CHAIN_NHOP];
+        if (len <= 0 || nhop <= 0) continue;
+        vc_forward_piece_quarter(vc_resolve(it[VC_CHAIN_SRC], sendbuf, recvbuf, stage), len, nhop,
+                                 [&](int k) { return vc_resolve(it[VC_CHAIN_HEAD + k], sendbuf, recvbuf, stage); });
+    }
 }
 
-__global__ __launch_bounds__(VC_WAVE) void vc_copy_items_quarter_kernel(const VcDesc *__restrict__ items, unsigned nitems,
+__global__ __launch_bounds__(VC_WAVE) void vc_copy_items_quarter_kernel(const VcDesc *__restrict__ items, unsigned nitems, int rounds,
                                                                         const char *__restrict__ sendbuf, char *__restrict__ recvbuf,
                                                                         char *__restrict__ stage) {
     const unsigned per = gridDim.x / VC_XCDS;
     const unsigned wave = (blockIdx.x % VC_XCDS) * per + blockIdx.x / VC_XCDS;
-    const int64_t idx = (int64_t)wave * VC_ITEMS_PER_WAVE + threadIdx.x / VC_QUARTER;
-    if (idx >= nitems) return;
-    const VcDesc d = items[idx];
-    if (d.len <= 0) return;
-    char *dst = vc_resolve(d.dst, sendbuf, recvbuf, stage);
-    vc_forward_piece_quarter(vc_resolve(d.src, sendbuf, recvbuf, stage), d.len, 1, [&](int) { return dst; });
+    for (int round = 0; round < rounds; round++) {
+        const int64_t idx = ((int64_t)wave * rounds + round) * VC_ITEMS_PER_WAVE + threadIdx.x / VC_QUARTER;
+        if (idx >= nitems) continue;
+        const VcDesc d = items[idx];
+        if (d.len <= 0) continue;
+        char *dst = vc_resolve(d.dst, sendbuf, recvbuf, stage);
+        vc_forward_piece_quarter(vc_resolve(d.src, sendbuf, recvbuf, stage), d.len, 1, [&](int) { return dst; });
+    }
 }
 
 // ---- fixed-stride staging in one launch (the `totals` of vc_launch_copy_blocks) ----
@@ -513,8 +519,12 @@ hipError_t vc_launch_copy_blocks(const VcSched &S, VcTables T, const int64_t *sl
 // Items of one launch: as many as VC_MAX_GRID workgroups or wavefronts take.
 static int64_t vc_items_per_launch(int lanes) { return lanes == VC_QUARTER ? VC_MAX_GRID * VC_ITEMS_PER_WAVE : VC_MAX_GRID; }
 
+// Groups of four items a wavefront of the quarter kernels takes: as many as leave every SIMD of the chip a few wavefronts.
+static int vc_quarter_rounds(int64_t items) { return items >= ((int64_t)1 << 19) ? 4 : (items >= ((int64_t)1 << 17) ? 2 : 1); }
+
 static unsigned vc_grid_for(int64_t items, int lanes) {
-    const int64_t units = lanes == VC_QUARTER ? (items + VC_ITEMS_PER_WAVE - 1) / VC_ITEMS_PER_WAVE : items;
+    const int64_t per = lanes == VC_QUARTER ? VC_ITEMS_PER_WAVE * vc_quarter_rounds(items) : 1;
+    const int64_t units = (items + per - 1) / per;
     return (unsigned)((units + VC_XCDS - 1) / VC_XCDS * VC_XCDS);
 }
 
@@ -526,7 +536,8 @@ hipError_t vc_launch_copy_chains(const int64_t *items, int stride, int64_t nitem
         const dim3 grid(vc_grid_for(now, lanes));
         const int64_t *first = items + done * stride;
         if (lanes == VC_QUARTER)
-            hipLaunchKernelGGL(vc_copy_chains_quarter_kernel, grid, dim3(VC_WAVE), 0, st, first, stride, (unsigned)now, sendbuf, recvbuf, stage);
+            hipLaunchKernelGGL(vc_copy_chains_quarter_kernel, grid, dim3(VC_WAVE), 0, st, first, stride, (unsigned)now, vc_quarter_rounds(now),
+                               sendbuf, recvbuf, stage);
         else if (lanes == VC_WAVE)
             hipLaunchKernelGGL(vc_copy_chains_kernel<VC_WAVE>, grid, dim3(VC_WAVE), 0, st, first, stride, (unsigned)now, sendbuf, recvbuf, stage);
         else
@@ -543,7 +554,8 @@ hipError_t vc_launch_copy_items(const VcDesc *items, int64_t nitems, int lanes, 
         const int64_t now = nitems - done < step ? nitems - done : step;
         const dim3 grid(vc_grid_for(now, lanes));
         if (lanes == VC_QUARTER)
-            hipLaunchKernelGGL(vc_copy_items_quarter_kernel, grid, dim3(VC_WAVE), 0, st, items + done, (unsigned)now, sendbuf, recvbuf, stage);
+            hipLaunchKernelGGL(vc_copy_items_quarter_kernel, grid, dim3(VC_WAVE), 0, st, items + done, (unsigned)now, vc_quarter_rounds(now),
+                               sendbuf, recvbuf, stage);
         else if (lanes == VC_WAVE)
             hipLaunchKernelGGL(vc_copy_items_kernel<VC_WAVE>, grid, dim3(VC_WAVE), 0, st, items + done, (unsigned)now, sendbuf, recvbuf, stage);
         else
