@@ -98,7 +98,9 @@ int vc_comm_set_forwarding(vc_comm_t comm, int enable);
  * per multi-hop offset and reuses it in every round (src/twophase_tunable_rbruckv-om.cpp:52-75).  Here, bounded:
  *  - one launch per digit: a staged block arrives in one digit phase and leaves in a later one; blocks with the same
  *    (arrival, departure) pair form a sub-region of the arena, and a sub-region is placed over the memory of sub-regions
- *    whose blocks have all left before it is written (first fit).  Calls with at least three staging regions; the
+ *    whose blocks have all left before it is written (first fit).  Calls with at least three staging regions whose
+ *    separate regions would take more than a thirty-second of the allowance below (about 1 GiB: planning for reuse costs
+ *    some tens of microseconds, and such a call is planned twice); the
  *    peak then stays below about 1.5 x the payload where separate regions need the sum over the blocks of
  *    (hops - 1) x bytes (configuration 5 with radix 2: 60 GB);
  *  - forwarded execution keeps every hop's copy of every block, because nothing reads them and so nothing says when one

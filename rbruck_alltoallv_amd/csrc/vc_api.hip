@@ -326,12 +326,21 @@ struct CallParams {
 // The schedule of a call in one of the two execution modes.  Launch-per-digit execution reuses staging memory when the
 // communicator bounds its staging (the default) and there is something to reuse: with fewer than three staging regions
 // no sub-region is written after another one has been read for the last time.
-static int make_schedule(const vc_comm *c, const CallParams &q, bool forward, VcSched &S, std::vector<VcLaunchInfo> &L) {
+// reuse: launch-per-digit execution on reused staging memory (where the schedule allows it).
+static int make_schedule(const vc_comm *c, const CallParams &q, bool forward, VcSched &S, std::vector<VcLaunchInfo> &L, bool reuse = false) {
     const int rc = vc_make_schedule(q.f, c->P, q.n, q.r, q.batch, q.esz, q.uniform, S, L, q.batch2, forward);
     if (rc) return rc;
     const int nreg = S.w + S.w2;
-    if (!forward && c->bound_staging && nreg >= 3 && nreg + 1 <= VC_RECYCLE_MAX_SLOTS) S.recycle = 1;
+    if (!forward && reuse && c->bound_staging && nreg >= 3 && nreg + 1 <= VC_RECYCLE_MAX_SLOTS) S.recycle = 1;
     return VC_OK;
+}
+
+// Reused staging costs planning time (one prefix sum per pair of hop slots, the allocator on one thread: 0.05 ms on 64
+// ranks), so a launch-per-digit call is planned with a region per digit first and planned again on reused staging
+// only when that would take more than a thirty-second of the communicator's staging allowance (about 1 GiB).
+static bool worth_reusing(const vc_comm *c, const VcSched &S, int64_t stage_bytes) {
+    const int nreg = S.w + S.w2;
+    return c->bound_staging && !S.recycle && nreg >= 3 && nreg + 1 <= VC_RECYCLE_MAX_SLOTS && stage_bytes > (c->staging_allowance >> 5);
 }
 
 // Forwarded execution keeps every hop's copy of every block (nothing reads them, so nothing says when one could be
@@ -510,10 +519,10 @@ static int plan_emit(vc_comm *c, const VcSched &S, std::vector<VcLaunchInfo> &L,
     return VC_OK;
 }
 
-static int build_plan(vc_comm *c, const CallParams &q, int recv_lo, VcTables T, DevBuf &items, PlanInfo &out, bool forward) {
+static int build_plan(vc_comm *c, const CallParams &q, int recv_lo, VcTables T, DevBuf &items, PlanInfo &out, bool forward, bool reuse = false) {
     VcSched S;
     std::vector<VcLaunchInfo> L;
-    int rc = make_schedule(c, q, forward, S, L);
+    int rc = make_schedule(c, q, forward, S, L, reuse);
     if (rc) return schedule_error(rc);
     S.recv_lo = recv_lo;
     rc = plan_sizes(c, S, L, T, forward);
@@ -521,7 +530,8 @@ static int build_plan(vc_comm *c, const CallParams &q, int recv_lo, VcTables T, 
     HIP_TRY(hipStreamSynchronize(c->stream));     // the staging arena and the item list are sized from the plan
     rc = plan_read(c, S, L, out, forward);
     if (rc) return rc;
-    if (forward && staging_out_of_bound(c, out.stage_bytes, out.payload_bytes)) return build_plan(c, q, recv_lo, T, items, out, false);
+    if (forward && staging_out_of_bound(c, out.stage_bytes, out.payload_bytes)) return build_plan(c, q, recv_lo, T, items, out, false, true);
+    if (!forward && worth_reusing(c, S, out.stage_bytes)) return build_plan(c, q, recv_lo, T, items, out, false, true);
     return plan_emit(c, S, L, T, items, out);
 }
 
@@ -705,10 +715,10 @@ static int try_strided(vc_comm *c, VcSched S, std::vector<VcLaunchInfo> &L, cons
     return rc ? rc : 1;
 }
 
-static int run_schedule(vc_comm *c, const CallParams &q, const char *sendbuf, char *recvbuf, VcTables T, bool forward) {
+static int run_schedule(vc_comm *c, const CallParams &q, const char *sendbuf, char *recvbuf, VcTables T, bool forward, bool reuse = false) {
     VcSched S;
     std::vector<VcLaunchInfo> L;
-    const int rc_sched = make_schedule(c, q, forward, S, L);
+    const int rc_sched = make_schedule(c, q, forward, S, L, reuse);
     if (rc_sched) return schedule_error(rc_sched);
     S.recv_lo = (int)((uintptr_t)recvbuf & 4095);
     PlanInfo pi;
@@ -755,7 +765,8 @@ static int run_schedule(vc_comm *c, const CallParams &q, const char *sendbuf, ch
         rc = plan_read(c, S, L, pi, forward);
         if (rc) return rc;
     }
-    if (forward && staging_out_of_bound(c, pi.stage_bytes, pi.payload_bytes)) return run_schedule(c, q, sendbuf, recvbuf, T, false);
+    if (forward && staging_out_of_bound(c, pi.stage_bytes, pi.payload_bytes)) return run_schedule(c, q, sendbuf, recvbuf, T, false, true);
+    if (!forward && worth_reusing(c, S, pi.stage_bytes)) return run_schedule(c, q, sendbuf, recvbuf, T, false, true);
     rc = plan_emit(c, S, L, T, c->desc, pi);
     if (rc) return rc;
     return run_items(c, pi, c->desc.p, sendbuf, recvbuf, true);

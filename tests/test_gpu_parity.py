@@ -935,7 +935,7 @@ def test_both_execution_modes_leave_the_same_staging(api):
             assert np.count_nonzero(snaps[0] != 0xAB) > sizes[0] // 4, name        # the slots were written
             # with the staging bound on (the default), launch-per-digit execution reuses staging memory: never more, and
             # the same result
-            dp.comm.set_staging_bound(True)
+            dp.comm.set_staging_bound(2)             # (an allowance of 2 MiB: calls as small as these are planned for reuse)
             dp.comm.set_forwarding(0)
             dr = dp.new_recv_arena(0xEE)
             assert fn(dp, ds, dr) == 0 and dp.verify(ds, dr) == 0, name
