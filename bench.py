@@ -119,7 +119,8 @@ def short_block_context(api, torch) -> dict:
     out = {}
     for key, P, hi, what, fn in (
             ("P64_blocks_0_4096B_twophase_r2", 64, 4096, "benchmark configuration 2", lambda dp, s, d: api.twophase_rbruck_alltoallv(2, dp, s, d)),
-            ("P1024_blocks_0_512B_ttpl_n32_r32", 1024, 512, "configuration 4's shape with short blocks", lambda dp, s, d: api.TTPL_BT_alltoallv_s1(32, 32, 0, dp, s, d))):
+            ("P1024_blocks_0_512B_ttpl_n32_r32", 1024, 512, "configuration 4's shape with short blocks", lambda dp, s, d: api.TTPL_BT_alltoallv_s1(32, 32, 0, dp, s, d)),
+            ("P1024_blocks_0_16B_ttpl_n32_r32", 1024, 16, "configuration 4's shape with very short blocks", lambda dp, s, d: api.TTPL_BT_alltoallv_s1(32, 32, 0, dp, s, d))):
         prob = W.make_problem(W.counts_uniform_random(P, hi, seed=0), 1, 0, 0)
         dp = api.DeviceProblem(prob)
         send, recv = dp.new_send_arena(), dp.new_recv_arena()
