@@ -73,6 +73,10 @@ def workload(name: str, seed: int):
         counts = W.counts_from_npz(os.path.join(ROOT, "tests", "golden", "inputs", f"global_comm_pattern_{P}proc.npz"))
         r = min(32, P)
         return counts, 1, "twophase_rbruck_alltoallv", dict(r=r), W.hops_flat(P, r)
+    if name.startswith("S"):
+        # configuration 4's shape with short blocks, S<bytes>: counts uniform in 0..bytes (what the Bruck family exists for)
+        counts = W.counts_uniform_random(1024, int(name[1:]), seed)
+        return counts, 1, "TTPL_BT_alltoallv_s1", dict(n=32, r=32, bblock=0), W.hops_twolayer(1024, 32, 32)
     if name.startswith("U"):
         # equal blocks of U<bytes> bytes at configuration 4's shape: separates the cost of variable, unaligned blocks
         counts = np.full((1024, 1024), int(name[1:]), dtype=np.int32)
@@ -436,6 +440,7 @@ def main() -> None:
         "config": {"workload": (f"benchmark configuration 4 with counts rounded to multiples of {args.workload[3:]} bytes" if args.workload.startswith("C4m") else
                                 f"benchmark configuration {args.workload[1:]}" if args.workload[0] == "C" else
                                 f"equal blocks of {args.workload[1:]} bytes" if args.workload[0] == "U" else
+                                f"blocks uniform in 0..{args.workload[1:]} bytes" if args.workload[0] == "S" else
                                 f"reference input matrix inputs/{prob.P}proc") + f": {func}, P={prob.P} virtual ranks, "
                                + ", ".join(f"{k}={v}" for k, v in tun.items()) + f", {esz}-byte elements",
                    "payload_bytes": S, "algorithmic_bytes": A, "physical_bytes": int(phys_call),
