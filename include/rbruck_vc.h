@@ -89,7 +89,8 @@ int vc_comm_set_bases(vc_comm_t comm, const int64_t *sbase_bytes, const int64_t 
  * 0: one kernel launch per digit phase (or per batch of its rounds, as b / bblock say); every hop reads the block
  *    where the previous hop left it.  This is the mode whose launches vc_comm_last_stats and vc_comm_last_traffic
  *    describe one by one.
- * Results, and the staging contents, are the same in all of them.  Applies to calls and to plans created afterwards
+ * Results are the same in all of them, and so are the staging contents wherever two modes use the same staging layout
+ * (a region per digit phase: staging bound off, no fixed stride).  Applies to calls and to plans created afterwards
  * (plans always hold a list). */
 int vc_comm_set_forwarding(vc_comm_t comm, int enable);
 
