@@ -149,41 +149,48 @@ def short_block_context(api, torch) -> dict:
     return out
 
 
-def cpu_baseline(name: str, seed: int, budget_s: float) -> dict:
-    """The same algorithm on this box's host cores, on a bounded sample of the workload.
+def cpu_sample(name: str, seed: int):
+    """The bounded sample of workload `name` the CPU leg runs: (rank count, counts, element size, the reference driver's function
+    name and arguments, this library's function name and tunables, what differs from the workload)."""
+    sample_P = {"C4": 256, "C5": 512, "C3": 256, "C2": 64}[name]
+    if name == "C4":
+        return (sample_P, W.counts_normal(sample_P, 4096.0, 1024.0, 0, 16384, seed), 1, "ttpl", dict(r=32, b=0, n=32, bblock=0),
+                "TTPL_BT_alltoallv", dict(n=32, r=32, bblock=0),
+                "same count distribution at a quarter of the ranks (the box caps processes near 1000)")
+    if name == "C5":
+        return (sample_P, W.counts_fft_rows(sample_P, 32, 16384), 8, "tuna", dict(r=32, b=0, n=0, bblock=0),
+                "tuna_algorithm", dict(r=32, b=0), "the configuration's rank count and pattern, blocks of 128 KiB instead of 1 MiB")
+    if name == "C3":
+        return (sample_P, W.counts_zipf(sample_P, 65536, 1.2, 5, seed), 4, "twophase", dict(r=16, b=0, n=0, bblock=0),
+                "twophase_rbruck_alltoallv", dict(r=16), "the configuration itself")
+    return (sample_P, W.counts_uniform_random(sample_P, 4096, seed), 1, "twophase", dict(r=2, b=0, n=0, bblock=0),
+            "twophase_rbruck_alltoallv", dict(r=2), "the configuration itself")
+
+
+def cpu_reference_leg(name: str, seed: int, budget_s: float) -> dict:
+    """The same algorithm on this box's host cores, on a bounded sample of the workload.  Runs BEFORE this process touches
+    the GPU (it starts child processes and needs nothing from the device).
 
     Preferred: the real reference functions (oracle/_ref/ref_driver, built in the build container from the
     reference's own sources) under `mpiexec -n P`, timed the reference's way (MPI_Wtime around the call, maximum
-    over ranks).  Configurations 2, 3 and 5 run at their real rank counts (64, 256, 512; configuration 5 with blocks of
-    128 KiB instead of 1 MiB, which bounds the time).  The box allows ~1000 processes, so configuration 4 (1024 ranks)
-    keeps its shape at P = 256 ranks (8 nodes of 32).  Fallback: the single-threaded C restatement (oracle/), "port".
+    over ranks, examples/rbruckv_example.cpp:101-131).  Configurations 2, 3 and 5 run at their real rank counts (64, 256,
+    512; configuration 5 with blocks of 128 KiB instead of 1 MiB, which bounds the time).  The box allows ~1000 processes,
+    so configuration 4 (1024 ranks) keeps its shape at P = 256 ranks (8 nodes of 32).  Fallback: the single-threaded C
+    restatement (oracle/), "port".  The per-rank digests of what the CPU side received are kept: same_run_parity()
+    runs the GPU path on the same sample afterwards and compares.
     """
     from oracle import oracle_py as O
     if name not in ("C2", "C3", "C4", "C5"):
         return {"value": None, "unit": "GB/s", "cores": 0, "kind": "port", "sample": "not measured for this workload"}
-    sample_P = {"C4": 256, "C5": 512, "C3": 256, "C2": 64}[name]
-    if name == "C4":
-        counts, esz = W.counts_normal(sample_P, 4096.0, 1024.0, 0, 16384, seed), 1
-        func, args = "ttpl", dict(r=32, b=0, n=32, bblock=0)
-    elif name == "C5":
-        counts, esz = W.counts_fft_rows(sample_P, 32, 16384), 8
-        func, args = "tuna", dict(r=32, b=0, n=0, bblock=0)
-    elif name == "C3":
-        counts, esz = W.counts_zipf(sample_P, 65536, 1.2, 5, seed), 4
-        func, args = "twophase", dict(r=16, b=0, n=0, bblock=0)
-    else:
-        counts, esz = W.counts_uniform_random(sample_P, 4096, seed), 1
-        func, args = "twophase", dict(r=2, b=0, n=0, bblock=0)
+    sample_P, counts, esz, func, args, gpu_func, gpu_tun, what = cpu_sample(name, seed)
     payload = int(counts.astype(np.int64).sum()) * esz
     cores = os.cpu_count() or 1
     try:
         cores = len(os.sched_getaffinity(0))
     except Exception:
         pass
-    what = {"C4": "same count distribution at a quarter of the ranks (the box caps processes near 1000)",
-            "C5": "the configuration's rank count and pattern, blocks of 128 KiB instead of 1 MiB",
-            "C3": "the configuration itself", "C2": "the configuration itself"}[name]
     sample = f"{func} P={sample_P}, {what}, payload {payload / 1e6:.1f} MB"
+    keep = {"_counts": counts, "_esz": esz, "_gpu_func": gpu_func, "_gpu_tun": gpu_tun, "_seed": seed}
     if os.path.exists(O.REF_DRIVER) and os.path.exists(O.MPIEXEC):
         try:
             with tempfile.TemporaryDirectory() as tmp:
@@ -195,12 +202,13 @@ def cpu_baseline(name: str, seed: int, budget_s: float) -> dict:
                 res = subprocess.run(cmd, capture_output=True, text=True, timeout=budget_s)
                 if res.returncode == 0:
                     times = [float(x) for x in open(out + ".times").read().split()]
+                    digests = open(out + ".digests").read().split()
                     t = float(np.median(times[1:])) if len(times) > 1 else times[0]
                     return {"value": payload / t / 1e9, "unit": "GB/s", "cores": cores, "kind": "reference",
                             "sample": sample + f"; mpiexec -n {sample_P} (MPICH 3.3.2) on {cores} cores, "
                                                f"{sample_P / cores:.0f}x oversubscribed, median of 2 after 1 warm-up, "
                                                f"max over ranks; result equal to MPI_Alltoallv",
-                            "seconds": t}
+                            "seconds": t, "_digests": digests, **keep}
         except (subprocess.TimeoutExpired, OSError, ValueError):
             pass
     prob = W.make_problem(counts, esz, 0, 0)
@@ -221,7 +229,30 @@ def cpu_baseline(name: str, seed: int, budget_s: float) -> dict:
     t = (time.perf_counter() - t0) / reps
     return {"value": payload / t / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
             "sample": sample + f"; single-threaded C restatement of the reference algorithm, mean of {reps} calls",
-            "seconds": t}
+            "seconds": t, "_digests": [f"{int(h):016x}" for h in O.digest_recv(prob, recv)], **keep}
+
+
+def same_run_parity(cpu: dict, api) -> dict:
+    """Runs this library's function on the very sample the CPU leg ran (same counts, seed, payload, function, tunables) and
+    compares each virtual rank's FNV-1a digest of its receive blocks with what the CPU ranks received — the check the
+    reference's drivers make inside their timed runs (examples/rbruckv_example.cpp:101-121).  Returns the public part of
+    the CPU leg's record with `digests_equal` added."""
+    from oracle import oracle_py as O
+    pub = {k: v for k, v in cpu.items() if not k.startswith("_")}
+    if "_digests" not in cpu:
+        return pub
+    prob = W.make_problem(cpu["_counts"], cpu["_esz"], 0, 0)
+    dp = api.DeviceProblem(prob)
+    send, recv = dp.new_send_arena(), dp.new_recv_arena(0xEE)
+    dp.fill_payload(0, cpu["_seed"], send)
+    rc = call(api, cpu["_gpu_func"], cpu["_gpu_tun"], dp, send, recv)
+    assert rc == 0, dp.comm.error()
+    got = [f"{int(h):016x}" for h in O.digest_recv(prob, recv.cpu().numpy())]
+    pub["digests_equal"] = got == cpu["_digests"]
+    pub["digests_compared"] = len(got)
+    pub["gpu_execution_on_sample"] = EXECUTION_NAMES[int(dp.comm.last_stats().execution)]
+    dp.comm.free()
+    return pub
 
 
 # vc_stats_t.execution of the timed calls (the library's default mode picks between the two forwarded kernels)
@@ -245,29 +276,136 @@ def kernel_name(st) -> str:
 
 
 def copy_ceiling(comm, torch, mib: int = 2048, reps: int = 5) -> dict:
-    """What a plain contiguous copy sustains on this GPU in this run: vc_calibration_copy (16-byte non-temporal loads and
-    stores, one vector per lane, the access pattern of the block mover without its scatter), HIP events on the
-    communicator's stream, best of `reps`."""
+    """What contiguous copies sustain on this GPU in this run: vc_calibration_copy (one read, one write: the mix of
+    launch-per-digit execution) and vc_calibration_copy2 (one read, two writes: the mix of the forwarded kernel on two-hop
+    routes), 16-byte non-temporal loads and stores, one vector per lane — the access pattern of the block movers without
+    their scatter.  HIP events on the communicator's stream, best of `reps`."""
     nb = mib << 20
     a = torch.zeros(nb, dtype=torch.uint8, device="cuda:0")
     b = torch.empty(nb, dtype=torch.uint8, device="cuda:0")
-    best = None
+    b2 = torch.empty(nb, dtype=torch.uint8, device="cuda:0")
+    best = {1: None, 2: None}
     for _ in range(reps + 1):
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        e0.record()
-        comm._check(comm.lib.vc_calibration_copy(b.data_ptr(), a.data_ptr(), nb, comm.handle))
-        e1.record()
-        torch.cuda.synchronize()
-        ms = e0.elapsed_time(e1)
-        best = ms if best is None or ms < best else best
-    del a, b
-    return {"GBps": round(2 * nb / (best * 1e-3) / 1e9, 1), "ms": round(best, 4), "bytes_each_way": nb}
+        for writes in (1, 2):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            if writes == 1:
+                comm._check(comm.lib.vc_calibration_copy(b.data_ptr(), a.data_ptr(), nb, comm.handle))
+            else:
+                comm._check(comm.lib.vc_calibration_copy2(b.data_ptr(), b2.data_ptr(), a.data_ptr(), nb, comm.handle))
+            e1.record()
+            torch.cuda.synchronize()
+            ms = e0.elapsed_time(e1)
+            best[writes] = ms if best[writes] is None or ms < best[writes] else best[writes]
+    del a, b, b2
+    return {"GBps": round(2 * nb / (best[1] * 1e-3) / 1e9, 1), "ms": round(best[1], 4), "bytes_each_way": nb,
+            "one_read_one_write_GBps": round(2 * nb / (best[1] * 1e-3) / 1e9, 1),
+            "one_read_two_writes_GBps": round(3 * nb / (best[2] * 1e-3) / 1e9, 1), "one_read_two_writes_ms": round(best[2], 4)}
+
+
+def ceiling_for_mix(ceiling: dict, writes_per_read: float) -> float:
+    """GB/s a contiguous copy with this many writes per read sustains: the two measured mixes, the time per byte read
+    interpolated (extrapolated beyond two writes) linearly between them."""
+    t1 = 2.0 / ceiling["one_read_one_write_GBps"]
+    t2 = 3.0 / ceiling["one_read_two_writes_GBps"]
+    t = t1 + (writes_per_read - 1.0) * (t2 - t1)
+    return (1.0 + writes_per_read) / t
 
 
 def physical_bytes(st) -> int:
     """Bytes the copy kernels of the last call had to move through HBM: one launch per digit reads and writes every hop;
     forwarded execution reads every block once and writes it once per hop."""
     return 2 * st.moved_bytes if st.execution == 0 else st.payload_bytes + st.moved_bytes
+
+
+def other_configurations(api, torch, ceiling: dict, seed: int) -> dict:
+    """The benchmark's other configurations beside the one `value` is quoted on, a few steps each in the default mode:
+    configuration 2 at its three radices, configuration 3, configuration 5 at r = 32 (what src/tuna.cpp:67-165 times) and at
+    r = 2.  Per entry: milliseconds per blocking call (wall clock), the copy kernels' bytes over their launch time (HIP
+    events on the communicator's stream) against the HBM peak, the execution the library chose, staging memory, and the
+    exact receiver-side check."""
+    out = {}
+    for key, name, radix, steps in (("C2_r2", "C2", 2, 50), ("C2_r4", "C2", 4, 50), ("C2_r8", "C2", 8, 50), ("C3_r16", "C3", 16, 10),
+                                    ("C5_r32", "C5", 32, 5), ("C5_r2", "C5", 2, 5)):
+        counts, esz, func, tun, _ = workload(name, seed)
+        tun = dict(tun, r=radix)
+        prob = W.make_problem(counts, esz, 0, 0)
+        dp = api.DeviceProblem(prob)
+        send, recv = dp.new_send_arena(), dp.new_recv_arena(0)
+        dp.fill_payload(0, seed, send)
+        for _ in range(3):
+            assert call(api, func, tun, dp, send, recv) == 0, dp.comm.error()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            call(api, func, tun, dp, send, recv)
+        torch.cuda.synchronize()
+        call_s = (time.perf_counter() - t0) / steps
+        # the same calls again with the library's events around every launch (they cost microseconds that matter at
+        # configuration 2, so the wall-clock figure above is taken without them)
+        dp.comm.set_timing(True)
+        kern_ms, phys = 0.0, 0
+        for _ in range(steps):
+            assert call(api, func, tun, dp, send, recv) == 0, dp.comm.error()
+            st = dp.comm.last_stats()
+            kern_ms += sum(st.launch_ms[k] for k in range(st.n_launches))
+            phys += physical_bytes(st)
+        st = dp.comm.last_stats()
+        achieved = phys / (kern_ms * 1e-3) / 1e9 if kern_ms > 0 else 0.0
+        mix = 1.0 if st.execution == 0 else st.moved_bytes / max(st.payload_bytes, 1)
+        out[key] = {"workload": f"benchmark configuration {name[1:]}: {func}, P={prob.P}, r={radix}, {esz}-byte elements",
+                    "payload_bytes": int(prob.payload_bytes), "ms_per_call": round(call_s * 1e3, 4),
+                    "GBps_effective": round(prob.payload_bytes / call_s / 1e9, 1),
+                    "kernel": kernel_name(st), "execution": EXECUTION_NAMES[int(st.execution)],
+                    "launches_per_call": int(st.n_launches), "kernel_ms_per_call": round(kern_ms / steps, 4),
+                    "kernel_GBps_physical": round(achieved, 1), "frac": round(achieved / HBM_PEAK_GBPS, 4),
+                    "frac_of_copy_ceiling": round(achieved / ceiling_for_mix(ceiling, mix), 4),
+                    "algorithmic_frac_whole_call": round(2 * st.moved_bytes / call_s / 1e9 / HBM_PEAK_GBPS, 4),
+                    "staging_bytes": int(st.staging_bytes), "steps": steps,
+                    "mismatched_bytes": int(dp.verify(send, recv))}
+        dp.comm.free()
+        del send, recv, dp
+        torch.cuda.empty_cache()
+    return out
+
+
+def metadata_calls(api, torch, counts) -> dict:
+    """The caller-side steps of the reference's drivers (examples/rbruckv_example.cpp:69-82) on configuration 4's tables:
+    count-matrix exchange, the two displacement scans, the two scans of arena bases, the global maximum — microseconds per
+    blocking call (each ends in a stream synchronisation), mean of 20, checked against numpy."""
+    P = counts.shape[0]
+    comm = api.VirtualComm(P)
+    lib, h = comm.lib, comm.handle
+    dev = "cuda:0"
+    sc = torch.from_numpy(np.ascontiguousarray(counts)).to(dev)
+    rc = torch.empty_like(sc)
+    sd, rd = torch.empty_like(sc), torch.empty_like(sc)
+    sext, rext = torch.empty(P, dtype=torch.int64, device=dev), torch.empty(P, dtype=torch.int64, device=dev)
+    sbase, rbase = torch.empty(P, dtype=torch.int64, device=dev), torch.empty(P, dtype=torch.int64, device=dev)
+    total = torch.empty(1, dtype=torch.int64, device=dev)
+    mx = torch.empty(1, dtype=torch.int32, device=dev)
+    steps = (("vc_alltoall_counts", lambda: lib.vc_alltoall_counts(sc.data_ptr(), rc.data_ptr(), h)),
+             ("vc_displs_from_counts_send", lambda: lib.vc_displs_from_counts(sc.data_ptr(), sd.data_ptr(), sext.data_ptr(), h)),
+             ("vc_displs_from_counts_recv", lambda: lib.vc_displs_from_counts(rc.data_ptr(), rd.data_ptr(), rext.data_ptr(), h)),
+             ("vc_bases_from_extents_send", lambda: lib.vc_bases_from_extents(sext.data_ptr(), 1, 256, sbase.data_ptr(), total.data_ptr(), h)),
+             ("vc_bases_from_extents_recv", lambda: lib.vc_bases_from_extents(rext.data_ptr(), 1, 256, rbase.data_ptr(), total.data_ptr(), h)),
+             ("vc_allreduce_max_count", lambda: lib.vc_allreduce_max_count(sc.data_ptr(), mx.data_ptr(), h)))
+    out, reps = {"P": P, "table_bytes": int(counts.nbytes)}, 20
+    for name, fn in steps:
+        assert fn() == 0, comm.error()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            fn()
+        out[name] = round((time.perf_counter() - t0) / reps * 1e6, 1)
+    out["total"] = round(sum(v for k, v in out.items() if k.startswith("vc_")), 1)
+    c64 = counts.astype(np.int64)
+    ok = (np.array_equal(rc.cpu().numpy(), counts.T) and np.array_equal(sd.cpu().numpy(), np.cumsum(c64, axis=1) - c64)
+          and np.array_equal(rd.cpu().numpy(), np.cumsum(c64.T, axis=1) - c64.T) and int(mx.item()) == int(counts.max())
+          and np.array_equal(sext.cpu().numpy(), c64.sum(axis=1)))
+    out["equal_to_numpy"] = bool(ok)
+    comm.free()
+    return out
 
 
 def main() -> None:
@@ -291,6 +429,9 @@ def main() -> None:
     args = ap.parse_args()
     if args.gpus != 1:
         raise SystemExit("bench.py: this build runs the virtual communicator on ONE GPU; --gpus N with N > 1 is not supported")
+
+    # the CPU leg starts child processes (mpiexec) and needs nothing from the GPU: it runs before anything here touches the device
+    cpu = None if args.no_cpu_baseline else cpu_reference_leg(args.workload, args.seed, args.cpu_budget)
 
     import torch
     from rbruck_alltoallv_amd import api
@@ -368,13 +509,18 @@ def main() -> None:
         achieved = t["phys_bytes"] / secs / 1e9 if secs > 0 else 0.0
         alg = t["alg_bytes"] / secs / 1e9 if secs > 0 else 0.0
         quoted = not (args.radix or args.seed or args.func)
+        # the contiguous copy with this execution's mix of reads and writes: one write per read when every hop is a launch
+        # of its own, (bytes of all hops) / payload writes per read when the blocks are forwarded
+        mix = 1.0 if st.execution == 0 else st.moved_bytes / max(st.payload_bytes, 1)
+        like = ceiling_for_mix(ceiling, mix)
         traffic, source = profiled_traffic(kern.split("<")[0], args.workload) if quoted else (None, None)
         r = {"bound": "hbm", "kernel": kern, "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
              "frac": round(achieved / HBM_PEAK_GBPS, 4), "frac_physical": round(achieved / HBM_PEAK_GBPS, 4),
              "physical_bytes_per_launch": int(t["phys_bytes"] / nk),
              "algorithmic_GBps": round(alg, 1), "algorithmic_frac": round(alg / HBM_PEAK_GBPS, 4),
              "algorithmic_bytes_per_launch": int(t["alg_bytes"] / nk),
-             "copy_ceiling_GBps": ceiling["GBps"], "frac_of_copy_ceiling": round(achieved / ceiling["GBps"], 4),
+             "copy_ceiling_writes_per_read": round(mix, 3), "copy_ceiling_GBps": round(like, 1),
+             "frac_of_copy_ceiling": round(achieved / like, 4),
              "traffic": traffic, "traffic_source": source,
              "avg_launch_ms": round(t["kern_ms"] / nk, 4), "launches_per_call": int(st.n_launches),
              "per_launch": None if t["per_launch_ms"] is None else [
@@ -496,13 +642,22 @@ def main() -> None:
         if args.workload == "C4" and args.func is None:
             out["short_block_calls"] = short_block_context(api, torch)
     out["roofline"] = roofline_of(t)
-    if not args.no_cpu_baseline:
-        del send, recv
-        torch.cuda.empty_cache()
-        out["cpu_baseline"] = cpu_baseline(args.workload, args.seed, args.cpu_budget)
+    dp.comm.free()
+    del send, recv, dp
+    torch.cuda.empty_cache()
+    if not args.no_context and args.workload == "C4" and args.func is None and not args.radix:
+        out["configs"] = other_configurations(api, torch, ceiling, args.seed)
+        out["metadata_us"] = metadata_calls(api, torch, counts)
+    if cpu is not None:
+        out["cpu_baseline"] = same_run_parity(cpu, api)
     print(json.dumps(out), flush=True)
     if bad:
         raise SystemExit(f"bench.py: {bad} bytes differ from the alltoallv definition")
+    if cpu is not None and out["cpu_baseline"].get("digests_equal") is False:
+        raise SystemExit("bench.py: the digests of the GPU's receive blocks differ from those of the CPU run on the same sample")
+    wrong = [k for k, v in out.get("configs", {}).items() if v["mismatched_bytes"]]
+    if wrong:
+        raise SystemExit(f"bench.py: configurations {wrong} differ from the alltoallv definition")
 
 
 if __name__ == "__main__":

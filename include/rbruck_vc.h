@@ -371,6 +371,11 @@ int vc_verify_alltoallv(const char *sendbuf, const int *sendcounts, const int *s
  * accesses the block mover uses: the transfer of known size against which hardware byte counters are scaled. */
 int vc_calibration_copy(char *dst, const char *src, int64_t nbytes, vc_comm_t comm);
 
+/* The same with every vector stored twice (to dst and to dst2): one read, two writes, the mix of the forwarded
+ * kernel on two-hop routes (the pack and unpack memcpys of src/twophase_twolayer_rbruck.cpp:334-343,368-377 in one
+ * pass).  The contiguous ceiling that kernel is held against. */
+int vc_calibration_copy2(char *dst, char *dst2, const char *src, int64_t nbytes, vc_comm_t comm);
+
 #ifdef __cplusplus
 }
 #endif

@@ -77,6 +77,7 @@ SYMBOLS = {
     "vc_fill_payload": (_I, [_I, _U64, _P, _P, _P, _I, _P]),
     "vc_verify_alltoallv": (_I, [_P, _P, _P, _I, _P, _P, _P, _I, C.POINTER(_I64), _P]),
     "vc_calibration_copy": (_I, [_P, _P, _I64, _P]),
+    "vc_calibration_copy2": (_I, [_P, _P, _P, _I64, _P]),
 }
 
 _lib = None

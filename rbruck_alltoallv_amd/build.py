@@ -49,6 +49,25 @@ def build_example(verbose: bool = False) -> list[str]:
     return built
 
 
+VARIANTS_BIN = os.path.join(PKG_DIR, "examples", "vc_copy_variants")
+
+
+def build_variants(verbose: bool = False) -> str:
+    """The A/B program of the forwarded copy kernel (examples/vc_copy_variants.hip includes csrc/vc_copy.hip): the
+    product kernel, the variants that were measured against it and the contiguous copies that bound them."""
+    cmd = [HIPCC, "-O3", "-std=c++17", "-Wall", "--offload-arch=gfx950", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+           os.path.join(PKG_DIR, "examples", "vc_copy_variants.hip"), "-o", VARIANTS_BIN]
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    if verbose or res.returncode != 0:
+        print(" ".join(cmd))
+        print(res.stdout)
+        print("\n".join(l for l in res.stderr.splitlines() if "packed-fp32-ops" not in l))
+    if res.returncode != 0:
+        raise RuntimeError("hipcc failed building examples/vc_copy_variants")
+    return VARIANTS_BIN
+
+
 if __name__ == "__main__":
     print(build_library(verbose=True))
     print(build_example(verbose=True))
+    print(build_variants(verbose=True))

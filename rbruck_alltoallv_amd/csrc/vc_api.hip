@@ -1226,7 +1226,7 @@ static int calibrate(vc_comm *c) {
     hipError_t e = hipSuccess;
     for (int rep = 0; rep < 4 && e == hipSuccess; rep++) {         // the first one warms up
         e = hipEventRecord(c->events[0], c->stream);
-        if (e == hipSuccess) e = vc_launch_calibration_copy(buf, buf + nb, (int64_t)nb, c->stream);
+        if (e == hipSuccess) e = vc_launch_calibration_copy(buf, buf + nb, nullptr, (int64_t)nb, c->stream);
         if (e == hipSuccess) e = hipEventRecord(c->events[1], c->stream);
         if (e == hipSuccess) e = hipEventSynchronize(c->events[1]);
         if (e == hipSuccess) e = hipEventElapsedTime(&ms, c->events[0], c->events[1]);
@@ -1396,7 +1396,15 @@ extern "C" int vc_verify_alltoallv(const char *sendbuf, const int *sendcounts, c
 extern "C" int vc_calibration_copy(char *dst, const char *src, int64_t nbytes, vc_comm_t c) {
     if (!c || !dst || !src || nbytes < 0 || (nbytes & 15) || ((uintptr_t)dst & 15) || ((uintptr_t)src & 15))
         return fail_arg("vc_calibration_copy: 16-byte aligned pointers and size needed");
-    HIP_TRY(vc_launch_calibration_copy(src, dst, nbytes, c->stream));
+    HIP_TRY(vc_launch_calibration_copy(src, dst, nullptr, nbytes, c->stream));
+    HIP_TRY(hipStreamSynchronize(c->stream));
+    return VC_OK;
+}
+
+extern "C" int vc_calibration_copy2(char *dst, char *dst2, const char *src, int64_t nbytes, vc_comm_t c) {
+    if (!c || !dst || !dst2 || !src || nbytes < 0 || (nbytes & 15) || ((uintptr_t)dst & 15) || ((uintptr_t)dst2 & 15) || ((uintptr_t)src & 15))
+        return fail_arg("vc_calibration_copy2: 16-byte aligned pointers and size needed");
+    HIP_TRY(vc_launch_calibration_copy(src, dst, dst2, nbytes, c->stream));
     HIP_TRY(hipStreamSynchronize(c->stream));
     return VC_OK;
 }

@@ -213,4 +213,5 @@ VC_HD bool vc_listless_ok(const int64_t *header, const VcListlessGuard &g) {
 hipError_t vc_launch_copy_blocks(const VcSched &S, VcTables T, const int64_t *slot_off, const int64_t *row_base, const int64_t *header,
                                  VcListlessGuard guard, int lanes, const char *sendbuf, char *recvbuf, char *stage, hipStream_t st,
                                  int64_t *header_host = nullptr, int64_t *header_zero = nullptr, int64_t *totals = nullptr);
-hipError_t vc_launch_calibration_copy(const char *src, char *dst, int64_t nbytes, hipStream_t st);
+// dst2 non-null: every vector is stored twice (one read, two writes)
+hipError_t vc_launch_calibration_copy(const char *src, char *dst, char *dst2, int64_t nbytes, hipStream_t st);

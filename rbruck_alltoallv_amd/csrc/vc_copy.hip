@@ -565,19 +565,31 @@ hipError_t vc_launch_copy_items(const VcDesc *items, int64_t nitems, int lanes, 
     return hipGetLastError();
 }
 
-// Plain contiguous copy of a known size: one 16-byte vector per lane, 4 KiB per workgroup.  It exists so that
-// hardware counters (bytes fetched / written per dispatch) can be scaled against a transfer whose size is known.
-__global__ __launch_bounds__(VC_THREADS) void vc_calibration_copy_kernel(const vc_u32x4 *__restrict__ src, vc_u32x4 *__restrict__ dst, int64_t nvec) {
+// Plain contiguous copy of a known size: one 16-byte vector per lane, 4 KiB per workgroup, WRITES stores per load.  It exists so
+// that hardware counters (bytes fetched / written per dispatch) can be scaled against a transfer whose size is known, and as
+// the ceiling the block movers are held against: WRITES = 1 for launch-per-digit execution (one read, one write per hop),
+// WRITES = 2 for the forwarded kernel on two-hop routes (one read, two writes).
+template <int WRITES>
+__global__ __launch_bounds__(VC_THREADS) void vc_calibration_copy_kernel(const vc_u32x4 *__restrict__ src, vc_u32x4 *__restrict__ dst,
+                                                                         vc_u32x4 *__restrict__ dst2, int64_t nvec) {
     const int64_t i = (int64_t)blockIdx.x * VC_THREADS + threadIdx.x;
-    if (i < nvec) __builtin_nontemporal_store(__builtin_nontemporal_load(&src[i]), &dst[i]);
+    if (i >= nvec) return;
+    const vc_u32x4 v = __builtin_nontemporal_load(&src[i]);
+    __builtin_nontemporal_store(v, &dst[i]);
+    if (WRITES == 2) __builtin_nontemporal_store(v, &dst2[i]);
 }
 
-hipError_t vc_launch_calibration_copy(const char *src, char *dst, int64_t nbytes, hipStream_t st) {
+hipError_t vc_launch_calibration_copy(const char *src, char *dst, char *dst2, int64_t nbytes, hipStream_t st) {
     const int64_t nvec = nbytes / 16;
     for (int64_t done = 0; done < nvec; done += VC_MAX_GRID * VC_THREADS) {
         const int64_t now = nvec - done < VC_MAX_GRID * VC_THREADS ? nvec - done : VC_MAX_GRID * VC_THREADS;
-        hipLaunchKernelGGL(vc_calibration_copy_kernel, dim3((unsigned)((now + VC_THREADS - 1) / VC_THREADS)), dim3(VC_THREADS), 0, st,
-                           reinterpret_cast<const vc_u32x4 *>(src) + done, reinterpret_cast<vc_u32x4 *>(dst) + done, now);
+        const dim3 grid((unsigned)((now + VC_THREADS - 1) / VC_THREADS));
+        if (dst2)
+            hipLaunchKernelGGL(vc_calibration_copy_kernel<2>, grid, dim3(VC_THREADS), 0, st, reinterpret_cast<const vc_u32x4 *>(src) + done,
+                               reinterpret_cast<vc_u32x4 *>(dst) + done, reinterpret_cast<vc_u32x4 *>(dst2) + done, now);
+        else
+            hipLaunchKernelGGL(vc_calibration_copy_kernel<1>, grid, dim3(VC_THREADS), 0, st, reinterpret_cast<const vc_u32x4 *>(src) + done,
+                               reinterpret_cast<vc_u32x4 *>(dst) + done, static_cast<vc_u32x4 *>(nullptr), now);
     }
     return hipGetLastError();
 }
