@@ -337,6 +337,13 @@ typedef struct {
                                     workgroup; 64: a wavefront (short pieces); 16: a quarter of one (pieces of a
                                     few hundred bytes); 1: a wavefront took a batch of pairs of ranks (many very short
                                     blocks).  Launch-per-digit execution: of the launch that moved the most bytes. */
+    int64_t block_pieces;        /* forwarded execution: pieces the blocks were cut into (the work items of the list); else 0 */
+    int64_t max_block_pieces;    /* ... the most pieces of one block */
+    int64_t max_block_bytes;     /* ... the longest block */
+    int64_t bad_table_entries;   /* table entries no set of ranks could have passed (negative ones, recvcounts[t][s] !=
+                                    sendcounts[s][t]; + 2^40 per rank whose packed receive layout overflows), as the device
+                                    counted them: 0 after a call that returned VC_OK, set by one that returned VC_ERR_TABLES
+                                    or VC_ERR_OVERFLOW (the other fields then still describe the call before it) */
 } vc_stats_t;
 
 /* Per-launch HIP-event timing of the following calls (0 = off, default). */

@@ -14,6 +14,7 @@
 #include <chrono>
 #include <cstdio>
 #include <cstring>
+#include <mutex>
 #include <string>
 #include <vector>
 
@@ -32,6 +33,8 @@ static thread_local std::string g_last_error;
 static __device__ __align__(256) unsigned char scratch[VC_NOALLOC_SCRATCH_BYTES];
 #define VC_MAX_DEVICES 64
 static unsigned char *g_scratch_ptr[VC_MAX_DEVICES];       // per device: where its copy of `scratch` lives (null: not resolved)
+static std::mutex g_scratch_mutex;                         // guards the resolution (communicators may be created from several threads)
+static std::atomic_flag g_scratch_busy[VC_MAX_DEVICES];    // per device: a call is using the array (all communicators on a GPU share it)
 
 static int fail_hip(hipError_t e, const char *what, int line) {
     char buf[256];
@@ -96,6 +99,12 @@ struct PlanBufs {
     int *rd_packed = nullptr;
 };
 
+// What a call asked for: enough to derive its schedule again in the other execution mode.
+struct CallParams {
+    VcFunc f;
+    int n, r, batch, esz, uniform, batch2;
+};
+
 struct vc_comm {
     int P = 0;
     int device = 0;
@@ -129,11 +138,14 @@ struct vc_comm {
         char *recvbuf = nullptr;
         int lanes = 0;
         int n_launch_infos = 0;
+        hipStream_t own_stream = nullptr; // the communicator's stream while the call runs on the caller's
+        CallParams q;                     // what was asked for (the call may have to be run again another way)
     } pending;
     PlanBufs B;                           // where the current call's plan lives
     const void *last_stage = nullptr;     // staging arena of the last call
     int64_t *h_header = nullptr;          // pinned, coherent: the planner writes its header straight into it
     int64_t *h_header_dev = nullptr;      // the same memory as the device sees it
+    int *h_flags = nullptr, *h_flags_dev = nullptr;   // pinned, coherent: the two flags of vc_displs_from_counts, as host and device see them
     VcLaunchInfo *h_launches = nullptr;   // pinned
     std::vector<hipEvent_t> events;
     vc_stats_t stats;
@@ -185,14 +197,19 @@ extern "C" int vc_comm_create(int nranks, vc_comm_t *comm_out) {
     c->P = nranks;
     memset(&c->stats, 0, sizeof c->stats);
     hipError_t e = hipGetDevice(&c->device);
-    if (e == hipSuccess && c->device >= 0 && c->device < VC_MAX_DEVICES && !g_scratch_ptr[c->device]) {
-        void *ptr = nullptr;                              // this device's copy of the static scratch array
-        e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
-        if (e == hipSuccess) g_scratch_ptr[c->device] = static_cast<unsigned char *>(ptr);
+    if (e == hipSuccess && c->device >= 0 && c->device < VC_MAX_DEVICES) {
+        std::lock_guard<std::mutex> lock(g_scratch_mutex);
+        if (!g_scratch_ptr[c->device]) {
+            void *ptr = nullptr;                          // this device's copy of the static scratch array
+            e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+            if (e == hipSuccess) g_scratch_ptr[c->device] = static_cast<unsigned char *>(ptr);
+        }
     }
     if (e == hipSuccess) e = hipHostMalloc((void **)&c->h_header, sizeof(int64_t) * VC_HEADER_WORDS(VC_MAX_LAUNCHES), hipHostMallocCoherent);
     if (e == hipSuccess) e = hipHostGetDevicePointer((void **)&c->h_header_dev, c->h_header, 0);
     if (e == hipSuccess) e = hipHostMalloc((void **)&c->h_launches, sizeof(VcLaunchInfo) * VC_MAX_LAUNCHES, hipHostMallocDefault);
+    if (e == hipSuccess) e = hipHostMalloc((void **)&c->h_flags, 2 * sizeof(int), hipHostMallocCoherent);
+    if (e == hipSuccess) e = hipHostGetDevicePointer((void **)&c->h_flags_dev, c->h_flags, 0);
     if (e != hipSuccess) {
         (void)vc_comm_free(c);
         return fail_hip(e, "vc_comm_create", __LINE__);
@@ -213,6 +230,7 @@ extern "C" int vc_comm_free(vc_comm_t c) {
     for (hipEvent_t e : c->events) (void)hipEventDestroy(e);
     if (c->h_header) (void)hipHostFree(c->h_header);
     if (c->h_launches) (void)hipHostFree(c->h_launches);
+    if (c->h_flags) (void)hipHostFree(c->h_flags);
     delete c;
     return VC_OK;
 }
@@ -278,14 +296,13 @@ extern "C" int vc_alltoall_counts(const int *sendcounts, int *recvcounts, vc_com
 
 extern "C" int vc_displs_from_counts(const int *counts, int *displs, int64_t *extent_out, vc_comm_t c) {
     if (!c || !counts || !displs) return fail_arg("vc_displs_from_counts: null argument");
-    HIP_TRY(c->scratch.reserve(2 * sizeof(int)));
-    int flags[2] = {0, 0};
-    HIP_TRY(hipMemsetAsync(c->scratch.p, 0, sizeof flags, c->stream));
-    HIP_TRY(vc_launch_row_scan(counts, displs, extent_out, c->scratch.as<int>(), c->P, c->stream));
-    HIP_TRY(hipMemcpyAsync(flags, c->scratch.p, sizeof flags, hipMemcpyDeviceToHost, c->stream));
+    VC_ONE_CALL(c);
+    // the kernel raises the two flags in pinned host memory: no clearing launch before it, no copy back after it
+    c->h_flags[0] = c->h_flags[1] = 0;
+    HIP_TRY(vc_launch_row_scan(counts, displs, extent_out, c->h_flags_dev, c->P, c->stream));
     HIP_TRY(hipStreamSynchronize(c->stream));
-    if (flags[1]) return fail_arg("vc_displs_from_counts: negative count", VC_ERR_TABLES);
-    if (flags[0]) return fail_arg("vc_displs_from_counts: a rank's counts sum past INT_MAX elements", VC_ERR_OVERFLOW);
+    if (c->h_flags[1]) return fail_arg("vc_displs_from_counts: negative count", VC_ERR_TABLES);
+    if (c->h_flags[0]) return fail_arg("vc_displs_from_counts: a rank's counts sum past INT_MAX elements", VC_ERR_OVERFLOW);
     return VC_OK;
 }
 
@@ -316,12 +333,6 @@ static int ensure_events(vc_comm *c, size_t n) {
 }
 
 static int schedule_error(int code);
-
-// What a call asked for: enough to derive its schedule again in the other execution mode.
-struct CallParams {
-    VcFunc f;
-    int n, r, batch, esz, uniform, batch2;
-};
 
 // The schedule of a call in one of the two execution modes.  Launch-per-digit execution reuses staging memory when the
 // communicator bounds its staging (the default) and there is something to reuse: with fewer than three staging regions
@@ -470,6 +481,7 @@ static int plan_read(vc_comm *c, const VcSched &S, const std::vector<VcLaunchInf
     const int nl = forward ? 1 : (int)L.size();           // forwarded execution: one launch, one set of totals
     const int64_t *h = c->h_header;
     out = PlanInfo();                                     // (a plan that is derived again in the other execution mode reuses `out`)
+    c->stats.bad_table_entries = h[VC_HEADER_BAD];
     if (h[VC_HEADER_BAD] >= VC_BAD_OVERFLOW)
         return fail_arg("a rank receives more than INT_MAX elements: the packed receive displacements of TTPL_BT_alltoallv do not fit an int",
                         VC_ERR_OVERFLOW);
@@ -561,6 +573,10 @@ static int finish_stats(vc_comm *c, const PlanInfo &pi, const void *items_any, b
     s.payload_bytes = pi.payload_bytes;
     s.moved_bytes = 0;
     s.execution = pi.chain ? (pi.listless ? (pi.strided ? 3 : 2) : 1) : 0;
+    s.block_pieces = pi.chain ? pi.chain_items : 0;
+    s.max_block_pieces = pi.chain ? pi.max_pieces : 0;
+    s.max_block_bytes = pi.chain ? pi.max_len : 0;
+    s.bad_table_entries = 0;
     s.plan_ms = s.total_ms = s.intra_ms = s.inter_ms = 0.f;
     if (pi.chain) {                                   // one launch that performs the hops of every digit
         for (int k = 0; k < pi.nl; k++) s.moved_bytes += pi.bytes[k];
@@ -775,7 +791,8 @@ static int run_schedule(vc_comm *c, const CallParams &q, const char *sendbuf, ch
 // The _async entry points: planning kernels and the listless copy kernel are enqueued and the call returns.  The copy
 // kernel checks the planner's verdict on the device (tables, staging arena) and touches nothing when it is bad;
 // vc_comm_wait reads the same verdict and reports it, or grows the arena and runs the copy again.
-static int enqueue_async(vc_comm *c, const VcSched &S, std::vector<VcLaunchInfo> &L, const char *sendbuf, char *recvbuf, VcTables T) {
+static int enqueue_async(vc_comm *c, const CallParams &q, const VcSched &S, std::vector<VcLaunchInfo> &L, const char *sendbuf, char *recvbuf,
+                         VcTables T) {
     int rc = plan_sizes(c, S, L, T, true);
     if (rc) return rc;
     hipStream_t st = c->stream;
@@ -790,15 +807,27 @@ static int enqueue_async(vc_comm *c, const VcSched &S, std::vector<VcLaunchInfo>
     c->pending.active = true;
     c->pending.S = S; c->pending.T = T; c->pending.sendbuf = sendbuf; c->pending.recvbuf = recvbuf; c->pending.lanes = lanes;
     c->pending.n_launch_infos = (int)L.size();
+    c->pending.q = q;
     return VC_OK;
 }
 
 extern "C" int vc_comm_wait(vc_comm_t c) {
     if (!c) return fail_arg("null communicator");
-    HIP_TRY(hipStreamSynchronize(c->stream));
-    if (!c->pending.active) return VC_OK;
+    if (!c->pending.active) {
+        HIP_TRY(hipStreamSynchronize(c->stream));
+        return VC_OK;
+    }
+    // whatever happens below, the call is over when this function returns: the communicator is free again and launches
+    // on its own stream, not on the caller's (which the caller may destroy once the call has been collected)
     c->pending.active = false;
-    struct Release { vc_comm *c; ~Release() { c->busy.clear(std::memory_order_release); } } release{c};
+    struct Release {
+        vc_comm *c;
+        ~Release() {
+            c->stream = c->pending.own_stream;
+            c->busy.clear(std::memory_order_release);
+        }
+    } release{c};
+    HIP_TRY(hipStreamSynchronize(c->stream));
     const VcSched &S = c->pending.S;
     std::vector<VcLaunchInfo> L((size_t)c->pending.n_launch_infos);     // plan_read only needs their number here
     PlanInfo pi;
@@ -806,6 +835,10 @@ extern "C" int vc_comm_wait(vc_comm_t c) {
     if (rc) return rc;
     VcListlessGuard guard = {c->stage.cap >= 64 ? (int64_t)c->stage.cap - 64 : 0, 0, 0, 0, 0};
     if (!vc_listless_ok(c->h_header, guard)) {            // the arena was too small: nothing has been moved yet
+        // a call whose forwarded staging is out of the communicator's bound runs one launch per digit on reused staging,
+        // like its blocking twin
+        if (staging_out_of_bound(c, pi.stage_bytes, pi.payload_bytes))
+            return run_schedule(c, c->pending.q, c->pending.sendbuf, c->pending.recvbuf, c->pending.T, false, true);
         HIP_TRY(reserve_stage(c, (size_t)pi.stage_bytes + 64));
         guard.stage_cap = (int64_t)c->stage.cap - 64;
         if (c->timing) HIP_TRY(hipEventRecord(c->events[2], c->stream));
@@ -862,9 +895,11 @@ static int run_v(VcFunc f, int n, int r, int batch, vc_comm *c, char *sendbuf, i
     rc = make_schedule(c, q, true, S, L);
     if (rc) return schedule_error(rc);
     S.recv_lo = (int)((uintptr_t)recvbuf & 4095);
+    c->pending.own_stream = c->stream;
     c->stream = static_cast<hipStream_t>(*async_stream);
-    rc = enqueue_async(c, S, L, sendbuf, recvbuf, make_tables(c, sendcounts, sdispls, recvcounts, rdispls));
+    rc = enqueue_async(c, q, S, L, sendbuf, recvbuf, make_tables(c, sendcounts, sdispls, recvcounts, rdispls));
     if (rc == VC_OK) busy_guard_.keep();
+    else c->stream = c->pending.own_stream;
     return rc;
 }
 
@@ -931,8 +966,21 @@ extern "C" int twophase_rbruck_alltoallv_noalloc(int r, char *sendbuf, int *send
     if (rc) return rc;
     VC_ONE_CALL(c);
     if (!sendcounts || !sdispls || !recvcounts || !rdispls) return fail_arg("null table");
-    unsigned char *base = c->device < VC_MAX_DEVICES ? g_scratch_ptr[c->device] : nullptr;
+    unsigned char *base = nullptr;
+    if (c->device < VC_MAX_DEVICES) {
+        std::lock_guard<std::mutex> lock(g_scratch_mutex);
+        base = g_scratch_ptr[c->device];
+    }
     if (!base) return fail_arg("the static scratch array was not resolved on this device", VC_ERR_HIP);
+    // every communicator on this GPU shares the one array: a second call that would overlap this one is refused
+    struct ScratchLock {
+        std::atomic_flag &f;
+        bool mine;
+        explicit ScratchLock(std::atomic_flag &flag) : f(flag), mine(!flag.test_and_set(std::memory_order_acquire)) {}
+        ~ScratchLock() { if (mine) f.clear(std::memory_order_release); }
+    } scratch_lock(g_scratch_busy[c->device]);
+    if (!scratch_lock.mine)
+        return fail_arg("twophase_rbruck_alltoallv_noalloc: another call on this GPU is using the static scratch array", VC_ERR_BUSY);
     VcSched S;
     std::vector<VcLaunchInfo> L;
     rc = vc_make_schedule(VC_F_TWOPHASE, c->P, 0, r, 0, sendtype_size, 0, S, L, 0, true);
@@ -1048,15 +1096,19 @@ static int run_uniform(VcFunc f, int n, int r, vc_comm *c, char *sendbuf, int se
     rc = make_schedule(c, q, forward, S, L);              // (validates the tunables before anything is enqueued)
     if (rc) return schedule_error(rc);
     S.recv_lo = (int)((uintptr_t)recvbuf & 4095);
-    if (async_stream) c->stream = static_cast<hipStream_t>(*async_stream);
     const size_t PP = (size_t)c->P * c->P;
     HIP_TRY(c->uni_counts.reserve(sizeof(int) * PP));
     HIP_TRY(c->uni_displs.reserve(sizeof(int) * PP));
-    HIP_TRY(vc_launch_uniform_tables(c->uni_counts.as<int>(), c->uni_displs.as<int>(), sendcount, c->P, c->stream));
+    hipStream_t const own = c->stream;
+    if (async_stream) c->stream = static_cast<hipStream_t>(*async_stream);
     const int *cnt = c->uni_counts.as<int>(), *dsp = c->uni_displs.as<int>();
+    hipError_t e = vc_launch_uniform_tables(c->uni_counts.as<int>(), c->uni_displs.as<int>(), sendcount, c->P, c->stream);
+    if (e != hipSuccess) { c->stream = own; return fail_hip(e, "vc_launch_uniform_tables", __LINE__); }
     if (!async_stream) return run_schedule(c, q, sendbuf, recvbuf, make_tables(c, cnt, dsp, cnt, dsp), forward);
-    rc = enqueue_async(c, S, L, sendbuf, recvbuf, make_tables(c, cnt, dsp, cnt, dsp));
+    c->pending.own_stream = own;
+    rc = enqueue_async(c, q, S, L, sendbuf, recvbuf, make_tables(c, cnt, dsp, cnt, dsp));
     if (rc == VC_OK) busy_guard_.keep();
+    else c->stream = own;
     return rc;
 }
 
@@ -1219,9 +1271,21 @@ static int calibrate(vc_comm *c) {
     if (c->cal_copy_bytes_per_s > 0) return VC_OK;
     int rc = ensure_events(c, 2);
     if (rc) return rc;
-    const size_t nb = (size_t)256 << 20;
+    // 2 x 256 MiB where the device has room, 2 x 16 MiB where it is nearly full; with no room at all the figures of an idle
+    // MI355X stand in (the suggestion then prices candidates with constants instead of measurements)
+    size_t nb = (size_t)256 << 20;
     char *buf = nullptr;
-    HIP_TRY(hipMalloc((void **)&buf, 2 * nb));
+    if (hipMalloc((void **)&buf, 2 * nb) != hipSuccess) {
+        (void)hipGetLastError();
+        nb = (size_t)16 << 20;
+        if (hipMalloc((void **)&buf, 2 * nb) != hipSuccess) {
+            (void)hipGetLastError();
+            c->cal_copy_bytes_per_s = 6.0e12;
+            c->cal_launch_s = 4.0e-6;
+            c->cal_sync_s = 15.0e-6;
+            return VC_OK;
+        }
+    }
     float best = 0.f, ms = 0.f;
     hipError_t e = hipSuccess;
     for (int rep = 0; rep < 4 && e == hipSuccess; rep++) {         // the first one warms up

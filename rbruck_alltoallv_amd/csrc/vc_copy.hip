@@ -233,12 +233,12 @@ __device__ __forceinline__ void vc_add_totals(const VcSched &S, const VcTables &
         const int to = (int)(idx / P), s = (int)(idx % P);
         const int64_t i = (int64_t)to * P + s, k = (int64_t)s * P + to;
         const int sc = T.sc[k], rc = T.rc[i];
-        bad += (sc < 0) | (rc != sc) | (T.sd[i] < 0) | (!S.packed_recv && T.rd[i] < 0);
+        bad += vc_pair_bad_entries(S, T, s, to);          // the same count the planner's row kernel makes
         // (a packed receive layout past INT_MAX elements shows as a negative packed displacement of a later source)
         if (S.packed_recv && (T.rd_packed[i] < 0 || (s == P - 1 && (int64_t)T.rd_packed[i] + rc > 0x7FFFFFFF))) bad += VC_BAD_OVERFLOW;
         const int64_t len = (int64_t)sc * S.esz;
         const int64_t cnt = sc > 0 ? vc_chain_count(S, T, s, to) : 0;
-        payload += len;
+        payload += (int64_t)rc * S.esz;                   // (what the receivers expect, as the planner counts it)
         items += cnt;
         moved += len * vc_block_hops(S, s, to);
         most = cnt > most ? cnt : most;

@@ -89,20 +89,22 @@ hipError_t vc_launch_bases(const int64_t *extent, int esz, int64_t align, int64_
 // ---------------------------------------------------------------------------
 // MPI_Allreduce(MAX) of the block length (src/twophase_tunable_rbruckv.cpp:40-44).
 // ---------------------------------------------------------------------------
+// One atomic per workgroup (the wavefronts' maxima meet in LDS first): 256 atomics on the one word instead of one per
+// wavefront, which is what the call waited for at 1024 ranks.
 __global__ __launch_bounds__(VC_THREADS) void vc_max_kernel(const int *__restrict__ counts, int *__restrict__ out, int64_t n) {
+    __shared__ int64_t lds[VC_WAVES_PER_BLOCK];
     int m = INT_MIN;
     for (int64_t i = (int64_t)blockIdx.x * VC_THREADS + threadIdx.x; i < n; i += (int64_t)gridDim.x * VC_THREADS) m = max(m, counts[i]);
-#pragma unroll
-    for (int o = VC_WAVE / 2; o > 0; o >>= 1) m = max(m, __shfl_xor(m, o, VC_WAVE));
-    if ((threadIdx.x & (VC_WAVE - 1)) == 0) atomicMax(out, m);
+    const int64_t all = vc_block_max(m, lds);
+    if (threadIdx.x == 0) atomicMax(out, (int)all);
 }
 
 __global__ void vc_lowest_int_kernel(int *p) { *p = INT_MIN; }
 
 hipError_t vc_launch_max(const int *counts, int *out, int64_t nelem, hipStream_t st) {
     hipLaunchKernelGGL(vc_lowest_int_kernel, dim3(1), dim3(1), 0, st, out);
-    int64_t blocks = (nelem + VC_THREADS - 1) / VC_THREADS;
-    if (blocks > 1024) blocks = 1024;
+    int64_t blocks = (nelem + 4 * VC_THREADS - 1) / (4 * VC_THREADS);
+    if (blocks > 256) blocks = 256;
     if (blocks < 1) blocks = 1;
     hipLaunchKernelGGL(vc_max_kernel, dim3((unsigned)blocks), dim3(VC_THREADS), 0, st, counts, out, nelem);
     return hipGetLastError();

@@ -105,11 +105,8 @@ __global__ __launch_bounds__(VC_THREADS) void vc_plan_rows(VcSched S, VcLaunchPa
                 cnt[u] = 0;
                 if (chunk0 + u >= nchunk || s >= P) continue;
                 cnt[u] = vc_chain_count(S, T, s, to);
-                const int64_t i = (int64_t)to * P + s;
-                const int expected = T.rc[i], sent = T.sc[(int64_t)s * P + to];
-                // the receiver must expect exactly what the source sends (the reference fails with an MPI truncation error)
-                bad += expected != sent;
-                bad += (T.sc[i] < 0) | (T.sd[i] < 0) | (expected < 0) | (!S.packed_recv && T.rd[i] < 0);
+                const int expected = T.rc[(int64_t)to * P + s], sent = T.sc[(int64_t)s * P + to];
+                bad += vc_pair_bad_entries(S, T, s, to);
                 payload += (int64_t)expected * S.esz;
                 most = cnt[u] > most ? cnt[u] : most;
                 const int64_t len = (int64_t)sent * S.esz;
@@ -137,10 +134,8 @@ __global__ __launch_bounds__(VC_THREADS) void vc_plan_rows(VcSched S, VcLaunchPa
     }
     if (L == 0 && !forward)                               // forwarded execution has done this above
         for (int id = threadIdx.x; id < P; id += VC_THREADS) {
-            const int64_t i = (int64_t)to * P + id;
-            payload += (int64_t)T.rc[i] * S.esz;
-            bad += (T.sc[i] < 0) | (T.sd[i] < 0) | (T.rc[i] < 0) | (!S.packed_recv && T.rd[i] < 0);
-            bad += T.rc[i] != T.sc[(int64_t)id * P + to];
+            payload += (int64_t)T.rc[(int64_t)to * P + id] * S.esz;
+            bad += vc_pair_bad_entries(S, T, id, to);
         }
     items = vc_block_sum(items, lds);
     if (forward) { most = vc_block_max(most, lds); longest = vc_block_max(longest, lds); } else bytes = vc_block_sum(bytes, lds);

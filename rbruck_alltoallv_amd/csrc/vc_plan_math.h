@@ -380,6 +380,16 @@ VC_HD int64_t vc_chain_count(const VcSched &S, const VcTables &T, int s, int t) 
     return vc_chunk_count(len, vc_phase(S, T, s, t), vc_chain_cut(S, T, s, t));
 }
 
+// Entries of the tables around the pair (source s, receiver t) that no set of ranks could have passed: the receiver must
+// expect exactly what the source sends (the reference fails with an MPI truncation error), and no count or displacement
+// of the receiver's own row may be negative.  Summed over all pairs this is header word VC_HEADER_BAD, whoever adds it
+// up (the planner's row kernel, or the copy kernel that plans nothing).
+VC_HD int vc_pair_bad_entries(const VcSched &S, const VcTables &T, int s, int t) {
+    const int64_t i = (int64_t)t * S.P + s;
+    const int expected = T.rc[i], sent = T.sc[(int64_t)s * S.P + t];
+    return (expected != sent) + (int)((T.sc[i] < 0) | (T.sd[i] < 0) | (expected < 0) | (!S.packed_recv && T.rd[i] < 0));
+}
+
 // Layout of a chain item, in int64 words; `stride` = VC_CHAIN_HEAD + hop slots of the call.
 #define VC_CHAIN_SRC 0    // space-tagged source offset of the piece (always in sendbuf)
 #define VC_CHAIN_LEN 1

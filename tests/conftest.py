@@ -10,6 +10,7 @@ if ROOT not in sys.path:
 
 def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu)")
+    config.addinivalue_line("markers", "perf: wall-clock assertions on a real MI355X (run with -m perf; not part of -m gpu)")
 
 
 @pytest.fixture(scope="session")

@@ -113,3 +113,43 @@ def fnv1a64_blocks(prob: W.Problem, recv: np.ndarray) -> list[str]:
                 h = ((h ^ byte) * 0x100000001B3) & 0xFFFFFFFFFFFFFFFF
         out.append(f"{h:016x}")
     return out
+
+
+COLLECTIVES = ("twophase_rbruck_alltoallv", "twophase_rbruck_alltoallv_om", "tuna_algorithm", "tuna2_algorithm", "TTPL_BT_alltoallv",
+               "TTPL_BT_alltoallv_s1", "TTPL_rbruck_alltoallv", "uniform_spreadout_twolayer", "uniform_inverse_isplit_r_bruck",
+               "MPICH_intra_scattered", "ompi_alltoallv_intra_basic_linear", "ompi_alltoallv_intra_pairwise", "exclisive_or_alltoallv",
+               "spreadout_alltoallv", "twolayer_communicator_linear", "twolayer_communicator_linear_s2")
+
+
+class CalledTwice:
+    """The package's API with every collective called twice.  In the library's default mode (vc_comm_set_forwarding 1) the
+    first call on a communicator goes through the work-item list and leaves the hint by which the next one picks its
+    kernel (listless, batched, fixed-stride staging): a test that makes one call per communicator would never reach those.
+    The receive arena is put back to what it held before the first call, the second call runs on the hint of the first,
+    and both must leave the same bytes; the test's own checks then see the second call's result."""
+
+    def __init__(self, module):
+        self._module = module
+
+    def __getattr__(self, name):
+        fn = getattr(self._module, name)
+        if name not in COLLECTIVES:
+            return fn
+
+        def twice(*args):
+            import torch
+            recv = args[-1]
+            small = recv.numel() <= (1 << 28)
+            before = recv.clone() if small else None
+            rc = fn(*args)
+            if rc != 0:
+                return rc
+            first = recv.clone() if small else None
+            if small:
+                recv.copy_(before)
+            rc = fn(*args)
+            assert rc == 0, "the second call failed where the first one passed"
+            if small:
+                assert torch.equal(first, recv), "the second call on a communicator left other bytes than the first"
+            return rc
+        return twice

@@ -8,7 +8,7 @@ import pytest
 
 from oracle import oracle_py as O
 from rbruck_alltoallv_amd import workloads as W
-from tests.helpers import digest_problem, load_golden, problem_for_case, run_on
+from tests.helpers import CalledTwice, digest_problem, load_golden, problem_for_case, run_on
 
 pytestmark = pytest.mark.gpu
 
@@ -17,7 +17,10 @@ CASES = load_golden()
 
 # vc_comm_set_forwarding: 2 forwarded through a work-item list, 3 / 4 / 5 forwarded without one (a workgroup / a quarter of a
 # wavefront per pair of ranks / a batch of pairs per wavefront), 0 one launch per digit phase
-MODES = {"forwarded": 2, "forwarded-listless": 3, "forwarded-listless-quarter": 4, "forwarded-listless-batch": 5, "launch-per-digit": 0}
+# "default": 1, the mode callers get: the library picks per call from what the last call on the communicator looked like, so
+# every collective is called twice there (tests.helpers.CalledTwice)
+MODES = {"forwarded": 2, "forwarded-listless": 3, "forwarded-listless-quarter": 4, "forwarded-listless-batch": 5, "launch-per-digit": 0,
+         "default": 1}
 
 
 @pytest.fixture(scope="module", params=list(MODES))
@@ -27,7 +30,7 @@ def api(request):
     assert torch.cuda.is_available(), "these tests need the GPU"
     from rbruck_alltoallv_amd import api as A
     A.DEFAULT_FORWARDING = MODES[request.param]
-    yield A
+    yield CalledTwice(A) if request.param == "default" else A
     A.DEFAULT_FORWARDING = None
 
 
@@ -485,7 +488,7 @@ def test_benchmark_configurations_at_full_size(api, name):
            "C4": [("ttpl n=32 r=32", lambda dp, s, d: api.TTPL_BT_alltoallv(32, 32, 0, dp, s, d), True),
                   ("ttpl_rbruck n=32 r=4", lambda dp, s, d: api.TTPL_rbruck_alltoallv(32, 4, dp, s, d), False)],
            "C5": [("tuna r=32", lambda dp, s, d: api.tuna_algorithm(32, 0, dp, s, d), False)]}[name]
-    if api.DEFAULT_FORWARDING in (0, 2):
+    if api.DEFAULT_FORWARDING in (0, 1, 2):
         # the other radices the configuration names, through the work-item list and one launch per digit (the listless
         # kernels give a 1 MiB block to 16 or 256 lanes: exact, shown above for one radix, but slow)
         fwd += {"C2": [("twophase r=4", lambda dp, s, d: api.twophase_rbruck_alltoallv(4, dp, s, d), False),
@@ -610,7 +613,7 @@ def test_reference_input_matrices_at_full_size(api, P):
     """The smallest and the largest of the reference's communication patterns at their real sizes (5.2 and 12.8 GB of
     payload, examples/MLinputs_example.cpp:96: twophase_rbruck_alltoallv on 1-byte elements), checked as the benchmark
     configurations are: definition check on the device, byte sum, and the transposed alltoallv by another function."""
-    if api.DEFAULT_FORWARDING not in (0, 2):
+    if api.DEFAULT_FORWARDING not in (0, 1, 2):
         pytest.skip("blocks of megabytes belong to the work-item list and to launch-per-digit execution")
     import os
     import torch
@@ -807,6 +810,8 @@ def test_default_mode_picks_the_listless_kernel_for_small_calls(api):
     """Mode 1 (the library's default): forwarded, and after a call of few short blocks the next one goes without the
     work-item list; a call with long blocks is refused by the listless kernel's own check of the plan and goes through
     the list.  Every call is exact whichever way it went."""
+    if isinstance(api, CalledTwice):
+        pytest.skip("this test lays out the sequence of calls itself")
     small = W.make_problem(W.counts_uniform_random(64, 4096, seed=0), 1, 0, 0)
     big_counts = W.counts_uniform_random(64, 4096, seed=1)
     big_counts[5, 9] = 200000                          # 49 pieces
@@ -862,7 +867,10 @@ def test_three_shapes_of_the_copy_kernel(api, hi, lanes):
         assert fn(dr) == 0, (name, dp.comm.error())
         assert dp.verify(ds, dr) == 0, name
         st = dp.comm.last_stats()
-        assert st.lanes_per_item == ({3: 256, 4: 16, 5: 1}[api.DEFAULT_FORWARDING] if st.execution == 2 else lanes), (name, st.lanes_per_item)
+        if api.DEFAULT_FORWARDING == 1 and st.execution in (2, 3):       # the default mode went without the list: by its own rule
+            assert st.lanes_per_item in (1, 16, 64, 256), (name, st.lanes_per_item)
+        else:
+            assert st.lanes_per_item == ({3: 256, 4: 16, 5: 1}[api.DEFAULT_FORWARDING] if st.execution == 2 else lanes), (name, st.lanes_per_item)
     dp.comm.free()
 
 
