@@ -41,8 +41,8 @@ typedef struct vc_comm *vc_comm_t;
 #define VC_ERR_ARG (-5)        /* null handle / pointer, element size < 1, bases not set */
 #define VC_ERR_NO_DEVICE (-6)  /* no HIP device */
 #define VC_ERR_TABLES (-7)     /* a negative count or displacement in the tables, or recvcounts[t][s] != sendcounts[s][t] (the reference
-                                  fails with an MPI truncation error); found on the device before anything is copied
-                                  (single-launch execution of small calls: before the pair's own block is) */
+                                  fails with an MPI truncation error); found on the device before anything is copied:
+                                  recvbuf is untouched */
 #define VC_ERR_OVERFLOW (-8)   /* a rank's counts sum past INT_MAX elements, where the reference's int displacements wrap
                                   (examples/rbruckv_example.cpp:69-72): vc_displs_from_counts, and the packed receive layout of
                                   TTPL_BT_alltoallv (src/twophase_twolayer_rbruck.cpp:406-418) */

@@ -20,6 +20,7 @@
 
 #include "../../include/rbruck_vc.h"
 #include "vc_common.h"
+#include "vc_dispatch.h"
 #include "vc_sched.h"
 #include "vc_plan_math.h"
 #include "vc_scan.h"
@@ -42,24 +43,6 @@ static int fail_hip(hipError_t e, const char *what, int line) {
     g_last_error = buf;
     return VC_ERR_HIP;
 }
-
-// Where the default mode goes without a work-item list (measured, blocking calls on MI355X):
-//  - blocks of a few hundred bytes, any number of ranks: a quarter of a wavefront per pair of ranks.  Average piece below
-//    768 B: 26 - 30 us per call at 64 ranks (through the list 42), 42 - 73 at 256 (51 - 88), 300 - 900 at 1024 (330 - 990).
-//  - at most 128 ranks and 32768 pieces, longer blocks: a workgroup per pair (26 - 42 us against 40 - 57 at 16 and 64 ranks
-//    with blocks up to 8 KB, 31 - 77 against 48 - 92 up to 32 KB; a few per cent at 128 ranks; at 256 ranks the list wins).
-//  - never after a call with a block of more than 8 (quarter) / 16 (workgroup) pieces: one group of lanes moves the
-//    pieces of a block in turn.
-#define VC_LISTLESS_MAX_PAIRS 16384           // "small communicator": at most 128 ranks
-#define VC_LISTLESS_MAX_ITEMS 32768           // pieces of a call for a workgroup per pair
-#define VC_LISTLESS_MAX_PIECES 8              // pieces of one block, quarter of a wavefront per pair
-#define VC_LISTLESS_WG_MAX_PIECES 16          // pieces of one block, workgroup per pair
-#define VC_LISTLESS_QUARTER_BELOW 768         // average piece, any communicator (at 1 KiB the two ways are even)
-#define VC_LISTLESS_BATCH_BELOW 384           // average piece below which a wavefront takes a batch of pairs
-// ... on communicators of at most 128 ranks, where the alternative is a workgroup per pair: never up to 32 ranks (1024
-// pairs leave room for as many workgroups: 26 us either way, the workgroup up to 1.3x faster on KiB blocks), below
-// 1.75 KiB up to 90 ranks (64 ranks: 27 - 33 us against 34 - 38), below 3 KiB above (128 ranks: 30 - 70 us against 64 - 84)
-static int64_t small_quarter_below(int64_t pairs) { return pairs <= 1024 ? 0 : (pairs < 8192 ? 1792 : 3072); }
 
 #define HIP_TRY(expr)                                                   \
     do {                                                                \
@@ -114,8 +97,7 @@ struct vc_comm {
     int forward = 1;                      // vc_comm_set_forwarding: 0 launch per digit, 1 forwarded (list or listless as the last
                                           // call suggests), 2 forwarded through a work-item list, 3 / 4 forwarded, listless with a
                                           // workgroup / a quarter of a wavefront per pair of ranks
-    bool hint_valid = false;              // what the last forwarded call on this communicator looked like
-    int64_t hint_items = 0, hint_max_pieces = 0, hint_payload = 0, hint_max_len = 0;
+    VcHint hint = {0, 0, 0, 0, 0};        // what the last forwarded call on this communicator looked like
     DevBuf chain_row_tot, chain_row_base;
     DevBuf strided_headers;               // fixed-stride calls: two headers used in turn
     bool strided_clean = false;           // ... and the one the next call will use is known to be zero
@@ -464,18 +446,6 @@ static int plan_sizes(vc_comm *c, const VcSched &S, std::vector<VcLaunchInfo> &L
     return enqueue_plan_sizes(c, S, L, T, forward, c->timing);
 }
 
-// Lanes per work item, from the average piece of the list.  Short pieces leave most of a workgroup idle, and what bounds
-// the launch is then the number of items in flight: a wavefront per item keeps four times as many as a workgroup, a
-// quarter of a wavefront sixteen times.  Measured on 1 Mi items (P = 1024, times of the copy kernel, workgroup /
-// wavefront / quarter): pieces uniform in 0..16 B 830 / 269 / 67 us, 0..256 B 882 / 351 / 189, 0..1 KiB 926 / 455 / 431,
-// 0..2 KiB 1105 / 693 / 770, 0..4 KiB 1449 / 1311 / 1462; around 4 KiB and above the workgroup is 5 - 8 % faster than the
-// wavefront.
-static int lanes_for(int64_t bytes, int64_t items) {
-    if (items <= 0) return VC_THREADS;
-    const int64_t average = bytes / items;
-    return average < 448 ? VC_QUARTER : (average < 3072 ? VC_WAVE : VC_THREADS);
-}
-
 // Step 3b, after the stream has been synchronised: what the planning kernels found.
 static int plan_read(vc_comm *c, const VcSched &S, const std::vector<VcLaunchInfo> &L, PlanInfo &out, bool forward) {
     const int nl = forward ? 1 : (int)L.size();           // forwarded execution: one launch, one set of totals
@@ -496,7 +466,7 @@ static int plan_read(vc_comm *c, const VcSched &S, const std::vector<VcLaunchInf
         out.chain = true;
         out.chain_stride = VC_CHAIN_HEAD + vc_hop_slots(S);
         out.chain_items = h[2];
-        out.chain_lanes = lanes_for(out.payload_bytes, out.chain_items);      // every chain item carries one piece of the payload
+        out.chain_lanes = vc_lanes_for_items(out.payload_bytes, out.chain_items);      // every chain item carries one piece of the payload
         out.max_pieces = h[VC_HEADER_MAX_PIECES];
         out.max_len = h[VC_HEADER_MAX_LEN];
         return VC_OK;
@@ -507,7 +477,7 @@ static int plan_read(vc_comm *c, const VcSched &S, const std::vector<VcLaunchInf
         out.bytes[k] = h[VC_HEADER_FIXED + k];
         out.first[k] = nitems;
         out.count[k] = h[VC_HEADER_FIXED + nl + k];
-        out.lanes[k] = lanes_for(out.bytes[k], out.count[k]);
+        out.lanes[k] = vc_lanes_for_items(out.bytes[k], out.count[k]);
         nitems += out.count[k];
     }
     out.items_total = nitems;
@@ -585,11 +555,7 @@ static int finish_stats(vc_comm *c, const PlanInfo &pi, const void *items_any, b
         if (c->timing) HIP_TRY(hipEventElapsedTime(&s.launch_ms[0], c->events[2], c->events[3]));
         s.intra_ms = s.launch_ms[0];
         s.lanes_per_item = pi.chain_lanes;
-        c->hint_valid = true;
-        c->hint_items = pi.chain_items;
-        c->hint_payload = pi.payload_bytes;
-        c->hint_max_pieces = pi.max_pieces;
-        c->hint_max_len = pi.max_len;
+        c->hint = VcHint{1, pi.chain_items, pi.payload_bytes, pi.max_pieces, pi.max_len};
     } else {
         int64_t most = -1;
         for (int k = 0; k < nl; k++) {
@@ -634,62 +600,20 @@ static int run_items(vc_comm *c, const PlanInfo &pi, const void *items_any, cons
     return finish_stats(c, pi, items_any, planned_now);
 }
 
-// Whether a forwarded call should try to go without the work-item list, and with how many lanes per pair of ranks
-// (0: through the list): worth it when writing the list (and waiting for its size before that) costs more than the
-// per-pair kernel loses by working out routes itself, i.e. for calls of short blocks.  The last forwarded call on the
-// communicator is the guide (mode 1), or the caller says so (modes 3 and 4).
-// Calls of short blocks: a quarter of a wavefront per pair, or, when the blocks are so short that working out the routes
-// costs more than moving the bytes, a batch of pairs per wavefront.  Measured on MI355X on 192 - 2048 ranks: the batches
-// are 5 - 40 % faster up to an average block of 256 bytes, even at 512, 3 - 16 % slower beyond.
-// Not on at most 128 ranks, where batches would leave most of the chip without a wavefront.
-static int short_block_lanes(const vc_comm *c, int P) {
-    if ((int64_t)P * P <= VC_LISTLESS_MAX_PAIRS) return VC_QUARTER;
-    return c->hint_payload / std::max<int64_t>(c->hint_items, 1) < VC_LISTLESS_BATCH_BELOW ? VC_BATCHED : VC_QUARTER;
-}
-
-static int listless_lanes(const vc_comm *c, const VcSched &S) {
-    if (c->forward == 3) return VC_THREADS;
-    if (c->forward == 4) return VC_QUARTER;
-    if (c->forward == 5) return VC_BATCHED;
-    if (c->forward != 1 || !c->hint_valid) return 0;
-    const int64_t average = c->hint_payload / std::max<int64_t>(c->hint_items, 1);
-    const bool small_comm = (int64_t)S.P * S.P <= VC_LISTLESS_MAX_PAIRS;
-    if (c->hint_max_pieces <= VC_LISTLESS_MAX_PIECES && average < (small_comm ? small_quarter_below((int64_t)S.P * S.P) : VC_LISTLESS_QUARTER_BELOW))
-        return short_block_lanes(c, S.P);
-    // a wavefront per pair when the blocks are a KiB or two (a workgroup would start four wavefronts for each of them and
-    // leave two or three without work), a workgroup per pair for longer ones
-    if (small_comm && c->hint_max_pieces <= VC_LISTLESS_WG_MAX_PIECES && c->hint_items <= VC_LISTLESS_MAX_ITEMS)
-        return average < 3072 ? VC_WAVE : VC_THREADS;
-    return 0;
-}
-
-// Fixed-stride staging for calls of short blocks (the default mode, after a call that the listless kernels could serve):
-// the reference's own layout, every slot as long as the longest block (src/twophase_tunable_rbruckv.cpp:59), makes slot
-// addresses closed forms, so the call needs neither the planner's prefix sums nor its slot tables, and no planner at all
-// before the copy kernel: the call is ONE launch and one host synchronisation.  The first wavefronts of the copy kernel
+// One launch on fixed-stride staging (vc_dispatch chose it: a small call in the default mode, after a call the listless
+// kernels could serve): no planner before the copy kernel, one host synchronisation.  The first wavefronts of the copy kernel
 // add up what the host wants to know afterwards (validation, totals, the longest block); every pair of ranks checks its
-// own table entries, and that its block fits a slot, before it moves anything.  The stride comes from the last call's
-// longest block; a call with a longer block is redone the general way, and a call with bad tables returns the same
-// code as elsewhere — but blocks of the pairs whose entries were in order may have been delivered by then (everywhere
-// else nothing moves before the tables have been checked).  Costs arena: regions x P x P x stride bytes, so only
-// up to VC_STRIDED_MAX_BYTES, and only on communicators of at most 192 ranks.  Measured on MI355X, microseconds per
-// blocking call: 64 ranks with blocks of 0 - 4 KiB 41 -> 29 with a pass over the tables before the copy kernel, 24.6 with
-// the pass inside it; 128 ranks, 0 - 512 B: 41 -> 25.6; 160 ranks: 31 - 42 -> 26 - 34; 192 ranks: 31 - 50 -> 30 - 42; but
-// 256 ranks 34 - 68 -> 44 - 68, 384 ranks 44 - 55 -> 85 - 88 (the atomics of the totals, six per 256 pairs on the same
-// words, and the arena grow with the square of the ranks), 1024 ranks with blocks of 0 - 512 B 380 -> 560 (805 MB of
-// slots 768 bytes apart instead of 270 MB of compact ones).
+// own table entries, and that its block fits a slot, before it forms an address from them, and holds its stores back
+// until all of those wavefronts have reported the tables in order (their verdict comes after one round of loads, about
+// when the copying wavefronts have their data): as everywhere else, a call with bad tables has touched nothing when it
+// returns.  A call with a longer block than the stride holds is redone the general way (the blocks that did fit have
+// been delivered by then, and are delivered again).
 // Returns 1 when the call has been served, 0 when it must go the general way, < 0 on errors.
-#define VC_STRIDED_MAX_BYTES ((int64_t)256 << 20)
-#define VC_STRIDED_MAX_PAIRS 36864           // 192 ranks
-static int try_strided(vc_comm *c, VcSched S, std::vector<VcLaunchInfo> &L, const char *sendbuf, char *recvbuf, VcTables T, int pair_lanes) {
-    if (c->forward != 1 || !pair_lanes || S.coalesce || vc_hop_slots(S) > VC_MAX_HOP_SLOTS) return 0;
-    if ((int64_t)S.P * S.P > VC_STRIDED_MAX_PAIRS) return 0;
-    if (pair_lanes == VC_BATCHED) pair_lanes = VC_QUARTER;      // (the batches come without the totals)
-    const int64_t stride = (c->hint_max_len + 2 * VC_LINE - 1) & ~(int64_t)(VC_LINE - 1);     // the block at any cache-line phase
-    if (stride > 0x7FFFFF80) return 0;
-    S.stride = (int)stride;
+static int try_strided(vc_comm *c, VcSched S, std::vector<VcLaunchInfo> &L, const char *sendbuf, char *recvbuf, VcTables T, const VcDispatch &d) {
+    if (d.stride <= 0) return 0;
+    const int pair_lanes = d.stride_lanes;
+    S.stride = d.stride;
     const int64_t need = vc_strided_stage_bytes(S);
-    if (need > VC_STRIDED_MAX_BYTES) return 0;
     hipStream_t st = c->stream;
     // two headers in turn: the planner adds up into one (with atomics, so it must start from zero) while the copy kernel
     // clears the other one for the next call
@@ -710,12 +634,13 @@ static int try_strided(vc_comm *c, VcSched S, std::vector<VcLaunchInfo> &L, cons
         HIP_TRY(vc_launch_row_scan(T.rc, c->rd_packed.as<int>(), nullptr, nullptr, S.P, st));
         T.rd_packed = c->rd_packed.as<int>();
     }
-    const bool quarter = pair_lanes == VC_QUARTER;
-    VcListlessGuard guard = {(int64_t)c->stage.cap - 64, quarter ? VC_LISTLESS_MAX_PIECES : VC_LISTLESS_WG_MAX_PIECES,
-                             quarter ? 0 : VC_LISTLESS_MAX_ITEMS, quarter ? 4096 : 0, stride - VC_LINE + 1};
+    VcListlessGuard guard = d.guard;
+    guard.stage_cap = (int64_t)c->stage.cap - 64;
     if (c->timing) { HIP_TRY(hipEventRecord(c->events[1], st)); HIP_TRY(hipEventRecord(c->events[2], st)); }
-    // the one launch of the call: its first wavefronts add the tables' totals up into `header`, every pair checks its own
-    // entries and the length of its block before it moves anything
+    c->h_header[VC_HEADER_STALLED] = 0;
+    // the one launch of the call: its first wavefronts check the tables and add their totals up into `header`; every pair
+    // checks its own entries and the length of its block before it forms an address, and stores nothing before all of
+    // the tables have been found in order
     HIP_TRY(vc_launch_copy_blocks(S, T, nullptr, nullptr, header, guard, pair_lanes, sendbuf, recvbuf, c->stage.as<char>(), st, c->h_header_dev,
                                   header_next, header));
     c->strided_clean = true;
@@ -724,6 +649,7 @@ static int try_strided(vc_comm *c, VcSched S, std::vector<VcLaunchInfo> &L, cons
     PlanInfo pi;
     int rc = plan_read(c, S, L, pi, true);
     if (rc) return rc;
+    if (c->h_header[VC_HEADER_STALLED]) return 0;          // a copying wavefront gave up waiting for the verdict and moved nothing
     if (!vc_listless_ok(c->h_header, guard)) return 0;     // longer blocks than the last call's, or not a call for this kernel
     pi.listless = pi.strided = true;
     pi.chain_lanes = pair_lanes;
@@ -739,8 +665,9 @@ static int run_schedule(vc_comm *c, const CallParams &q, const char *sendbuf, ch
     S.recv_lo = (int)((uintptr_t)recvbuf & 4095);
     PlanInfo pi;
     hipStream_t st = c->stream;
-    const int pair_lanes = forward ? listless_lanes(c, S) : 0;
-    int rc = try_strided(c, S, L, sendbuf, recvbuf, T, pair_lanes);
+    const VcDispatch d = forward ? vc_dispatch(c->forward, VC_CALL_BLOCKING, c->hint, S) : VcDispatch{0, 0, 0, {0, 0, 0, 0, 0}};
+    const int pair_lanes = d.lanes;
+    int rc = try_strided(c, S, L, sendbuf, recvbuf, T, d);
     if (rc) return rc < 0 ? rc : VC_OK;
     rc = plan_sizes(c, S, L, T, forward);
     if (rc) return rc;
@@ -749,13 +676,8 @@ static int run_schedule(vc_comm *c, const CallParams &q, const char *sendbuf, ch
         // the copy kernel goes out right behind the planning kernels and checks their verdict on the device: when the
         // staging arena turns out too small it has touched nothing and goes out once more behind a larger arena; when the
         // call is not of the kind the last one made the host expect, the call continues through the list
-        VcListlessGuard guard = {0, 0, 0, 0, 0};
-        if (c->forward == 1) {
-            const bool quarter = pair_lanes == VC_QUARTER || pair_lanes == VC_BATCHED;
-            guard.max_pieces = quarter ? VC_LISTLESS_MAX_PIECES : VC_LISTLESS_WG_MAX_PIECES;
-            guard.max_items = quarter ? 0 : VC_LISTLESS_MAX_ITEMS;
-            guard.max_average = quarter ? 4096 : 0;
-        }
+        VcListlessGuard guard = d.guard;
+        guard.max_len = 0;                                // (the limit of fixed-stride slots: compact ones hold any block)
         for (int attempt = 0; attempt < 2 && !pi.listless; attempt++) {
             guard.stage_cap = c->stage.cap >= 64 ? (int64_t)c->stage.cap - 64 : 0;
             if (c->timing) {
@@ -796,10 +718,7 @@ static int enqueue_async(vc_comm *c, const CallParams &q, const VcSched &S, std:
     int rc = plan_sizes(c, S, L, T, true);
     if (rc) return rc;
     hipStream_t st = c->stream;
-    // a quarter of a wavefront per pair of ranks after a call of short blocks on this communicator, else a workgroup
-    const bool quarter = c->hint_valid && c->hint_max_pieces <= VC_LISTLESS_MAX_PIECES &&
-                         c->hint_payload / std::max<int64_t>(c->hint_items, 1) < VC_LISTLESS_QUARTER_BELOW;
-    const int lanes = quarter ? short_block_lanes(c, S.P) : VC_THREADS;
+    const int lanes = vc_dispatch(c->forward, VC_CALL_LISTLESS_ONLY, c->hint, S).lanes;
     const VcListlessGuard guard = {c->stage.cap >= 64 ? (int64_t)c->stage.cap - 64 : 0, 0, 0, 0, 0};
     if (c->timing) { HIP_TRY(hipEventRecord(c->events[1], st)); HIP_TRY(hipEventRecord(c->events[2], st)); }
     HIP_TRY(vc_launch_copy_blocks(S, T, c->B.slot_off, c->B.row_base, c->B.header, guard, lanes, sendbuf, recvbuf, c->stage.as<char>(), st));
@@ -1010,10 +929,7 @@ extern "C" int twophase_rbruck_alltoallv_noalloc(int r, char *sendbuf, int *send
     VcTables T = make_tables(c, sendcounts, sdispls, recvcounts, rdispls);
     rc = enqueue_plan_sizes(c, S, L, T, true, false);
     if (rc) return rc;
-    // a quarter of a wavefront per pair of ranks after a call of short blocks on this communicator, else a workgroup
-    const bool quarter = c->hint_valid && c->hint_max_pieces <= VC_LISTLESS_MAX_PIECES &&
-                         c->hint_payload / std::max<int64_t>(c->hint_items, 1) < VC_LISTLESS_QUARTER_BELOW;
-    const int lanes = quarter ? short_block_lanes(c, S.P) : VC_THREADS;
+    const int lanes = vc_dispatch(c->forward, VC_CALL_LISTLESS_ONLY, c->hint, S).lanes;
     HIP_TRY(vc_launch_copy_blocks(S, T, B.slot_off, B.row_base, B.header, guard, lanes, sendbuf, recvbuf, stage, c->stream));
     HIP_TRY(hipStreamSynchronize(c->stream));
     PlanInfo pi;

@@ -147,6 +147,11 @@ hipError_t vc_launch_empty(hipStream_t st);
 #define VC_HEADER_MAX_PIECES 4
 // fixed-stride staging: wavefronts that have added their part of the tables' totals into the header
 #define VC_HEADER_SYNC (VC_HEADER_MAX_LEN + 1)
+// ... wavefronts that have checked their part of the tables and added what they found to VC_HEADER_BAD: the copying
+// wavefronts of the same launch store nothing before all of them have
+#define VC_HEADER_VERDICT (VC_HEADER_SYNC + 1)
+// ... set (in the host's copy of the header only) by a copying wavefront that gave up waiting for that: the call is redone
+#define VC_HEADER_STALLED (VC_HEADER_SYNC + 2)
 #define VC_HEADER_WORDS(nl) (VC_HEADER_FIXED + 2 * (nl))
 // Passes 1 and 2: staging prefix sums and the number of work items of every launch (sizes only).  The launch table
 // travels as a kernel argument when it has at most VC_LAUNCH_PACK entries (launches_dev is then not read).  With chain_row_tot /

@@ -9,7 +9,7 @@
 // sides (the data is touched once per hop).  For pieces of several KiB a 256-lane workgroup per item is fastest (many
 // small workgroups beat persistent or wider ones for a plain copy on this chip, and the same holds for the scattered
 // variable-size blocks of an alltoallv); lists of short pieces are bound by the number of items in flight and get a
-// wavefront, or a quarter of one, per item.  The host chooses per launch (lanes_for in vc_api.hip).
+// wavefront, or a quarter of one, per item.  The host chooses per launch (vc_lanes_for_items in vc_dispatch.h).
 //
 // Workgroups are handed to the 8 XCDs of the chip in turn (workgroup b runs on XCD
 // b mod 8) and every XCD has its own L2.  Work items that follow each other in the
@@ -19,6 +19,7 @@
 // through its own range of addresses.  Measured: +3 % on 4 KiB blocks, +15 % on
 // 1 MiB blocks cut into pieces.
 #include "vc_common.h"
+#include "vc_dispatch.h"
 #include "vc_plan_math.h"
 #include "vc_scan.h"
 
@@ -57,8 +58,11 @@ __device__ __forceinline__ char *vc_resolve(int64_t loc, const char *sendbuf, ch
 // With nhop > 1 this is forwarded execution: the piece is read once, from sendbuf, and every hop stores the same
 // registers (all destinations of a block share the offset inside their cache line, so one mapping of lanes to window
 // vectors serves them all).  dst_of(k) is where hop k puts the piece.
-template <int LANES, class DstOf>
-__device__ __forceinline__ void vc_forward_piece(const char *src, int64_t len, int nhop, DstOf dst_of) {
+// go() is asked once, after the loads have been issued and before the first store: false leaves the piece where it is.
+struct VcAlwaysGo { __device__ __forceinline__ bool operator()() const { return true; } };
+
+template <int LANES, class DstOf, class Go = VcAlwaysGo>
+__device__ __forceinline__ void vc_forward_piece(const char *src, int64_t len, int nhop, DstOf dst_of, Go go = Go()) {
     constexpr int VECS = VC_CHUNK / 16 / LANES;           // window vectors per lane: 2 for a workgroup of 256, 8 for one wavefront
     char *dst = dst_of(0);
     const int t = threadIdx.x;
@@ -80,6 +84,7 @@ __device__ __forceinline__ void vc_forward_piece(const char *src, int64_t len, i
     const int64_t edge = t < 16 ? (t < head ? t : -1) : (t < 32 && done + (t - 16) < len ? done + (t - 16) : -1);
     char edge_byte = 0;
     if (edge >= 0) edge_byte = src[edge];
+    if (!go()) return;
     for (int k = 0; k < nhop; k++) {
         if (k) dst = dst_of(k);
         char *dw = dst - w;
@@ -127,8 +132,8 @@ __global__ __launch_bounds__(LANES) void vc_copy_items_kernel(const VcDesc *__re
 // such a launch is bound by how many items are in flight, not by HBM, and a piece of 100 bytes has work for 7 lanes.
 // Every group of 16 lanes reads its own item; lane t of the group owns window vectors t, t + 16 of every 512-byte pass
 // (most items need one pass; longer ones loop), and moves head byte t and tail byte t.
-template <class DstOf>
-__device__ __forceinline__ void vc_forward_piece_quarter(const char *src, int64_t len, int nhop, DstOf dst_of) {
+template <class DstOf, class Go = VcAlwaysGo>
+__device__ __forceinline__ void vc_forward_piece_quarter(const char *src, int64_t len, int nhop, DstOf dst_of, Go go = Go()) {
     const int t = threadIdx.x & 15;
     char *dst = dst_of(0);
     const int64_t w = (int64_t)((uintptr_t)dst & (VC_LINE - 1));
@@ -148,6 +153,7 @@ __device__ __forceinline__ void vc_forward_piece_quarter(const char *src, int64_
         vc_u32x4 v0, v1;
         if (has0) v0 = vc_load16(sw + (j << 4));
         if (has1) v1 = vc_load16(sw + ((j + 16) << 4));
+        if (first_pass && !go()) return;
         for (int k = 0; k < nhop; k++) {
             if (k || !first_pass) dst = dst_of(k);
             char *dw = dst - w;
@@ -219,13 +225,36 @@ __device__ __forceinline__ int64_t vc_wave_max(int64_t v) {
 // have passed, [4] the most pieces of a block, [5] hop-weighted bytes, [6] the longest block.  The wavefront that finishes
 // last hands the words to the host.
 #define VC_TOTALS_PER_LANE 4
+// wavefronts that add up the totals of a call on P ranks
+__host__ __device__ __forceinline__ int64_t vc_totals_waves(int P) {
+    const int64_t per_wave = VC_WAVE * VC_TOTALS_PER_LANE;
+    return ((int64_t)P * P + per_wave - 1) / per_wave;
+}
+
 __device__ __forceinline__ void vc_add_totals(const VcSched &S, const VcTables &T, int64_t *totals, int64_t *header_host) {
     const int P = S.P;
-    const int64_t pairs = (int64_t)P * P, per_wave = VC_WAVE * VC_TOTALS_PER_LANE, nwaves = (pairs + per_wave - 1) / per_wave;
+    const int64_t pairs = (int64_t)P * P, per_wave = VC_WAVE * VC_TOTALS_PER_LANE, nwaves = vc_totals_waves(P);
     const int64_t wave = (int64_t)blockIdx.x * (blockDim.x / VC_WAVE) + threadIdx.x / VC_WAVE;
     if (wave >= nwaves) return;
     const int lane = threadIdx.x & (VC_WAVE - 1);
+    unsigned long long *h = reinterpret_cast<unsigned long long *>(totals);
     int64_t payload = 0, items = 0, bad = 0, most = 0, moved = 0, longest = 0;
+    // The verdict on the tables first, with nothing but one round of loads in front of it: the copying wavefronts of this
+    // launch hold their stores back until every totalling wavefront has reported (vc_wait_verdict).
+#pragma unroll
+    for (int u = 0; u < VC_TOTALS_PER_LANE; u++) {
+        const int64_t idx = wave * per_wave + u * VC_WAVE + lane;
+        if (idx >= pairs) continue;
+        const int to = (int)(idx / P), s = (int)(idx % P);
+        const int64_t i = (int64_t)to * P + s;
+        bad += vc_pair_bad_entries(S, T, s, to);          // the same count the planner's row kernel makes
+        // (a packed receive layout past INT_MAX elements shows as a negative packed displacement of a later source)
+        if (S.packed_recv && (T.rd_packed[i] < 0 || (s == P - 1 && (int64_t)T.rd_packed[i] + T.rc[i] > 0x7FFFFFFF))) bad += VC_BAD_OVERFLOW;
+    }
+    bad = vc_wave_sum(bad);
+    // one word says it all, so one atomic publishes it: wavefronts that have reported in the low half, wavefronts that
+    // found something wrong in the high half
+    if (lane == 0) atomicAdd(&h[VC_HEADER_VERDICT], 1ull | (bad ? 1ull << 32 : 0ull));
 #pragma unroll
     for (int u = 0; u < VC_TOTALS_PER_LANE; u++) {
         const int64_t idx = wave * per_wave + u * VC_WAVE + lane;
@@ -233,9 +262,6 @@ __device__ __forceinline__ void vc_add_totals(const VcSched &S, const VcTables &
         const int to = (int)(idx / P), s = (int)(idx % P);
         const int64_t i = (int64_t)to * P + s, k = (int64_t)s * P + to;
         const int sc = T.sc[k], rc = T.rc[i];
-        bad += vc_pair_bad_entries(S, T, s, to);          // the same count the planner's row kernel makes
-        // (a packed receive layout past INT_MAX elements shows as a negative packed displacement of a later source)
-        if (S.packed_recv && (T.rd_packed[i] < 0 || (s == P - 1 && (int64_t)T.rd_packed[i] + rc > 0x7FFFFFFF))) bad += VC_BAD_OVERFLOW;
         const int64_t len = (int64_t)sc * S.esz;
         const int64_t cnt = sc > 0 ? vc_chain_count(S, T, s, to) : 0;
         payload += (int64_t)rc * S.esz;                   // (what the receivers expect, as the planner counts it)
@@ -246,11 +272,9 @@ __device__ __forceinline__ void vc_add_totals(const VcSched &S, const VcTables &
     }
     payload = vc_wave_sum(payload);
     items = vc_wave_sum(items);
-    bad = vc_wave_sum(bad);
     moved = vc_wave_sum(moved);
     most = vc_wave_max(most);
     longest = vc_wave_max(longest);
-    unsigned long long *h = reinterpret_cast<unsigned long long *>(totals);
     int last = 0;
     if (lane == 0) {
         // The count below must not be seen before the words above.  A release fence would do, but at device scope it writes
@@ -272,6 +296,34 @@ __device__ __forceinline__ void vc_add_totals(const VcSched &S, const VcTables &
         header_host[lane] = lane == 0 ? vc_strided_stage_bytes(S)
                                       : (int64_t)__hip_atomic_load(&h[lane], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
+
+// A copying wavefront of the single launch asks before its first store: have all totalling wavefronts checked their part of
+// the tables, and did they find them in order?  The totalling workgroups are the first of the grid, so they are resident
+// before any copying one; the wait is bounded all the same (VC_VERDICT_SPINS polls, a few milliseconds): a wavefront that
+// gives up moves nothing and says so in the host's copy of the header, and the host redoes the call the general way.
+#define VC_VERDICT_SPINS (1 << 15)
+__device__ __forceinline__ unsigned long long vc_verdict_word(int64_t *totals) {
+    return __hip_atomic_load(reinterpret_cast<unsigned long long *>(totals) + VC_HEADER_VERDICT, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// Asked by the piece movers between their loads and their stores (see vc_forward_piece).  Without `totals` there is nothing
+// to wait for (the planner's verdict was checked before the block's route was worked out).  look() reads the word once
+// ahead of the block's loads, so that a verdict that is already in costs no round trip of its own.
+struct VcVerdictGate {
+    int64_t *totals, *header_host;
+    unsigned long long nwaves, word;
+    int state;                                            // 0 not known yet, 1 go, 2 leave everything where it is
+    __device__ __forceinline__ void look() { if (totals) word = vc_verdict_word(totals); }
+    __device__ __forceinline__ bool operator()() {
+        if (!totals) return true;
+        for (int spin = 0; state == 0; spin++) {
+            if ((word & 0xFFFFFFFFull) >= nwaves) state = (word >> 32) ? 2 : 1;
+            else if (spin >= VC_VERDICT_SPINS) { header_host[VC_HEADER_STALLED] = 1; state = 2; }
+            else { __builtin_amdgcn_s_sleep(4); word = vc_verdict_word(totals); }
+        }
+        return state == 1;
+    }
+};
 
 // Workgroups at the head of the grid that only add up the totals (none without `totals`): their round trips run beside the
 // copying instead of in front of it.  A multiple of VC_XCDS, so that the workgroups behind them keep their XCDs.
@@ -328,7 +380,7 @@ __global__ __launch_bounds__(LANES) void vc_copy_blocks_kernel(VcSched S, VcTabl
     const int64_t recv_off = vc_recv_offset(S, T, s, t);
     int64_t dst = 0;
     const bool moves = threadIdx.x < VC_WAVE && (int)threadIdx.x < vc_hop_slots(S) && vc_block_hop(S, T, slot_off, row_base, s, t, threadIdx.x, dst);
-    if (block == 0 && first_pair == 0 && threadIdx.x <= VC_HEADER_SYNC) {
+    if (block == 0 && first_pair == 0 && threadIdx.x <= VC_HEADER_VERDICT) {
         if (header_host && !totals && threadIdx.x <= VC_HEADER_MAX_LEN) header_host[threadIdx.x] = header[threadIdx.x];
         if (header_zero) header_zero[threadIdx.x] = 0;    // the header the next call will add up into
     }
@@ -345,10 +397,13 @@ __global__ __launch_bounds__(LANES) void vc_copy_blocks_kernel(VcSched S, VcTabl
     const char *src = sendbuf + send_off;
     const int phase = (int)((recv_off + S.recv_lo) & (VC_LINE - 1)), cut = (int)((recv_off + S.recv_lo) & (VC_PIECE - 1));
     const int64_t pieces = vc_chunk_count(len, phase, cut);
+    VcVerdictGate gate = {totals, header_host, (unsigned long long)vc_totals_waves(S.P), 0, 0};
+    gate.look();
     for (int64_t c = 0; c < pieces; c++) {                // the same cuts as the chain items of this block
         int64_t lo, hi;
         vc_piece_range(len, phase, cut, c, lo, hi);
-        vc_forward_piece<LANES>(src + lo, hi - lo, nhop, [&](int k) { return vc_resolve(route[k] + lo, sendbuf, recvbuf, stage); });
+        vc_forward_piece<LANES>(src + lo, hi - lo, nhop, [&](int k) { return vc_resolve(route[k] + lo, sendbuf, recvbuf, stage); },
+                                [&]() { return gate(); });
     }
 }
 
@@ -381,7 +436,7 @@ __global__ __launch_bounds__(VC_WAVE) void vc_copy_blocks_quarter_kernel(VcSched
     int64_t d0 = 0, d1 = 0;
     const bool m0 = active && q < nslots && vc_block_hop(S, T, slot_off, row_base, s, t, q, d0);
     const bool m1 = active && q + VC_QUARTER < nslots && vc_block_hop(S, T, slot_off, row_base, s, t, q + VC_QUARTER, d1);
-    if (block == 0 && first_pair == 0 && threadIdx.x <= VC_HEADER_SYNC) {
+    if (block == 0 && first_pair == 0 && threadIdx.x <= VC_HEADER_VERDICT) {
         if (header_host && !totals && threadIdx.x <= VC_HEADER_MAX_LEN) header_host[threadIdx.x] = header[threadIdx.x];
         if (header_zero) header_zero[threadIdx.x] = 0;
     }
@@ -396,10 +451,13 @@ __global__ __launch_bounds__(VC_WAVE) void vc_copy_blocks_quarter_kernel(VcSched
     const char *src = sendbuf + send_off;
     const int phase = (int)((recv_off + S.recv_lo) & (VC_LINE - 1)), cut = (int)((recv_off + S.recv_lo) & (VC_PIECE - 1));
     const int64_t pieces = vc_chunk_count(len, phase, cut);
+    VcVerdictGate gate = {totals, header_host, (unsigned long long)vc_totals_waves(S.P), 0, 0};
+    gate.look();
     for (int64_t c = 0; c < pieces; c++) {
         int64_t lo, hi;
         vc_piece_range(len, phase, cut, c, lo, hi);
-        vc_forward_piece_quarter(src + lo, hi - lo, nhop, [&](int k) { return vc_resolve(route[g][k] + lo, sendbuf, recvbuf, stage); });
+        vc_forward_piece_quarter(src + lo, hi - lo, nhop, [&](int k) { return vc_resolve(route[g][k] + lo, sendbuf, recvbuf, stage); },
+                                 [&]() { return gate(); });
     }
 }
 
@@ -481,9 +539,6 @@ static void vc_launch_batch(int64_t pairs, const VcSched &S, VcTables T, const i
                        T, slot_off, row_base, header, guard, first_pair, sendbuf, recvbuf, stage, header_host, header_zero);
 }
 
-// Pairs per wavefront of vc_copy_blocks_batch_kernel: as many as leave every SIMD of the chip a few wavefronts.
-int vc_batch_pairs(int64_t pairs) { return pairs >= ((int64_t)1 << 19) ? 64 : (pairs >= ((int64_t)1 << 17) ? 32 : 16); }
-
 hipError_t vc_launch_copy_blocks(const VcSched &S, VcTables T, const int64_t *slot_off, const int64_t *row_base, const int64_t *header,
                                  VcListlessGuard guard, int lanes, const char *sendbuf, char *recvbuf, char *stage, hipStream_t st,
                                  int64_t *header_host, int64_t *header_zero, int64_t *totals) {
@@ -518,9 +573,6 @@ hipError_t vc_launch_copy_blocks(const VcSched &S, VcTables T, const int64_t *sl
 
 // Items of one launch: as many as VC_MAX_GRID workgroups or wavefronts take.
 static int64_t vc_items_per_launch(int lanes) { return lanes == VC_QUARTER ? VC_MAX_GRID * VC_ITEMS_PER_WAVE : VC_MAX_GRID; }
-
-// Groups of four items a wavefront of the quarter kernels takes: as many as leave every SIMD of the chip a few wavefronts.
-static int vc_quarter_rounds(int64_t items) { return items >= ((int64_t)1 << 19) ? 4 : (items >= ((int64_t)1 << 17) ? 2 : 1); }
 
 static unsigned vc_grid_for(int64_t items, int lanes) {
     const int64_t per = lanes == VC_QUARTER ? VC_ITEMS_PER_WAVE * vc_quarter_rounds(items) : 1;

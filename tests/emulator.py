@@ -19,7 +19,7 @@ MAX_LAUNCHES = 64
 
 
 def build() -> str:
-    deps = [SRC] + [os.path.join(CSRC, f) for f in ("vc_plan_math.h", "vc_sched.h", "vc_common.h")]
+    deps = [SRC] + [os.path.join(CSRC, f) for f in ("vc_plan_math.h", "vc_sched.h", "vc_common.h", "vc_dispatch.h", "vc_scan.h")]
     if not os.path.exists(LIB) or os.path.getmtime(LIB) < max(os.path.getmtime(d) for d in deps):
         os.makedirs(os.path.dirname(LIB), exist_ok=True)
         tmp = f"{LIB}.{os.getpid()}.tmp"                      # parallel test workers may build at the same time
@@ -146,3 +146,24 @@ def twolayer_communicator_linear(n, prob, send, recv):
 
 def twolayer_communicator_linear_s2(n, bblock1, bblock2, prob, send, recv):
     return _run(F_TWOLAYER_LINEAR_S2, prob, send, recv, n=n, batch=bblock1, batch2=bblock2)
+
+
+def dispatch(func, P, hint, mode=1, call_kind=0, n=0, r=2):
+    """csrc/vc_dispatch.h on the CPU: hint = (valid, block pieces, payload bytes, most pieces of a block, longest block).
+    Returns dict(lanes, stride, stride_lanes, max_pieces, max_items, max_average, max_len)."""
+    global _lib
+    if _lib is None:
+        _lib = C.CDLL(build())
+    out = np.zeros(7, dtype=np.int64)
+    valid, items, payload, max_pieces, max_len = hint
+    rc = _lib.dispatch_decision(C.c_int(func), C.c_int(P), C.c_int(n), C.c_int(r), C.c_int(mode), C.c_int(call_kind), C.c_int(int(valid)),
+                                C.c_int64(items), C.c_int64(payload), C.c_int64(max_pieces), C.c_int64(max_len), _p(out))
+    assert rc == 0, rc
+    return dict(zip(("lanes", "stride", "stride_lanes", "max_pieces", "max_items", "max_average", "max_len"), (int(v) for v in out)))
+
+
+def lanes_for_items(nbytes, items):
+    global _lib
+    if _lib is None:
+        _lib = C.CDLL(build())
+    return _lib.lanes_for_items(C.c_int64(nbytes), C.c_int64(items))

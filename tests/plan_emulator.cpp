@@ -15,6 +15,7 @@
 #include <cstring>
 #include <vector>
 
+#include "../rbruck_alltoallv_amd/csrc/vc_dispatch.h"
 #include "../rbruck_alltoallv_amd/csrc/vc_plan_math.h"
 #include "../rbruck_alltoallv_amd/csrc/vc_sched.h"
 
@@ -289,3 +290,22 @@ extern "C" int64_t staging_allocate(int w, int w2, int msd, int coalesce, const 
     std::vector<int64_t> lo(VC_RECYCLE_MAX_PAIRS), hi(VC_RECYCLE_MAX_PAIRS);
     return vc_allocate_staging(S, size, base, lo.data(), hi.data());
 }
+
+
+// The library's choice of kernel (csrc/vc_dispatch.h) for a call of function `func` on P ranks whose last forwarded call
+// left the hint (valid, items, payload, max_pieces, max_len).  out: lanes, stride, stride_lanes, guard.max_pieces,
+// guard.max_items, guard.max_average, guard.max_len.  Returns the schedule's error code.
+extern "C" int dispatch_decision(int func, int P, int n, int r, int mode, int call_kind, int valid, int64_t items, int64_t payload,
+                                 int64_t max_pieces, int64_t max_len, int64_t *out) {
+    VcSched S;
+    std::vector<VcLaunchInfo> L;
+    const int code = vc_make_schedule((VcFunc)func, P, n, r, 0, 1, 0, S, L, 0, true);
+    if (code) return code;
+    const VcHint h = {valid, items, payload, max_pieces, max_len};
+    const VcDispatch d = vc_dispatch(mode, call_kind, h, S);
+    out[0] = d.lanes; out[1] = d.stride; out[2] = d.stride_lanes; out[3] = d.guard.max_pieces; out[4] = d.guard.max_items;
+    out[5] = d.guard.max_average; out[6] = d.guard.max_len;
+    return 0;
+}
+
+extern "C" int lanes_for_items(int64_t bytes, int64_t items) { return vc_lanes_for_items(bytes, items); }
