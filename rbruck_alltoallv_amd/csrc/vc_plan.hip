@@ -434,11 +434,46 @@ __global__ __launch_bounds__(VC_THREADS) void vc_chain_emit(VcSched S, VcTables 
     int64_t total;
     const int64_t at = carry + vc_block_exclusive_scan(cnt, lds, total);
     const bool big = cnt > 4;
-    if (!big)
+    if (cached && cnt > 0) {
+        // the block's route once, in registers (hop slot k in d[k], statically indexed; its table reads go out together); the
+        // pieces of a block of few pieces are then arithmetic and stores only — evaluating the route again for every piece
+        // was a chain of dependent reads per item
+        int64_t d[VC_ROUTE_CACHE];
+        unsigned moves = 0;
+        const int nslots = vc_hop_slots(S);
+#pragma unroll
+        for (int k = 0; k < VC_ROUTE_CACHE; k++) {
+            d[k] = 0;
+            if (k < nslots && vc_block_hop(S, T, slot_off, row_base, s, t, k, d[k])) moves |= 1u << k;
+        }
+        const int nhop = __popc(moves);
+        if (!big) {
+            const int64_t src = VC_SPACE_SEND | vc_send_offset(S, T, s, t), len = (int64_t)T.sc[(int64_t)s * P + t] * S.esz;
+            const int phase = vc_phase(S, T, s, t), cut = vc_chain_cut(S, T, s, t);
+            for (int64_t c = 0; c < cnt; c++) {
+                int64_t lo, hi;
+                vc_piece_range(len, phase, cut, c, lo, hi);
+                int64_t *item = items + (at + c) * stride;
+                item[VC_CHAIN_SRC] = src + lo;
+                item[VC_CHAIN_LEN] = hi - lo;
+                item[VC_CHAIN_NHOP] = nhop;
+                int n = 0;
+#pragma unroll
+                for (int k = 0; k < VC_ROUTE_CACHE; k++)
+                    if (moves >> k & 1) item[VC_CHAIN_HEAD + n++] = d[k] + lo;
+            }
+        } else {
+            big_at[threadIdx.x] = at;
+            big_nhop[threadIdx.x] = nhop;
+            int n = 0;
+#pragma unroll
+            for (int k = 0; k < VC_ROUTE_CACHE; k++)
+                if (moves >> k & 1) big_dst[threadIdx.x][n++] = d[k];
+        }
+    } else if (!big) {
         for (int64_t c = 0; c < cnt; c++) vc_chain_item(S, T, slot_off, row_base, s, t, c, items + (at + c) * stride);
-    else {
+    } else {
         big_at[threadIdx.x] = at;
-        if (cached) big_nhop[threadIdx.x] = vc_chain_route(S, T, slot_off, row_base, s, t, big_dst[threadIdx.x]);
     }
     if (__syncthreads_or(big)) {
         int64_t btotal;
@@ -465,7 +500,11 @@ hipError_t vc_launch_chain_plan(const VcSched &S, VcTables T, const int64_t *slo
                                 const int64_t *chain_row_base, const int64_t *chain_chunk_pre, int64_t *items, int64_t nitems,
                                 hipStream_t st) {
     const int nchunk = (S.P + VC_THREADS - 1) / VC_THREADS;
-    const int slices = nchunk > 1 ? 1 : vc_emit_slices(nitems, S.P);
+    // at least ~1024 workgroups (four per compute unit): the kernel is a chain of dependent table reads per workgroup, and
+    // one workgroup per compute unit hides none of them (256 ranks: 23.5 us with one slice)
+    int slices = nchunk > 1 ? 1 : vc_emit_slices(nitems, S.P);
+    if (nchunk == 1)
+        while (slices < 16 && (int64_t)S.P * slices < 1024 && S.P / (slices * 2) >= 16) slices *= 2;
     hipLaunchKernelGGL(vc_chain_emit, dim3(S.P, nchunk * slices), dim3(VC_THREADS), 0, st, S, T, slot_off, row_base, chain_row_base,
                        chain_chunk_pre, slices, items);
     return hipGetLastError();
