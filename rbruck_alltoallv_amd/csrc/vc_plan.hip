@@ -216,10 +216,11 @@ __global__ __launch_bounds__(VC_THREADS) void vc_plan_bases(VcSched S, int P, in
         return;
     }
     if (L == nl && recycle) {
-        // reused staging: row bases inside every sub-region, the sub-regions' sizes, their places in the arena
-        __shared__ int64_t family_size[VC_RECYCLE_MAX_PAIRS], family_base[VC_RECYCLE_MAX_PAIRS], hole_lo[VC_RECYCLE_MAX_PAIRS],
-            hole_hi[VC_RECYCLE_MAX_PAIRS];
-        const int ns = nreg + 1, nfam = ns * ns + 1;
+        // reused staging: row offsets inside every sub-region, the sizes of the sub-regions' pieces (the rows of
+        // vc_recycle_rows_per_segment(P) consecutive receivers each), their places in the arena
+        __shared__ int64_t piece_size[VC_RECYCLE_MAX_PAIRS * VC_RECYCLE_SEGMENTS], piece_base[VC_RECYCLE_MAX_PAIRS * VC_RECYCLE_SEGMENTS],
+            hole_lo[VC_RECYCLE_MAX_HOLES], hole_hi[VC_RECYCLE_MAX_HOLES];
+        const int ns = nreg + 1, nfam = ns * ns + 1, nseg = VC_RECYCLE_SEGMENTS, rps = vc_recycle_rows_per_segment(P);
         for (int f = 0; f < nfam; f++) {
             const int ka = f / ns, kd = f % ns;
             const bool used = f == ns * ns ? w > nreg : (ka < nreg && vc_slot_time(S, kd) > vc_slot_time(S, ka));
@@ -229,16 +230,28 @@ __global__ __launch_bounds__(VC_THREADS) void vc_plan_bases(VcSched S, int P, in
                     const int i = b0 + threadIdx.x;
                     int64_t total;
                     const int64_t ex = vc_block_exclusive_scan((i < P) ? row_tot[(int64_t)f * P + i] : 0, lds, total);
-                    if (i < P) row_base[(int64_t)f * P + i] = fam_carry + ex;
+                    if (i < P) {
+                        row_base[(int64_t)f * P + i] = fam_carry + ex;
+                        if (i % rps == 0) piece_base[f * nseg + i / rps] = fam_carry + ex;      // where the piece starts (for now)
+                    }
                     fam_carry += total;
                 }
-            if (threadIdx.x == 0) family_size[f] = fam_carry;
+            __syncthreads();
+            if ((int)threadIdx.x < nseg) {
+                const int g = threadIdx.x;
+                const bool has = used && g * rps < P, more = g + 1 < nseg && (g + 1) * rps < P;
+                piece_size[f * nseg + g] = has ? (more ? piece_base[f * nseg + g + 1] : fam_carry) - piece_base[f * nseg + g] : 0;
+            }
+            __syncthreads();
         }
+        if (threadIdx.x == 0) carry = vc_allocate_staging(S, piece_size, piece_base, hole_lo, hole_hi);
         __syncthreads();
-        if (threadIdx.x == 0) carry = vc_allocate_staging(S, family_size, family_base, hole_lo, hole_hi);
-        __syncthreads();
-        for (int64_t i = threadIdx.x; i < (int64_t)nfam * P; i += VC_THREADS)
-            if (family_size[i / P] > 0) row_base[i] += family_base[i / P];
+        for (int64_t i = threadIdx.x; i < (int64_t)nfam * P; i += VC_THREADS) {
+            const int f = (int)(i / P), g = (int)(i % P) / rps;
+            int64_t start = 0;                            // offset of the piece's first row inside the sub-region
+            for (int k = 0; k < g; k++) start += piece_size[f * nseg + k];
+            if (piece_size[f * nseg + g] > 0) row_base[i] += piece_base[f * nseg + g] - start;
+        }
         int64_t bad = 0;
         for (int i = threadIdx.x; i < P; i += VC_THREADS) { bytes += row_bytes[(int64_t)nsum * P + i]; bad += row_bytes[(int64_t)(nsum + 1) * P + i]; }
         bytes = vc_block_sum(bytes, lds);

@@ -425,58 +425,84 @@ VC_HD int vc_next_hop(const VcSched &S, int s, int t, int k) {
     return -1;
 }
 
-// Where the sub-regions of reused staging go.  size[family] (family = arrival slot * slots + departure slot; the
-// organized region at slots * slots) are the bytes of the sub-regions, multiples of VC_LINE; base[family] receives
-// their offsets in the arena; returns the arena's size.  A sub-region is written in the launches of its arrival slot
-// and read for the last time in those of its departure slot, so its memory is free for sub-regions that arrive in
-// any later slot.  First fit, the longest-lived sub-regions of an arrival slot first.  hole_lo / hole_hi: work space of
-// VC_RECYCLE_MAX_PAIRS entries each.
+// Where the sub-regions of reused staging go.  A sub-region (family = arrival slot * slots + departure slot; the organized
+// region at slots * slots) is written in the launches of its arrival slot and read for the last time in those of its
+// departure slot, so its memory is free for sub-regions that arrive in any later slot.  A hole seldom has the size of a
+// whole sub-region, so sub-regions are placed in VC_RECYCLE_SEGMENTS pieces, each the rows of a run of consecutive
+// receiving ranks: size[family * VC_RECYCLE_SEGMENTS + g] are the bytes of the pieces (multiples of VC_LINE), base[...]
+// receives their offsets in the arena; returns the arena's size.  First fit from the low end of the arena, the
+// longest-lived sub-regions of an arrival slot first; the holes are kept sorted and merged, so the pieces of a sub-region
+// that leaves become one hole again where they were neighbours.  This is the reference's economy — only the P - K - 1
+// multi-hop slots, reused every round (src/twophase_tunable_rbruckv-om.cpp:52-86, src/tuna.cpp:36-52,93-97) — for compact
+// slots of variable length.  hole_lo / hole_hi: work space of VC_RECYCLE_MAX_HOLES entries each.
+#define VC_RECYCLE_SEGMENTS 8
+#define VC_RECYCLE_MAX_HOLES 256
+
+VC_HD void vc_hole_add(int64_t *lo, int64_t *hi, int &nh, int64_t a, int64_t b, int64_t &top) {
+    if (a >= b) return;
+    int i = 0;
+    while (i < nh && lo[i] < a) i++;
+    if (i > 0 && hi[i - 1] == a) {
+        hi[--i] = b;                                      // grows the hole below it
+    } else {
+        if (nh == VC_RECYCLE_MAX_HOLES) return;           // (the bytes stay unused for the rest of the call)
+        for (int k = nh; k > i; k--) { lo[k] = lo[k - 1]; hi[k] = hi[k - 1]; }
+        lo[i] = a; hi[i] = b; nh++;
+    }
+    if (i + 1 < nh && hi[i] == lo[i + 1]) {               // ... and meets the hole above it
+        hi[i] = hi[i + 1];
+        for (int k = i + 1; k + 1 < nh; k++) { lo[k] = lo[k + 1]; hi[k] = hi[k + 1]; }
+        nh--;
+    }
+    if (hi[nh - 1] == top) top = lo[--nh];                // the top of the arena comes back
+}
+
+VC_HD int64_t vc_hole_take(int64_t *lo, int64_t *hi, int &nh, int64_t size, int64_t &top, int64_t &peak) {
+    for (int i = 0; i < nh; i++)
+        if (hi[i] - lo[i] >= size) {
+            const int64_t at = lo[i];
+            lo[i] += size;
+            if (lo[i] == hi[i]) {
+                for (int k = i; k + 1 < nh; k++) { lo[k] = lo[k + 1]; hi[k] = hi[k + 1]; }
+                nh--;
+            }
+            return at;
+        }
+    const int64_t at = top;
+    top += size;
+    if (top > peak) peak = top;
+    return at;
+}
+
 VC_HD int64_t vc_allocate_staging(const VcSched &S, const int64_t *size, int64_t *base, int64_t *hole_lo, int64_t *hole_hi) {
-    const int ns = S.w + S.w2 + 1, org = ns * ns;
+    const int ns = S.w + S.w2 + 1, org = ns * ns, nseg = VC_RECYCLE_SEGMENTS;
     int nh = 0;
     int64_t top = 0, peak = 0;
-    base[org] = 0;                                        // lives from the first launch to the last
-    top = peak = size[org];
+    for (int g = 0; g < nseg; g++)                        // the organized region lives from the first launch to the last
+        base[org * nseg + g] = size[org * nseg + g] > 0 ? vc_hole_take(hole_lo, hole_hi, nh, size[org * nseg + g], top, peak) : 0;
     for (int ta = 0; ta < ns; ta++) {
         if (ta >= 1) {                                    // what the launches of the slot before have read for the last time
             const int kd = vc_slot_time(S, ta - 1);
             for (int ka = 0; ka < ns - 1; ka++)
-                if (size[ka * ns + kd] > 0 && vc_slot_time(S, ka) < ta - 1) {
-                    hole_lo[nh] = base[ka * ns + kd]; hole_hi[nh] = hole_lo[nh] + size[ka * ns + kd]; nh++;
-                }
-            for (bool again = true; again;) {             // merge neighbours, give the top of the arena back
-                again = false;
-                for (int a = 0; a < nh && !again; a++) {
-                    if (hole_hi[a] == top) { top = hole_lo[a]; hole_lo[a] = hole_lo[nh - 1]; hole_hi[a] = hole_hi[nh - 1]; nh--; again = true; break; }
-                    for (int b = 0; b < nh; b++)
-                        if (b != a && hole_hi[a] == hole_lo[b]) {
-                            hole_hi[a] = hole_hi[b]; hole_lo[b] = hole_lo[nh - 1]; hole_hi[b] = hole_hi[nh - 1]; nh--; again = true; break;
-                        }
-                }
-            }
+                if (vc_slot_time(S, ka) < ta - 1)
+                    for (int g = 0; g < nseg; g++) {
+                        const int u = (ka * ns + kd) * nseg + g;
+                        if (size[u] > 0) vc_hole_add(hole_lo, hole_hi, nh, base[u], base[u] + size[u], top);
+                    }
         }
         const int ka = vc_slot_time(S, ta);
         if (ka >= ns - 1) continue;                       // the last slot has no staging region
         for (int td = ns - 1; td > ta; td--) {
             const int f = ka * ns + vc_slot_time(S, td);
-            const int64_t sz = size[f];
-            if (sz <= 0) { base[f] = 0; continue; }
-            int best = -1;
-            for (int a = 0; a < nh; a++)
-                if (hole_hi[a] - hole_lo[a] >= sz && (best < 0 || hole_lo[a] < hole_lo[best])) best = a;
-            if (best >= 0) {
-                base[f] = hole_lo[best];
-                hole_lo[best] += sz;
-                if (hole_lo[best] == hole_hi[best]) { hole_lo[best] = hole_lo[nh - 1]; hole_hi[best] = hole_hi[nh - 1]; nh--; }
-            } else {
-                base[f] = top;
-                top += sz;
-                if (top > peak) peak = top;
-            }
+            for (int g = 0; g < nseg; g++)
+                base[f * nseg + g] = size[f * nseg + g] > 0 ? vc_hole_take(hole_lo, hole_hi, nh, size[f * nseg + g], top, peak) : 0;
         }
     }
     return peak;
 }
+
+// Receiving ranks per piece of a sub-region, and the piece a rank's row belongs to.
+VC_HD int vc_recycle_rows_per_segment(int P) { return (P + VC_RECYCLE_SEGMENTS - 1) / VC_RECYCLE_SEGMENTS; }
 
 // The route of block (s, t) in closed form: does it move in hop slot k, and where to?  After digit x of a Bruck that
 // runs least significant digit first a block has travelled (offset mod r^(x+1)) ranks down from its source, most

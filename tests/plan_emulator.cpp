@@ -79,7 +79,9 @@ extern "C" int plan_emulate(int func, int P, int n, int r, int batch, int esz, i
         // the planner's passes for reused staging: slots numbered per (arrival, departure) family, rows inside a family,
         // families placed by the allocator the planning kernel uses
         const int ns = S.w + S.w2 + 1, nfam = ns * ns + 1;
-        std::vector<int64_t> row_tot((int64_t)nfam * P, 0), fam_size(nfam, 0), fam_base(nfam, 0), hole_lo(VC_RECYCLE_MAX_PAIRS), hole_hi(VC_RECYCLE_MAX_PAIRS);
+        const int nseg = VC_RECYCLE_SEGMENTS, rps = vc_recycle_rows_per_segment(P);
+        std::vector<int64_t> row_tot((int64_t)nfam * P, 0), piece_size((size_t)nfam * nseg, 0), piece_base((size_t)nfam * nseg, 0),
+            hole_lo(VC_RECYCLE_MAX_HOLES), hole_hi(VC_RECYCLE_MAX_HOLES);
         for (int y = 0; y < S.w + S.w2; y++)
             for (int to = 0; to < P; to++) {
                 std::vector<int64_t> carry(ns, 0);
@@ -103,15 +105,25 @@ extern "C" int plan_emulate(int func, int P, int n, int r, int batch, int esz, i
                     slot_off[((int64_t)S.w * P + to) * P + id] = run_base[id / S.n] + vc_org_slot_rel(S, T, to, id);
                 row_tot[(int64_t)(ns * ns) * P + to] = acc;
             }
+        // a sub-region is placed in pieces: the rows of rps consecutive receivers each
         for (int f = 0; f < nfam; f++) {
             int64_t acc = 0;
-            for (int to = 0; to < P; to++) { row_base[(int64_t)f * P + to] = acc; acc += row_tot[(int64_t)f * P + to]; }
-            fam_size[f] = acc;
+            for (int to = 0; to < P; to++) {
+                row_base[(int64_t)f * P + to] = acc;
+                piece_size[(size_t)f * nseg + to / rps] += row_tot[(int64_t)f * P + to];
+                acc += row_tot[(int64_t)f * P + to];
+            }
         }
-        stage_bytes = vc_allocate_staging(S, fam_size.data(), fam_base.data(), hole_lo.data(), hole_hi.data());
+        stage_bytes = vc_allocate_staging(S, piece_size.data(), piece_base.data(), hole_lo.data(), hole_hi.data());
         for (int f = 0; f < nfam; f++) {
-            if (fam_size[f] > 0 && fam_base[f] + fam_size[f] > stage_bytes) return -102;
-            for (int to = 0; to < P; to++) row_base[(int64_t)f * P + to] += fam_base[f];
+            int64_t start = 0;
+            for (int g = 0; g < nseg; g++) {
+                const size_t u = (size_t)f * nseg + g;
+                if (piece_size[u] > 0 && piece_base[u] + piece_size[u] > stage_bytes) return -102;
+                for (int to = g * rps; to < P && to < (g + 1) * rps; to++)
+                    if (piece_size[u] > 0) row_base[(int64_t)f * P + to] += piece_base[u] - start;
+                start += piece_size[u];
+            }
         }
     }
     for (int x = 0; x < S.w + S.w2 && !S.stride && !S.recycle; x++) {
@@ -282,12 +294,13 @@ extern "C" int plan_emulate(int func, int P, int n, int r, int batch, int esz, i
     return 0;
 }
 
-// The staging allocator of the planning kernel on its own: sizes per (arrival, departure) family in, bases out.
+// The staging allocator of the planning kernel on its own: sizes per piece of every (arrival, departure) family in
+// (VC_RECYCLE_SEGMENTS pieces per family), bases out.
 extern "C" int64_t staging_allocate(int w, int w2, int msd, int coalesce, const int64_t *size, int64_t *base) {
     VcSched S;
     memset(&S, 0, sizeof S);
     S.w = w; S.w2 = w2; S.msd = msd; S.coalesce = coalesce; S.recycle = 1;
-    std::vector<int64_t> lo(VC_RECYCLE_MAX_PAIRS), hi(VC_RECYCLE_MAX_PAIRS);
+    std::vector<int64_t> lo(VC_RECYCLE_MAX_HOLES), hi(VC_RECYCLE_MAX_HOLES);
     return vc_allocate_staging(S, size, base, lo.data(), hi.data());
 }
 
@@ -307,5 +320,7 @@ extern "C" int dispatch_decision(int func, int P, int n, int r, int mode, int ca
     out[5] = d.guard.max_average; out[6] = d.guard.max_len;
     return 0;
 }
+
+extern "C" int recycle_segments() { return VC_RECYCLE_SEGMENTS; }
 
 extern "C" int lanes_for_items(int64_t bytes, int64_t items) { return vc_lanes_for_items(bytes, items); }

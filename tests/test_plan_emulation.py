@@ -536,10 +536,10 @@ def test_strided_plans_all_radices(P, strided):
 
 @pytest.mark.parametrize("P,r,func", [(64, 2, "tuna"), (64, 2, "twophase"), (81, 3, "om"), (100, 2, "twophase"), (50, 3, "tuna"),
                                       (64, 4, "om"), (128, 2, "tuna")])
-def test_reused_staging_is_smaller_and_stays_below_twice_the_payload(P, r, func):
+def test_reused_staging_is_smaller_and_stays_below_one_and_a_half_payloads(P, r, func):
     """A sub-region of staging takes the memory of sub-regions whose blocks have all left before it is written.  The
     emulator checks every launch (nothing lands on bytes that still wait for their next hop, every staged byte is read
-    exactly once, all have left at the end); here: the arena shrinks and stays below twice the payload, on all-pairs
+    exactly once, all have left at the end); here: the arena shrinks and stays below 1.5 x the payload, on all-pairs
     traffic and on the pencil pattern of configuration 5 (rows of a grid)."""
     fn = {"tuna": lambda rec, p, s, d: E.emulate(E.F_TUNA, p, s, d, r=r, recycle=rec),
           "twophase": lambda rec, p, s, d: E.emulate(E.F_TWOPHASE, p, s, d, r=r, recycle=rec),
@@ -555,8 +555,9 @@ def test_reused_staging_is_smaller_and_stays_below_twice_the_payload(P, r, func)
             assert res.rc == 0 and res.errors == 0, (P, r, func, rec, res.errors)
             assert np.array_equal(recv, want)
             sizes.append(res.stage_bytes)
-        assert sizes[1] <= sizes[0] and (r > 2 or sizes[1] < 0.8 * sizes[0]), sizes      # (first fit: a hole must hold a whole sub-region)
-        assert sizes[1] <= 2 * prob.payload_bytes + 128 * P * P, (sizes, prob.payload_bytes)
+        assert sizes[1] <= sizes[0] and (r > 2 or sizes[1] < 0.8 * sizes[0]), sizes
+        # sub-regions are placed in pieces (a hole need not hold a whole one): close to what is alive at the worst moment
+        assert sizes[1] <= 1.5 * prob.payload_bytes + 128 * P * P, (sizes, prob.payload_bytes)
 
 
 @pytest.mark.parametrize("P,n,r", [(64, 8, 2), (64, 16, 2), (81, 27, 3), (128, 32, 2), (64, 8, 3)])
@@ -585,34 +586,41 @@ def test_reused_staging_twolayer(P, n, r):
 
 @pytest.mark.parametrize("msd", [0, 1])
 def test_staging_allocator_never_overlaps_live_sub_regions(msd):
-    """vc_allocate_staging on random sizes: two sub-regions whose lifetimes (arrival slot .. departure slot, in the call's
-    order) touch never share memory; the arena is no larger than separate regions and no smaller than the most bytes alive
-    during any digit's launches."""
+    """vc_allocate_staging on random sizes: the pieces of two sub-regions whose lifetimes (arrival slot .. departure slot, in
+    the call's order) touch never share memory, nor do two pieces of one sub-region; the arena is no larger than separate
+    regions and no smaller than the most bytes alive during any digit's launches."""
     import ctypes as C
     lib = C.CDLL(E.build())
     lib.staging_allocate.restype = C.c_int64
+    nseg = lib.recycle_segments()
     rng = np.random.default_rng(7 + msd)
+    excess = []
     for trial in range(300):
         w = int(rng.integers(1, 9))
         w2 = int(rng.integers(0, 11 - w)) if not msd else 0
         ns = w + w2 + 1
         time = lambda k: (w - 1 - k) if (k < w and msd) else k
-        size = np.zeros(ns * ns + 1, dtype=np.int64)
+        size = np.zeros((ns * ns + 1, nseg), dtype=np.int64)
         fams = [(ka, kd) for ka in range(ns - 1) for kd in range(ns) if time(kd) > time(ka)]
         for ka, kd in fams:
             if rng.random() < 0.8:
-                size[ka * ns + kd] = 128 * int(rng.integers(1, 2000))
+                size[ka * ns + kd] = 128 * rng.integers(0, 300, size=nseg) * (rng.random(nseg) < 0.9)
         if rng.random() < 0.3:
-            size[ns * ns] = 128 * int(rng.integers(1, 500))
+            size[ns * ns] = 128 * rng.integers(1, 70, size=nseg)
         base = np.zeros_like(size)
-        peak = lib.staging_allocate(w, w2, msd, int(size[ns * ns] > 0), size.ctypes.data_as(C.c_void_p), base.ctypes.data_as(C.c_void_p))
-        live = [(time(ka), time(kd), int(base[ka * ns + kd]), int(size[ka * ns + kd])) for ka, kd in fams if size[ka * ns + kd]]
-        if size[ns * ns]:
-            live.append((0, ns - 1, int(base[ns * ns]), int(size[ns * ns])))
+        peak = lib.staging_allocate(w, w2, msd, int(size[ns * ns].sum() > 0), size.ctypes.data_as(C.c_void_p), base.ctypes.data_as(C.c_void_p))
+        live = [(time(ka), time(kd), int(base[ka * ns + kd, g]), int(size[ka * ns + kd, g])) for ka, kd in fams for g in range(nseg)
+                if size[ka * ns + kd, g]]
+        live += [(0, ns - 1, int(base[ns * ns, g]), int(size[ns * ns, g])) for g in range(nseg) if size[ns * ns, g]]
         for i, (a0, d0, b0, s0) in enumerate(live):
             assert 0 <= b0 and b0 + s0 <= peak
             for a1, d1, b1, s1 in live[i + 1:]:
                 if a0 <= d1 and a1 <= d0:                      # alive during the launches of a common slot
                     assert b0 + s0 <= b1 or b1 + s1 <= b0, (trial, (a0, d0, b0, s0), (a1, d1, b1, s1))
         assert peak <= int(size.sum())
-        assert peak >= max(sum(s for a, d, _, s in live if a <= t <= d) for t in range(ns))
+        need = max(sum(s for a, d, _, s in live if a <= t <= d) for t in range(ns)) if live else 0
+        assert peak >= need
+        if need:
+            excess.append(peak / need)
+    # placing sub-regions in pieces keeps the arena close to what is alive at the worst moment
+    assert np.median(excess) < 1.1 and max(excess) < 1.6, (np.median(excess), max(excess))
