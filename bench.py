@@ -424,6 +424,8 @@ def main() -> None:
     ap.add_argument("--no-context", action="store_true", help="skip the context figures beside the metric (plans, graph, the other "
                                                              "execution mode, comparator, short-block calls): for profiling runs")
     ap.add_argument("--cpu-budget", type=float, default=150.0)
+    ap.add_argument("--only-metadata", action="store_true",
+                    help="only the caller-side metadata steps on the workload's count table (for profiling their kernels); prints their record")
     ap.add_argument("--calibration-copy", type=int, default=0, metavar="MiB",
                     help="also run one plain copy of this many MiB before the timed region (for scaling rocprofv3 --pmc byte counters)")
     args = ap.parse_args()
@@ -431,12 +433,23 @@ def main() -> None:
         raise SystemExit("bench.py: this build runs the virtual communicator on ONE GPU; --gpus N with N > 1 is not supported")
 
     # the CPU leg starts child processes (mpiexec) and needs nothing from the GPU: it runs before anything here touches the device
-    cpu = None if args.no_cpu_baseline else cpu_reference_leg(args.workload, args.seed, args.cpu_budget)
+    cpu = None if args.no_cpu_baseline or args.only_metadata else cpu_reference_leg(args.workload, args.seed, args.cpu_budget)
 
     import torch
     from rbruck_alltoallv_amd import api
 
     counts, esz, func, tun, hops = workload(args.workload, args.seed)
+    if args.only_metadata:
+        if args.calibration_copy:                          # the transfer of known size the byte counters are scaled against
+            comm = api.VirtualComm(2)
+            nb = args.calibration_copy << 20
+            a = torch.zeros(nb, dtype=torch.uint8, device="cuda:0")
+            b = torch.zeros(nb, dtype=torch.uint8, device="cuda:0")
+            comm._check(comm.lib.vc_calibration_copy(b.data_ptr(), a.data_ptr(), nb, comm.handle))
+            comm.free()
+            del a, b
+        print(json.dumps({"metadata_us": metadata_calls(api, torch, counts)}), flush=True)
+        return
     if args.func:
         func = args.func
     if args.radix:
