@@ -149,7 +149,7 @@ hipError_t vc_launch_empty(hipStream_t st);
 #define VC_HEADER_SYNC (VC_HEADER_MAX_LEN + 1)
 // ... wavefronts that have checked their part of the tables and added what they found to VC_HEADER_BAD: the copying
 // wavefronts of the same launch store nothing before all of them have
-#define VC_HEADER_VERDICT (VC_HEADER_SYNC + 1)
+#define VC_HEADER_CHECKED (VC_HEADER_SYNC + 1)
 // ... set (in the host's copy of the header only) by a copying wavefront that gave up waiting for that: the call is redone
 #define VC_HEADER_STALLED (VC_HEADER_SYNC + 2)
 #define VC_HEADER_WORDS(nl) (VC_HEADER_FIXED + 2 * (nl))

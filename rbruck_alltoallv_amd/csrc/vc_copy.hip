@@ -254,7 +254,7 @@ __device__ __forceinline__ void vc_add_totals(const VcSched &S, const VcTables &
     bad = vc_wave_sum(bad);
     // one word says it all, so one atomic publishes it: wavefronts that have reported in the low half, wavefronts that
     // found something wrong in the high half
-    if (lane == 0) atomicAdd(&h[VC_HEADER_VERDICT], 1ull | (bad ? 1ull << 32 : 0ull));
+    if (lane == 0) atomicAdd(&h[VC_HEADER_CHECKED], 1ull | (bad ? 1ull << 32 : 0ull));
 #pragma unroll
     for (int u = 0; u < VC_TOTALS_PER_LANE; u++) {
         const int64_t idx = wave * per_wave + u * VC_WAVE + lane;
@@ -299,11 +299,11 @@ __device__ __forceinline__ void vc_add_totals(const VcSched &S, const VcTables &
 
 // A copying wavefront of the single launch asks before its first store: have all totalling wavefronts checked their part of
 // the tables, and did they find them in order?  The totalling workgroups are the first of the grid, so they are resident
-// before any copying one; the wait is bounded all the same (VC_VERDICT_SPINS polls, a few milliseconds): a wavefront that
+// before any copying one; the wait is bounded all the same (VC_CHECK_SPINS polls, a few milliseconds): a wavefront that
 // gives up moves nothing and says so in the host's copy of the header, and the host redoes the call the general way.
-#define VC_VERDICT_SPINS (1 << 15)
+#define VC_CHECK_SPINS (1 << 15)
 __device__ __forceinline__ unsigned long long vc_verdict_word(int64_t *totals) {
-    return __hip_atomic_load(reinterpret_cast<unsigned long long *>(totals) + VC_HEADER_VERDICT, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    return __hip_atomic_load(reinterpret_cast<unsigned long long *>(totals) + VC_HEADER_CHECKED, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 // Asked by the piece movers between their loads and their stores (see vc_forward_piece).  Without `totals` there is nothing
@@ -318,7 +318,7 @@ struct VcVerdictGate {
         if (!totals) return true;
         for (int spin = 0; state == 0; spin++) {
             if ((word & 0xFFFFFFFFull) >= nwaves) state = (word >> 32) ? 2 : 1;
-            else if (spin >= VC_VERDICT_SPINS) { header_host[VC_HEADER_STALLED] = 1; state = 2; }
+            else if (spin >= VC_CHECK_SPINS) { header_host[VC_HEADER_STALLED] = 1; state = 2; }
             else { __builtin_amdgcn_s_sleep(4); word = vc_verdict_word(totals); }
         }
         return state == 1;
@@ -380,7 +380,7 @@ __global__ __launch_bounds__(LANES) void vc_copy_blocks_kernel(VcSched S, VcTabl
     const int64_t recv_off = vc_recv_offset(S, T, s, t);
     int64_t dst = 0;
     const bool moves = threadIdx.x < VC_WAVE && (int)threadIdx.x < vc_hop_slots(S) && vc_block_hop(S, T, slot_off, row_base, s, t, threadIdx.x, dst);
-    if (block == 0 && first_pair == 0 && threadIdx.x <= VC_HEADER_VERDICT) {
+    if (block == 0 && first_pair == 0 && threadIdx.x <= VC_HEADER_CHECKED) {
         if (header_host && !totals && threadIdx.x <= VC_HEADER_MAX_LEN) header_host[threadIdx.x] = header[threadIdx.x];
         if (header_zero) header_zero[threadIdx.x] = 0;    // the header the next call will add up into
     }
@@ -436,7 +436,7 @@ __global__ __launch_bounds__(VC_WAVE) void vc_copy_blocks_quarter_kernel(VcSched
     int64_t d0 = 0, d1 = 0;
     const bool m0 = active && q < nslots && vc_block_hop(S, T, slot_off, row_base, s, t, q, d0);
     const bool m1 = active && q + VC_QUARTER < nslots && vc_block_hop(S, T, slot_off, row_base, s, t, q + VC_QUARTER, d1);
-    if (block == 0 && first_pair == 0 && threadIdx.x <= VC_HEADER_VERDICT) {
+    if (block == 0 && first_pair == 0 && threadIdx.x <= VC_HEADER_CHECKED) {
         if (header_host && !totals && threadIdx.x <= VC_HEADER_MAX_LEN) header_host[threadIdx.x] = header[threadIdx.x];
         if (header_zero) header_zero[threadIdx.x] = 0;
     }
