@@ -31,7 +31,7 @@ from rbruck_alltoallv_amd import workloads as W  # noqa: E402
 HBM_PEAK_GBPS = 8000.0
 METRIC = "effective alltoallv GB/s + % HBM peak, P=64..1024 virtual ranks, 1 GPU"
 # the sources the copy kernels are built from: a counter profile under profiles/ is only quoted while they are unchanged
-KERNEL_SOURCES = ("vc_copy.hip", "vc_plan.hip", "vc_plan_math.h", "vc_common.h", "vc_scan.h")
+KERNEL_SOURCES = ("vc_copy.hip", "vc_plan.hip", "vc_plan_math.h", "vc_common.h", "vc_scan.h", "vc_dispatch.h")
 
 
 def kernel_sources_sha() -> str:

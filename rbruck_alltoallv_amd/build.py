@@ -7,7 +7,7 @@ import subprocess
 PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(PKG_DIR, "csrc")
 LIB_PATH = os.path.join(PKG_DIR, "librbruck_vc.so")
-SOURCES = ["vc_meta.hip", "vc_plan.hip", "vc_copy.hip", "vc_api.hip"]
+SOURCES = ["vc_meta.hip", "vc_plan.hip", "vc_copy.hip", "vc_api.hip", "vc_tools.hip"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 # packed FP32 instructions stay off for every HIP translation unit of this library
 FLAGS = ["--offload-arch=gfx950", "-O3", "-fPIC", "-shared", "-std=c++17", "-Wall",
