@@ -200,7 +200,7 @@ static PlanBufSizes plan_buf_sizes(const VcSched &S, int nl, bool forward) {
     z.org_run_base = sizeof(int64_t) * P * (size_t)std::max(S.G, 1);
     z.item_row_tot = z.item_row_base = sizeof(int64_t) * P * (size_t)std::max(nl, 1);
     z.row_bytes = sizeof(int64_t) * P * (size_t)(std::max(nl, S.w + S.w2) + 3);
-    z.chain_row_tot = forward ? sizeof(int64_t) * (2 + (P + VC_THREADS - 1) / VC_THREADS) * P : 0;
+    z.chain_row_tot = forward ? sizeof(int64_t) * (2 + VC_TILES(P)) * P : 0;
     z.chain_row_base = forward ? sizeof(int64_t) * P : 0;
     z.header = sizeof(int64_t) * VC_HEADER_WORDS(VC_MAX_LAUNCHES);
     z.launches = sizeof(VcLaunchInfo) * VC_MAX_LAUNCHES;
@@ -311,8 +311,8 @@ static int plan_emit(vc_comm *c, const VcSched &S, std::vector<VcLaunchInfo> &L,
     if (pi.chain) {
         if (!c->B.chain_row_base || !c->B.chain_row_tot) return fail_arg("internal: chain items asked for a plan that was not sized for them", VC_ERR_HIP);
         HIP_TRY(items.reserve(sizeof(int64_t) * (size_t)pi.chain_stride * (size_t)std::max<int64_t>(pi.chain_items, 1)));
-        HIP_TRY(vc_launch_chain_plan(S, T, c->B.slot_off, c->B.row_base, c->B.chain_row_base, c->B.chain_row_tot + 2 * (size_t)S.P,
-                                     items.as<int64_t>(), pi.chain_items, st));
+        HIP_TRY(vc_launch_chain_plan(S, T, c->B.slot_off, c->B.row_base, c->B.chain_row_tot + 2 * (size_t)S.P, items.as<int64_t>(),
+                                     pi.chain_items, st));
     } else {
         HIP_TRY(items.reserve(sizeof(VcDesc) * (size_t)std::max<int64_t>(pi.items_total, 1)));
         HIP_TRY(vc_launch_plan_emit(S, L.data(), c->B.launches, pi.nl, T, c->B.slot_off, c->B.row_base, c->B.item_row_base, c->B.header,

@@ -102,6 +102,12 @@ struct VcLaunchInfo {
     int self;      // also performs every rank's copy to itself
 };
 
+// Forwarded execution lists its chain items in tiles of VC_TILE_RANKS receivers x VC_TILE_RANKS sources (receiver by
+// receiver inside a tile) instead of all sources of a receiver in a row: neighbours in the list then read from few send
+// buffers and write to few receive buffers, each in runs of consecutive blocks.
+#define VC_TILE_RANKS 32
+#define VC_TILES(P) (((P) + VC_TILE_RANKS - 1) / VC_TILE_RANKS)
+
 #define VC_LAUNCH_PACK 16
 struct VcLaunchPack { VcLaunchInfo info[VC_LAUNCH_PACK]; };
 
@@ -155,7 +161,8 @@ hipError_t vc_launch_empty(hipStream_t st);
 #define VC_HEADER_WORDS(nl) (VC_HEADER_FIXED + 2 * (nl))
 // Passes 1 and 2: staging prefix sums and the number of work items of every launch (sizes only).  The launch table
 // travels as a kernel argument when it has at most VC_LAUNCH_PACK entries (launches_dev is then not read).  With chain_row_tot /
-// chain_row_base ((2 + ceil(P / VC_THREADS)) P and P int64, or null) also the chain items per final receiver, their total in header[2] and the most
+// chain_row_base ((2 + VC_TILES(P)) P and P int64, or null) also the chain items per final receiver, the first item of every
+// (receiver, tile of sources) in the list's tiled order (behind chain_row_tot's first 2 P words), their total in header[2] and the most
 // pieces of any block in header[4].
 hipError_t vc_launch_plan_sizes(const VcSched &S, const VcLaunchInfo *launches_host, const VcLaunchInfo *launches_dev, int nlaunch,
                                 VcTables T, int64_t *slot_off,
@@ -163,11 +170,10 @@ hipError_t vc_launch_plan_sizes(const VcSched &S, const VcLaunchInfo *launches_h
                                 int64_t *item_row_base, int64_t *row_bytes, int64_t *chain_row_tot, int64_t *chain_row_base,
                                 int64_t *header, int64_t *header_host, hipStream_t st);
 // Forwarded execution: the chain items (every block's route in closed form, staging addresses from the plan tables).
-// chain_chunk_pre: [P][chunks of VC_THREADS sources] items of a receiver before each chunk (vc_launch_plan_sizes leaves it
-// behind chain_row_tot's first 2 P words).
+// chain_tile_base: [P][VC_TILES(P)] first item of every (receiver, tile of sources) (vc_launch_plan_sizes leaves it behind
+// chain_row_tot's first 2 P words).
 hipError_t vc_launch_chain_plan(const VcSched &S, VcTables T, const int64_t *slot_off, const int64_t *row_base,
-                                const int64_t *chain_row_base, const int64_t *chain_chunk_pre, int64_t *items, int64_t nitems,
-                                hipStream_t st);
+                                const int64_t *chain_tile_base, int64_t *items, int64_t nitems, hipStream_t st);
 // Pass 3: writes the work items (needs the item buffer, sized from the header).
 hipError_t vc_launch_plan_emit(const VcSched &S, const VcLaunchInfo *launches_host, const VcLaunchInfo *launches_dev, int nlaunch,
                                VcTables T, const int64_t *slot_off,

@@ -92,10 +92,11 @@ __global__ __launch_bounds__(VC_THREADS) void vc_plan_rows(VcSched S, VcLaunchPa
     int64_t bad = 0;                                      // entries of this rank's rows no rank could have passed
     const int L = blockIdx.y - nreg;
     if (forward) {
-        // sources in chunks of VC_THREADS: the items before each chunk let vc_chain_emit give every chunk a workgroup.
+        // sources in chunks of VC_THREADS; the items of every tile of VC_TILE_RANKS sources (half a wavefront) are left for
+        // vc_plan_bases, which turns them into the first item of every (receiver, tile) in the list's tiled order.
         // Four chunks at a time, so that the table reads of all of them travel together before the first sum needs them;
         // the checks of this rank's own rows (the loop over ids below, for launch-per-digit execution) ride along.
-        const int nchunk = (P + VC_THREADS - 1) / VC_THREADS;
+        const int nchunk = (P + VC_THREADS - 1) / VC_THREADS, ntile = VC_TILES(P);
         int64_t before = 0;
         for (int chunk0 = 0; chunk0 < nchunk; chunk0 += 4) {
             int64_t cnt[4];
@@ -115,7 +116,11 @@ __global__ __launch_bounds__(VC_THREADS) void vc_plan_rows(VcSched S, VcLaunchPa
 #pragma unroll
             for (int u = 0; u < 4; u++) {
                 if (chunk0 + u >= nchunk) break;
-                if (threadIdx.x == 0) chain_row_tot[2 * (int64_t)P + (int64_t)to * nchunk + chunk0 + u] = before;
+                int64_t tile = cnt[u];
+#pragma unroll
+                for (int o = VC_TILE_RANKS / 2; o > 0; o >>= 1) tile += __shfl_xor(tile, o, VC_TILE_RANKS);
+                const int s = (chunk0 + u) * VC_THREADS + threadIdx.x;
+                if (threadIdx.x % VC_TILE_RANKS == 0 && s < P) chain_row_tot[2 * (int64_t)P + (int64_t)to * ntile + s / VC_TILE_RANKS] = tile;
                 before += vc_block_sum(cnt[u], lds);
             }
         }
@@ -181,18 +186,39 @@ __global__ __launch_bounds__(VC_THREADS) void vc_plan_org_rows(VcSched S, VcTabl
 // took twice as long that way.)
 // Launch-per-digit execution: grid (nl + 1).  Workgroup L < nl: item bases of launch L's rows (relative to the launch's
 // first item), its item count and moved bytes.  Workgroup nl: staging row bases, staging bytes, payload bytes, negative
-// table entries.  Forwarded execution (chain_row_tot != null, nl = 0): grid (2).  Workgroup 0 as workgroup nl above, and
-// the moved bytes = payload + bytes of the staged blocks as those of launch 0; workgroup 1: chain item bases.
+// table entries.  Forwarded execution (chain_row_tot != null, nl = 0): grid (2 + tile rows).  Workgroup 0 as workgroup nl above,
+// and the moved bytes = payload + bytes of the staged blocks as those of launch 0; workgroup 1: chain items per receiver summed up
+// (their total, the most pieces, the longest block); workgroup 2 + k: first item of every (receiver, tile of sources) of tile row k.
 __global__ __launch_bounds__(VC_THREADS) void vc_plan_bases(VcSched S, int P, int w, int nreg, int nl, const int64_t *__restrict__ row_tot,
                                                             int64_t *__restrict__ row_base, const int64_t *__restrict__ item_row_tot,
                                                             int64_t *__restrict__ item_row_base, const int64_t *__restrict__ row_bytes,
-                                                            const int64_t *__restrict__ chain_row_tot, int64_t *__restrict__ chain_row_base,
+                                                            int64_t *chain_row_tot, int64_t *__restrict__ chain_row_base,
                                                             int64_t *__restrict__ header, int64_t *__restrict__ header_host) {
     __shared__ int64_t lds[VC_WAVES_PER_BLOCK];
     const int L = blockIdx.x;
     const bool forward = chain_row_tot != nullptr, recycle = S.recycle != 0;
     const int nsum = forward ? nreg : nl;                 // rows of row_bytes before the payload row
     int64_t carry = 0, bytes = 0;
+    if (forward && L >= 2) {
+        // tile row L - 2: the receivers [t0, t1).  The list holds, tile row after tile row, the tiles of sources in turn and
+        // inside a tile the receivers in turn: an exclusive scan over (tile of sources, receiver) of the counts vc_plan_rows
+        // left, in place, started at the items of all receivers before t0.
+        const int ntile = VC_TILES(P), t0 = (L - 2) * VC_TILE_RANKS, rows = (t0 + VC_TILE_RANKS < P ? t0 + VC_TILE_RANKS : P) - t0;
+        int64_t *tile = chain_row_tot + 2 * (int64_t)P;
+        int64_t earlier = 0;
+        for (int i = threadIdx.x; i < t0; i += VC_THREADS) earlier += chain_row_tot[i];
+        carry = vc_block_sum(earlier, lds);
+        const int per = VC_THREADS / VC_TILE_RANKS;       // tiles of sources per pass
+        for (int sb0 = 0; sb0 < ntile; sb0 += per) {
+            const int sb = sb0 + threadIdx.x / VC_TILE_RANKS, row = threadIdx.x % VC_TILE_RANKS;
+            const bool inside = sb < ntile && row < rows;
+            int64_t total;
+            const int64_t ex = vc_block_exclusive_scan(inside ? tile[(int64_t)(t0 + row) * ntile + sb] : 0, lds, total);
+            if (inside) tile[(int64_t)(t0 + row) * ntile + sb] = carry + ex;
+            carry += total;
+        }
+        return;
+    }
     if (forward && L == 1) {                              // first chain item of every final receiver
         int64_t most = 0, longest = 0;
         for (int b0 = 0; b0 < P; b0 += VC_THREADS) {
@@ -399,7 +425,7 @@ hipError_t vc_launch_plan_sizes(const VcSched &S, const VcLaunchInfo *launches_h
                        row_tot, item_row_tot, row_bytes, chain_row_tot);
     if (S.coalesce)
         hipLaunchKernelGGL(vc_plan_org_rows, dim3(S.P), dim3(VC_THREADS), 0, st, S, T, slot_off, row_tot, org_run_base);
-    hipLaunchKernelGGL(vc_plan_bases, dim3(forward ? 2 : nl + 1), dim3(VC_THREADS), 0, st, S, S.P, vc_regions(S), nreg, nl, row_tot, row_base,
+    hipLaunchKernelGGL(vc_plan_bases, dim3(forward ? 2 + VC_TILES(S.P) : nl + 1), dim3(VC_THREADS), 0, st, S, S.P, vc_regions(S), nreg, nl, row_tot, row_base,
                        item_row_tot, item_row_base, row_bytes, chain_row_tot, chain_row_base, header, header_host);
     return hipGetLastError();
 }
@@ -415,14 +441,15 @@ hipError_t vc_launch_plan_emit(const VcSched &S, const VcLaunchInfo *launches_ho
 }
 
 // ---- forwarded execution ----
-// grid (P, chunks x Z): the chain items of the blocks that end on rank t, in source order.  The sources come in chunks of
-// VC_THREADS (vc_plan_rows has counted the items before each chunk); Z workgroups share a chunk when there are few ranks
-// with huge blocks, which would otherwise leave most of the chip idle: workgroup (t, chunk, z) writes the items of the
-// z-th slice of the chunk's sources.  Big blocks are written by the whole workgroup as in vc_plan_emit.
+// grid (P, chunks x Z): the chain items of the blocks that end on rank t.  The list is ordered in tiles of VC_TILE_RANKS
+// receivers x VC_TILE_RANKS sources, receiver by receiver inside a tile (vc_plan_bases has left the first item of every
+// (receiver, tile of sources)); the sources come in chunks of VC_THREADS, and Z workgroups share a chunk (each a whole number
+// of tiles) when there are few ranks, which would otherwise leave most of the chip idle: the kernel is a chain of dependent
+// table reads per workgroup, and one workgroup per compute unit hides none of them.  Big blocks are written by the whole
+// workgroup as in vc_plan_emit.
 __global__ __launch_bounds__(VC_THREADS) void vc_chain_emit(VcSched S, VcTables T, const int64_t *__restrict__ slot_off,
                                                             const int64_t *__restrict__ row_base,
-                                                            const int64_t *__restrict__ chain_row_base,
-                                                            const int64_t *__restrict__ chain_chunk_pre, int slices,
+                                                            const int64_t *__restrict__ chain_tile_base, int slices,
                                                             int64_t *__restrict__ items) {
     __shared__ int64_t lds[VC_WAVES_PER_BLOCK];
     __shared__ int64_t big_at[VC_THREADS], big_pre[VC_THREADS];
@@ -434,18 +461,20 @@ __global__ __launch_bounds__(VC_THREADS) void vc_chain_emit(VcSched S, VcTables 
     const int t = blockIdx.x, P = S.P;
     const int stride = VC_CHAIN_HEAD + vc_hop_slots(S);
     const bool cached = vc_hop_slots(S) <= VC_ROUTE_CACHE;
-    const int nchunk = (P + VC_THREADS - 1) / VC_THREADS;
     const int chunk = (int)blockIdx.y / slices, z = (int)blockIdx.y % slices;
     const int c_lo = chunk * VC_THREADS, c_hi = c_lo + VC_THREADS < P ? c_lo + VC_THREADS : P;
-    const int per = (c_hi - c_lo + slices - 1) / slices;
+    const int per = ((c_hi - c_lo + slices - 1) / slices + VC_TILE_RANKS - 1) / VC_TILE_RANKS * VC_TILE_RANKS;      // whole tiles
     const int s_lo = c_lo + z * per < c_hi ? c_lo + z * per : c_hi, s_hi = s_lo + per < c_hi ? s_lo + per : c_hi;
-    int64_t before = 0;                                   // items of the chunk's earlier sources
-    if (c_lo + (int)threadIdx.x < s_lo) before = vc_chain_count(S, T, c_lo + threadIdx.x, t);
-    const int64_t carry = chain_row_base[t] + chain_chunk_pre[(int64_t)t * nchunk + chunk] + vc_block_sum(before, lds);
     const int s = s_lo + threadIdx.x;                     // one source per lane: a slice has at most VC_THREADS of them
     const int64_t cnt = s < s_hi ? vc_chain_count(S, T, s, t) : 0;
-    int64_t total;
-    const int64_t at = carry + vc_block_exclusive_scan(cnt, lds, total);
+    // the block's first item: the first item of its (receiver, tile of sources) + the items of the tile's earlier sources
+    int64_t upto = cnt;
+#pragma unroll
+    for (int o = 1; o < VC_TILE_RANKS; o <<= 1) {
+        const int64_t below = __shfl_up(upto, o, VC_TILE_RANKS);
+        if ((int)(threadIdx.x % VC_TILE_RANKS) >= o) upto += below;
+    }
+    const int64_t at = (s < s_hi ? chain_tile_base[(int64_t)t * VC_TILES(P) + s / VC_TILE_RANKS] : 0) + upto - cnt;
     const bool big = cnt > 4;
     if (cached && cnt > 0) {
         // the block's route once, in registers (hop slot k in d[k], statically indexed; its table reads go out together); the
@@ -510,16 +539,14 @@ __global__ __launch_bounds__(VC_THREADS) void vc_chain_emit(VcSched S, VcTables 
 }
 
 hipError_t vc_launch_chain_plan(const VcSched &S, VcTables T, const int64_t *slot_off, const int64_t *row_base,
-                                const int64_t *chain_row_base, const int64_t *chain_chunk_pre, int64_t *items, int64_t nitems,
-                                hipStream_t st) {
+                                const int64_t *chain_tile_base, int64_t *items, int64_t nitems, hipStream_t st) {
     const int nchunk = (S.P + VC_THREADS - 1) / VC_THREADS;
-    // at least ~1024 workgroups (four per compute unit): the kernel is a chain of dependent table reads per workgroup, and
-    // one workgroup per compute unit hides none of them (256 ranks: 23.5 us with one slice)
+    // at least ~1024 workgroups (four per compute unit), each a whole number of tiles of sources
     int slices = nchunk > 1 ? 1 : vc_emit_slices(nitems, S.P);
     if (nchunk == 1)
-        while (slices < 16 && (int64_t)S.P * slices < 1024 && S.P / (slices * 2) >= 16) slices *= 2;
-    hipLaunchKernelGGL(vc_chain_emit, dim3(S.P, nchunk * slices), dim3(VC_THREADS), 0, st, S, T, slot_off, row_base, chain_row_base,
-                       chain_chunk_pre, slices, items);
+        while (slices < 8 && (int64_t)S.P * slices < 1024 && S.P / (slices * 2) >= VC_TILE_RANKS) slices *= 2;
+    hipLaunchKernelGGL(vc_chain_emit, dim3(S.P, nchunk * slices), dim3(VC_THREADS), 0, st, S, T, slot_off, row_base, chain_tile_base,
+                       slices, items);
     return hipGetLastError();
 }
 

@@ -3,9 +3,10 @@
 // The program builds the chain items of benchmark configuration 4 on the host (TTPL_BT_alltoallv, 1024 ranks, 32 per
 // node, r = 32, 1-byte elements, counts ~ Normal(4096, 1024): one read from sendbuf, one write into the staging slot of the
 // intermediate holder, one write into recvbuf; src/twophase_twolayer_rbruck.cpp:334-343,368-377 are the pack / unpack
-// memcpys this replaces), runs the library's own kernel on them (this file includes csrc/vc_copy.hip, so the first row IS
-// the product kernel), then every variant that was tried against it, and the contiguous copies that bound them.  Every
-// variant's receive and staging arenas are compared with the product kernel's, vector by vector.
+// memcpys this replaces) in the order the library's planner writes them (tiles of VC_TILE_RANKS receivers x VC_TILE_RANKS
+// sources), runs the library's own kernel on them (this file includes csrc/vc_copy.hip, so the first row IS the product
+// kernel), then every variant that was tried against it, other orders of the list among them, and the contiguous copies
+// that bound them.  Every variant's receive and staging arenas are compared with the product kernel's, vector by vector.
 //
 //   vc_copy_variants [reps]        (default 7; the best of `reps` launches is printed)
 //
@@ -271,7 +272,7 @@ int main(int argc, char **argv) {
                 stage_bytes += (count[k] + phase + VC_LINE - 1) & ~(int64_t)(VC_LINE - 1);
             }
     }
-    std::vector<int64_t> items(N * ITEM_WORDS);      // by destination, then source: the order vc_chain_emit writes
+    std::vector<int64_t> items(N * ITEM_WORDS);      // by receiver, then source; reordered below
     for (int t = 0; t < P; t++)
         for (int s = 0; s < P; s++) {
             const int64_t k = (int64_t)s * P + t;
@@ -307,7 +308,22 @@ int main(int argc, char **argv) {
         for (auto &w : bytes) { x ^= x << 13; x ^= x >> 7; x ^= x << 17; w = x; }
         CK(hipMemcpy(sendbuf, bytes.data(), cap, hipMemcpyHostToDevice));
     }
-    CK(hipMemcpy(items_dev, items.data(), sizeof(int64_t) * items.size(), hipMemcpyHostToDevice));
+    // the list in tiles of TT receivers x TS sources, receiver by receiver inside a tile; vc_chain_emit writes tiles of
+    // VC_TILE_RANKS x VC_TILE_RANKS, which is the order every kernel below runs on unless its row says otherwise
+    auto in_tiles = [&](int TT, int TS) {
+        std::vector<int64_t> tiled(items.size());
+        int64_t o = 0;
+        for (int tb = 0; tb < P; tb += TT)
+            for (int sb = 0; sb < P; sb += TS)
+                for (int t = tb; t < tb + TT; t++)
+                    for (int s = sb; s < sb + TS; s++) {
+                        std::copy(&items[((int64_t)t * P + s) * ITEM_WORDS], &items[((int64_t)t * P + s) * ITEM_WORDS] + ITEM_WORDS, &tiled[o]);
+                        o += ITEM_WORDS;
+                    }
+        return tiled;
+    };
+    const std::vector<int64_t> library_order = in_tiles(VC_TILE_RANKS, VC_TILE_RANKS);
+    CK(hipMemcpy(items_dev, library_order.data(), sizeof(int64_t) * library_order.size(), hipMemcpyHostToDevice));
     const double physical = (double)payload + (double)moved;      // one read, one write per hop
     printf("configuration 4 as chain items: payload %.3f GB, staging %.3f GB, bytes the launch must move %.3f GB, %lld items, best of %d launches\n",
            payload / 1e9, stage_bytes / 1e9, physical / 1e9, (long long)N, reps);
@@ -373,29 +389,22 @@ int main(int argc, char **argv) {
     VARIANT("8 items per workgroup, loads one item ahead of the stores", 8, true, false, 0, false);
     VARIANT("aligned loads, realigned in registers (DPP wave_shl + v_alignbyte)", 1, false, true, 0, false);
     VARIANT("aligned loads + one round trip + touched 1024 ahead", 1, false, true, 1024, true);
-    {   // the order of the item list: tiles of TT receivers x TS sources instead of all sources of a receiver in a row
-        std::vector<int64_t> tiled(items.size());
-        const int shapes[][2] = {{32, 32}, {64, 64}, {128, 128}, {32, 1024}};
+    {   // other orders of the item list
+        const int shapes[][2] = {{1, 1024}, {64, 64}, {128, 128}, {32, 1024}};
         for (int v = 0; v < 4; v++) {
             const int TT = shapes[v][0], TS = shapes[v][1];
-            int64_t o = 0;
-            for (int tb = 0; tb < P; tb += TT)
-                for (int sb = 0; sb < P; sb += TS)
-                    for (int t = tb; t < tb + TT; t++)
-                        for (int s = sb; s < sb + TS; s++) {
-                            std::copy(&items[((int64_t)t * P + s) * ITEM_WORDS], &items[((int64_t)t * P + s) * ITEM_WORDS] + ITEM_WORDS, &tiled[o]);
-                            o += ITEM_WORDS;
-                        }
+            const std::vector<int64_t> tiled = in_tiles(TT, TS);
             CK(hipMemcpy(items_dev, tiled.data(), sizeof(int64_t) * tiled.size(), hipMemcpyHostToDevice));
             char name[128];
-            snprintf(name, sizeof name, "item list in tiles of %d receivers x %d sources", TT, TS);
+            if (TT == 1) snprintf(name, sizeof name, "item list receiver after receiver, all sources of a receiver in a row");
+            else snprintf(name, sizeof name, "item list in tiles of %d receivers x %d sources", TT, TS);
             const auto launch = [&](auto kernel) { hipLaunchKernelGGL(kernel, dim3((unsigned)N), dim3(VC_THREADS), 0, 0, items_dev, (unsigned)N, (unsigned)(N / VC_XCDS), sendbuf, recvbuf, stage); };
             if (v == 0) failures += row(name, [&] { launch(variant_kernel<1, false, false, 0, false, 1>); });
             if (v == 1) failures += row(name, [&] { launch(variant_kernel<1, false, false, 0, false, 2>); });
             if (v == 2) failures += row(name, [&] { launch(variant_kernel<1, false, false, 0, false, 3>); });
             if (v == 3) failures += row(name, [&] { launch(variant_kernel<1, false, false, 0, false, 4>); });
         }
-        CK(hipMemcpy(items_dev, items.data(), sizeof(int64_t) * items.size(), hipMemcpyHostToDevice));
+        CK(hipMemcpy(items_dev, library_order.data(), sizeof(int64_t) * library_order.size(), hipMemcpyHostToDevice));
     }
     failures += row("vc_copy_chains_kernel<256> once more", product);
     // what contiguous copies of the payload sustain in the same process
