@@ -118,7 +118,7 @@ __device__ __forceinline__ void piece_store(char *dst, const PieceRegs &R) {
 //        item's cache line is in the L2 when that workgroup starts (the value is looked at after the stores only)
 // WHOLE  M = 1: all five words of the item are fetched in one scalar round trip before anything is decided from them
 //        (the library's kernel fetches length and hop count first, then the addresses, then one destination per hop)
-// ORDER  only names the instance: the same kernel on another order of the item list
+// ORDER  only names the instance: the same kernel on another order of the item list, or with fewer workgroups resident
 template <int M, bool PIPE, bool ALIGNED, int AHEAD, bool WHOLE, int ORDER>
 __global__ __launch_bounds__(VC_THREADS) void variant_kernel(const int64_t *__restrict__ items, unsigned nitems, unsigned per,
                                                              const char *__restrict__ sendbuf, char *__restrict__ recvbuf,
@@ -405,6 +405,14 @@ int main(int argc, char **argv) {
             if (v == 3) failures += row(name, [&] { launch(variant_kernel<1, false, false, 0, false, 4>); });
         }
         CK(hipMemcpy(items_dev, library_order.data(), sizeof(int64_t) * library_order.size(), hipMemcpyHostToDevice));
+    }
+    {   // fewer workgroups resident per compute unit (the kernel itself fits 8): dynamic LDS that it never touches takes the room
+        const auto launch = [&](auto kernel, unsigned lds_kib) {
+            hipLaunchKernelGGL(kernel, dim3((unsigned)N), dim3(VC_THREADS), lds_kib << 10, 0, items_dev, (unsigned)N, (unsigned)(N / VC_XCDS), sendbuf, recvbuf, stage);
+        };
+        failures += row("restated kernel + 26 KiB of unused LDS per workgroup (fewer resident)", [&] { launch(variant_kernel<1, false, false, 0, false, 26>, 26); });
+        failures += row("restated kernel + 40 KiB of unused LDS per workgroup", [&] { launch(variant_kernel<1, false, false, 0, false, 40>, 40); });
+        failures += row("restated kernel + 53 KiB of unused LDS per workgroup", [&] { launch(variant_kernel<1, false, false, 0, false, 53>, 53); });
     }
     failures += row("vc_copy_chains_kernel<256> once more", product);
     // what contiguous copies of the payload sustain in the same process
