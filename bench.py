@@ -275,32 +275,39 @@ def kernel_name(st) -> str:
     return base + "_kernel" + f"<{lanes}>"
 
 
-def copy_ceiling(comm, torch, mib: int = 2048, reps: int = 5) -> dict:
+def copy_ceiling(comm, torch, mib: int = 2048, reps: int = 4) -> dict:
     """What contiguous copies sustain on this GPU in this run: vc_calibration_copy (one read, one write: the mix of
     launch-per-digit execution) and vc_calibration_copy2 (one read, two writes: the mix of the forwarded kernel on two-hop
     routes), 16-byte non-temporal loads and stores, one vector per lane — the access pattern of the block movers without
-    their scatter.  HIP events on the communicator's stream, best of `reps`."""
+    their scatter.  HIP events on the communicator's stream.  What the two-writes copy sustains depends on which
+    allocations it runs on (up to 10 % inside one process), so four buffers take the three roles in turn and the
+    ceiling is the best of all launches; the slowest placement's best is reported beside it."""
     nb = mib << 20
-    a = torch.zeros(nb, dtype=torch.uint8, device="cuda:0")
-    b = torch.empty(nb, dtype=torch.uint8, device="cuda:0")
-    b2 = torch.empty(nb, dtype=torch.uint8, device="cuda:0")
-    best = {1: None, 2: None}
-    for _ in range(reps + 1):
+    bufs = [torch.zeros(nb, dtype=torch.uint8, device="cuda:0") for _ in range(4)]
+    per_placement = {1: [], 2: []}
+    for shift in range(4):
+        a, b, b2 = (bufs[(shift + k) % 4] for k in range(3))
+        best = {1: None, 2: None}
+        for _ in range(reps + 1):
+            for writes in (1, 2):
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record()
+                if writes == 1:
+                    comm._check(comm.lib.vc_calibration_copy(b.data_ptr(), a.data_ptr(), nb, comm.handle))
+                else:
+                    comm._check(comm.lib.vc_calibration_copy2(b.data_ptr(), b2.data_ptr(), a.data_ptr(), nb, comm.handle))
+                e1.record()
+                torch.cuda.synchronize()
+                ms = e0.elapsed_time(e1)
+                best[writes] = ms if best[writes] is None or ms < best[writes] else best[writes]
         for writes in (1, 2):
-            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            e0.record()
-            if writes == 1:
-                comm._check(comm.lib.vc_calibration_copy(b.data_ptr(), a.data_ptr(), nb, comm.handle))
-            else:
-                comm._check(comm.lib.vc_calibration_copy2(b.data_ptr(), b2.data_ptr(), a.data_ptr(), nb, comm.handle))
-            e1.record()
-            torch.cuda.synchronize()
-            ms = e0.elapsed_time(e1)
-            best[writes] = ms if best[writes] is None or ms < best[writes] else best[writes]
-    del a, b, b2
-    return {"GBps": round(2 * nb / (best[1] * 1e-3) / 1e9, 1), "ms": round(best[1], 4), "bytes_each_way": nb,
-            "one_read_one_write_GBps": round(2 * nb / (best[1] * 1e-3) / 1e9, 1),
-            "one_read_two_writes_GBps": round(3 * nb / (best[2] * 1e-3) / 1e9, 1), "one_read_two_writes_ms": round(best[2], 4)}
+            per_placement[writes].append(best[writes])
+    del bufs
+    ms1, ms2 = min(per_placement[1]), min(per_placement[2])
+    return {"GBps": round(2 * nb / (ms1 * 1e-3) / 1e9, 1), "ms": round(ms1, 4), "bytes_each_way": nb, "placements": 4,
+            "one_read_one_write_GBps": round(2 * nb / (ms1 * 1e-3) / 1e9, 1),
+            "one_read_two_writes_GBps": round(3 * nb / (ms2 * 1e-3) / 1e9, 1), "one_read_two_writes_ms": round(ms2, 4),
+            "one_read_two_writes_GBps_slowest_placement": round(3 * nb / (max(per_placement[2]) * 1e-3) / 1e9, 1)}
 
 
 def ceiling_for_mix(ceiling: dict, writes_per_read: float) -> float:
