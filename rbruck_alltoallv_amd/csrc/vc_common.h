@@ -40,6 +40,36 @@ struct VcDesc {
     int32_t to;
 };
 
+#if defined(__HIPCC__)
+#define VC_HD __host__ __device__ __forceinline__
+#else
+#define VC_HD inline
+#endif
+
+// Division of a non-negative int (below 2^31) by a divisor that is the same for the whole call — ranks per node, nodes,
+// the radix, ranks — as a multiplication and a shift with constants the host works out once per call: an integer
+// division is 30-odd instructions on this chip, and the route of one block takes a dozen of them.
+// floor(x / d) = (x * mul) >> shift for all 0 <= x < 2^31, with shift = 31 + ceil(log2 d) and mul = floor(2^shift / d) + 1 < 2^32
+// (2^shift <= mul * d <= 2^shift + 2^ceil(log2 d)).
+struct VcDivisor {
+    int d;
+    unsigned mul;
+    int shift;
+};
+
+VC_HD VcDivisor vc_make_divisor(int d) {          // d >= 1
+    int l = 0;
+    while (((int64_t)1 << l) < d) l++;
+    VcDivisor v;
+    v.d = d;
+    v.shift = 31 + l;
+    v.mul = (unsigned)((((uint64_t)1 << v.shift) / (uint64_t)d) + 1);
+    return v;
+}
+
+VC_HD int vc_div(int x, const VcDivisor &v) { return (int)(((uint64_t)(unsigned)x * v.mul) >> v.shift); }
+VC_HD int vc_mod(int x, const VcDivisor &v) { return x - vc_div(x, v) * v.d; }
+
 // What kind of algorithm the call runs; fixed for the whole call.
 struct VcSched {
     int P;            // ranks
@@ -70,13 +100,16 @@ struct VcSched {
                       //    holds for one destination rank back to back in source order — so that an inter-node message
                       //    is a contiguous copy (TTPL_BT_alltoallv, src/twophase_twolayer_rbruck.cpp:388-398, 430-453).
                       //    The organized region is staging region number w.
+    // set by vc_set_divisors once n, G, r and P are final:
+    VcDivisor dn, dG, dr, dP;                     // division by n, G, r, P
 };
 
-#if defined(__HIPCC__)
-#define VC_HD __host__ __device__ __forceinline__
-#else
-#define VC_HD inline
-#endif
+VC_HD void vc_set_divisors(VcSched &S) {
+    S.dn = vc_make_divisor(S.n > 0 ? S.n : 1);
+    S.dG = vc_make_divisor(S.G > 0 ? S.G : 1);
+    S.dr = vc_make_divisor(S.r > 0 ? S.r : 1);
+    S.dP = vc_make_divisor(S.P > 0 ? S.P : 1);
+}
 
 // Staging regions of a call: one per intra-node digit, one per inter-node digit, the organized region.
 VC_HD int vc_regions(const VcSched &S) { return S.w + S.w2 + S.coalesce; }

@@ -245,7 +245,7 @@ __device__ __forceinline__ void vc_add_totals(const VcSched &S, const VcTables &
     for (int u = 0; u < VC_TOTALS_PER_LANE; u++) {
         const int64_t idx = wave * per_wave + u * VC_WAVE + lane;
         if (idx >= pairs) continue;
-        const int to = (int)(idx / P), s = (int)(idx % P);
+        const int to = vc_div((int)idx, S.dP), s = (int)idx - to * P;      // (idx < P^2 <= 2^30)
         const int64_t i = (int64_t)to * P + s;
         bad += vc_pair_bad_entries(S, T, s, to);          // the same count the planner's row kernel makes
         // (a packed receive layout past INT_MAX elements shows as a negative packed displacement of a later source)
@@ -259,7 +259,7 @@ __device__ __forceinline__ void vc_add_totals(const VcSched &S, const VcTables &
     for (int u = 0; u < VC_TOTALS_PER_LANE; u++) {
         const int64_t idx = wave * per_wave + u * VC_WAVE + lane;
         if (idx >= pairs) continue;
-        const int to = (int)(idx / P), s = (int)(idx % P);
+        const int to = vc_div((int)idx, S.dP), s = (int)idx - to * P;      // (idx < P^2 <= 2^30)
         const int64_t i = (int64_t)to * P + s, k = (int64_t)s * P + to;
         const int sc = T.sc[k], rc = T.rc[i];
         const int64_t len = (int64_t)sc * S.esz;
@@ -371,7 +371,7 @@ __global__ __launch_bounds__(LANES) void vc_copy_blocks_kernel(VcSched S, VcTabl
     const int64_t per = (gridDim.x - head) / VC_XCDS;
     const int64_t idx = first_pair + (int64_t)(block % VC_XCDS) * per + block / VC_XCDS;
     const bool inside = idx < (int64_t)S.P * S.P;
-    const int t = inside ? (int)(idx / S.P) : 0, s = inside ? (int)(idx % S.P) : 0;
+    const int t = inside ? vc_div((int)idx, S.dP) : 0, s = inside ? (int)idx - t * S.P : 0;       // (idx < P^2 <= 2^30)
     // Everything the block's addresses depend on is loaded before the planner's verdict is looked at: the loads are
     // independent of each other and of the verdict (tables are always readable), so they travel together instead of one
     // memory round trip after the other; nothing is stored before the verdict is known.
@@ -425,7 +425,7 @@ __global__ __launch_bounds__(VC_WAVE) void vc_copy_blocks_quarter_kernel(VcSched
     const int g = threadIdx.x / VC_QUARTER, q = threadIdx.x % VC_QUARTER;
     const int64_t idx = first_pair + wave * VC_ITEMS_PER_WAVE + g;
     const bool inside = idx < (int64_t)S.P * S.P;
-    const int t = inside ? (int)(idx / S.P) : 0, s = inside ? (int)(idx % S.P) : 0;
+    const int t = inside ? vc_div((int)idx, S.dP) : 0, s = inside ? (int)idx - t * S.P : 0;       // (idx < P^2 <= 2^30)
     // all loads the addresses depend on go out before the planner's verdict is looked at (see vc_copy_blocks_kernel)
     const int64_t len = inside ? (int64_t)T.sc[(int64_t)s * S.P + t] * S.esz : 0;
     const int64_t send_off = vc_send_offset(S, T, s, t);
@@ -483,7 +483,7 @@ __global__ __launch_bounds__(VC_WAVE) void vc_copy_blocks_batch_kernel(VcSched S
     const int p = threadIdx.x % BATCH, kq = threadIdx.x / BATCH;
     const int64_t idx = first_pair + wave * BATCH + p;
     const bool inside = idx < (int64_t)S.P * S.P;
-    const int t = inside ? (int)(idx / S.P) : 0, s = inside ? (int)(idx % S.P) : 0;
+    const int t = inside ? vc_div((int)idx, S.dP) : 0, s = inside ? (int)idx - t * S.P : 0;       // (idx < P^2 <= 2^30)
     // all loads the addresses depend on go out before the planner's verdict is looked at (see vc_copy_blocks_kernel)
     const int64_t len = inside ? (int64_t)T.sc[(int64_t)s * S.P + t] * S.esz : 0;
     const int64_t send_off = vc_send_offset(S, T, s, t);

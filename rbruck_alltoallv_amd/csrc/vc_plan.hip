@@ -176,7 +176,7 @@ __global__ __launch_bounds__(VC_THREADS) void vc_plan_org_rows(VcSched S, VcTabl
     if (threadIdx.x == 0) row_tot[(int64_t)(S.recycle ? ns * ns : S.w) * P + to] = carry;
     __syncthreads();                                      // org_run_base of this rank is complete (same workgroup wrote it)
     for (int id = threadIdx.x; id < P; id += VC_THREADS)
-        slot_off[((int64_t)S.w * P + to) * P + id] = org_run_base[(int64_t)to * G + id / S.n] + vc_org_slot_rel(S, T, to, id);
+        slot_off[((int64_t)S.w * P + to) * P + id] = org_run_base[(int64_t)to * G + vc_div(id, S.dn)] + vc_org_slot_rel(S, T, to, id);
 }
 
 // ---- pass 2: prefix sums over the rows ----

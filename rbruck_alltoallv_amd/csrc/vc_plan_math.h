@@ -19,47 +19,65 @@ struct VcBlock {
     bool to_org;     // ... in its organized region (last intra-node hop of a block that still has to change node)
 };
 
-VC_HD int vc_top_digit(int v, int r) {     // position of the highest non-zero digit, v > 0
+VC_HD int vc_top_digit(int v, const VcDivisor &r) {     // position of the highest non-zero digit, v > 0
     int x = -1;
-    while (v) { v /= r; x++; }
+    while (v) { v = vc_div(v, r); x++; }
     return x;
 }
 
-VC_HD int vc_low_digit(int v, int r) {     // position of the lowest non-zero digit, v > 0
+VC_HD int vc_low_digit(int v, const VcDivisor &r) {     // position of the lowest non-zero digit, v > 0
     int x = 0;
-    while (v % r == 0) { v /= r; x++; }
-    return x;
+    for (;;) {
+        const int q = vc_div(v, r);
+        if (q * r.d != v) return x;
+        v = q; x++;
+    }
+}
+
+// a mod n for 0 <= a < 2n
+VC_HD int vc_wrap(int a, int n) { return a >= n ? a - n : a; }
+
+// Offset j < span without its x lowest base-r digits (j div r^x), and r^x in `dist`: x divisions by the radix.  The power
+// stops growing once it has reached the span (spans are at most 32768 ranks, the radix no more than the span: r^x and
+// r^(x+1) stay below 2^30); the quotient is 0 then, as no offset reaches it.
+VC_HD int vc_upper_digits(const VcSched &S, int j, int x, int span, int &dist) {
+    int upper = j;
+    dist = 1;
+    for (int i = 0; i < x && dist < span; i++) { upper = vc_div(upper, S.dr); dist *= S.r; }
+    return upper;
 }
 
 // Block that arrives in slot `id` of rank `to` during digit x (dist = r^x), if any.
 VC_HD bool vc_intra_block(const VcSched &S, int x, int dist, int to, int id, VcBlock &b) {
-    const int n = S.n, r = S.r;
-    const int gs = to / n, lr = to % n;
-    const int g = id / n;
-    const int j = (id % n - lr + n) % n;
+    const int n = S.n;
+    const int gs = vc_div(to, S.dn), lr = to - gs * n;
+    const int g = vc_div(id, S.dn);
+    const int j = vc_wrap(id - g * n - lr + n, n);
     b.z = 0;
     if (j == 0) return false;
-    const int z = (j / dist) % r;
+    const int upper = vc_upper_digits(S, j, x, n, dist);  // the digits from x upwards (dist = r^x as the launch says, or past n)
+    const int higher = vc_div(upper, S.dr);               // ... from x + 1 upwards
+    const int z = upper - higher * S.r;
     if (z == 0) return false;
-    const int lfrom = (lr + z * dist) % n;
-    const int64_t nd = (int64_t)dist * r;
+    const int nd = dist * S.r;                            // z != 0: dist <= j < n
+    const int lfrom = vc_wrap(lr + z * dist, n);          // z r^x <= j < n
     int above;        // how far the source is above the sender
     bool last;
     if (!S.msd) {
-        above = j % dist;
-        last = j < nd;
-        b.xprev = above ? vc_top_digit(above, r) : -1;
+        above = j - upper * dist;
+        last = higher == 0;
+        b.xprev = above ? vc_top_digit(above, S.dr) : -1;
     } else {
-        above = (int)((j / nd) * nd);
-        last = (j % dist) == 0;
-        b.xprev = above ? vc_low_digit(above, r) : -1;
+        above = higher * nd;
+        last = upper * dist == j;
+        b.xprev = above ? vc_low_digit(above, S.dr) : -1;
     }
-    const int ls = (lfrom + above) % n;
+    const int ls = vc_wrap(lfrom + above, n);             // above <= j < n
     b.s = gs * n + ls;
-    b.t = g * n + (ls - j + n) % n;
+    b.t = g * n + vc_wrap(ls - j + n, n);
     b.from = gs * n + lfrom;
     b.z = z;
-    b.id_from = g * n + (j + lfrom) % n;
+    b.id_from = g * n + vc_wrap(j + lfrom, n);
     b.to_stage = !(last && g == gs);
     b.to_org = S.coalesce && last && g != gs;
     return true;
@@ -81,24 +99,26 @@ struct VcEntry {
 // spoint*n below, group slots (j + gid) % ngroup, n blocks per group slot).  Entry id = jg*n + jj of rank `to`
 // is the block of source local index jj that arrives there in digit x (dist = r^x nodes), if any.
 VC_HD bool vc_inter_block(const VcSched &S, int x, int dist, int to, int id, VcEntry &e, int &z) {
-    const int n = S.n, G = S.G, r = S.r;
-    const int gto = to / n, l = to % n;
-    const int jg = id / n, jj = id % n;
-    z = (jg / dist) % r;
+    const int n = S.n, G = S.G;
+    const int gto = vc_div(to, S.dn), l = to - gto * n;
+    const int jg = vc_div(id, S.dn), jj = id - jg * n;
+    const int upper = vc_upper_digits(S, jg, x, G, dist);
+    const int higher = vc_div(upper, S.dr);
+    z = upper - higher * S.r;
     if (z == 0) return false;
-    const int low = jg % dist;                        // part of the offset travelled in earlier digits
-    const int gfrom = (gto + z * dist) % G;
-    const int gs = (gfrom + low) % G;
-    const int gt = (gs - jg + G) % G;
+    const int low = jg - upper * dist;                // part of the offset travelled in earlier digits
+    const int gfrom = vc_wrap(gto + z * dist, G);
+    const int gs = vc_wrap(gfrom + low, G);
+    const int gt = vc_wrap(gs - jg + G, G);
     e.s = gs * n + jj; e.t = gt * n + l; e.from = gfrom * n + l; e.nblk = 1;
     if (low) {
-        e.xprev = S.w + vc_top_digit(low, r); e.id_from = id;
+        e.xprev = S.w + vc_top_digit(low, S.dr); e.id_from = id;
     } else {                                          // still where the intra-node phase left it
-        const int j = (jj - l + n) % n;
-        e.xprev = j == 0 ? -1 : vc_top_digit(j, r);
+        const int j = vc_wrap(jj - l + n, n);
+        e.xprev = j == 0 ? -1 : vc_top_digit(j, S.dr);
         e.id_from = gt * n + jj;
     }
-    e.xdst = jg < (int64_t)dist * r ? -1 : S.w + x;
+    e.xdst = higher == 0 ? -1 : S.w + x;
     e.id_to = id;
     return true;
 }
@@ -172,11 +192,21 @@ VC_HD int64_t vc_strided_stage_bytes(const VcSched &S) { return (int64_t)(S.w + 
 // Hops of block (s, t): the digit rounds it moves in, plus the hop that is no digit round (vc_block_hop's last slot).
 VC_HD int vc_block_hops(const VcSched &S, int s, int t) {
     if (s == t) return 1;
-    const int n = S.n, G = S.G, r = S.r;
-    const int gs = s / n, gt = t / n;
+    const int n = S.n, G = S.G;
+    const int gs = vc_div(s, S.dn), gt = vc_div(t, S.dn);
     int hops = (S.last_hop == 2 || (S.last_hop == 1 && gs != gt)) ? 1 : 0;
-    if (S.w) for (int j = (s % n - t % n + n) % n; j; j /= r) hops += (j % r) != 0;
-    if (S.w2) for (int j = (gs - gt + G) % G; j; j /= r) hops += (j % r) != 0;
+    if (S.w)
+        for (int j = vc_wrap((s - gs * n) - (t - gt * n) + n, n); j;) {
+            const int q = vc_div(j, S.dr);
+            hops += q * S.r != j;
+            j = q;
+        }
+    if (S.w2)
+        for (int j = vc_wrap(gs - gt + G, G); j;) {
+            const int q = vc_div(j, S.dr);
+            hops += q * S.r != j;
+            j = q;
+        }
     return hops;
 }
 
@@ -204,7 +234,7 @@ VC_HD int64_t vc_org_run_prefix(const VcSched &S, const VcTables &T, int gs, int
 
 // size of the run rank `to` keeps for group g (multiple of VC_LINE; 0 for its own group)
 VC_HD int64_t vc_org_run_size(const VcSched &S, const VcTables &T, int to, int g) {
-    const int gs = to / S.n, t = g * S.n + to % S.n;
+    const int gs = vc_div(to, S.dn), t = g * S.n + (to - gs * S.n);
     if (g == gs) return 0;
     const int64_t phase = (vc_org_run_dst(S, T, gs, t) + S.recv_lo) & (VC_LINE - 1);
     return (phase + vc_org_run_prefix(S, T, gs, t, S.n) + VC_LINE - 1) & ~(int64_t)(VC_LINE - 1);
@@ -212,7 +242,7 @@ VC_HD int64_t vc_org_run_size(const VcSched &S, const VcTables &T, int to, int g
 
 // line-aligned part of the offset of slot id = g*n + m inside the run (vc_stage_addr adds the block's own phase)
 VC_HD int64_t vc_org_slot_rel(const VcSched &S, const VcTables &T, int to, int id) {
-    const int gs = to / S.n, g = id / S.n, m = id % S.n, t = g * S.n + to % S.n;
+    const int gs = vc_div(to, S.dn), g = vc_div(id, S.dn), m = id - g * S.n, t = g * S.n + (to - gs * S.n);
     if (g == gs) return 0;
     const int64_t phase = (vc_org_run_dst(S, T, gs, t) + S.recv_lo) & (VC_LINE - 1);
     return (phase + vc_org_run_prefix(S, T, gs, t, m)) & ~(int64_t)(VC_LINE - 1);
@@ -230,9 +260,9 @@ VC_HD bool vc_entry_block(const VcSched &S, const VcLaunchInfo &info, int to, in
     if (info.kind == 3) {
         // coalesced inter-node message from rank (gs, lt) to rank `to` = (gt, lt), in three contiguous parts: the
         // blocks of local ranks below lt (organized region), the block of lt itself (still in sendbuf), those above
-        const int gs = id / 3, part = id % 3, gt = to / n, lt = to % n;
+        const int gs = id / 3, part = id % 3, gt = vc_div(to, S.dn), lt = to - gt * n;
         if (gs == gt) return false;
-        const int q = ((gs - gt + S.G) % S.G) * n;
+        const int q = vc_wrap(gs - gt + S.G, S.G) * n;
         if (q < info.qlo || q >= info.qhi) return false;
         const int m0 = part == 0 ? 0 : (part == 1 ? lt : lt + 1);
         const int m1 = part == 0 ? lt : (part == 1 ? lt + 1 : n);
@@ -246,13 +276,15 @@ VC_HD bool vc_entry_block(const VcSched &S, const VcLaunchInfo &info, int to, in
         // (src/MPICH_scattered.cpp:44-45: receive from rank + i + ii)
         int q;
         if (info.x == 1) {                                  // inside the node: local rank distance (twolayer_communicator_linear.cpp:45)
-            if (id / n != to / n) return false;
-            q = (id % n - to % n + n) % n;
+            const int gi = vc_div(id, S.dn), gt = vc_div(to, S.dn);
+            if (gi != gt) return false;
+            q = vc_wrap((id - gi * n) - (to - gt * n) + n, n);
         } else if (info.x == 2) {                           // between nodes: (group distance)*n + source local index (:146-153)
-            if (id / n == to / n) return false;
-            q = ((to / n - id / n + S.G) % S.G) * n + id % n;
+            const int gi = vc_div(id, S.dn), gt = vc_div(to, S.dn);
+            if (gi == gt) return false;
+            q = vc_wrap(gt - gi + S.G, S.G) * n + (id - gi * n);
         } else {
-            q = (id - to + S.P) % S.P;
+            q = vc_wrap(id - to + S.P, S.P);
         }
         if (q < info.qlo || q >= info.qhi) return false;
         e.s = id; e.t = to; e.from = id; e.xprev = -1; e.id_from = to; e.xdst = -1; e.id_to = id;
@@ -277,20 +309,20 @@ VC_HD bool vc_entry_block(const VcSched &S, const VcLaunchInfo &info, int to, in
     // inter-node: `id` is the source rank s; the block waits on the rank of s's node that has
     // the receiver's local index (src/twophase_twolayer_rbruck.cpp:430-453, 634-671)
     const int s = id, t = to;
-    const int gs = s / n, gt = t / n, ls = s % n, lt = t % n;
+    const int gs = vc_div(s, S.dn), gt = vc_div(t, S.dn), ls = s - gs * n, lt = t - gt * n;
     if (gs == gt) return false;
-    const int q = ((gs - gt + S.G) % S.G) * n + ls;
+    const int q = vc_wrap(gs - gt + S.G, S.G) * n + ls;
     if (q < info.qlo || q >= info.qhi) return false;
-    const int j = (ls - lt + n) % n;
+    const int j = vc_wrap(ls - lt + n, n);
     e.s = s; e.t = t; e.from = gs * n + lt;
-    e.xprev = j == 0 ? -1 : (S.msd ? vc_low_digit(j, S.r) : vc_top_digit(j, S.r));
+    e.xprev = j == 0 ? -1 : (S.msd ? vc_low_digit(j, S.dr) : vc_top_digit(j, S.dr));
     e.id_from = gt * n + ls; e.xdst = -1; e.id_to = id;
     return true;
 }
 
 VC_HD int64_t vc_entry_len(const VcSched &S, const VcTables &T, const VcEntry &e) {
     if (e.nblk == 1) return (int64_t)T.sc[(int64_t)e.s * S.P + e.t] * S.esz;
-    const int gs = e.s / S.n, m0 = e.s % S.n;
+    const int gs = vc_div(e.s, S.dn), m0 = e.s - gs * S.n;
     return vc_org_run_prefix(S, T, gs, e.t, m0 + e.nblk) - vc_org_run_prefix(S, T, gs, e.t, m0);
 }
 
@@ -402,17 +434,17 @@ VC_HD int vc_slot_time(const VcSched &S, int k) { return (k < S.w && S.msd) ? S.
 
 // Whether block (s, t) moves in hop slot k (vc_block_hop without the destination).
 VC_HD bool vc_block_moves(const VcSched &S, int s, int t, int k) {
-    const int n = S.n, G = S.G, r = S.r, final_slot = S.w + S.w2;
+    const int n = S.n, G = S.G, final_slot = S.w + S.w2;
     if (s == t) return k == final_slot;
-    const int gs = s / n, gt = t / n;
+    const int gs = vc_div(s, S.dn), gt = vc_div(t, S.dn);
     if (k == final_slot) return S.last_hop == 2 || (S.last_hop == 1 && gs != gt);
     const bool intra = k < S.w;
     const int x = intra ? k : k - S.w;
     const int span = intra ? n : G;
-    const int j = intra ? (s % n - t % n + n) % n : (gs - gt + G) % G;
-    int64_t dist = 1;
-    for (int i = 0; i < x; i++) dist *= r;
-    return dist < span && (j / dist) % r != 0;
+    const int j = intra ? vc_wrap((s - gs * n) - (t - gt * n) + n, n) : vc_wrap(gs - gt + G, G);
+    int dist;
+    const int upper = vc_upper_digits(S, j, x, span, dist);
+    return dist < span && vc_mod(upper, S.dr) != 0;
 }
 
 // The hop slot in which block (s, t) moves next after hop slot k (in the call's order), or -1.
@@ -511,25 +543,26 @@ VC_HD int vc_recycle_rows_per_segment(int P) { return (P + VC_RECYCLE_SEGMENTS -
 // destination's node.  The CPU check of the plan compares this with what the launches' entries say, block by block.
 VC_HD bool vc_block_hop(const VcSched &S, const VcTables &T, const int64_t *slot_off, const int64_t *row_base, int s, int t, int k,
                         int64_t &dst) {
-    const int n = S.n, G = S.G, r = S.r, final_slot = S.w + S.w2;
+    const int n = S.n, G = S.G, final_slot = S.w + S.w2;
     const int64_t to_recv = VC_SPACE_RECV | vc_recv_offset(S, T, s, t);
     if (s == t) { dst = to_recv; return k == final_slot; }
-    const int gs = s / n, gt = t / n, ls = s % n, lt = t % n;
+    const int gs = vc_div(s, S.dn), gt = vc_div(t, S.dn), ls = s - gs * n, lt = t - gt * n;
     if (k == final_slot) { dst = to_recv; return S.last_hop == 2 || (S.last_hop == 1 && gs != gt); }
     const bool intra = k < S.w;
     const int x = intra ? k : k - S.w;
     const int span = intra ? n : G;
-    const int j = intra ? (ls - lt + n) % n : (gs - gt + G) % G;       // offset inside the node / between the nodes
-    int64_t dist = 1;
-    for (int i = 0; i < x; i++) dist *= r;
-    if (dist >= span || (j / dist) % r == 0) return false;
-    const int64_t nd = dist * r;
+    const int j = intra ? vc_wrap(ls - lt + n, n) : vc_wrap(gs - gt + G, G);      // offset inside the node / between the nodes
+    int dist;
+    const int upper = vc_upper_digits(S, j, x, span, dist);       // the digits from x upwards
+    if (dist >= span) return false;
+    const int higher = vc_div(upper, S.dr);                       // ... from x + 1 upwards
+    if (upper == higher * S.r) return false;
     const bool msd = intra && S.msd;
-    const int64_t travelled = msd ? (j / dist) * dist : j % nd;
-    const bool last = msd ? j % dist == 0 : j < nd;
-    const int pos = (int)((((intra ? ls : gs) - travelled) % span + span) % span);   // local rank / node of the holder after the hop
+    const int travelled = msd ? upper * dist : j - higher * dist * S.r;           // at most j < span
+    const bool last = msd ? upper * dist == j : higher == 0;
+    const int pos = vc_wrap((intra ? ls : gs) - travelled + span, span);            // local rank / node of the holder after the hop
     const int to = intra ? gs * n + pos : pos * n + lt;
-    const int id = intra ? gt * n + (j + pos) % n : j * n + ls;
+    const int id = intra ? gt * n + vc_wrap(j + pos, n) : j * n + ls;
     dst = (last && (intra ? gs == gt : true)) ? to_recv : (VC_SPACE_STAGE | vc_stage_addr(S, T, slot_off, row_base, k, to, id, s, t));
     return true;
 }

@@ -225,5 +225,6 @@ inline int vc_make_schedule(VcFunc f, int P, int n, int r, int batch, int esz, i
         L.push_back(li);
     }
     if (L[0].kind != 2) L[0].self = 1;                      // direct launches carry the self block as distance 0
+    vc_set_divisors(S);
     return VC_OK;
 }

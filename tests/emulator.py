@@ -167,3 +167,13 @@ def lanes_for_items(nbytes, items):
     if _lib is None:
         _lib = C.CDLL(build())
     return _lib.lanes_for_items(C.c_int64(nbytes), C.c_int64(items))
+
+
+def division_mismatches(d_lo, d_hi, samples=64):
+    """Numerators below 2^31 for which vc_div / vc_mod (csrc/vc_common.h) differ from the hardware division, over the divisors
+    d_lo .. d_hi."""
+    global _lib
+    if _lib is None:
+        _lib = C.CDLL(build())
+    _lib.division_mismatches.restype = C.c_int64
+    return int(_lib.division_mismatches(C.c_int(d_lo), C.c_int(d_hi), C.c_int(samples)))

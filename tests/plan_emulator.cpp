@@ -324,3 +324,28 @@ extern "C" int dispatch_decision(int func, int P, int n, int r, int mode, int ca
 extern "C" int recycle_segments() { return VC_RECYCLE_SEGMENTS; }
 
 extern "C" int lanes_for_items(int64_t bytes, int64_t items) { return vc_lanes_for_items(bytes, items); }
+
+// vc_div / vc_mod (csrc/vc_common.h) against the hardware division for every divisor in [d_lo, d_hi]: numerators around every
+// multiple of the divisor along a geometric walk up to 2^31 - 1, the ends of the range, and `samples` pseudo-random ones.
+// Returns the number of numerators whose quotient or remainder differs.
+extern "C" int64_t division_mismatches(int d_lo, int d_hi, int samples) {
+    int64_t wrong = 0;
+    uint64_t state = 0x9E3779B97F4A7C15ull;
+    for (int64_t d = d_lo; d <= d_hi; d++) {
+        const VcDivisor v = vc_make_divisor((int)d);
+        auto check = [&](int64_t x) {
+            if (x < 0 || x > 0x7FFFFFFF) return;
+            wrong += vc_div((int)x, v) != (int)(x / d) || vc_mod((int)x, v) != (int)(x % d);
+        };
+        for (int64_t q = 0; q * d <= 0x7FFFFFFF; q = q < 16 ? q + 1 : q + q / 3) {
+            check(q * d - 1); check(q * d); check(q * d + 1); check(q * d + d - 1);
+        }
+        const int64_t top = 0x7FFFFFFF / d;
+        check(top * d - 1); check(top * d); check(0x7FFFFFFF); check(0x7FFFFFFE);
+        for (int i = 0; i < samples; i++) {
+            state ^= state << 13; state ^= state >> 7; state ^= state << 17;
+            check((int64_t)(state >> 33));
+        }
+    }
+    return wrong;
+}

@@ -624,3 +624,14 @@ def test_staging_allocator_never_overlaps_live_sub_regions(msd):
             excess.append(peak / need)
     # placing sub-regions in pieces keeps the arena close to what is alive at the worst moment
     assert np.median(excess) < 1.1 and max(excess) < 1.6, (np.median(excess), max(excess))
+
+
+def test_multiply_and_shift_division_is_exact():
+    """The route arithmetic divides by the call's constants (ranks per node, nodes, radix and its powers, ranks) with a
+    multiplication and a shift (vc_div, csrc/vc_common.h).  Exact for every divisor a call can have — 1 .. 32768, and the
+    stand-in for a power of the radix beyond every span — and, as a property of the construction, for any other divisor
+    below 2^31: around every multiple of the divisor, at the ends of the numerators' range and on random numerators."""
+    assert E.division_mismatches(1, 32768) == 0
+    assert E.division_mismatches(1 << 30, 1 << 30) == 0
+    for d in (32769, 65535, 65536, 65537, 1000003, (1 << 24) - 1, (1 << 30) - 1, (1 << 30) + 1, (1 << 31) - 1):
+        assert E.division_mismatches(d, d, 4096) == 0, d
