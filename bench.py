@@ -266,12 +266,17 @@ EXECUTION_KERNELS = {0: "vc_copy_items", 1: "vc_copy_chains", 2: "vc_copy_blocks
 
 
 def kernel_name(st) -> str:
-    """Name of the copy kernel the timed calls launched, from vc_stats_t.execution and .lanes_per_item."""
+    """Name of the copy kernel the timed calls launched, from vc_stats_t.execution, .lanes_per_item and .host_waits (a
+    list-driven call whose launches all went out before the host had seen the plan runs the instance of the kernel that
+    checks the plan on the device: second template argument true)."""
     base, lanes = EXECUTION_KERNELS[int(st.execution)], int(st.lanes_per_item)
+    enqueued = int(st.execution) == 1 and int(st.host_waits) == 1
     if lanes == 16:
-        return base + "_quarter_kernel"
+        return base + "_quarter_kernel" + ("<true>" if enqueued else "<false>" if int(st.execution) == 1 else "")
     if lanes == 1:
         return base + "_batch_kernel"
+    if int(st.execution) == 1:
+        return base + "_kernel" + f"<{lanes}, {'true' if enqueued else 'false'}>"
     return base + "_kernel" + f"<{lanes}>"
 
 
@@ -364,7 +369,8 @@ def other_configurations(api, torch, ceiling: dict, seed: int) -> dict:
                     "payload_bytes": int(prob.payload_bytes), "ms_per_call": round(call_s * 1e3, 4),
                     "GBps_effective": round(prob.payload_bytes / call_s / 1e9, 1),
                     "kernel": kernel_name(st), "execution": EXECUTION_NAMES[int(st.execution)],
-                    "launches_per_call": int(st.n_launches), "kernel_ms_per_call": round(kern_ms / steps, 4),
+                    "launches_per_call": int(st.n_launches), "host_waits_per_call": int(st.host_waits),
+                    "kernel_ms_per_call": round(kern_ms / steps, 4),
                     "kernel_GBps_physical": round(achieved, 1), "frac": round(achieved / HBM_PEAK_GBPS, 4),
                     "frac_of_copy_ceiling": round(achieved / ceiling_for_mix(ceiling, mix), 4),
                     "algorithmic_frac_whole_call": round(2 * st.moved_bytes / call_s / 1e9 / HBM_PEAK_GBPS, 4),
@@ -619,6 +625,7 @@ def main() -> None:
         "plan_ms_per_step": round(t["plan_ms"] / args.steps, 4),
         "mismatched_bytes": int(bad),
         "execution": EXECUTION_NAMES[int(st.execution)],
+        "host_waits_per_call": int(st.host_waits),
         "kernel_sources_sha256": kernel_sources_sha(),
         "copy_ceiling": ceiling,
     }

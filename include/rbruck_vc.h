@@ -71,17 +71,23 @@ int vc_comm_set_bases(vc_comm_t comm, const int64_t *sbase_bytes, const int64_t 
  *    once (from sendbuf) and written once per hop (into the staging slot of every intermediate holder, then into
  *    recvbuf).  The batching tunables (b, bblock) then have no effect, and TTPL_BT_alltoallv sends its inter-node data
  *    per block instead of coalesced.  The copy kernel normally works through a list of block pieces that a planning
- *    kernel writes first (after the host has learnt its size).  When the last call on the communicator consisted of
+ *    kernel writes first, after the host has learnt its size (vc_stats_t.host_waits 2).  Once two calls in a row on the
+ *    communicator were of a kind (the second no more than twice the pieces of the first), list and copy kernel are
+ *    enqueued right behind the size computation, the list's length taken from the last call, and check the plan on the
+ *    device instead (tables, room in the list and in the staging arena, the staging bound: host_waits 1); a call they
+ *    cannot serve has moved nothing and is redone the usual way, a longer list than guessed gets a second launch.
+ *    When the last call on the communicator consisted of
  *    short blocks, the next one goes without the list: every pair of ranks gets a workgroup (at most 128 ranks) or a
  *    quarter of a wavefront (short blocks: average piece below 768 B on any number of ranks, below 1.75 - 3 KiB on 33 - 128) that derives its block's route itself; the
  *    kernel is enqueued right behind the size computation and the call needs one host synchronisation instead of two.
  *    Such a call also gets the reference's own staging layout, every slot as long as the longest block
  *    (src/twophase_tunable_rbruckv.cpp:59; the stride comes from the last call's longest block): slot addresses are then
  *    closed forms and the call is a single kernel launch, without a planner before it.  Every pair of ranks checks its own
- *    table entries, and that its block fits a slot, before it moves anything, and the kernel's first wavefronts add up
- *    what the host needs afterwards; a call with a longer block is redone the general way.  Only on at most 192 ranks
- *    and while regions x P x P x stride stays below 256 MiB.  This is the one execution in which a call that returns
- *    VC_ERR_TABLES may already have delivered the blocks of the pairs whose entries were in order.
+ *    table entries, and that its block fits a slot, before it forms an address from them; the kernel's first wavefronts
+ *    check all of the tables and add up what the host needs afterwards, and the copying wavefronts hold their stores
+ *    back until those have reported the tables in order (a call that returns VC_ERR_TABLES has written nothing here
+ *    either); a call with a longer block is redone the general way.  Only on at most 192 ranks and while
+ *    regions x P x P x stride stays below 256 MiB.
  *    On more than 192 ranks and blocks below 384 B on average a wavefront takes a batch of 16 - 64 pairs instead: a lane per
  *    pair works out the route, then the quarters of the wavefront carry the blocks one after the other.
  * 2: forwarded, always through the list.   3 / 4 / 5: forwarded, always without it, a workgroup / a quarter of a
@@ -344,6 +350,9 @@ typedef struct {
                                     sendcounts[s][t]; + 2^40 per rank whose packed receive layout overflows), as the device
                                     counted them: 0 after a call that returned VC_OK, set by one that returned VC_ERR_TABLES
                                     or VC_ERR_OVERFLOW (the other fields then still describe the call before it) */
+    int64_t host_waits;          /* times the host waited for the device inside the call: 1 when everything the call needed was
+                                    enqueued at once, 2 when the host looked at the plan in mid-call to size the work-item list
+                                    and the staging arena, more when a launch had to be repeated behind larger buffers */
 } vc_stats_t;
 
 /* Per-launch HIP-event timing of the following calls (0 = off, default). */

@@ -21,7 +21,7 @@ class VcStats(C.Structure):
                 ("launch_bytes", C.c_int64 * VC_MAX_LAUNCHES),
                 ("launch_ms", C.c_float * VC_MAX_LAUNCHES), ("execution", C.c_int32), ("lanes_per_item", C.c_int32),
                 ("block_pieces", C.c_int64), ("max_block_pieces", C.c_int64), ("max_block_bytes", C.c_int64),
-                ("bad_table_entries", C.c_int64)]
+                ("bad_table_entries", C.c_int64), ("host_waits", C.c_int64)]
 
 
 # every symbol include/rbruck_vc.h declares: name -> (restype, argtypes)

@@ -330,7 +330,7 @@ static int build_plan(vc_comm *c, const CallParams &q, int recv_lo, VcTables T, 
     S.recv_lo = recv_lo;
     rc = plan_sizes(c, S, L, T, forward);
     if (rc) return rc;
-    HIP_TRY(hipStreamSynchronize(c->stream));     // the staging arena and the item list are sized from the plan
+    HIP_TRY(VC_WAIT(c));     // the staging arena and the item list are sized from the plan
     rc = plan_read(c, S, L, out, forward);
     if (rc) return rc;
     if (forward && staging_out_of_bound(c, out.stage_bytes, out.payload_bytes)) return build_plan(c, q, recv_lo, T, items, out, false, true);
@@ -368,6 +368,7 @@ static int finish_stats(vc_comm *c, const PlanInfo &pi, const void *items_any, b
     s.max_block_pieces = pi.chain ? pi.max_pieces : 0;
     s.max_block_bytes = pi.chain ? pi.max_len : 0;
     s.bad_table_entries = 0;
+    s.host_waits = c->waits;
     s.plan_ms = s.total_ms = s.intra_ms = s.inter_ms = 0.f;
     if (pi.chain) {                                   // one launch that performs the hops of every digit
         for (int k = 0; k < pi.nl; k++) s.moved_bytes += pi.bytes[k];
@@ -376,6 +377,7 @@ static int finish_stats(vc_comm *c, const PlanInfo &pi, const void *items_any, b
         if (c->timing) HIP_TRY(hipEventElapsedTime(&s.launch_ms[0], c->events[2], c->events[3]));
         s.intra_ms = s.launch_ms[0];
         s.lanes_per_item = pi.chain_lanes;
+        c->items_before_last = c->hint.valid ? c->hint.items : 0;
         c->hint = VcHint{1, pi.chain_items, pi.payload_bytes, pi.max_pieces, pi.max_len};
     } else {
         int64_t most = -1;
@@ -417,7 +419,7 @@ static int run_items(vc_comm *c, const PlanInfo &pi, const void *items_any, cons
         }
     }
     if (c->timing) HIP_TRY(hipEventRecord(c->events[2 + nl], st));
-    HIP_TRY(hipStreamSynchronize(st));
+    HIP_TRY(VC_WAIT(c));
     return finish_stats(c, pi, items_any, planned_now);
 }
 
@@ -466,7 +468,7 @@ static int try_strided(vc_comm *c, VcSched S, std::vector<VcLaunchInfo> &L, cons
                                   header_next, header));
     c->strided_clean = true;
     if (c->timing) HIP_TRY(hipEventRecord(c->events[3], st));
-    HIP_TRY(hipStreamSynchronize(st));
+    HIP_TRY(VC_WAIT(c));
     PlanInfo pi;
     int rc = plan_read(c, S, L, pi, true);
     if (rc) return rc;
@@ -475,6 +477,49 @@ static int try_strided(vc_comm *c, VcSched S, std::vector<VcLaunchInfo> &L, cons
     pi.listless = pi.strided = true;
     pi.chain_lanes = pair_lanes;
     rc = finish_stats(c, pi, nullptr, true);
+    return rc ? rc : 1;
+}
+
+// A forwarded call through the work-item list, without the host's look at the plan in mid-call (a round trip of ~10 us):
+// the list kernel and the copy kernel go out right behind the sizing kernels, the list's length guessed from the last
+// forwarded call on the communicator, and check on the device what the host checks otherwise — tables in order, the list
+// and the staging arena large enough, the staging within the communicator's bound (VcChainGuard).  The host reads the
+// same header after the one synchronisation of the call: a plan the launches could not serve has moved nothing and goes
+// the general way; a list longer than guessed gets a second launch for the rest.
+// Returns 1: served; 0: nothing moved, `pi` holds the plan (the stream is synchronised); 2: not tried; < 0: errors.
+static int try_enqueued_list(vc_comm *c, const VcSched &S, std::vector<VcLaunchInfo> &L, const VcTables &T, const char *sendbuf, char *recvbuf,
+                             PlanInfo &pi) {
+    const int stride = VC_CHAIN_HEAD + vc_hop_slots(S);
+    VcChainGuard guard;
+    guard.cap_items = (int64_t)(c->desc.cap / (sizeof(int64_t) * (size_t)stride));
+    guard.stage_cap = c->stage.cap >= 64 ? (int64_t)c->stage.cap - 64 : 0;
+    guard.allowance = c->bound_staging ? c->staging_allowance : INT64_MAX;
+    const int64_t guess = std::min<int64_t>(c->hint.items, guard.cap_items);
+    if (!c->hint.valid || guess <= 0 || !c->B.chain_row_tot) return 2;
+    // a guess far above the call's real length costs a workgroup that starts and ends for every item there is not: only
+    // while the communicator's calls stay of a kind (the last one no more than twice the one before)
+    if (c->hint.items > 2 * c->items_before_last) return 2;
+    hipStream_t st = c->stream;
+    const int lanes = vc_lanes_for_items(c->hint.payload, c->hint.items);
+    HIP_TRY(vc_launch_chain_plan(S, T, c->B.slot_off, c->B.row_base, c->B.chain_row_tot + 2 * (size_t)S.P, c->desc.as<int64_t>(), guess, st,
+                                 c->B.header, guard.cap_items));
+    if (c->timing) { HIP_TRY(hipEventRecord(c->events[1], st)); HIP_TRY(hipEventRecord(c->events[2], st)); }
+    int64_t done = 0;                                     // items the guarded launch was sized for
+    HIP_TRY(vc_launch_copy_chains_guarded(c->desc.as<int64_t>(), stride, guess, lanes, sendbuf, recvbuf, c->stage.as<char>(), st, c->B.header,
+                                          guard, &done));
+    if (c->timing) HIP_TRY(hipEventRecord(c->events[3], st));
+    HIP_TRY(VC_WAIT(c));
+    int rc = plan_read(c, S, L, pi, true);
+    if (rc) return rc;                                    // (bad tables: the launches have moved nothing)
+    if (!vc_chain_guard_ok(c->h_header, guard)) return 0;
+    pi.chain_lanes = lanes;
+    if (pi.chain_items > done) {                          // more pieces than the last call had
+        HIP_TRY(vc_launch_copy_chains(c->desc.as<int64_t>() + done * stride, stride, pi.chain_items - done, lanes, sendbuf, recvbuf,
+                                      c->stage.as<char>(), st));
+        if (c->timing) HIP_TRY(hipEventRecord(c->events[3], st));
+        HIP_TRY(VC_WAIT(c));
+    }
+    rc = finish_stats(c, pi, c->desc.p, true);
     return rc ? rc : 1;
 }
 
@@ -508,7 +553,7 @@ static int run_schedule(vc_comm *c, const CallParams &q, const char *sendbuf, ch
             HIP_TRY(vc_launch_copy_blocks(S, T, c->B.slot_off, c->B.row_base, c->B.header, guard, pair_lanes, sendbuf, recvbuf,
                                           c->stage.as<char>(), st));
             if (c->timing) HIP_TRY(hipEventRecord(c->events[3], st));
-            HIP_TRY(hipStreamSynchronize(st));
+            HIP_TRY(VC_WAIT(c));
             synced = true;
             rc = plan_read(c, S, L, pi, true);
             if (rc) return rc;
@@ -519,8 +564,14 @@ static int run_schedule(vc_comm *c, const CallParams &q, const char *sendbuf, ch
         }
         if (pi.listless) return finish_stats(c, pi, nullptr, true);
     }
+    if (!synced && forward) {
+        rc = try_enqueued_list(c, S, L, T, sendbuf, recvbuf, pi);
+        if (rc == 1) return VC_OK;
+        if (rc < 0) return rc;
+        synced = rc == 0;
+    }
     if (!synced) {
-        HIP_TRY(hipStreamSynchronize(st));         // the staging arena and the item list are sized from the plan
+        HIP_TRY(VC_WAIT(c));         // the staging arena and the item list are sized from the plan
         rc = plan_read(c, S, L, pi, forward);
         if (rc) return rc;
     }
@@ -554,7 +605,7 @@ static int enqueue_async(vc_comm *c, const CallParams &q, const VcSched &S, std:
 extern "C" int vc_comm_wait(vc_comm_t c) {
     if (!c) return fail_arg("null communicator");
     if (!c->pending.active) {
-        HIP_TRY(hipStreamSynchronize(c->stream));
+        HIP_TRY(VC_WAIT(c));
         return VC_OK;
     }
     // whatever happens below, the call is over when this function returns: the communicator is free again and launches
@@ -567,7 +618,7 @@ extern "C" int vc_comm_wait(vc_comm_t c) {
             c->busy.clear(std::memory_order_release);
         }
     } release{c};
-    HIP_TRY(hipStreamSynchronize(c->stream));
+    HIP_TRY(VC_WAIT(c));
     const VcSched &S = c->pending.S;
     std::vector<VcLaunchInfo> L((size_t)c->pending.n_launch_infos);     // plan_read only needs their number here
     PlanInfo pi;
@@ -585,7 +636,7 @@ extern "C" int vc_comm_wait(vc_comm_t c) {
         HIP_TRY(vc_launch_copy_blocks(S, c->pending.T, c->B.slot_off, c->B.row_base, c->B.header, guard, c->pending.lanes,
                                       c->pending.sendbuf, c->pending.recvbuf, c->stage.as<char>(), c->stream));
         if (c->timing) HIP_TRY(hipEventRecord(c->events[3], c->stream));
-        HIP_TRY(hipStreamSynchronize(c->stream));
+        HIP_TRY(VC_WAIT(c));
     }
     pi.listless = true;
     pi.chain_lanes = c->pending.lanes;
@@ -752,7 +803,7 @@ extern "C" int twophase_rbruck_alltoallv_noalloc(int r, char *sendbuf, int *send
     if (rc) return rc;
     const int lanes = vc_dispatch(c->forward, VC_CALL_LISTLESS_ONLY, c->hint, S).lanes;
     HIP_TRY(vc_launch_copy_blocks(S, T, B.slot_off, B.row_base, B.header, guard, lanes, sendbuf, recvbuf, stage, c->stream));
-    HIP_TRY(hipStreamSynchronize(c->stream));
+    HIP_TRY(VC_WAIT(c));
     PlanInfo pi;
     rc = plan_read(c, S, L, pi, true);
     if (rc) return rc;

@@ -205,8 +205,11 @@ hipError_t vc_launch_plan_sizes(const VcSched &S, const VcLaunchInfo *launches_h
 // Forwarded execution: the chain items (every block's route in closed form, staging addresses from the plan tables).
 // chain_tile_base: [P][VC_TILES(P)] first item of every (receiver, tile of sources) (vc_launch_plan_sizes leaves it behind
 // chain_row_tot's first 2 P words).
+// header + cap_items (optional): the launch was enqueued before the host knew the plan; it writes nothing unless the
+// device header the sizing kernels left says the tables are in order and the list holds all header[2] items.
 hipError_t vc_launch_chain_plan(const VcSched &S, VcTables T, const int64_t *slot_off, const int64_t *row_base,
-                                const int64_t *chain_tile_base, int64_t *items, int64_t nitems, hipStream_t st);
+                                const int64_t *chain_tile_base, int64_t *items, int64_t nitems, hipStream_t st,
+                                const int64_t *header = nullptr, int64_t cap_items = 0);
 // Pass 3: writes the work items (needs the item buffer, sized from the header).
 hipError_t vc_launch_plan_emit(const VcSched &S, const VcLaunchInfo *launches_host, const VcLaunchInfo *launches_dev, int nlaunch,
                                VcTables T, const int64_t *slot_off,
@@ -221,6 +224,25 @@ hipError_t vc_launch_copy_items(const VcDesc *items, int64_t nitems, int lanes, 
                                 hipStream_t st);
 hipError_t vc_launch_copy_chains(const int64_t *items, int stride, int64_t nitems, int lanes, const char *sendbuf, char *recvbuf,
                                  char *stage, hipStream_t st);
+// What the plan of a call must look like for a list and a copy launch that were enqueued right behind the sizing kernels,
+// before the host had seen the plan, to do their work.  Kernels and host evaluate it on the same header, so both agree on
+// whether anything was moved.
+struct VcChainGuard {
+    int64_t cap_items;      // chain items the list has room for
+    int64_t stage_cap;      // bytes of staging arena there are
+    int64_t allowance;      // staging a forwarded call may take before its ratio to the payload counts (INT64_MAX: no bound)
+};
+
+VC_HD bool vc_chain_guard_ok(const int64_t *header, const VcChainGuard &g) {
+    if (header[VC_HEADER_BAD] != 0 || header[2] > g.cap_items || header[0] > g.stage_cap) return false;
+    return !(header[0] > g.allowance && header[0] > 3 * header[1]);
+}
+
+// The same launch for a list whose length the host only guesses (grid_items: work items the grid is sized for): every
+// workgroup checks vc_chain_guard_ok on the device header and takes an item only if there is one at its index
+// (header[2] items exist).  Items beyond `covered` (grid_items, or what one launch holds) are left for a second, ordinary launch.
+hipError_t vc_launch_copy_chains_guarded(const int64_t *items, int stride, int64_t grid_items, int lanes, const char *sendbuf,
+                                         char *recvbuf, char *stage, hipStream_t st, const int64_t *header, VcChainGuard guard, int64_t *covered);
 // What the plan of a call must look like for the listless kernels to run it; 0 = no limit.  The kernels evaluate it on
 // the device header, the host on its copy after the synchronisation: both then agree on whether anything was moved.
 struct VcListlessGuard {
@@ -253,7 +275,9 @@ VC_HD bool vc_listless_ok(const int64_t *header, const VcListlessGuard &g) {
 // copies the words to header_host, with [0] = the bytes the fixed-stride arena takes; `header` is not read.  Every pair
 // checks its own table entries and the guard's max_len / max_pieces and leaves its block alone when one of them fails, so
 // no address is formed from a bad entry; the host, which evaluates the same conditions on the totals afterwards, reports
-// the call as refused then.  Blocks of the other pairs may already have been delivered.
+// the call as refused then.  With bad table entries nothing has been stored by then: the copying wavefronts hold their
+// stores back until the totalling ones have reported on all of the tables.  With a block longer than a slot the blocks of
+// the other pairs may already have been delivered; they are delivered again when the host redoes the call.
 hipError_t vc_launch_copy_blocks(const VcSched &S, VcTables T, const int64_t *slot_off, const int64_t *row_base, const int64_t *header,
                                  VcListlessGuard guard, int lanes, const char *sendbuf, char *recvbuf, char *stage, hipStream_t st,
                                  int64_t *header_host = nullptr, int64_t *header_zero = nullptr, int64_t *totals = nullptr);

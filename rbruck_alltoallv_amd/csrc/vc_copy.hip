@@ -98,13 +98,17 @@ __device__ __forceinline__ void vc_forward_piece(const char *src, int64_t len, i
 // LANES = VC_THREADS: one workgroup of four wavefronts per item, the shape that moves blocks of several KiB fastest.
 // LANES = VC_WAVE: one wavefront per item, for lists of short pieces: four times as many items in flight per compute
 // unit, and no wavefronts that start only to find nothing left for them in a piece of a few hundred bytes.
-template <int LANES>
+// GUARDED: the launch was enqueued before the host had seen the plan (see VcChainGuard): `nitems` is a guess, header[2] the
+// truth, and nothing moves unless the plan is one this launch can serve.
+template <int LANES, bool GUARDED = false>
 __global__ __launch_bounds__(LANES) void vc_copy_chains_kernel(const int64_t *__restrict__ items, int stride, unsigned nitems,
                                                                const char *__restrict__ sendbuf, char *__restrict__ recvbuf,
-                                                               char *__restrict__ stage) {
+                                                               char *__restrict__ stage, const int64_t *__restrict__ header = nullptr,
+                                                               VcChainGuard guard = VcChainGuard()) {
     const unsigned per = gridDim.x / VC_XCDS;
     const unsigned idx = (blockIdx.x % VC_XCDS) * per + blockIdx.x / VC_XCDS;
     if (idx >= nitems) return;
+    if (GUARDED && (!vc_chain_guard_ok(header, guard) || (int64_t)idx >= header[2])) return;
     const int64_t *it = items + (int64_t)idx * stride;
     const int64_t len = it[VC_CHAIN_LEN];
     const int nhop = (int)it[VC_CHAIN_NHOP];
@@ -171,14 +175,18 @@ __device__ __forceinline__ void vc_forward_piece_quarter(const char *src, int64_
 // gridDim.x wavefronts, a multiple of VC_XCDS; XCD k works through the k-th eighth of them, each taking four items in a row
 // `rounds`: groups of four items in a row a wavefront takes, one after the other (long lists of very short pieces: fewer
 // wavefronts, each paying its start-up once for more items)
+template <bool GUARDED = false>
 __global__ __launch_bounds__(VC_WAVE) void vc_copy_chains_quarter_kernel(const int64_t *__restrict__ items, int stride, unsigned nitems,
                                                                          int rounds, const char *__restrict__ sendbuf,
-                                                                         char *__restrict__ recvbuf, char *__restrict__ stage) {
+                                                                         char *__restrict__ recvbuf, char *__restrict__ stage,
+                                                                         const int64_t *__restrict__ header = nullptr,
+                                                                         VcChainGuard guard = VcChainGuard()) {
     const unsigned per = gridDim.x / VC_XCDS;
     const unsigned wave = (blockIdx.x % VC_XCDS) * per + blockIdx.x / VC_XCDS;
+    if (GUARDED && !vc_chain_guard_ok(header, guard)) return;
     for (int round = 0; round < rounds; round++) {
         const int64_t idx = ((int64_t)wave * rounds + round) * VC_ITEMS_PER_WAVE + threadIdx.x / VC_QUARTER;
-        if (idx >= nitems) continue;
+        if (idx >= nitems || (GUARDED && idx >= header[2])) continue;
         const int64_t *it = items + idx * stride;
         const int64_t len = it[VC_CHAIN_LEN];
         const int nhop = (int)it[VC_CHAIN_NHOP];
@@ -588,14 +596,35 @@ hipError_t vc_launch_copy_chains(const int64_t *items, int stride, int64_t nitem
         const dim3 grid(vc_grid_for(now, lanes));
         const int64_t *first = items + done * stride;
         if (lanes == VC_QUARTER)
-            hipLaunchKernelGGL(vc_copy_chains_quarter_kernel, grid, dim3(VC_WAVE), 0, st, first, stride, (unsigned)now, vc_quarter_rounds(now),
-                               sendbuf, recvbuf, stage);
+            hipLaunchKernelGGL(vc_copy_chains_quarter_kernel<false>, grid, dim3(VC_WAVE), 0, st, first, stride, (unsigned)now,
+                               vc_quarter_rounds(now), sendbuf, recvbuf, stage, nullptr, VcChainGuard());
         else if (lanes == VC_WAVE)
-            hipLaunchKernelGGL(vc_copy_chains_kernel<VC_WAVE>, grid, dim3(VC_WAVE), 0, st, first, stride, (unsigned)now, sendbuf, recvbuf, stage);
+            hipLaunchKernelGGL((vc_copy_chains_kernel<VC_WAVE, false>), grid, dim3(VC_WAVE), 0, st, first, stride, (unsigned)now, sendbuf, recvbuf,
+                               stage, nullptr, VcChainGuard());
         else
-            hipLaunchKernelGGL(vc_copy_chains_kernel<VC_THREADS>, grid, dim3(VC_THREADS), 0, st, first, stride, (unsigned)now, sendbuf, recvbuf,
-                               stage);
+            hipLaunchKernelGGL((vc_copy_chains_kernel<VC_THREADS, false>), grid, dim3(VC_THREADS), 0, st, first, stride, (unsigned)now, sendbuf,
+                               recvbuf, stage, nullptr, VcChainGuard());
     }
+    return hipGetLastError();
+}
+
+// One launch (a guessed list longer than a launch holds is cut to what one holds; the rest is the caller's second launch).
+hipError_t vc_launch_copy_chains_guarded(const int64_t *items, int stride, int64_t grid_items, int lanes, const char *sendbuf,
+                                         char *recvbuf, char *stage, hipStream_t st, const int64_t *header, VcChainGuard guard, int64_t *covered) {
+    const int64_t step = vc_items_per_launch(lanes);
+    const int64_t now = grid_items < step ? grid_items : step;
+    *covered = now > 0 ? now : 0;
+    if (now <= 0) return hipSuccess;
+    const dim3 grid(vc_grid_for(now, lanes));
+    if (lanes == VC_QUARTER)
+        hipLaunchKernelGGL(vc_copy_chains_quarter_kernel<true>, grid, dim3(VC_WAVE), 0, st, items, stride, (unsigned)now, vc_quarter_rounds(now),
+                           sendbuf, recvbuf, stage, header, guard);
+    else if (lanes == VC_WAVE)
+        hipLaunchKernelGGL((vc_copy_chains_kernel<VC_WAVE, true>), grid, dim3(VC_WAVE), 0, st, items, stride, (unsigned)now, sendbuf, recvbuf,
+                           stage, header, guard);
+    else
+        hipLaunchKernelGGL((vc_copy_chains_kernel<VC_THREADS, true>), grid, dim3(VC_THREADS), 0, st, items, stride, (unsigned)now, sendbuf,
+                           recvbuf, stage, header, guard);
     return hipGetLastError();
 }
 

@@ -81,6 +81,8 @@ struct vc_comm {
                                           // call suggests), 2 forwarded through a work-item list, 3 / 4 forwarded, listless with a
                                           // workgroup / a quarter of a wavefront per pair of ranks
     VcHint hint = {0, 0, 0, 0, 0};        // what the last forwarded call on this communicator looked like
+    int waits = 0;                        // times the host has waited for the stream in the call in progress
+    int64_t items_before_last = 0;        // block pieces of the forwarded call before the one `hint` describes (0: there was none)
     DevBuf chain_row_tot, chain_row_base;
     DevBuf strided_headers;               // fixed-stride calls: two headers used in turn
     bool strided_clean = false;           // ... and the one the next call will use is known to be zero
@@ -140,11 +142,16 @@ inline void free_retired_stage(vc_comm *c) {
 struct BusyGuard {
     vc_comm *c;
     bool mine;
-    explicit BusyGuard(vc_comm *comm) : c(comm), mine(comm && !comm->busy.test_and_set(std::memory_order_acquire)) {}
+    explicit BusyGuard(vc_comm *comm) : c(comm), mine(comm && !comm->busy.test_and_set(std::memory_order_acquire)) {
+        if (mine) c->waits = 0;
+    }
     ~BusyGuard() { if (mine) c->busy.clear(std::memory_order_release); }
     bool ok() const { return !c || mine; }
     void keep() { mine = false; }         // the call stays in progress after the entry point returns (vc_comm_wait ends it)
 };
+// the host waits for the communicator's stream (counted: vc_stats_t.host_waits)
+#define VC_WAIT(c) ((c)->waits++, hipStreamSynchronize((c)->stream))
+
 #define VC_ONE_CALL(c)                                                                                              \
     BusyGuard busy_guard_(c);                                                                                       \
     if (!busy_guard_.ok()) return fail_arg("the communicator is serving another call (one call at a time)", VC_ERR_BUSY)

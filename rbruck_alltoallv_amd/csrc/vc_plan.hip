@@ -450,7 +450,11 @@ hipError_t vc_launch_plan_emit(const VcSched &S, const VcLaunchInfo *launches_ho
 __global__ __launch_bounds__(VC_THREADS) void vc_chain_emit(VcSched S, VcTables T, const int64_t *__restrict__ slot_off,
                                                             const int64_t *__restrict__ row_base,
                                                             const int64_t *__restrict__ chain_tile_base, int slices,
-                                                            int64_t *__restrict__ items) {
+                                                            int64_t *__restrict__ items, const int64_t *__restrict__ header,
+                                                            int64_t cap_items) {
+    // a launch that was enqueued before the host had seen the plan: nothing is written unless the tables are in order
+    // (their entries could point anywhere) and the list has room for every item
+    if (header && (header[VC_HEADER_BAD] != 0 || header[2] > cap_items)) return;
     __shared__ int64_t lds[VC_WAVES_PER_BLOCK];
     __shared__ int64_t big_at[VC_THREADS], big_pre[VC_THREADS];
     // a block of many pieces keeps its route here while the whole workgroup writes its items (routes of more hops than
@@ -539,14 +543,15 @@ __global__ __launch_bounds__(VC_THREADS) void vc_chain_emit(VcSched S, VcTables 
 }
 
 hipError_t vc_launch_chain_plan(const VcSched &S, VcTables T, const int64_t *slot_off, const int64_t *row_base,
-                                const int64_t *chain_tile_base, int64_t *items, int64_t nitems, hipStream_t st) {
+                                const int64_t *chain_tile_base, int64_t *items, int64_t nitems, hipStream_t st, const int64_t *header,
+                                int64_t cap_items) {
     const int nchunk = (S.P + VC_THREADS - 1) / VC_THREADS;
     // at least ~1024 workgroups (four per compute unit), each a whole number of tiles of sources
     int slices = nchunk > 1 ? 1 : vc_emit_slices(nitems, S.P);
     if (nchunk == 1)
         while (slices < 8 && (int64_t)S.P * slices < 1024 && S.P / (slices * 2) >= VC_TILE_RANKS) slices *= 2;
     hipLaunchKernelGGL(vc_chain_emit, dim3(S.P, nchunk * slices), dim3(VC_THREADS), 0, st, S, T, slot_off, row_base, chain_tile_base,
-                       slices, items);
+                       slices, items, header, cap_items);
     return hipGetLastError();
 }
 

@@ -37,11 +37,11 @@ def test_library_exports_every_declared_symbol():
 def test_stats_struct_layout_matches_header():
     text = open(os.path.join(ROOT, "include", "rbruck_vc.h")).read()
     assert f"#define VC_MAX_LAUNCHES {_lib.VC_MAX_LAUNCHES}" in text
-    # two int32, three int64, four float, the two per-launch arrays, two int32, four int64
-    fields = 2 * 4 + 3 * 8 + 4 * 4 + _lib.VC_MAX_LAUNCHES * (8 + 4) + 2 * 4 + 4 * 8
+    # two int32, three int64, four float, the two per-launch arrays, two int32, five int64
+    fields = 2 * 4 + 3 * 8 + 4 * 4 + _lib.VC_MAX_LAUNCHES * (8 + 4) + 2 * 4 + 5 * 8
     assert ctypes.sizeof(_lib.VcStats) == fields and fields % 8 == 0
-    assert _lib.VcStats.launch_bytes.offset == 48 and _lib.VcStats.execution.offset == fields - 8 - 4 * 8
-    assert _lib.VcStats.bad_table_entries.offset == fields - 8
+    assert _lib.VcStats.launch_bytes.offset == 48 and _lib.VcStats.execution.offset == fields - 8 - 5 * 8
+    assert _lib.VcStats.bad_table_entries.offset == fields - 16 and _lib.VcStats.host_waits.offset == fields - 8
 
 
 def test_argument_errors_need_no_gpu():

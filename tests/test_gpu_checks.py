@@ -538,3 +538,81 @@ def test_staging_bound(api):
     assert (int(dp2.comm.last_stats().execution), int(dp2.comm.last_stats().staging_bytes)) == seen[(True, 0)][:2]
     assert api.tuna_algorithm(32, 0, dp2, ds, dr2) == 0 and dp2.verify(ds, dr2) == 0      # the communicator is free and on its own stream again
     dp2.comm.free()
+
+
+def test_list_and_copy_enqueued_behind_the_sizing_kernels(api):
+    """A forwarded call through the work-item list normally waits for the sizing kernels in mid-call (vc_stats_t.host_waits
+    2).  Once two calls of a kind have been seen on a communicator, the list and the copy go out right behind the sizing
+    kernels, sized from the last call, and check the plan on the device (host_waits 1).  Every way that can end, against
+    the definition's bytes: the guess fits; the call needs a longer list and a larger arena than there are (nothing moves,
+    the call goes the general way); the call is shorter than guessed; its tables disagree (refused, recvbuf untouched);
+    it is longer than guessed (a second launch takes the rest); its staging is out of the communicator's bound (one
+    launch per digit instead)."""
+    import torch
+    P = 96
+    comm = api.VirtualComm(P)
+    base = W.counts_uniform_random(P, 3000, seed=11)
+    more = W.counts_uniform_random(P, 5000, seed=12)
+    more[::5, ::6] = 40000                                                            # + 320 blocks of 10 pieces
+    less = W.counts_uniform_random(P, 900, seed=13)
+    less[less % 5 != 0] = 0                                                           # four blocks in five are empty
+    probs = {"base": W.make_problem(base, 1, 0, 0), "more": W.make_problem(more, 1, 1, 1), "less": W.make_problem(less, 1, 0, 0)}
+
+    def call(name, func=None, expect=0, spoil=False):
+        prob = probs[name]
+        send = W.fill_send_arena(prob, 0, 21)
+        want = W.expected_recv_arena(prob, send)
+        dp = api.DeviceProblem(prob, comm=comm)
+        comm.set_forwarding(2)                                                        # forwarded, through the list
+        ds = torch.from_numpy(send).to("cuda:0")
+        dr = dp.new_recv_arena(0xEE)
+        if spoil:
+            dp.recvcounts[9, 4] += 2
+        rc = api.twophase_rbruck_alltoallv(4, dp, ds, dr) if func is None else func(dp, ds, dr)
+        assert rc == expect, (name, rc, comm.error())
+        got = dr.cpu().numpy()
+        if expect == 0:
+            assert np.array_equal(got, want), name
+        else:
+            assert bool((got == 0xEE).all()), "a refused call wrote into recvbuf"
+        st = comm.last_stats()
+        return int(st.host_waits), int(st.execution), int(st.block_pieces), int(st.staging_bytes)
+
+    seen = [call("base"), call("base"), call("base")]
+    assert [w for w, _, _, _ in seen] == [2, 2, 1] and all(e == 1 for _, e, _, _ in seen), seen
+    grown = call("more")                               # longer list, larger arena: refused on the device, redone the general way
+    assert grown[:2] == (2, 1) and seen[0][2] < grown[2] <= 2 * seen[0][2] and grown[3] > seen[0][3], (seen, grown)
+    assert call("more")[0] == 1                        # now the guess fits again
+    shorter = call("less")                             # fewer pieces than guessed: the surplus workgroups find nothing
+    assert shorter[0] == 1 and 2 * shorter[2] < grown[2], (shorter, grown)
+    call("base", expect=_lib.VC_ERR_TABLES, spoil=True)        # enqueued like the others: the device-side check refuses it
+    longer = call("more")                              # more pieces than guessed (the last good call was the short one): a second launch
+    assert longer[0] == 2 and longer[2] == grown[2], (longer, grown)
+    assert call("base")[0] == 2                        # after a short and a long call: not of a kind, the host looks first
+    assert call("base")[0] == 1
+    # the packed receive layout of the two-layer function
+    two_layer = [call("base", func=lambda dp, ds, dr: api.TTPL_BT_alltoallv(8, 4, 0, dp, ds, dr)) for _ in range(3)]
+    assert two_layer[-1][:2] == (1, 1), two_layer
+    comm.free()
+
+    # out of the staging bound: 512 ranks, radix 2 (4.5 hops per block: staging 3.5 x the payload), an allowance of 2 MiB
+    P = 512
+    comm = api.VirtualComm(P)
+    prob = W.make_problem(W.counts_uniform_random(P, 64, seed=14), 1, 0, 0)
+    send = W.fill_send_arena(prob, 0, 22)
+    want = W.expected_recv_arena(prob, send)
+    dp = api.DeviceProblem(prob, comm=comm)
+    ds = torch.from_numpy(send).to("cuda:0")
+    comm.set_forwarding(2)
+    comm.set_staging_bound(0)
+    for expected_waits in (2, 2, 1):
+        dr = dp.new_recv_arena(0xEE)
+        assert api.tuna_algorithm(2, 0, dp, ds, dr) == 0, comm.error()
+        st = comm.last_stats()
+        assert int(st.host_waits) == expected_waits and st.execution == 1 and np.array_equal(dr.cpu().numpy(), want)
+    comm.set_staging_bound(2)
+    dr = dp.new_recv_arena(0xEE)
+    assert api.tuna_algorithm(2, 0, dp, ds, dr) == 0, comm.error()
+    st = comm.last_stats()
+    assert st.execution == 0 and np.array_equal(dr.cpu().numpy(), want)      # refused on the device, run one launch per digit
+    comm.free()
