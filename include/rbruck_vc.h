@@ -355,7 +355,8 @@ typedef struct {
                                     and the staging arena, more when a launch had to be repeated behind larger buffers */
 } vc_stats_t;
 
-/* Per-launch HIP-event timing of the following calls (0 = off, default). */
+/* Per-launch HIP-event timing of the following calls (0 = off, default).  While it is on, a list-driven call keeps the
+ * host's look at the plan in mid-call (host_waits 2), so that the events bracket the copy kernel alone. */
 int vc_comm_set_timing(vc_comm_t comm, int enable);
 int vc_comm_last_stats(vc_comm_t comm, vc_stats_t *out);
 

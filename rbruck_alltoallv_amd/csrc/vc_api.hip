@@ -264,6 +264,7 @@ static int plan_sizes(vc_comm *c, const VcSched &S, std::vector<VcLaunchInfo> &L
     int rc = reserve_plan_bufs(c, S, nl, forward);
     if (rc) return rc;
     if (c->timing) { rc = ensure_events(c, (size_t)nl + 4); if (rc) return rc; }
+    c->plan_end = 2;                                      // the planning ends where the first copy launch begins: one event for both
     return enqueue_plan_sizes(c, S, L, T, forward, c->timing);
 }
 
@@ -318,7 +319,6 @@ static int plan_emit(vc_comm *c, const VcSched &S, std::vector<VcLaunchInfo> &L,
         HIP_TRY(vc_launch_plan_emit(S, L.data(), c->B.launches, pi.nl, T, c->B.slot_off, c->B.row_base, c->B.item_row_base, c->B.header,
                                     items.as<VcDesc>(), pi.items_total, st));
     }
-    if (c->timing) HIP_TRY(hipEventRecord(c->events[1], st));
     return VC_OK;
 }
 
@@ -393,7 +393,7 @@ static int finish_stats(vc_comm *c, const PlanInfo &pi, const void *items_any, b
         }
     }
     if (c->timing) {
-        if (planned_now) HIP_TRY(hipEventElapsedTime(&s.plan_ms, c->events[0], c->events[1]));
+        if (planned_now) HIP_TRY(hipEventElapsedTime(&s.plan_ms, c->events[0], c->events[c->plan_end]));
         HIP_TRY(hipEventElapsedTime(&s.total_ms, c->events[planned_now ? 0 : 2], c->events[2 + nl]));
     }
     c->last_nlaunch = pi.chain ? 0 : nl;              // per-launch traffic can only be inspected after launch-per-digit execution
@@ -459,7 +459,7 @@ static int try_strided(vc_comm *c, VcSched S, std::vector<VcLaunchInfo> &L, cons
     }
     VcListlessGuard guard = d.guard;
     guard.stage_cap = (int64_t)c->stage.cap - 64;
-    if (c->timing) { HIP_TRY(hipEventRecord(c->events[1], st)); HIP_TRY(hipEventRecord(c->events[2], st)); }
+    if (c->timing) HIP_TRY(hipEventRecord(c->events[2], st));
     c->h_header[VC_HEADER_STALLED] = 0;
     // the one launch of the call: its first wavefronts check the tables and add their totals up into `header`; every pair
     // checks its own entries and the length of its block before it forms an address, and stores nothing before all of
@@ -496,6 +496,9 @@ static int try_enqueued_list(vc_comm *c, const VcSched &S, std::vector<VcLaunchI
     guard.allowance = c->bound_staging ? c->staging_allowance : INT64_MAX;
     const int64_t guess = std::min<int64_t>(c->hint.items, guard.cap_items);
     if (!c->hint.valid || guess <= 0 || !c->B.chain_row_tot) return 2;
+    // with per-launch timing on the host keeps its look at the plan: an event between the list kernel and the copy kernel
+    // would sit in the stream's critical path (4 - 8 us a piece) and be counted as time of the copy kernel
+    if (c->timing) return 2;
     // a guess far above the call's real length costs a workgroup that starts and ends for every item there is not: only
     // while the communicator's calls stay of a kind (the last one no more than twice the one before)
     if (c->hint.items > 2 * c->items_before_last) return 2;
@@ -503,7 +506,7 @@ static int try_enqueued_list(vc_comm *c, const VcSched &S, std::vector<VcLaunchI
     const int lanes = vc_lanes_for_items(c->hint.payload, c->hint.items);
     HIP_TRY(vc_launch_chain_plan(S, T, c->B.slot_off, c->B.row_base, c->B.chain_row_tot + 2 * (size_t)S.P, c->desc.as<int64_t>(), guess, st,
                                  c->B.header, guard.cap_items));
-    if (c->timing) { HIP_TRY(hipEventRecord(c->events[1], st)); HIP_TRY(hipEventRecord(c->events[2], st)); }
+    if (c->timing) HIP_TRY(hipEventRecord(c->events[2], st));
     int64_t done = 0;                                     // items the guarded launch was sized for
     HIP_TRY(vc_launch_copy_chains_guarded(c->desc.as<int64_t>(), stride, guess, lanes, sendbuf, recvbuf, c->stage.as<char>(), st, c->B.header,
                                           guard, &done));
@@ -547,7 +550,8 @@ static int run_schedule(vc_comm *c, const CallParams &q, const char *sendbuf, ch
         for (int attempt = 0; attempt < 2 && !pi.listless; attempt++) {
             guard.stage_cap = c->stage.cap >= 64 ? (int64_t)c->stage.cap - 64 : 0;
             if (c->timing) {
-                if (attempt == 0) HIP_TRY(hipEventRecord(c->events[1], st));
+                // (the planning ended where the first attempt began: its event stays as events[1])
+                if (attempt == 1) { std::swap(c->events[1], c->events[2]); c->plan_end = 1; }
                 HIP_TRY(hipEventRecord(c->events[2], st));
             }
             HIP_TRY(vc_launch_copy_blocks(S, T, c->B.slot_off, c->B.row_base, c->B.header, guard, pair_lanes, sendbuf, recvbuf,
@@ -592,7 +596,7 @@ static int enqueue_async(vc_comm *c, const CallParams &q, const VcSched &S, std:
     hipStream_t st = c->stream;
     const int lanes = vc_dispatch(c->forward, VC_CALL_LISTLESS_ONLY, c->hint, S).lanes;
     const VcListlessGuard guard = {c->stage.cap >= 64 ? (int64_t)c->stage.cap - 64 : 0, 0, 0, 0, 0};
-    if (c->timing) { HIP_TRY(hipEventRecord(c->events[1], st)); HIP_TRY(hipEventRecord(c->events[2], st)); }
+    if (c->timing) HIP_TRY(hipEventRecord(c->events[2], st));
     HIP_TRY(vc_launch_copy_blocks(S, T, c->B.slot_off, c->B.row_base, c->B.header, guard, lanes, sendbuf, recvbuf, c->stage.as<char>(), st));
     if (c->timing) HIP_TRY(hipEventRecord(c->events[3], st));
     c->pending.active = true;
@@ -632,7 +636,11 @@ extern "C" int vc_comm_wait(vc_comm_t c) {
             return run_schedule(c, c->pending.q, c->pending.sendbuf, c->pending.recvbuf, c->pending.T, false, true);
         HIP_TRY(reserve_stage(c, (size_t)pi.stage_bytes + 64));
         guard.stage_cap = (int64_t)c->stage.cap - 64;
-        if (c->timing) HIP_TRY(hipEventRecord(c->events[2], c->stream));
+        if (c->timing) {
+            std::swap(c->events[1], c->events[2]);        // (the planning ended where the first attempt began)
+            c->plan_end = 1;
+            HIP_TRY(hipEventRecord(c->events[2], c->stream));
+        }
         HIP_TRY(vc_launch_copy_blocks(S, c->pending.T, c->B.slot_off, c->B.row_base, c->B.header, guard, c->pending.lanes,
                                       c->pending.sendbuf, c->pending.recvbuf, c->stage.as<char>(), c->stream));
         if (c->timing) HIP_TRY(hipEventRecord(c->events[3], c->stream));

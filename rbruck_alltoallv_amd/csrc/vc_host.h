@@ -81,6 +81,7 @@ struct vc_comm {
                                           // call suggests), 2 forwarded through a work-item list, 3 / 4 forwarded, listless with a
                                           // workgroup / a quarter of a wavefront per pair of ranks
     VcHint hint = {0, 0, 0, 0, 0};        // what the last forwarded call on this communicator looked like
+    int plan_end = 2;                     // which event marks the end of the planning kernels of the call in progress
     int waits = 0;                        // times the host has waited for the stream in the call in progress
     int64_t items_before_last = 0;        // block pieces of the forwarded call before the one `hint` describes (0: there was none)
     DevBuf chain_row_tot, chain_row_base;
