@@ -506,10 +506,14 @@ def main() -> None:
         t0 = time.perf_counter()
         kern_ms, phys_bytes, alg_bytes, nkern, plan_ms = 0.0, 0, 0, 0, 0.0
         per_launch_ms = None
+        every = []                                      # the statistics of every call; added up after the timed region
         for _ in range(steps):
             rc = call(api, func, tun, dp, send, recv)
             assert rc == 0, dp.comm.error()
-            st = dp.comm.last_stats()
+            every.append(dp.comm.last_stats())
+        torch.cuda.synchronize()
+        elapsed = time.perf_counter() - t0
+        for st in every:
             for k in range(st.n_launches):
                 kern_ms += st.launch_ms[k]
                 nkern += 1
@@ -519,8 +523,6 @@ def main() -> None:
             if st.n_launches <= 16:
                 now = [st.launch_ms[k] for k in range(st.n_launches)]
                 per_launch_ms = now if per_launch_ms is None else [a + b for a, b in zip(per_launch_ms, now)]
-        torch.cuda.synchronize()
-        elapsed = time.perf_counter() - t0
         st = dp.comm.last_stats()
         assert 2 * st.moved_bytes == A, (st.moved_bytes, A)
         assert st.payload_bytes == S
